@@ -1,0 +1,189 @@
+"""Pin the CPU oracle before anything is compared with it.
+
+The reference holds no golden vectors (its test file has no ``test_*`` functions and no data
+files); what pins results there is a live comparison with PyTorch math SDPA under forward-mode AD
+(reference ``tests/test_jvp_attention.py:548-561``, ``:595-597``).  So the oracle is pinned by
+(1) that same library route, (2) finite differences, which share nothing with autograd or with the
+closed form, (3) invariants of the mathematics, and (4) agreement of the tile-loop restatement with
+the dense closed form for several tile sizes, ragged L included.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dense, sdpa_jvp, tiled
+
+torch.manual_seed(0)
+
+
+def _inputs(Z=2, H=2, L=32, D=16, seed=0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(Z, H, L, D, generator=g, dtype=dtype) for _ in range(8)]
+
+
+def _masks(Z, H, L, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(L // 2, L + 1, (Z,), generator=g)
+    keypad = (torch.arange(L)[None, :] < lens[:, None]).view(Z, 1, 1, L)
+    bias = torch.randn(Z, H, L, L, generator=g, dtype=torch.float64)
+    rnd = torch.rand(Z, H, L, L, generator=g) > 0.7
+    rnd[..., 0] = True  # no fully masked row
+    return {"none": (None, False), "causal": (None, True), "keypad": (keypad, False),
+            "bias": (bias, False), "random_bool": (rnd, False)}
+
+
+MODES = ["none", "causal", "keypad", "bias", "random_bool"]
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_dense_matches_sdpa_library_route(mode):
+    q, k, v, qt, kt, vt, go, gt = _inputs()
+    mask, causal = _masks(2, 2, 32)[mode]
+    o, ot, grads = sdpa_jvp.forward_backward(q, k, v, qt, kt, vt, go, gt, attn_mask=mask, causal=causal)
+    npm = None if mask is None else mask.numpy()
+    f = dense.forward(*(x.numpy() for x in (q, k, v, qt, kt, vt)), mask=npm, causal=causal)
+    b = dense.backward(*(x.numpy() for x in (q, k, v, qt, kt, vt, go, gt)), mask=npm, causal=causal)
+    assert np.abs(f["O"] - o.numpy()).max() < 1e-12
+    assert np.abs(f["Ot"] - ot.numpy()).max() < 1e-12
+    for name, ref in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        assert np.abs(b[name] - ref.numpy()).max() < 1e-11, name
+    # gT = None is the reference's first-order backward
+    _, _, g1 = sdpa_jvp.forward_backward(q, k, v, qt, kt, vt, go, None, attn_mask=mask, causal=causal)
+    b1 = dense.backward(*(x.numpy() for x in (q, k, v, qt, kt, vt, go)), None, mask=npm, causal=causal)
+    for name, ref in zip(("dq", "dk", "dv"), g1):
+        assert np.abs(b1[name] - ref.numpy()).max() < 1e-11, name
+    for name in ("dqt", "dkt", "dvt"):
+        assert np.abs(b1[name]).max() == 0.0
+
+
+def test_dense_M_and_mu_definitions():
+    q, k, v, qt, kt, vt, _, _ = _inputs()
+    f = dense.forward(*(x.numpy() for x in (q, k, v, qt, kt, vt)))
+    s = (q @ k.transpose(-1, -2)) * q.shape[-1] ** -0.5
+    assert np.abs(f["M"] - (torch.logsumexp(s, -1) * dense.LOG2E).numpy()).max() < 1e-12
+    assert np.abs(f["P"].sum(-1) - 1).max() < 1e-12
+
+
+@pytest.mark.parametrize("mode", ["none", "causal", "bias"])
+def test_tangent_is_directional_derivative_by_finite_difference(mode):
+    q, k, v, qt, kt, vt, _, _ = [x.numpy() for x in _inputs(Z=1, H=1, L=32, D=8, seed=3)]
+    mask, causal = _masks(1, 1, 32)[mode]
+    npm = None if mask is None else mask.numpy()
+    eps = 1e-6
+    fp = dense.forward(q + eps * qt, k + eps * kt, v + eps * vt, mask=npm, causal=causal)["O"]
+    fm = dense.forward(q - eps * qt, k - eps * kt, v - eps * vt, mask=npm, causal=causal)["O"]
+    fd = (fp - fm) / (2 * eps)
+    ot = dense.forward(q, k, v, qt, kt, vt, mask=npm, causal=causal)["Ot"]
+    assert np.abs(fd - ot).max() < 1e-7
+
+
+@pytest.mark.parametrize("mode", ["none", "causal", "keypad"])
+def test_backward_by_brute_force_finite_difference(mode):
+    """d/dx [<gO,O> + <gT,O'>] entry by entry on a tiny problem; no autograd, no closed form."""
+    Z, H, L, D = 1, 1, 8, 4
+    xs = [x.numpy() for x in _inputs(Z, H, L, D, seed=5)]
+    q, k, v, qt, kt, vt, go, gt = xs
+    mask, causal = _masks(Z, H, L)[mode]
+    npm = None if mask is None else mask.numpy()
+
+    def loss(args):
+        f = dense.forward(*args, mask=npm, causal=causal)
+        return (f["O"] * go).sum() + (f["Ot"] * gt).sum()
+
+    b = dense.backward(q, k, v, qt, kt, vt, go, gt, mask=npm, causal=causal)
+    eps = 1e-6
+    for idx, name in enumerate(("dq", "dk", "dv", "dqt", "dkt", "dvt")):
+        fd = np.zeros_like(xs[idx])
+        for pos in np.ndindex(*xs[idx].shape):
+            args_p = [a.copy() for a in xs[:6]]
+            args_m = [a.copy() for a in xs[:6]]
+            args_p[idx][pos] += eps
+            args_m[idx][pos] -= eps
+            fd[pos] = (loss(args_p) - loss(args_m)) / (2 * eps)
+        assert np.abs(fd - b[name]).max() < 1e-7, name
+
+
+def test_invariants():
+    q, k, v, qt, kt, vt, go, gt = [x.numpy() for x in _inputs(seed=7)]
+    # rows of P' sum to zero: constant V and V' = 0 give O' = 0
+    f = dense.forward(q, k, np.ones_like(v) * 3.0, qt, kt, np.zeros_like(vt))
+    assert np.abs(f["Ot"]).max() < 1e-12
+    assert np.abs(f["Pp"].sum(-1)).max() < 1e-12
+    # O' is linear in the tangents
+    f1 = dense.forward(q, k, v, qt, kt, vt)["Ot"]
+    f2 = dense.forward(q, k, v, 2 * qt, 2 * kt, 2 * vt)["Ot"]
+    assert np.abs(f2 - 2 * f1).max() < 1e-12
+    fa = dense.forward(q, k, v, qt, 0 * kt, 0 * vt)["Ot"]
+    fb = dense.forward(q, k, v, 0 * qt, kt, 0 * vt)["Ot"]
+    fc = dense.forward(q, k, v, 0 * qt, 0 * kt, vt)["Ot"]
+    assert np.abs(fa + fb + fc - f1).max() < 1e-12
+    # V' only: O' = P V'
+    assert np.abs(fc - dense.forward(q, k, vt)["O"]).max() < 1e-12
+    # single key attended (L=1 effectively via mask): O = V row, O' = V' row
+    L = q.shape[-2]
+    only0 = np.zeros((1, 1, L, L), dtype=bool)
+    only0[..., 0] = True
+    f0 = dense.forward(q, k, v, qt, kt, vt, mask=only0)
+    assert np.abs(f0["O"] - v[:, :, :1]).max() < 1e-12
+    assert np.abs(f0["Ot"] - vt[:, :, :1]).max() < 1e-12
+    # dV' = P^T gT is the transpose-action of O' = ... + P V'
+    b = dense.backward(q, k, v, qt, kt, vt, go, gt)
+    P = dense.forward(q, k, v)["P"]
+    assert np.abs(b["dvt"] - np.swapaxes(P, -1, -2) @ gt).max() < 1e-12
+
+
+def test_fully_masked_rows_give_zeros():
+    q, k, v, qt, kt, vt, go, gt = [x.numpy() for x in _inputs(Z=1, H=1, L=16, D=8, seed=9)]
+    mask = np.ones((1, 1, 16, 16), dtype=bool)
+    mask[0, 0, 3, :] = False
+    f = dense.forward(q, k, v, qt, kt, vt, mask=mask)
+    assert np.all(f["O"][0, 0, 3] == 0) and np.all(f["Ot"][0, 0, 3] == 0)
+    assert np.isposinf(f["M"][0, 0, 3])
+    b = dense.backward(q, k, v, qt, kt, vt, go, gt, mask=mask)
+    assert np.all(b["dq"][0, 0, 3] == 0) and np.all(np.isfinite(b["dk"]))
+    o, ot, M, mu = tiled.forward(*(torch.from_numpy(x) for x in (q, k, v, qt, kt, vt)),
+                                 mask=torch.from_numpy(mask), bm=8, bn=8)
+    assert torch.all(o[0, 0, 3] == 0) and torch.all(ot[0, 0, 3] == 0) and math.isinf(M[0, 0, 3])
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("L,bm,bn", [(32, 32, 32), (64, 32, 16), (64, 16, 64), (40, 16, 32), (96, 64, 32)])
+def test_tiled_matches_dense(mode, L, bm, bn):
+    Z, H, D = 2, 2, 16
+    q, k, v, qt, kt, vt, go, gt = _inputs(Z, H, L, D, seed=11)
+    mask, causal = _masks(Z, H, L)[mode]
+    npm = None if mask is None else mask.numpy()
+    f = dense.forward(*(x.numpy() for x in (q, k, v, qt, kt, vt)), mask=npm, causal=causal)
+    o, ot, M, mu = tiled.forward(q, k, v, qt, kt, vt, mask=mask, causal=causal, bm=bm, bn=bn)
+    assert np.abs(o.numpy() - f["O"]).max() < 1e-12
+    assert np.abs(ot.numpy() - f["Ot"]).max() < 1e-11
+    assert np.abs(M.numpy() - f["M"]).max() < 1e-12
+    assert np.abs(mu.numpy() - f["mu"]).max() < 1e-12
+    b = dense.backward(*(x.numpy() for x in (q, k, v, qt, kt, vt, go, gt)), mask=npm, causal=causal)
+    g = tiled.backward(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask=mask, causal=causal, bm=bm, bn=bn)
+    for name in b:
+        assert np.abs(g[name].numpy() - b[name]).max() < 1e-11, name
+    # plain forward + first-order backward (tangent-free path)
+    o1, none_t, M1, none_mu = tiled.forward(q, k, v, mask=mask, causal=causal, bm=bm, bn=bn)
+    assert none_t is None and none_mu is None and torch.equal(o1, o)
+    g1 = tiled.backward(q, k, v, None, None, None, o1, None, M1, None, go, None, mask=mask,
+                        causal=causal, bm=bm, bn=bn)
+    b1 = dense.backward(*(x.numpy() for x in (q, k, v)), None, None, None, go.numpy(), None,
+                        mask=npm, causal=causal)
+    for name in ("dq", "dk", "dv"):
+        assert np.abs(g1[name].numpy() - b1[name]).max() < 1e-11, name
+
+
+def test_config1_cpu_plumbing_fp32():
+    """BASELINE config 1: fp32 B2 H4 L128 D64, seed 0, N(0,1); SDPA route vs tiled restatement."""
+    g = torch.Generator().manual_seed(0)
+    q, k, v, qt, kt, vt, go, gt = [torch.randn(2, 4, 128, 64, generator=g) for _ in range(8)]
+    o_ref, ot_ref, grads = sdpa_jvp.forward_backward(q, k, v, qt, kt, vt, go, gt)
+    o, ot, M, mu = tiled.forward(q, k, v, qt, kt, vt)
+    gr = tiled.backward(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt)
+    assert (o - o_ref).abs().max() < 1e-5
+    assert (ot - ot_ref).abs().max() < 1e-4
+    for name, ref in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        assert (gr[name] - ref).abs().max() < 2e-4 * max(1.0, ref.abs().max().item()), name
