@@ -1,0 +1,122 @@
+/*
+ * jvpfa.h -- C ABI of the MI355X (gfx950) JVP flash-attention kernels.
+ *
+ * Plain pointers and sizes only; no torch types.  Every entry point is
+ * stateless, launches asynchronously on the HIP stream it is given, owns no
+ * memory and allocates none: the caller passes every input, output and
+ * workspace buffer as a device pointer.  Return value: 0 on success, a
+ * negative JVPFA_E_* code otherwise (jvpfa_error_string() names it).  Safe to
+ * call from any thread; two calls that write the same buffers race.
+ *
+ * Tensors q, k, v, their tangents, outputs and gradients are dense row-major
+ * (Z, H, L, D); row statistics are fp32 (Z, H, L).  The mask, when present,
+ * is addressed with four element strides (0 = broadcast along that axis), so
+ * a key-padding mask of shape [Z,1,1,L] is read in place.
+ *
+ * Each function names the part of the reference
+ * (jvp_flash_attention/jvp_attention.py, "JA") whose device work it replaces.
+ */
+#ifndef JVPFA_H
+#define JVPFA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JVPFA_ABI_VERSION 1
+
+enum jvpfa_dtype { JVPFA_BF16 = 0, JVPFA_FP16 = 1, JVPFA_FP32 = 2 };
+
+/* JA:2429-2446 classifies masks as 0 none / 1 boolean / 2 additive float. */
+enum jvpfa_mask_kind { JVPFA_MASK_NONE = 0, JVPFA_MASK_BOOL = 1, JVPFA_MASK_ADD = 2 };
+
+enum jvpfa_status {
+  JVPFA_OK = 0,
+  JVPFA_E_NULL = -1,      /* a required pointer is NULL */
+  JVPFA_E_SHAPE = -2,     /* Z,H,L < 1, or D not in {32, 64, 128} */
+  JVPFA_E_DTYPE = -3,     /* dtype / mask_kind out of range */
+  JVPFA_E_ALIGN = -4,     /* a tensor pointer is not 16-byte aligned */
+  JVPFA_E_CONFLICT = -5,  /* causal together with a mask (JA:2380-2381 raises ValueError) */
+  JVPFA_E_LAUNCH = -6,    /* hipGetLastError() reported a launch failure */
+  JVPFA_E_ABI = -7        /* struct_size does not match this library */
+};
+
+/* Shape, numeric type and masking shared by forward and backward. */
+typedef struct jvpfa_problem {
+  int32_t Z, H, L, D;
+  int32_t dtype;      /* enum jvpfa_dtype: element type of q,k,v,o and their tangents/gradients */
+  int32_t causal;     /* 0/1; lower-triangular (query index >= key index), JA:253-258 */
+  int32_t mask_kind;  /* enum jvpfa_mask_kind */
+  float sm_scale;     /* logits = sm_scale * q.k (+ additive mask); JA:2395-2396 default D^-0.5 */
+  const void *mask;   /* bool: uint8, nonzero = attend (JA:241-245); additive: same dtype as q,
+                         added to the scaled logits (SDPA semantics) */
+  int64_t mask_stride[4]; /* element strides over (z, h, query, key); 0 broadcasts */
+} jvpfa_problem;
+
+/*
+ * Fused dual forward.  Replaces the device work of JA:662-1033 (_attn_fwd) with
+ * its inner loop JA:125-336, launched from JVPAttn.forward (JA:2592-2631).
+ * With qt = kt = vt = NULL it is the plain forward (ENABLE_JVP False, JA:2365)
+ * and ot / mu may be NULL.
+ *   o  = softmax(S) v
+ *   ot = (P * (S' - mu)) v + P vt,   S' = sm_scale (qt k^T + q kt^T)
+ *   M  = log2-domain log-sum-exp of S per query row (JA:1017-1022); +inf for a row
+ *        with every key masked (such rows give o = ot = 0, JA:1011-1015)
+ *   mu = rowsum(P * S'), saved for the backward (the reference does not keep it)
+ */
+typedef struct jvpfa_fwd_args {
+  uint32_t struct_size; /* sizeof(jvpfa_fwd_args) */
+  jvpfa_problem p;
+  const void *q, *k, *v;
+  const void *qt, *kt, *vt; /* all three NULL, or all three set */
+  void *o, *ot;
+  float *M, *mu;
+} jvpfa_fwd_args;
+
+int jvpfa_fwd(const jvpfa_fwd_args *args, void *hip_stream);
+
+/*
+ * Backward of  Loss = <go, o> + <gt, ot>.  Replaces the device work of
+ * _attn_bwd_preprocess (JA:1384-1411), _attn_bwd / _attn_bwd_causal
+ * (JA:2008-2233, JA:1710-2005) with their inner loops JA:1415-1707, launched
+ * from JVPAttn.backward (JA:2921-2974), and adds the gradient through the
+ * tangent output, which the reference lacks (JA:2831 ignores its second
+ * incoming gradient).
+ *   gt == NULL            first-order backward: needs q,k,v,o,M,go -> dq,dk,dv
+ *                         (tangent pointers and ot, mu may be NULL)
+ *   gt != NULL            needs all of q,k,v,qt,kt,vt,o,ot,M,mu; go may be NULL (= 0)
+ *   dqt,dkt,dvt           optional outputs (all NULL or all set; need gt != NULL):
+ *                         gradients w.r.t. the tangent inputs
+ * workspace: jvpfa_bwd_workspace_bytes(Z,H,L) bytes of device memory, 16-byte
+ * aligned, contents don't-care on entry (row statistics of the pre-pass).
+ */
+typedef struct jvpfa_bwd_args {
+  uint32_t struct_size; /* sizeof(jvpfa_bwd_args) */
+  jvpfa_problem p;
+  const void *q, *k, *v;
+  const void *qt, *kt, *vt;
+  const void *o, *ot;
+  const float *M, *mu;
+  const void *go, *gt;
+  void *dq, *dk, *dv;
+  void *dqt, *dkt, *dvt;
+  void *workspace;
+} jvpfa_bwd_args;
+
+int jvpfa_bwd(const jvpfa_bwd_args *args, void *hip_stream);
+
+size_t jvpfa_bwd_workspace_bytes(int32_t Z, int32_t H, int32_t L);
+
+/* JVPFA_ABI_VERSION of the loaded library. */
+int jvpfa_abi_version(void);
+
+/* Static, NUL-terminated description of a jvpfa_status value. */
+const char *jvpfa_error_string(int status);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JVPFA_H */

@@ -1,0 +1,7 @@
+"""Drop-in import path of the reference (``jvp_flash_attention.jvp_attention``)."""
+from jvp_flash_attention_amd.jvp_attention import (  # noqa: F401
+    MASK_CONST,
+    MIN_SEQUENCE_LENGTH,
+    JVPAttn,
+    attention,
+)

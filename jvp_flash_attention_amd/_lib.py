@@ -1,0 +1,185 @@
+"""ctypes binding of ``libjvpfa.so`` (the C ABI declared in ``include/jvpfa.h``).
+
+The library is loaded after ``import torch`` so that the HIP runtime torch already mapped is the
+one the kernels launch on.  There is no fallback: if the library is missing, or a tensor is not
+on a GPU, the call raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libjvpfa.so")
+
+ABI_VERSION = 1
+DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
+EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_bwd_workspace_bytes", "jvpfa_abi_version", "jvpfa_error_string")
+
+
+class Problem(C.Structure):
+    _fields_ = [
+        ("Z", C.c_int32), ("H", C.c_int32), ("L", C.c_int32), ("D", C.c_int32),
+        ("dtype", C.c_int32), ("causal", C.c_int32), ("mask_kind", C.c_int32),
+        ("sm_scale", C.c_float),
+        ("mask", C.c_void_p),
+        ("mask_stride", C.c_int64 * 4),
+    ]
+
+
+class FwdArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("p", Problem),
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p),
+        ("qt", C.c_void_p), ("kt", C.c_void_p), ("vt", C.c_void_p),
+        ("o", C.c_void_p), ("ot", C.c_void_p),
+        ("M", C.c_void_p), ("mu", C.c_void_p),
+    ]
+
+
+class BwdArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("p", Problem),
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p),
+        ("qt", C.c_void_p), ("kt", C.c_void_p), ("vt", C.c_void_p),
+        ("o", C.c_void_p), ("ot", C.c_void_p),
+        ("M", C.c_void_p), ("mu", C.c_void_p),
+        ("go", C.c_void_p), ("gt", C.c_void_p),
+        ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
+        ("dqt", C.c_void_p), ("dkt", C.c_void_p), ("dvt", C.c_void_p),
+        ("workspace", C.c_void_p),
+    ]
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m jvp_flash_attention_amd.build` "
+                "(there is no non-HIP fallback)"
+            )
+        lib = C.CDLL(LIB_PATH)
+        lib.jvpfa_fwd.argtypes = [C.POINTER(FwdArgs), C.c_void_p]
+        lib.jvpfa_fwd.restype = C.c_int
+        lib.jvpfa_bwd.argtypes = [C.POINTER(BwdArgs), C.c_void_p]
+        lib.jvpfa_bwd.restype = C.c_int
+        lib.jvpfa_bwd_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+        lib.jvpfa_bwd_workspace_bytes.restype = C.c_size_t
+        lib.jvpfa_abi_version.argtypes = []
+        lib.jvpfa_abi_version.restype = C.c_int
+        lib.jvpfa_error_string.argtypes = [C.c_int]
+        lib.jvpfa_error_string.restype = C.c_char_p
+        if lib.jvpfa_abi_version() != ABI_VERSION:
+            raise RuntimeError("libjvpfa.so ABI version mismatch; rebuild the library")
+        _lib = lib
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        msg = load().jvpfa_error_string(status).decode()
+        raise RuntimeError(f"libjvpfa: {msg} (status {status})")
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def make_problem(q, mask, mask_kind, causal, sm_scale) -> Problem:
+    Z, H, L, D = q.shape
+    p = Problem()
+    p.Z, p.H, p.L, p.D = Z, H, L, D
+    p.dtype = DTYPES[q.dtype]
+    p.causal = int(bool(causal))
+    p.mask_kind = mask_kind
+    p.sm_scale = float(sm_scale)
+    if mask_kind != MASK_NONE:
+        p.mask = mask.data_ptr()
+        # a size-1 axis broadcasts, whatever stride torch reports for it
+        strides = [0 if mask.shape[i] == 1 else mask.stride(i) for i in range(4)]
+        p.mask_stride = (C.c_int64 * 4)(*strides)
+    else:
+        p.mask = None
+        p.mask_stride = (C.c_int64 * 4)(0, 0, 0, 0)
+    return p
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "jvp_flash_attention_amd runs on an AMD GPU only (HIP kernels); got a tensor on "
+                f"{t.device}.  There is no CPU path."
+            )
+
+
+def _stream(t) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class HipBackend:
+    """Device work of the forward and the backward, through the C ABI."""
+
+    name = "hip"
+
+    def fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
+        """Returns (o, ot, M, mu); ot and mu are None for a plain forward."""
+        _require_gpu(q, k, v, qt, kt, vt, mask)
+        lib = load()
+        dual = qt is not None
+        o = torch.empty_like(q)
+        ot = torch.empty_like(q) if dual else None
+        Z, H, L, _ = q.shape
+        M = torch.empty((Z, H, L), device=q.device, dtype=torch.float32)
+        mu = torch.empty((Z, H, L), device=q.device, dtype=torch.float32) if dual else None
+        a = FwdArgs()
+        a.struct_size = C.sizeof(FwdArgs)
+        a.p = make_problem(q, mask, mask_kind, causal, sm_scale)
+        a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
+        a.qt, a.kt, a.vt = _ptr(qt), _ptr(kt), _ptr(vt)
+        a.o, a.ot, a.M, a.mu = _ptr(o), _ptr(ot), _ptr(M), _ptr(mu)
+        with torch.cuda.device(q.device):
+            check(lib.jvpfa_fwd(C.byref(a), _stream(q)))
+        return o, ot, M, mu
+
+    def bwd(self, q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
+            want_tangent_grads=False):
+        """Returns (dq, dk, dv, dqt, dkt, dvt); the last three are None unless requested."""
+        _require_gpu(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask)
+        lib = load()
+        Z, H, L, _ = q.shape
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dqt = dkt = dvt = None
+        if want_tangent_grads:
+            dqt, dkt, dvt = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        ws = torch.empty(lib.jvpfa_bwd_workspace_bytes(Z, H, L), device=q.device, dtype=torch.uint8)
+        a = BwdArgs()
+        a.struct_size = C.sizeof(BwdArgs)
+        a.p = make_problem(q, mask, mask_kind, causal, sm_scale)
+        a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
+        a.qt, a.kt, a.vt = _ptr(qt), _ptr(kt), _ptr(vt)
+        a.o, a.ot, a.M, a.mu = _ptr(o), _ptr(ot), _ptr(M), _ptr(mu)
+        a.go, a.gt = _ptr(go), _ptr(gt)
+        a.dq, a.dk, a.dv = _ptr(dq), _ptr(dk), _ptr(dv)
+        a.dqt, a.dkt, a.dvt = _ptr(dqt), _ptr(dkt), _ptr(dvt)
+        a.workspace = _ptr(ws)
+        with torch.cuda.device(q.device):
+            check(lib.jvpfa_bwd(C.byref(a), _stream(q)))
+        return dq, dk, dv, dqt, dkt, dvt
+
+
+_backend = HipBackend()
+
+
+def backend():
+    return _backend

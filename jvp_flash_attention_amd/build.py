@@ -1,0 +1,76 @@
+"""Build ``libjvpfa.so`` (HIP kernels + C ABI) in-tree for gfx950 with hipcc.
+
+``python -m jvp_flash_attention_amd.build`` compiles every translation unit (one per element
+type x head dim for the forward and for the backward, plus the C ABI files) in parallel and
+links them into ``jvp_flash_attention_amd/libjvpfa.so``.  hipcc cross-compiles, so no GPU is
+needed to build.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(CSRC, "build")
+LIB = os.path.join(HERE, "libjvpfa.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wno-unused-value",
+    # keep hipcc from forming packed-fp32 VALU ops out of scalar float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+TYPES = {"bf16": "__bf16", "fp16": "_Float16", "fp32": "float"}
+DIMS = (32, 64, 128)
+
+
+def units():
+    """(object name, source, extra defines) for every translation unit."""
+    out = []
+    for kind in ("fwd", "bwd"):
+        src = os.path.join(CSRC, f"{kind}_inst.hip")
+        if not os.path.exists(src):
+            continue
+        for tag, ctype in TYPES.items():
+            for d in DIMS:
+                name = f"{kind}_{tag}_{d}"
+                out.append((name, src, [f"-DJVPFA_T={ctype}", f"-DJVPFA_D={d}", f"-DJVPFA_NAME={name}"]))
+    for api in ("api_fwd", "api_bwd"):
+        src = os.path.join(CSRC, f"{api}.hip")
+        if os.path.exists(src):
+            out.append((api, src, []))
+    return out
+
+
+def _compile(unit):
+    name, src, defs = unit
+    obj = os.path.join(OBJ, name + ".o")
+    cmd = [HIPCC, *FLAGS, *defs, "-c", src, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {name}:\n{' '.join(cmd)}\n{r.stderr[-4000:]}")
+    return obj
+
+
+def build(jobs: int | None = None, verbose: bool = True) -> str:
+    os.makedirs(OBJ, exist_ok=True)
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    us = units()
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(_compile, us))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
+    if verbose:
+        print(f"built {LIB} from {len(objs)} objects", flush=True)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

@@ -1,0 +1,41 @@
+// Argument validation shared by the C ABI entry points.
+#pragma once
+#include <stdint.h>
+
+#include "../../include/jvpfa.h"
+#include "params.hpp"
+
+namespace jvpfa {
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int check_problem(const jvpfa_problem &p) {
+  if (p.Z < 1 || p.H < 1 || p.L < 1) return JVPFA_E_SHAPE;
+  if (p.D != 32 && p.D != 64 && p.D != 128) return JVPFA_E_SHAPE;
+  if (p.dtype < JVPFA_BF16 || p.dtype > JVPFA_FP32) return JVPFA_E_DTYPE;
+  if (p.mask_kind < JVPFA_MASK_NONE || p.mask_kind > JVPFA_MASK_ADD) return JVPFA_E_DTYPE;
+  if (p.mask_kind != JVPFA_MASK_NONE) {
+    if (p.causal) return JVPFA_E_CONFLICT;
+    if (!p.mask) return JVPFA_E_NULL;
+    for (int i = 0; i < 4; ++i)
+      if (p.mask_stride[i] < 0) return JVPFA_E_SHAPE;
+  }
+  return JVPFA_OK;
+}
+
+inline Problem to_problem(const jvpfa_problem &p) {
+  Problem r;
+  r.Z = p.Z;
+  r.H = p.H;
+  r.L = p.L;
+  r.causal = p.causal ? 1 : 0;
+  r.scale = p.sm_scale;
+  r.mask = p.mask_kind == JVPFA_MASK_NONE ? nullptr : p.mask;
+  for (int i = 0; i < 4; ++i) r.ms[i] = p.mask_kind == JVPFA_MASK_NONE ? 0 : p.mask_stride[i];
+  return r;
+}
+
+// 0..8: (dtype, head-dim) slot in the launcher tables.
+inline int slot(const jvpfa_problem &p) { return p.dtype * 3 + (p.D == 32 ? 0 : p.D == 64 ? 1 : 2); }
+
+}  // namespace jvpfa

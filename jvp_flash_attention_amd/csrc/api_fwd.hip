@@ -1,0 +1,55 @@
+// C ABI: jvpfa_fwd and the small query functions.
+#include <hip/hip_runtime.h>
+
+#include "api_common.hpp"
+
+namespace jvpfa {
+#define JVPFA_DECL(name) int name(const FwdParams &, bool, int, hipStream_t);
+JVPFA_DECL(fwd_bf16_32) JVPFA_DECL(fwd_bf16_64) JVPFA_DECL(fwd_bf16_128)
+JVPFA_DECL(fwd_fp16_32) JVPFA_DECL(fwd_fp16_64) JVPFA_DECL(fwd_fp16_128)
+JVPFA_DECL(fwd_fp32_32) JVPFA_DECL(fwd_fp32_64) JVPFA_DECL(fwd_fp32_128)
+#undef JVPFA_DECL
+typedef int (*fwd_launcher)(const FwdParams &, bool, int, hipStream_t);
+static const fwd_launcher kFwd[9] = {fwd_bf16_32, fwd_bf16_64, fwd_bf16_128, fwd_fp16_32, fwd_fp16_64,
+                                     fwd_fp16_128, fwd_fp32_32, fwd_fp32_64, fwd_fp32_128};
+}  // namespace jvpfa
+
+using namespace jvpfa;
+
+extern "C" int jvpfa_fwd(const jvpfa_fwd_args *a, void *hip_stream) {
+  if (!a) return JVPFA_E_NULL;
+  if (a->struct_size != sizeof(jvpfa_fwd_args)) return JVPFA_E_ABI;
+  int rc = check_problem(a->p);
+  if (rc != JVPFA_OK) return rc;
+  if (!a->q || !a->k || !a->v || !a->o || !a->M) return JVPFA_E_NULL;
+  const int ntan = (a->qt != nullptr) + (a->kt != nullptr) + (a->vt != nullptr);
+  if (ntan != 0 && ntan != 3) return JVPFA_E_NULL;
+  const bool dual = ntan == 3;
+  if (dual && (!a->ot || !a->mu)) return JVPFA_E_NULL;
+  const void *ptrs[] = {a->q, a->k, a->v, a->qt, a->kt, a->vt, a->o, a->ot};
+  for (const void *ptr : ptrs)
+    if (ptr && !aligned16(ptr)) return JVPFA_E_ALIGN;
+
+  FwdParams p;
+  p.pr = to_problem(a->p);
+  p.q = a->q; p.k = a->k; p.v = a->v;
+  p.qt = a->qt; p.kt = a->kt; p.vt = a->vt;
+  p.o = a->o; p.ot = a->ot; p.M = a->M; p.mu = a->mu;
+  return kFwd[slot(a->p)](p, dual, a->p.mask_kind, static_cast<hipStream_t>(hip_stream));
+}
+
+extern "C" int jvpfa_abi_version(void) { return JVPFA_ABI_VERSION; }
+
+extern "C" const char *jvpfa_error_string(int status) {
+  switch (status) {
+    case JVPFA_OK: return "ok";
+    case JVPFA_E_NULL: return "a required pointer is NULL";
+    case JVPFA_E_SHAPE: return "unsupported shape (Z,H,L >= 1 and D in {32,64,128} required)";
+    case JVPFA_E_DTYPE: return "dtype or mask kind out of range";
+    case JVPFA_E_ALIGN: return "tensor pointer not 16-byte aligned";
+    case JVPFA_E_CONFLICT: return "causal attention does not take a mask";
+    case JVPFA_E_LAUNCH: return "HIP kernel launch failed";
+    case JVPFA_E_ABI: return "struct_size does not match this library";
+  }
+  return "unknown status";
+}

@@ -1,0 +1,48 @@
+// One translation unit per (element type, head dim): compiled with
+//   -DJVPFA_T=<__bf16|_Float16|float> -DJVPFA_D=<32|64|128> -DJVPFA_NAME=<symbol>
+// and exporting  int JVPFA_NAME(const BwdParams&, int mask_kind, bool dual, bool tangent_grads,
+// hipStream_t): pre-pass, then the dq and dk/dv kernels of every requested mode.
+#include "bwd_kernel.hpp"
+#include "launch.hpp"
+
+namespace jvpfa {
+
+template <typename T, int D, int MODE, int MASK>
+static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
+  using Cfg = BwdCfg<T, D, MODE>;
+  const int nb = (p.pr.L + BWD_BLK - 1) / BWD_BLK;
+  const long long blocks = (long long)nb * p.pr.Z * p.pr.H;
+  if (blocks > 0x7fffffffLL) return -2;
+  auto kq = bwd_dq_kernel<T, D, MODE, MASK>;
+  auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK>;
+  int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);
+  if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg::DKV_LDS);
+  if (rc != 0) return rc;
+  hipLaunchKernelGGL(kkv, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+  hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DQ_LDS, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : -6;
+}
+
+template <typename T, int D, int MASK>
+static int launch_bwd_mask(const BwdParams &p, bool dual, bool tangent_grads, hipStream_t stream) {
+  const long long rows = (long long)p.pr.Z * p.pr.H * p.pr.L;
+  constexpr int RPB = BWD_NT / (D / 8);
+  hipLaunchKernelGGL((bwd_prepass_kernel<T, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(BWD_NT), 0,
+                     stream, p, rows, dual ? 1 : 0);
+  if (hipGetLastError() != hipSuccess) return -6;
+  if (!dual) return launch_bwd_mode<T, D, BWD_PLAIN, MASK>(p, stream);
+  int rc = launch_bwd_mode<T, D, BWD_DUAL, MASK>(p, stream);
+  if (rc == 0 && tangent_grads) rc = launch_bwd_mode<T, D, BWD_TANGENT, MASK>(p, stream);
+  return rc;
+}
+
+int JVPFA_NAME(const BwdParams &p, int mask, bool dual, bool tangent_grads, hipStream_t stream) {
+  switch (mask) {
+    case MASK_NONE: return launch_bwd_mask<JVPFA_T, JVPFA_D, MASK_NONE>(p, dual, tangent_grads, stream);
+    case MASK_BOOL: return launch_bwd_mask<JVPFA_T, JVPFA_D, MASK_BOOL>(p, dual, tangent_grads, stream);
+    case MASK_ADD: return launch_bwd_mask<JVPFA_T, JVPFA_D, MASK_ADD>(p, dual, tangent_grads, stream);
+  }
+  return -3;
+}
+
+}  // namespace jvpfa

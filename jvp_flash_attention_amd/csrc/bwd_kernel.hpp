@@ -1,0 +1,441 @@
+// Backward kernels for  Loss = <gO, O> + <gT, O'>  with P recomputed from the saved
+// log-sum-exp M (and mu for the tangent path).
+//
+//   prepass   d1 = rowsum(gO*O), a = rowsum(gT*O), d2 = rowsum(gT*O') - a*mu
+//   dq        one workgroup per 128 query rows, loop over key tiles
+//   dkdv      one workgroup per 128 key rows, loop over query tiles
+//
+// Replaces the reference's _attn_bwd_preprocess (jvp_attention.py:1384-1411), _attn_bwd_dq
+// (:1567-1707) and _attn_bwd_dkdv (:1415-1563), which handle gO only; the gT terms follow
+//   dS' = P*(A - a),  dS = P*(gO V^T - d1 + B + A*(S' - mu) - a*S' - d2),  P' = P*(S' - mu)
+//   A = gT V^T,  B = gT V'^T
+//   dQ = s(dS K + dS' K'), dK = s(dS^T Q + dS'^T Q'), dV = P^T gO + P'^T gT
+//   dQ' = s dS' K,         dK' = s dS'^T Q,           dV' = P^T gT          (s = sm_scale)
+// Unlike the reference (:1519-1522, :1669-1671) an additive mask is part of the recomputed
+// logits.
+#pragma once
+#include "common.hpp"
+#include "mask.hpp"
+#include "params.hpp"
+
+namespace jvpfa {
+
+constexpr int BWD_NT = 256;
+constexpr int BWD_BLK = 128;  // rows owned by a workgroup (32 per wave)
+constexpr int BWD_T = 32;     // rows of the streamed tile
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void bwd_prepass_kernel(const BwdParams p, long long rows, int dual) {
+  constexpr int LPR = D / 8;  // lanes per row, 8 elements each
+  const long long row = (long long)blockIdx.x * (BWD_NT / LPR) + threadIdx.x / LPR;
+  const int part = threadIdx.x % LPR;
+  float s1 = 0.f, sa = 0.f, s2 = 0.f;
+  if (row < rows) {
+    const size_t off = (size_t)row * D + part * 8;
+    Frag<T> o = ld8<T>(reinterpret_cast<const T *>(p.o) + off);
+    if (p.go) {
+      Frag<T> go = ld8<T>(reinterpret_cast<const T *>(p.go) + off);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s1 += (float)go[e] * (float)o[e];
+    }
+    if (dual) {
+      Frag<T> gt = ld8<T>(reinterpret_cast<const T *>(p.gt) + off);
+      Frag<T> ot = ld8<T>(reinterpret_cast<const T *>(p.ot) + off);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        sa += (float)gt[e] * (float)o[e];
+        s2 += (float)gt[e] * (float)ot[e];
+      }
+    }
+  }
+#pragma unroll
+  for (int w = LPR / 2; w >= 1; w /= 2) {
+    s1 += __shfl_xor(s1, w, 64);
+    sa += __shfl_xor(sa, w, 64);
+    s2 += __shfl_xor(s2, w, 64);
+  }
+  if (row < rows && part == 0) {
+    p.d1[row] = s1;
+    if (dual) {
+      p.a[row] = sa;
+      p.d2[row] = s2 - sa * p.mu[row];
+    }
+  }
+}
+
+template <typename T, int D, int MODE> struct BwdCfg {
+  static constexpr int PAD = 16 / sizeof(T);
+  static constexpr int LDN = D + PAD;       // row-major streamed tiles (32 x D)
+  static constexpr int LDT = BWD_T + PAD;   // transposed streamed tiles (D x 32)
+  static constexpr int N_ELEMS = BWD_T * LDN;
+  static constexpr int T_ELEMS = D * LDT;
+  // dq:   PLAIN K,V,K^T | DUAL K,K',V,V',K^T,K'^T | TANGENT K,V,K^T
+  // dkdv: PLAIN Q,gO,Q^T,gO^T | DUAL Q,Q',gO,gT + 4 transposed | TANGENT Q,gT,Q^T,gT^T
+  static constexpr int DQ_NAT = MODE == BWD_DUAL ? 4 : 2;
+  static constexpr int DQ_TR = MODE == BWD_DUAL ? 2 : 1;
+  static constexpr int DKV_NAT = MODE == BWD_DUAL ? 4 : 2;
+  static constexpr int DKV_TR = MODE == BWD_DUAL ? 4 : 2;
+  static constexpr size_t DQ_LDS = (size_t)(DQ_NAT * N_ELEMS + DQ_TR * T_ELEMS) * sizeof(T);
+  static constexpr size_t DKV_LDS = (size_t)(DKV_NAT * N_ELEMS + DKV_TR * T_ELEMS) * sizeof(T) + 5 * BWD_T * sizeof(float);
+};
+
+template <int KK, typename T>
+__device__ __forceinline__ void load_row_frags(Frag<T> *f, const T *row, int g) {
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) f[kk] = ld8<T>(row + 16 * kk + 8 * g);
+}
+
+template <int KK, typename T>
+__device__ __forceinline__ void gemm_tile(f32x16 &acc, const T *tile, int ld, int arow, int g, const Frag<T> *b) {
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) mma(acc, lds_frag(tile + arow * ld + 16 * kk + 8 * g), b[kk]);
+}
+
+__device__ __forceinline__ void zero16(f32x16 &x) {
+#pragma unroll
+  for (int e = 0; e < 16; ++e) x[e] = 0.f;
+}
+
+// ------------------------------------------------------------------------------------------------
+// dq (MODE PLAIN / DUAL) or dq' (MODE TANGENT).  Scores are transposed (lane = query), as in the
+// forward, so ds is already the B operand of dQ^T += K^T dS^T.
+template <typename T, int D, int MODE, int MASK>
+__global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
+  using Cfg = BwdCfg<T, D, MODE>;
+  constexpr int KK = D / 16, DB = D / 32;
+  constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
+  constexpr float NEG_INF = -__builtin_inff();
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T *Kn = reinterpret_cast<T *>(smem_raw);
+  T *Vn = Kn + Cfg::N_ELEMS;
+  T *KT = Vn + Cfg::N_ELEMS;
+  T *Ktn = KT + Cfg::T_ELEMS;     // DUAL only from here on
+  T *Vtn = Ktn + Cfg::N_ELEMS;
+  T *KtT = Vtn + Cfg::N_ELEMS;
+
+  const Problem &pr = p.pr;
+  const int L = pr.L;
+  const int nqb = (L + BWD_BLK - 1) / BWD_BLK;
+  const int total = nqb * pr.Z * pr.H;
+  const int id = xcd_remap(blockIdx.x, total);
+  const int zh = id / nqb;
+  const int qb = pr.causal ? nqb - 1 - id % nqb : id % nqb;
+  const int z = zh / pr.H, h = zh % pr.H;
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 32, g = lane / 32, pr32 = perm32(r);
+
+  const size_t head = (size_t)zh * L * D;
+  const size_t srow = (size_t)zh * L;
+  const int q0 = qb * BWD_BLK;
+  const int qrow = q0 + wave * 32 + r;
+  const int qld = qrow < L ? qrow : L - 1;
+  const bool has_go = p.go != nullptr;
+
+  Frag<T> Qf[KK], gOf[TAN ? 1 : KK], Qtf[DUAL ? KK : 1], gTf[(DUAL || TAN) ? KK : 1];
+  load_row_frags<KK>(Qf, reinterpret_cast<const T *>(p.q) + head + (size_t)qld * D, g);
+  if constexpr (!TAN) {
+    if (has_go) load_row_frags<KK>(gOf, reinterpret_cast<const T *>(p.go) + head + (size_t)qld * D, g);
+  }
+  if constexpr (DUAL) load_row_frags<KK>(Qtf, reinterpret_cast<const T *>(p.qt) + head + (size_t)qld * D, g);
+  if constexpr (DUAL || TAN) load_row_frags<KK>(gTf, reinterpret_cast<const T *>(p.gt) + head + (size_t)qld * D, g);
+
+  const float Mq = qrow < L ? p.M[srow + qld] : __builtin_inff();
+  const float d1 = (!TAN && has_go) ? p.d1[srow + qld] : 0.f;
+  const float mu = (DUAL) ? p.mu[srow + qld] : 0.f;
+  const float av = (DUAL || TAN) ? p.a[srow + qld] : 0.f;
+  const float d2 = (DUAL) ? p.d2[srow + qld] : 0.f;
+
+  f32x16 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) zero16(acc[db]);
+
+  const float sl2 = pr.scale * LOG2E;
+  const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
+  const T *Kg = reinterpret_cast<const T *>(p.k) + head;
+  const T *Vg = reinterpret_cast<const T *>(p.v) + head;
+  const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + head : nullptr;
+  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + head : nullptr;
+
+  const int kend = pr.causal ? min(L, q0 + BWD_BLK) : L;
+  for (int j0 = 0; j0 < kend; j0 += BWD_T) {
+    __syncthreads();
+    const int nvalid = L - j0;
+    copy_rows<T, BWD_T, D, BWD_NT>(Kn, Cfg::LDN, Kg + (size_t)j0 * D, nvalid, tid);
+    copy_rows<T, BWD_T, D, BWD_NT>(Vn, Cfg::LDN, Vg + (size_t)j0 * D, nvalid, tid);
+    copy_rows_transposed<T, BWD_T, D, BWD_NT>(KT, Cfg::LDT, Kg + (size_t)j0 * D, nvalid, tid);
+    if constexpr (DUAL) {
+      copy_rows<T, BWD_T, D, BWD_NT>(Ktn, Cfg::LDN, Ktg + (size_t)j0 * D, nvalid, tid);
+      copy_rows<T, BWD_T, D, BWD_NT>(Vtn, Cfg::LDN, Vtg + (size_t)j0 * D, nvalid, tid);
+      copy_rows_transposed<T, BWD_T, D, BWD_NT>(KtT, Cfg::LDT, Ktg + (size_t)j0 * D, nvalid, tid);
+    }
+    __syncthreads();
+
+    f32x16 S, dP, Sp, At, Bt;
+    zero16(S);
+    gemm_tile<KK>(S, Kn, Cfg::LDN, pr32, g, Qf);
+    if constexpr (!TAN) {
+      zero16(dP);
+      if (has_go) gemm_tile<KK>(dP, Vn, Cfg::LDN, pr32, g, gOf);
+    }
+    if constexpr (DUAL) {
+      zero16(Sp);
+      gemm_tile<KK>(Sp, Kn, Cfg::LDN, pr32, g, Qtf);
+      gemm_tile<KK>(Sp, Ktn, Cfg::LDN, pr32, g, Qf);
+      zero16(Bt);
+      gemm_tile<KK>(Bt, Vtn, Cfg::LDN, pr32, g, gTf);
+    }
+    if constexpr (DUAL || TAN) {
+      zero16(At);
+      gemm_tile<KK>(At, Vn, Cfg::LDN, pr32, g, gTf);
+    }
+
+    const bool diag = pr.causal && (j0 + BWD_T - 1 > q0 + wave * 32);
+    const bool ragged = j0 + BWD_T > L;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int key0 = j0 + 16 * hf + 8 * g;
+      float bias[8];
+      bool keep[8];
+      if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
+      if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int i = 8 * hf + e;
+        float s = S[i] * sl2;
+        if constexpr (MASK == MASK_ADD) s += bias[e];
+        float pv = fast_exp2(s - Mq);
+        if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
+        if (diag) pv = (key0 + e <= qrow) ? pv : 0.f;
+        if (ragged) pv = (key0 + e < L) ? pv : 0.f;
+        if constexpr (MODE == BWD_PLAIN) {
+          S[i] = pv * (dP[i] - d1);
+        } else if constexpr (DUAL) {
+          const float sp = Sp[i] * pr.scale;
+          Sp[i] = pv * (At[i] - av);
+          S[i] = pv * (dP[i] - d1 + Bt[i] + At[i] * (sp - mu) - av * sp - d2);
+        } else {
+          S[i] = pv * (At[i] - av);
+        }
+      }
+    }
+
+#pragma unroll
+    for (int c = 0; c < BWD_T / 16; ++c) {
+      Frag<T> dsf = to_frag<T>(S, c);
+      Frag<T> dspf;
+      if constexpr (DUAL) dspf = to_frag<T>(Sp, c);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        mma(acc[db], lds_frag(KT + (32 * db + pr32) * Cfg::LDT + 16 * c + 8 * g), dsf);
+        if constexpr (DUAL) mma(acc[db], lds_frag(KtT + (32 * db + pr32) * Cfg::LDT + 16 * c + 8 * g), dspf);
+      }
+    }
+  }
+
+  if (qrow < L) {
+    T *out = reinterpret_cast<T *>(TAN ? p.dqt : p.dq) + head + (size_t)qrow * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = acc[db][8 * hf + e] * pr.scale;
+        store8<T>(out + 32 * db + 16 * hf + 8 * g, x);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// dk, dv (MODE PLAIN / DUAL) or dk', dv' (MODE TANGENT).  Scores are S = Q K^T (lane = key,
+// registers = queries), so P and dS are the B operands of dV^T += gO^T P and dK^T += Q^T dS.
+template <typename T, int D, int MODE, int MASK>
+__global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
+  using Cfg = BwdCfg<T, D, MODE>;
+  constexpr int KK = D / 16, DB = D / 32;
+  constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  // row-major tiles first, then transposed ones, then the row statistics
+  T *Qn = reinterpret_cast<T *>(smem_raw);
+  T *Gn = Qn + Cfg::N_ELEMS;                         // gO (PLAIN, DUAL) or gT (TANGENT)
+  T *Qtn = Gn + Cfg::N_ELEMS;                        // DUAL: Q'
+  T *GTn = Qtn + Cfg::N_ELEMS;                       // DUAL: gT
+  T *trbase = Qn + Cfg::DKV_NAT * Cfg::N_ELEMS;
+  T *QT = trbase;
+  T *GT = QT + Cfg::T_ELEMS;
+  T *QtT = GT + Cfg::T_ELEMS;                        // DUAL
+  T *GTT = QtT + Cfg::T_ELEMS;                       // DUAL
+  float *stats = reinterpret_cast<float *>(trbase + Cfg::DKV_TR * Cfg::T_ELEMS);
+  float *sM = stats, *sd1 = stats + BWD_T, *smu = stats + 2 * BWD_T, *sa = stats + 3 * BWD_T, *sd2 = stats + 4 * BWD_T;
+
+  const Problem &pr = p.pr;
+  const int L = pr.L;
+  const int nkb = (L + BWD_BLK - 1) / BWD_BLK;
+  const int total = nkb * pr.Z * pr.H;
+  const int id = xcd_remap(blockIdx.x, total);
+  const int zh = id / nkb;
+  const int kb = id % nkb;  // causal: the first key blocks have the longest query loops
+  const int z = zh / pr.H, h = zh % pr.H;
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 32, g = lane / 32, pr32 = perm32(r);
+
+  const size_t head = (size_t)zh * L * D;
+  const size_t srow = (size_t)zh * L;
+  const int k0 = kb * BWD_BLK;
+  const int krow = k0 + wave * 32 + r;
+  const int kld = krow < L ? krow : L - 1;
+  const bool has_go = p.go != nullptr;
+
+  Frag<T> Kf[KK], Vf[KK], Ktf[DUAL ? KK : 1], Vtf[DUAL ? KK : 1];
+  load_row_frags<KK>(Kf, reinterpret_cast<const T *>(p.k) + head + (size_t)kld * D, g);
+  load_row_frags<KK>(Vf, reinterpret_cast<const T *>(p.v) + head + (size_t)kld * D, g);
+  if constexpr (DUAL) {
+    load_row_frags<KK>(Ktf, reinterpret_cast<const T *>(p.kt) + head + (size_t)kld * D, g);
+    load_row_frags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + head + (size_t)kld * D, g);
+  }
+
+  f32x16 dK[DB], dV[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    zero16(dK[db]);
+    zero16(dV[db]);
+  }
+
+  const float sl2 = pr.scale * LOG2E;
+  const T *Qg = reinterpret_cast<const T *>(p.q) + head;
+  const T *Qtg = DUAL ? reinterpret_cast<const T *>(p.qt) + head : nullptr;
+  const T *gOg = (!TAN && has_go) ? reinterpret_cast<const T *>(p.go) + head : nullptr;
+  const T *gTg = (DUAL || TAN) ? reinterpret_cast<const T *>(p.gt) + head : nullptr;
+  const T *Gg = TAN ? gTg : gOg;  // tensor staged in Gn / GT
+
+  const int istart = pr.causal ? (k0 / BWD_T) * BWD_T : 0;
+  for (int i0 = istart; i0 < L; i0 += BWD_T) {
+    __syncthreads();
+    const int nvalid = L - i0;
+    copy_rows<T, BWD_T, D, BWD_NT>(Qn, Cfg::LDN, Qg + (size_t)i0 * D, nvalid, tid);
+    copy_rows_transposed<T, BWD_T, D, BWD_NT>(QT, Cfg::LDT, Qg + (size_t)i0 * D, nvalid, tid);
+    if (Gg) {
+      copy_rows<T, BWD_T, D, BWD_NT>(Gn, Cfg::LDN, Gg + (size_t)i0 * D, nvalid, tid);
+      copy_rows_transposed<T, BWD_T, D, BWD_NT>(GT, Cfg::LDT, Gg + (size_t)i0 * D, nvalid, tid);
+    }
+    if constexpr (DUAL) {
+      copy_rows<T, BWD_T, D, BWD_NT>(Qtn, Cfg::LDN, Qtg + (size_t)i0 * D, nvalid, tid);
+      copy_rows_transposed<T, BWD_T, D, BWD_NT>(QtT, Cfg::LDT, Qtg + (size_t)i0 * D, nvalid, tid);
+      copy_rows<T, BWD_T, D, BWD_NT>(GTn, Cfg::LDN, gTg + (size_t)i0 * D, nvalid, tid);
+      copy_rows_transposed<T, BWD_T, D, BWD_NT>(GTT, Cfg::LDT, gTg + (size_t)i0 * D, nvalid, tid);
+    }
+    if (tid < BWD_T) {
+      const bool ok = i0 + tid < L;
+      const size_t si = srow + (ok ? i0 + tid : 0);
+      sM[tid] = ok ? p.M[si] : __builtin_inff();
+      sd1[tid] = (ok && !TAN && has_go) ? p.d1[si] : 0.f;
+      smu[tid] = (ok && DUAL) ? p.mu[si] : 0.f;
+      sa[tid] = (ok && (DUAL || TAN)) ? p.a[si] : 0.f;
+      sd2[tid] = (ok && DUAL) ? p.d2[si] : 0.f;
+    }
+    __syncthreads();
+
+    f32x16 S, dP, Sp, At, Bt;
+    zero16(S);
+    gemm_tile<KK>(S, Qn, Cfg::LDN, pr32, g, Kf);
+    if constexpr (!TAN) {
+      zero16(dP);
+      if (has_go) gemm_tile<KK>(dP, Gn, Cfg::LDN, pr32, g, Vf);
+    }
+    if constexpr (DUAL) {
+      zero16(Sp);
+      gemm_tile<KK>(Sp, Qtn, Cfg::LDN, pr32, g, Kf);
+      gemm_tile<KK>(Sp, Qn, Cfg::LDN, pr32, g, Ktf);
+      zero16(At);
+      gemm_tile<KK>(At, GTn, Cfg::LDN, pr32, g, Vf);
+      zero16(Bt);
+      gemm_tile<KK>(Bt, GTn, Cfg::LDN, pr32, g, Vtf);
+    }
+    if constexpr (TAN) {
+      zero16(At);
+      gemm_tile<KK>(At, Gn, Cfg::LDN, pr32, g, Vf);
+    }
+
+    const bool diag = pr.causal && (i0 < k0 + wave * 32 + 31);  // some query may precede a key
+    f32x16 Pp;  // DUAL: P*(S'-mu); TANGENT: unused
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int ql = 16 * (e / 8) + 8 * g + (e % 8);  // query row within the tile
+      const int qi = i0 + ql;
+      float s = S[e] * sl2;
+      bool keep = true;
+      if constexpr (MASK != MASK_NONE) {
+        const int qc = qi < L ? qi : L - 1;
+        const int64_t off = z * pr.ms[0] + h * pr.ms[1] + (int64_t)qc * pr.ms[2] + (int64_t)kld * pr.ms[3];
+        if constexpr (MASK == MASK_ADD) s += (float)reinterpret_cast<const T *>(pr.mask)[off] * LOG2E;
+        if constexpr (MASK == MASK_BOOL) keep = reinterpret_cast<const uint8_t *>(pr.mask)[off] != 0;
+      }
+      float pv = fast_exp2(s - sM[ql]);
+      if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
+      if (diag) pv = (krow <= qi) ? pv : 0.f;
+      if constexpr (MODE == BWD_PLAIN) {
+        S[e] = pv;
+        dP[e] = pv * (dP[e] - sd1[ql]);
+      } else if constexpr (DUAL) {
+        const float sp = Sp[e] * pr.scale, m_ = smu[ql], a_ = sa[ql];
+        S[e] = pv;
+        Pp[e] = pv * (sp - m_);
+        Sp[e] = pv * (At[e] - a_);
+        dP[e] = pv * (dP[e] - sd1[ql] + Bt[e] + At[e] * (sp - m_) - a_ * sp - sd2[ql]);
+      } else {
+        S[e] = pv;
+        Sp[e] = pv * (At[e] - sa[ql]);
+      }
+    }
+
+#pragma unroll
+    for (int c = 0; c < BWD_T / 16; ++c) {
+      Frag<T> pf = to_frag<T>(S, c);
+      Frag<T> dsf, dspf, ppf;
+      if constexpr (!TAN) dsf = to_frag<T>(dP, c);
+      if constexpr (DUAL || TAN) dspf = to_frag<T>(Sp, c);
+      if constexpr (DUAL) ppf = to_frag<T>(Pp, c);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int off = (32 * db + pr32) * Cfg::LDT + 16 * c + 8 * g;
+        Frag<T> qT = lds_frag(QT + off);
+        if constexpr (MODE == BWD_PLAIN) {
+          mma(dK[db], qT, dsf);
+          mma(dV[db], lds_frag(GT + off), pf);
+        } else if constexpr (DUAL) {
+          mma(dK[db], qT, dsf);
+          mma(dK[db], lds_frag(QtT + off), dspf);
+          if (has_go) mma(dV[db], lds_frag(GT + off), pf);
+          mma(dV[db], lds_frag(GTT + off), ppf);
+        } else {
+          mma(dK[db], qT, dspf);
+          mma(dV[db], lds_frag(GT + off), pf);
+        }
+      }
+    }
+  }
+
+  if (krow < L) {
+    T *outk = reinterpret_cast<T *>(TAN ? p.dkt : p.dk) + head + (size_t)krow * D;
+    T *outv = reinterpret_cast<T *>(TAN ? p.dvt : p.dv) + head + (size_t)krow * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        float xk[8], xv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xk[e] = dK[db][8 * hf + e] * pr.scale;
+          xv[e] = dV[db][8 * hf + e];
+        }
+        store8<T>(outk + 32 * db + 16 * hf + 8 * g, xk);
+        store8<T>(outv + 32 * db + 16 * hf + 8 * g, xv);
+      }
+    }
+  }
+}
+
+}  // namespace jvpfa

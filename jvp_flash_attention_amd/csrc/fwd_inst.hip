@@ -1,0 +1,38 @@
+// One translation unit per (element type, head dim): compiled with
+//   -DJVPFA_T=<__bf16|_Float16|float> -DJVPFA_D=<32|64|128> -DJVPFA_NAME=<symbol>
+// and exporting  int JVPFA_NAME(const FwdParams&, bool dual, int mask_kind, hipStream_t).
+#include "fwd_kernel.hpp"
+#include "launch.hpp"
+
+namespace jvpfa {
+
+template <typename T, int D, int BN, bool DUAL, int MASK>
+static int launch_fwd_one(const FwdParams &p, hipStream_t stream) {
+  using Cfg = FwdCfg<T, D, BN, DUAL>;
+  auto kern = fwd_kernel<T, D, BN, DUAL, MASK>;
+  int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
+  if (rc != 0) return rc;
+  const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
+  const long long blocks = (long long)nqb * p.pr.Z * p.pr.H;
+  if (blocks > 0x7fffffffLL) return -2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : -6;
+}
+
+template <typename T, int D, int BN, bool DUAL>
+static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
+  switch (mask) {
+    case MASK_NONE: return launch_fwd_one<T, D, BN, DUAL, MASK_NONE>(p, stream);
+    case MASK_BOOL: return launch_fwd_one<T, D, BN, DUAL, MASK_BOOL>(p, stream);
+    case MASK_ADD: return launch_fwd_one<T, D, BN, DUAL, MASK_ADD>(p, stream);
+  }
+  return -3;
+}
+
+int JVPFA_NAME(const FwdParams &p, bool dual, int mask, hipStream_t stream) {
+  constexpr int BN = sizeof(JVPFA_T) == 4 ? 32 : 64;
+  return dual ? launch_fwd_mask<JVPFA_T, JVPFA_D, BN, true>(p, mask, stream)
+              : launch_fwd_mask<JVPFA_T, JVPFA_D, BN, false>(p, mask, stream);
+}
+
+}  // namespace jvpfa

@@ -1,0 +1,367 @@
+"""JVP flash attention for MI355X: the Python surface of amorehead/jvp_flash_attention on HIP kernels.
+
+Mirrors ``jvp_flash_attention/jvp_attention.py`` of the reference ("JA" below): the same names
+(``JVPAttn``, ``JVPAttn.fwd``, ``JVPAttn.fwd_dual``, ``attention``, ``MASK_CONST``), the same
+13-argument ``JVPAttn.forward`` (JA:2311-2325), the same ``(o, ctx_tuple)`` result of
+``JVPAttn.apply`` (JA:2633-2647) and 13-slot ``backward`` (JA:2285-2300).  The device work goes
+through the C ABI of ``libjvpfa.so`` (hand-written gfx950 kernels); there is no other code path.
+
+Differences from the reference, all deliberate:
+
+* Float masks follow ``scaled_dot_product_attention``: they are added to the *scaled* logits and
+  are part of the backward recomputation (the reference scales the mask too, JA:247-251, and
+  leaves it out of the backward, JA:1519-1522).  A float mask without any ``MASK_CONST`` entry is
+  accepted (the reference raises ``UserWarning``, JA:2459-2462).
+* Masks may broadcast: any shape whose axes are 1 or (Z, H, L, L); a key-padding mask
+  ``[Z,1,1,L]`` is read in place.  The reference requires the full shape (JA:2383-2388).
+* ``fwd_dual`` returns an output whose tangent O' carries an autograd graph, so gradients of
+  functions of O' (Hessian-vector products) reach q, k, v and the input tangents.  The
+  reference's tangent is a constant (JA:2399, JA:2828) and its backward ignores it (JA:2831).
+* Any sequence length L >= 1 and head dims {32, 64, 128} (the reference: L a multiple of 32,
+  D in {32, 64, 128, 256}, JA:2371-2378, JA:2892).
+"""
+from __future__ import annotations
+
+from typing import Any, Literal, NamedTuple
+
+import torch
+import torch.autograd.forward_ad as fwAD
+from torch import Tensor
+from torch.autograd import Function
+from torch.autograd.function import FunctionCtx, once_differentiable
+
+from . import _lib
+
+MASK_CONST = -100.0  # JA:48-50: value float masks use for "masked"; far below any real logit
+MIN_SEQUENCE_LENGTH = 32  # JA:51; kept for importers, not a limit of these kernels
+SUPPORTED_HEAD_DIMS = (32, 64, 128)
+BLOCK_M = 128  # query rows per workgroup of the forward kernel (only reported through Grid)
+
+
+def _validate(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dropout_p: float, causal: bool):
+    """Argument checks of JA:2356-2392, with this build's shape limits."""
+    if dropout_p != 0.0:
+        raise NotImplementedError("Dropout is not currently supported in JVP attention.")
+    assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be (Z, H, N_CTX, HEAD_DIM)"
+    Z, H, N_CTX, HEAD_DIM_Q = q.shape
+    HEAD_DIM_K, HEAD_DIM_V = k.shape[-1], v.shape[-1]
+    assert HEAD_DIM_Q == HEAD_DIM_K and HEAD_DIM_K == HEAD_DIM_V, (
+        "JVP attention requires HEAD_DIM_Q == HEAD_DIM_K == HEAD_DIM_V"
+        f" but got HEAD_DIM_Q={HEAD_DIM_Q}, HEAD_DIM_K={HEAD_DIM_K}, HEAD_DIM_V={HEAD_DIM_V}"
+    )
+    assert HEAD_DIM_K in SUPPORTED_HEAD_DIMS, (
+        f"JVP attention only supports HEAD_DIM_K in {set(SUPPORTED_HEAD_DIMS)}, but got HEAD_DIM_K={HEAD_DIM_K}"
+    )
+    assert k.shape == q.shape and v.shape == q.shape, (
+        "JVP attention requires q, k, v of one shape (no cross-attention or grouped heads),"
+        f" but got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}"
+    )
+    assert N_CTX >= 1, f"JVP attention requires N_CTX >= 1, but got N_CTX={N_CTX}"
+    assert q.dtype in _lib.DTYPES and k.dtype == q.dtype and v.dtype == q.dtype, (
+        f"q, k, v must share one dtype out of bfloat16/float16/float32, got {q.dtype}, {k.dtype}, {v.dtype}"
+    )
+    if causal and attn_mask is not None:
+        raise ValueError("Causal attention does not support an attention mask.")
+    if attn_mask is not None:
+        assert attn_mask.dim() == 4 and all(
+            m in (1, full) for m, full in zip(attn_mask.shape, (Z, H, N_CTX, N_CTX))
+        ), "The provided attention mask must have 4 dimensions broadcastable to (Z, H, N_CTX, N_CTX)."
+        assert attn_mask.dtype in {torch.bool, q.dtype}, (
+            "The attention mask must be of the dtype bool or that of the query tensor."
+        )
+
+
+def _classify_mask(attn_mask: Tensor | None, q: Tensor, verify_attn_mask: bool):
+    """Mask kind and the tensor the kernels read (JA:2429-2462)."""
+    if attn_mask is None:
+        return torch.empty(0, device=q.device, dtype=q.dtype), _lib.MASK_NONE
+    if attn_mask.dtype == torch.bool:
+        mask_tensor = attn_mask
+        if verify_attn_mask:
+            assert mask_tensor.any(dim=-1).any(dim=-1).all(), (
+                "The attention mask cannot be all False for any head."
+            )
+        return mask_tensor, _lib.MASK_BOOL
+    mask_tensor = attn_mask.to(q.dtype)
+    if verify_attn_mask:
+        assert not torch.isnan(mask_tensor).any(), "The attention mask cannot contain NaNs."
+        assert not torch.isposinf(mask_tensor).any(), "The attention mask cannot contain +inf."
+    return mask_tensor, _lib.MASK_ADD
+
+
+def _unwrap(x):
+    """Strip functorch wrappers from a saved tensor (JA:2846-2855)."""
+    while isinstance(x, Tensor) and torch._C._functorch.is_functorch_wrapped_tensor(x):
+        x = torch._C._functorch.get_unwrapped(x)
+    return x
+
+
+def _dense(t: Tensor | None) -> Tensor | None:
+    return None if t is None else (t if t.is_contiguous() else t.contiguous())
+
+
+class _DualCore(Function):
+    """(q, k, v, q', k', v') -> (O, O', M, mu), differentiable in all six tensor inputs.
+
+    The backward is the closed form for ``<gO,O> + <gT,O'>``; with gT = 0 it is the reference's
+    backward (JA:1541-1553, JA:1687-1697).
+    """
+
+    @staticmethod
+    def forward(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale):
+        o, o_t, M, mu = _lib.backend().fwd(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale)
+        return o, o_t, M, mu
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale = inputs
+        o, o_t, M, mu = outputs
+        ctx.mark_non_differentiable(M, mu)
+        ctx.save_for_backward(q, k, v, q_t, k_t, v_t, o, o_t, M, mu)
+        ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale = mask_tensor, MASK_TYPE, causal, sm_scale
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, go, gt, _gM, _gmu):
+        q, k, v, q_t, k_t, v_t, o, o_t, M, mu = (_unwrap(t) for t in ctx.saved_tensors)
+        want_t = any(ctx.needs_input_grad[3:6])
+        dq, dk, dv, dqt, dkt, dvt = _lib.backend().bwd(
+            q, k, v, q_t, k_t, v_t, o, o_t, M, mu, _dense(go), _dense(gt),
+            ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale, want_tangent_grads=want_t,
+        )
+        return dq, dk, dv, dqt, dkt, dvt, None, None, None, None
+
+
+class _AttachTangent(Function):
+    """Identity on O whose forward-mode tangent is the precomputed O' (the reference's trick of
+    JA:2688 and JA:2828, with O' an input so that it keeps its autograd graph)."""
+
+    @staticmethod
+    def forward(o, o_t, q, k, v):
+        return o.view_as(o)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        ctx.save_for_forward(inputs[1])
+
+    @staticmethod
+    def jvp(ctx, *_tangents):
+        return ctx.saved_for_forward[0]
+
+    @staticmethod
+    def backward(ctx, g):
+        return g, None, None, None, None
+
+
+class JVPAttn(Function):
+    """JVP (Jacobian-Vector Product) for Attention Mechanism."""
+
+    class Grid(NamedTuple):
+        """Launch grid of the forward kernel."""
+
+        M_BLOCKS: int
+        Z_H: int
+        ONE: Literal[1]
+
+    class FnCtx(FunctionCtx):
+        """Function context for JVP Attention."""
+
+        sm_scale: float
+        HEAD_DIM_K: int
+        causal: bool
+        grid: "JVPAttn.Grid"
+        mask_tensor: Tensor
+        MASK_TYPE: int
+        dropout_p: float
+        philox_seed: int
+        ENABLE_DROPOUT: bool
+
+    class FwdOutCtxContrib(NamedTuple):
+        """Forward output context contributions for JVP Attention."""
+
+        o_t: Tensor | None
+        M: Tensor
+        grid: "JVPAttn.Grid"
+        HEAD_DIM_K: int
+        sm_scale: float
+        mask_tensor: Tensor
+        MASK_TYPE: int
+        dropout_p: float
+        philox_seed: int
+        ENABLE_DROPOUT: bool
+
+    class FwdOut(NamedTuple):
+        """Forward output for JVP Attention."""
+
+        o: Tensor
+        ctx: "JVPAttn.FwdOutCtxContrib"
+
+    class JVPOut(NamedTuple):
+        """JVP output for JVP Attention."""
+
+        o: Tensor
+        ctx: None
+
+    class BwdOut(NamedTuple):
+        """Backward output for JVP Attention."""
+
+        q: Tensor
+        k: Tensor
+        v: Tensor
+        q_t: None
+        k_t: None
+        v_t: None
+        attn_mask: None
+        dropout_p: None
+        causal: None
+        sm_scale: None
+        warp_specialize: None
+        USE_TMA: None
+        verify_attn_mask: None
+
+    class Strides(NamedTuple):
+        """Strides for JVP Attention."""
+
+        z: int
+        h: int
+        n_ctx: int
+        head_dim: int
+
+    @staticmethod
+    def forward(
+        q: Tensor,
+        k: Tensor,
+        v: Tensor,
+        q_t: Tensor | None,
+        k_t: Tensor | None,
+        v_t: Tensor | None,
+        attn_mask: Tensor | None = None,
+        dropout_p: float = 0.0,
+        causal: bool = False,
+        sm_scale: float | None = None,
+        warp_specialize: bool = True,
+        USE_TMA: bool = True,
+        verify_attn_mask: bool = True,
+    ) -> "JVPAttn.FwdOut":
+        """Forward pass (JA:2310-2647): one fused kernel gives ``o`` and, when tangents are
+        passed, ``o_t``.  ``warp_specialize`` and ``USE_TMA`` are accepted and ignored (they
+        select NVIDIA-specific code in the reference)."""
+        _validate(q, k, v, attn_mask, dropout_p, causal)
+        Z, H, N_CTX, HEAD_DIM_K = q.shape
+        if sm_scale is None:
+            sm_scale = HEAD_DIM_K**-0.5
+        mask_tensor, MASK_TYPE = _classify_mask(attn_mask, q, verify_attn_mask)
+        ENABLE_JVP = q_t is not None
+        q, k, v = _dense(_unwrap(q)), _dense(_unwrap(k)), _dense(_unwrap(v))
+        if ENABLE_JVP:
+            q_t = _dense(_unwrap(q_t))
+            k_t = torch.zeros_like(k) if k_t is None else _dense(_unwrap(k_t))
+            v_t = torch.zeros_like(v) if v_t is None else _dense(_unwrap(v_t))
+        o, o_t, M, _mu = _lib.backend().fwd(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale)
+        grid = JVPAttn.Grid((N_CTX + BLOCK_M - 1) // BLOCK_M, Z * H, 1)
+        return JVPAttn.FwdOut(
+            o,
+            JVPAttn.FwdOutCtxContrib(o_t, M, grid, HEAD_DIM_K, sm_scale, mask_tensor, MASK_TYPE, dropout_p, 0, False),
+        )
+
+    @staticmethod
+    def setup_context(ctx: "JVPAttn.FnCtx", inputs, outputs: "JVPAttn.FwdOut") -> None:
+        """JA:2649-2698."""
+        q, k, v, _q_t, _k_t, _v_t, _mask, _dropout_p, causal, _scale, _ws, _tma, _verify = inputs
+        o, (o_t, M, grid, HEAD_DIM_K, sm_scale, mask_tensor, MASK_TYPE, dropout_p, philox_seed, ENABLE_DROPOUT) = outputs
+        ctx.grid = grid
+        ctx.save_for_forward(o_t)
+        ctx.save_for_backward(q, k, v, o, M)
+        ctx.sm_scale = sm_scale
+        ctx.HEAD_DIM_K = HEAD_DIM_K
+        ctx.causal = causal
+        ctx.mask_tensor = mask_tensor
+        ctx.MASK_TYPE = MASK_TYPE
+        ctx.dropout_p = dropout_p
+        ctx.philox_seed = philox_seed
+        ctx.ENABLE_DROPOUT = ENABLE_DROPOUT
+
+    @staticmethod
+    def fwd(
+        q: Tensor,
+        k: Tensor,
+        v: Tensor,
+        attn_mask: Tensor | None = None,
+        dropout_p: float = 0.0,
+        causal: bool = False,
+        sm_scale: float | None = None,
+        warp_specialize: bool = True,
+        USE_TMA: bool = True,
+    ) -> Tensor:
+        """Plain attention forward, differentiable in q, k, v (JA:2700-2752)."""
+        if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+            q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        out: JVPAttn.FwdOut = JVPAttn.apply(
+            q, k, v, None, None, None, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA
+        )
+        a, _ = out
+        return a
+
+    @staticmethod
+    def fwd_dual(
+        q: Tensor,
+        k: Tensor,
+        v: Tensor,
+        attn_mask: Tensor | None = None,
+        dropout_p: float = 0.0,
+        causal: bool = False,
+        sm_scale: float | None = None,
+        warp_specialize: bool = True,
+        USE_TMA: bool = True,
+    ) -> Tensor:
+        """Attention on dual tensors (JA:2754-2813): inside ``fwAD.dual_level()`` or
+        ``torch.func.jvp`` the result is a dual tensor whose tangent is O', computed by the same
+        kernel pass as O.  Both O and O' are differentiable (reverse mode) in q, k, v and in the
+        input tangents."""
+        if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+            q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        q_p, q_t = fwAD.unpack_dual(q)
+        k_p, k_t = fwAD.unpack_dual(k)
+        v_p, v_t = fwAD.unpack_dual(v)
+        if q_t is None and k_t is None and v_t is None:
+            return JVPAttn.fwd(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
+
+        _validate(q_p, k_p, v_p, attn_mask, dropout_p, causal)
+        if sm_scale is None:
+            sm_scale = q_p.shape[-1] ** -0.5
+        mask_tensor, MASK_TYPE = _classify_mask(attn_mask, q_p, True)
+        q_t = torch.zeros_like(q_p) if q_t is None else _dense(q_t)
+        k_t = torch.zeros_like(k_p) if k_t is None else _dense(k_t)
+        v_t = torch.zeros_like(v_p) if v_t is None else _dense(v_t)
+        o, o_t, _M, _mu = _DualCore.apply(
+            _dense(q_p), _dense(k_p), _dense(v_p), q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale
+        )
+        # NOTE: q, k, v are passed as dual tensors so that autograd calls jvp(), which hands back O'.
+        return _AttachTangent.apply(o, o_t, q, k, v)
+
+    @staticmethod
+    def jvp(ctx: "JVPAttn.FnCtx", gq: Tensor, gk: Tensor, gv: Tensor, *_) -> "JVPAttn.JVPOut":
+        """JA:2815-2828: the tangent was computed in forward(); hand it back."""
+        return JVPAttn.JVPOut(ctx.saved_for_forward[0], None)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, do, _) -> "JVPAttn.BwdOut":
+        """First-order backward from the gradient of ``o`` (JA:2830-2978)."""
+        q, k, v, o, M = (_unwrap(t) for t in ctx.saved_tensors)
+        if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and o.is_contiguous()):
+            raise ValueError(
+                "JVPAttn expected q, k, v, o to be contiguous; got "
+                f"q.is_contiguous()={q.is_contiguous()}, k.is_contiguous()={k.is_contiguous()}, "
+                f"v.is_contiguous()={v.is_contiguous()}, o.is_contiguous()={o.is_contiguous()}, "
+                f"do.is_contiguous()={do.is_contiguous()}"
+            )
+        do = _dense(_unwrap(do))
+        dq, dk, dv, _, _, _ = _lib.backend().bwd(
+            q, k, v, None, None, None, o, None, M, None, do, None,
+            ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale,
+        )
+        return JVPAttn.BwdOut(dq, dk, dv, None, None, None, None, None, None, None, None, None, None)
+
+
+attention = JVPAttn.fwd

@@ -1,0 +1,55 @@
+"""A stand-in for the HIP backend so that the host logic (argument checks, autograd wiring,
+dual-tensor handling) can be exercised on a machine without a GPU.  It computes with the oracle's
+tile-loop restatement on CPU tensors.  Test infrastructure only: the shipped package never
+imports it."""
+import contextlib
+
+import torch
+
+from jvp_flash_attention_amd import _lib
+from oracle import tiled
+
+
+class OracleBackend:
+    name = "oracle-cpu"
+
+    def __init__(self):
+        self.calls = []
+
+    @staticmethod
+    def _mask(mask, kind):
+        return None if kind == _lib.MASK_NONE else mask
+
+    def fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
+        self.calls.append(("fwd", qt is not None, mask_kind, bool(causal)))
+        f = lambda t: None if t is None else t.double()  # noqa: E731
+        m = self._mask(mask, mask_kind)
+        m = m if m is None or m.dtype == torch.bool else m.double()
+        o, ot, M, mu = tiled.forward(f(q), f(k), f(v), f(qt), f(kt), f(vt), mask=m, causal=causal, scale=sm_scale)
+        c = lambda t: None if t is None else t.to(q.dtype)  # noqa: E731
+        return c(o), c(ot), M.float(), None if mu is None else mu.float()
+
+    def bwd(self, q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
+            want_tangent_grads=False):
+        self.calls.append(("bwd", gt is not None, mask_kind, bool(causal), want_tangent_grads))
+        f = lambda t: None if t is None else t.double()  # noqa: E731
+        m = self._mask(mask, mask_kind)
+        m = m if m is None or m.dtype == torch.bool else m.double()
+        if go is None:
+            go = torch.zeros_like(q)
+        g = tiled.backward(f(q), f(k), f(v), f(qt), f(kt), f(vt), f(o), f(ot), f(M), f(mu), f(go), f(gt),
+                           mask=m, causal=causal, scale=sm_scale)
+        c = lambda t: t.to(q.dtype)  # noqa: E731
+        tg = (c(g["dqt"]), c(g["dkt"]), c(g["dvt"])) if want_tangent_grads else (None, None, None)
+        return (c(g["dq"]), c(g["dk"]), c(g["dv"]), *tg)
+
+
+@contextlib.contextmanager
+def oracle_backend():
+    saved = _lib._backend
+    fake = OracleBackend()
+    _lib._backend = fake
+    try:
+        yield fake
+    finally:
+        _lib._backend = saved

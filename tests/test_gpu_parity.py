@@ -1,0 +1,180 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle.
+
+Tolerances (BASELINE north star): fp32 max-abs <= 1e-4; bf16 / fp16 relative error
+``max|x - ref| / max|ref| <= 2e-2``.  The oracle is the dense fp64 closed form evaluated on the
+same, already rounded, inputs (it is itself pinned against PyTorch's math SDPA under
+``torch.func.jvp`` in ``test_oracle.py``).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dense
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
+
+
+def _tol_check(name, got, ref, dtype):
+    got = got.detach().double().cpu().numpy()
+    assert np.isfinite(got).all(), f"{name}: non-finite values"
+    err = np.abs(got - ref).max()
+    if dtype == torch.float32:
+        assert err <= 1e-4, f"{name}: max-abs {err:.3e} > 1e-4"
+    else:
+        # the floor only matters when the exact answer is (nearly) zero, e.g. dq for L = 1
+        rel = err / max(np.abs(ref).max(), 1e-2)
+        assert rel <= 2e-2, f"{name}: relative {rel:.3e} > 2e-2"
+
+
+def _make(Z, H, L, D, dtype, seed, tangent_std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    t = [torch.randn(Z, H, L, D, generator=g) for _ in range(8)]
+    for i in (3, 4, 5):
+        t[i] = t[i] * tangent_std
+    return [x.to(dtype) for x in t]
+
+
+def _mask(mode, Z, H, L, dtype, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    if mode in ("none", "causal"):
+        return None
+    if mode == "keypad":  # BASELINE config 4(a): per-batch valid length uniform in [L/2, L]
+        lens = torch.randint(L // 2, L + 1, (Z,), generator=g)
+        return (torch.arange(L)[None, :] < lens[:, None]).view(Z, 1, 1, L)
+    if mode == "bias":  # BASELINE config 4(b)
+        return torch.randn(Z, H, L, L, generator=g).to(dtype)
+    if mode == "bool_full":  # the reference's test masks: random, keep-probability 0.1 (test file :334-363)
+        m = torch.rand(Z, H, L, L, generator=g) > 0.9
+        m[..., 0] = True
+        return m
+    if mode == "bias_bcast":
+        return torch.randn(1, H, L, L, generator=g).to(dtype)
+    raise ValueError(mode)
+
+
+def _run_case(Z, H, L, D, dtype, mode, seed=0, tangent_std=1.0, plain=False, tangent_grads=True):
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    q, k, v, qt, kt, vt, go, gt = _make(Z, H, L, D, dtype, seed, tangent_std)
+    mask = _mask(mode, Z, H, L, dtype)
+    causal = mode == "causal"
+    kind = _lib.MASK_NONE if mask is None else (_lib.MASK_BOOL if mask.dtype == torch.bool else _lib.MASK_ADD)
+    scale = D**-0.5
+    npm = None if mask is None else (mask.numpy() if mask.dtype == torch.bool else mask.double().numpy())
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dmask = None if mask is None else mask.cuda()
+    print(f"case Z{Z} H{H} L{L} D{D} {dtype} {mode} plain={plain}", flush=True)
+    if plain:
+        ref = dense.forward(*f64[:3], mask=npm, causal=causal, scale=scale)
+        rb = dense.backward(*f64[:3], None, None, None, f64[6], None, mask=npm, causal=causal, scale=scale)
+        o, ot, M, mu = be.fwd(dev[0], dev[1], dev[2], None, None, None, dmask, kind, causal, scale)
+        assert ot is None and mu is None
+        _tol_check("O", o, ref["O"], dtype)
+        assert np.abs(M.double().cpu().numpy() - ref["M"]).max() < (1e-4 if dtype == torch.float32 else 2e-2)
+        dq, dk, dv, *_ = be.bwd(dev[0], dev[1], dev[2], None, None, None, o, None, M, None, dev[6], None,
+                                dmask, kind, causal, scale)
+        for n, t in (("dq", dq), ("dk", dk), ("dv", dv)):
+            _tol_check(n, t, rb[n], dtype)
+        return
+    ref = dense.forward(*f64[:6], mask=npm, causal=causal, scale=scale)
+    o, ot, M, mu = be.fwd(*dev[:6], dmask, kind, causal, scale)
+    _tol_check("O", o, ref["O"], dtype)
+    _tol_check("O'", ot, ref["Ot"], dtype)
+    stat_tol = 1e-4 if dtype == torch.float32 else 2e-2
+    assert np.abs(M.double().cpu().numpy() - ref["M"]).max() < stat_tol
+    assert np.abs(mu.double().cpu().numpy() - ref["mu"]).max() < stat_tol * max(1.0, np.abs(ref["mu"]).max())
+    rb = dense.backward(*f64, mask=npm, causal=causal, scale=scale)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, kind, causal, scale,
+                   want_tangent_grads=tangent_grads)
+    names = ("dq", "dk", "dv", "dqt", "dkt", "dvt")
+    for n, t in zip(names, grads):
+        if t is not None:
+            _tol_check(n, t, rb[n], dtype)
+    # first-order backward from gO only through the same saved state (reference's backward)
+    rb1 = dense.backward(*f64[:7], None, mask=npm, causal=causal, scale=scale)
+    g1 = be.bwd(dev[0], dev[1], dev[2], None, None, None, o, None, M, None, dev[6], None, dmask, kind, causal, scale)
+    for n, t in zip(names[:3], g1[:3]):
+        _tol_check(n + "(gO only)", t, rb1[n], dtype)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("mode", ["none", "causal"])
+def test_dual_fwd_bwd_dense_and_causal(dt, D, mode):
+    _run_case(2, 2, 256, D, DTYPES[dt], mode)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("mode", ["keypad", "bias", "bool_full", "bias_bcast"])
+def test_dual_fwd_bwd_masks(dt, mode):
+    _run_case(2, 3, 192, 64, DTYPES[dt], mode)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+@pytest.mark.parametrize("mode", ["keypad", "bias"])
+def test_masks_d128(dt, mode):
+    _run_case(2, 2, 128, 128, DTYPES[dt], mode)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+@pytest.mark.parametrize("L", [1, 31, 40, 100, 130, 333])
+@pytest.mark.parametrize("mode", ["none", "causal", "keypad"])
+def test_ragged_lengths(dt, L, mode):
+    _run_case(1, 2, L, 64, DTYPES[dt], mode)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("mode", ["none", "causal", "keypad", "bias"])
+def test_plain_forward_and_first_order_backward(dt, mode):
+    _run_case(2, 2, 160, 64, DTYPES[dt], mode, plain=True)
+    _run_case(1, 2, 128, 128, DTYPES[dt], mode, plain=True)
+
+
+def test_small_tangents_config2_shape_slice():
+    # BASELINE config 2 statistics (tangents ~ N(0, 0.1^2)) on a slice of its shape
+    _run_case(1, 4, 512, 64, torch.bfloat16, "none", tangent_std=0.1)
+
+
+def test_fully_masked_rows_are_zero():
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    Z, H, L, D = 1, 2, 64, 64
+    q, k, v, qt, kt, vt, go, gt = [x.cuda() for x in _make(Z, H, L, D, torch.float32, 3)]
+    mask = torch.ones(Z, H, L, L, dtype=torch.bool)
+    mask[0, 1, 5, :] = False
+    mask[0, 0, 40, :] = False
+    mask = mask.cuda()
+    o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, mask, _lib.MASK_BOOL, False, D**-0.5)
+    for t in (o, ot):
+        assert torch.all(t[0, 1, 5] == 0) and torch.all(t[0, 0, 40] == 0) and torch.isfinite(t).all()
+    assert torch.isposinf(M[0, 1, 5]) and mu[0, 1, 5] == 0
+    grads = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, _lib.MASK_BOOL, False, D**-0.5,
+                   want_tangent_grads=True)
+    for gname, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        assert torch.isfinite(t).all(), gname
+    assert torch.all(grads[0][0, 1, 5] == 0) and torch.all(grads[3][0, 0, 40] == 0)
+    f64 = [x.double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    rb = dense.backward(*f64, mask=mask.cpu().numpy(), scale=D**-0.5)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        _tol_check(n, t, rb[n], torch.float32)
+
+
+def test_only_tangent_gradient_hvp_style():
+    """gO absent (loss is a function of O' only), the Hessian-vector-product use."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    Z, H, L, D = 1, 2, 256, 128
+    xs = _make(Z, H, L, D, torch.bfloat16, 5)
+    f64 = [x.double().numpy() for x in xs]
+    dev = [x.cuda() for x in xs]
+    o, ot, M, mu = be.fwd(*dev[:6], None, _lib.MASK_NONE, True, D**-0.5)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, None, dev[7], None, _lib.MASK_NONE, True, D**-0.5)
+    rb = dense.backward(*f64[:6], np.zeros_like(f64[6]), f64[7], causal=True, scale=D**-0.5)
+    for n, t in zip(("dq", "dk", "dv"), grads[:3]):
+        _tol_check(n, t, rb[n], torch.bfloat16)
