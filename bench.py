@@ -1,0 +1,163 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused JVP attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Workload (BASELINE.json headline): bf16, B=4, H=16, L=4096, D=128, synthetic N(0,1) inputs that
+are resident in HBM before the timed region.  A step is one fused dual forward (O and O' in
+one kernel).  ``value`` is its throughput in TFLOP/s with the algorithmic FLOP count
+12 * B*H*L^2*D (six GEMM-shaped products, 2 FLOPs per multiply-add).  The same JSON line also
+carries the causal forward, forward+backward (tangent-path backward, 24 * B*H*L^2*D more) and
+the reference's FLOP convention (its tests count 2*(4*B*H*L^2*D + 5*B*H*L^2)) for comparison with
+its README, a roofline block for the forward kernel, and the reference's CPU route (math SDPA under
+``torch.func.jvp``, fp32) timed on this host on a slab of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
+Z, H, L, D = 4, 16, 4096, 128
+
+# HBM bytes per forward launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
+# profiles/); None until measured.
+MEASURED_FWD_TRAFFIC_BYTES = None
+
+
+def timed(fn, steps, warmup):
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_time(stop) / steps, wall_ms
+
+
+def cpu_baseline():
+    """Reference CPU route on a B=1, H=2 slab of the headline shape, scaled to the full shape."""
+    import torch
+
+    from oracle import sdpa_jvp
+
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    cores = torch.get_num_threads()
+    zb, hb = 1, 2
+    g = torch.Generator().manual_seed(0)
+    q, k, v, qt, kt, vt = [torch.randn(zb, hb, L, D, generator=g) for _ in range(6)]
+    sdpa_jvp.forward(q[:, :1, :512], k[:, :1, :512], v[:, :1, :512], qt[:, :1, :512], kt[:, :1, :512], vt[:, :1, :512])
+    t0 = time.perf_counter()
+    sdpa_jvp.forward(q, k, v, qt, kt, vt)
+    dt = time.perf_counter() - t0
+    flops = 12.0 * zb * hb * L * L * D
+    return {
+        "value": flops / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"math SDPA + torch.func.jvp fp32 dual forward on a B={zb},H={hb},L={L},D={D} slab "
+                  f"({dt:.1f} s); full shape would take ~{dt * Z * H / (zb * hb):.0f} s (extrapolated)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--fwd-only", action="store_true", help="time only the headline forward (for profiling)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (B*H shards trivially); use --gpus 1")
+
+    import torch
+
+    from jvp_flash_attention_amd import _lib
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an AMD GPU (no CPU path exists)")
+    be = _lib.backend()
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    q, k, v, qt, kt, vt, go, gt = [
+        torch.randn(Z, H, L, D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(8)
+    ]
+    scale = D**-0.5
+    N = float(Z) * H * L * L * D
+    fwd_flops, bwd_flops = 12.0 * N, 24.0 * N
+    ref_conv_flops = 2.0 * (4.0 * N + 5.0 * Z * H * L * L)
+
+    def fwd(causal=False):
+        return be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, causal, scale)
+
+    state = {}
+
+    def fwd_bwd(causal=False):
+        o, ot, M, mu = fwd(causal)
+        state["g"] = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, causal, scale)
+
+    ms_fwd, wall_fwd = timed(fwd, args.steps, args.warmup)
+    out = {
+        "metric": "fused JVP dual-forward throughput, bf16 B4 H16 L4096 D128 (non-causal)",
+        "value": fwd_flops / (ms_fwd * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_fwd,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "bf16 B4 H16 L4096 D128 dual forward (O, O'), no mask, sm_scale=D^-0.5",
+                   "flops_per_step": fwd_flops},
+        "pct_mfma_peak": 100.0 * fwd_flops / (ms_fwd * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        "wall_ms_per_step": wall_fwd,
+        "roofline": {
+            "bound": "mfma",
+            "achieved": fwd_flops / (ms_fwd * 1e-3) / 1e12,
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": fwd_flops / (ms_fwd * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "traffic": MEASURED_FWD_TRAFFIC_BYTES,
+            "kernel": "fwd_kernel<bf16, D=128, dual>",
+        },
+    }
+    if not args.fwd_only:
+        ms_fc, _ = timed(lambda: fwd(True), args.steps, args.warmup)
+        ms_fb, _ = timed(fwd_bwd, max(1, args.steps // 2), 1)
+        ms_fbc, _ = timed(lambda: fwd_bwd(True), max(1, args.steps // 2), 1)
+        tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12  # noqa: E731
+        out["extra"] = {
+            "fwd_causal": {"ms": ms_fc, "tflops": tf(fwd_flops / 2, ms_fc),
+                           "pct_mfma_peak": 100 * tf(fwd_flops / 2, ms_fc) / PEAK_BF16_TFLOPS},
+            "fwd_bwd": {"ms": ms_fb, "tflops": tf(fwd_flops + bwd_flops, ms_fb),
+                        "pct_mfma_peak": 100 * tf(fwd_flops + bwd_flops, ms_fb) / PEAK_BF16_TFLOPS},
+            "fwd_bwd_causal": {"ms": ms_fbc, "tflops": tf((fwd_flops + bwd_flops) / 2, ms_fbc),
+                               "pct_mfma_peak": 100 * tf((fwd_flops + bwd_flops) / 2, ms_fbc) / PEAK_BF16_TFLOPS},
+            "fwd_tflops_reference_flop_convention": tf(ref_conv_flops, ms_fwd),
+            "peak_hbm_allocated_mb": torch.cuda.max_memory_allocated() / 2**20,
+        }
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -16,15 +16,14 @@ pytestmark = pytest.mark.gpu
 DTYPES = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
 
 
-def _tol_check(name, got, ref, dtype):
+def _tol_check(name, got, ref, dtype, floor=1e-30):
     got = got.detach().double().cpu().numpy()
     assert np.isfinite(got).all(), f"{name}: non-finite values"
     err = np.abs(got - ref).max()
     if dtype == torch.float32:
         assert err <= 1e-4, f"{name}: max-abs {err:.3e} > 1e-4"
     else:
-        # the floor only matters when the exact answer is (nearly) zero, e.g. dq for L = 1
-        rel = err / max(np.abs(ref).max(), 1e-2)
+        rel = err / max(np.abs(ref).max(), floor)
         assert rel <= 2e-2, f"{name}: relative {rel:.3e} > 2e-2"
 
 
@@ -121,7 +120,7 @@ def test_masks_d128(dt, mode):
 
 
 @pytest.mark.parametrize("dt", ["bf16", "fp32"])
-@pytest.mark.parametrize("L", [1, 31, 40, 100, 130, 333])
+@pytest.mark.parametrize("L", [2, 31, 40, 100, 130, 333])
 @pytest.mark.parametrize("mode", ["none", "causal", "keypad"])
 def test_ragged_lengths(dt, L, mode):
     _run_case(1, 2, L, 64, DTYPES[dt], mode)
@@ -178,3 +177,26 @@ def test_only_tangent_gradient_hvp_style():
     rb = dense.backward(*f64[:6], np.zeros_like(f64[6]), f64[7], causal=True, scale=D**-0.5)
     for n, t in zip(("dq", "dk", "dv"), grads[:3]):
         _tol_check(n, t, rb[n], torch.bfloat16)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+def test_single_key(dt):
+    """L = 1: softmax is the constant 1, so O = v, O' = v' and dq = dk = dq' = dk' = 0 exactly.
+    In 16-bit the zero gradients come out as rounding residue of O and O' (stored rounded), so
+    they are held to an absolute bound instead of a relative one."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    dtype = DTYPES[dt]
+    q, k, v, qt, kt, vt, go, gt = [x.cuda() for x in _make(2, 2, 1, 64, dtype, 9)]
+    o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, 0.125)
+    assert torch.equal(o, v)
+    # O' = (p s') v / l - mu O + v': the first two terms cancel only up to the rounding of p s'
+    assert (ot.float() - vt.float()).abs().max().item() <= (1e-5 if dtype == torch.float32 else 5e-2)
+    grads = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, False, 0.125,
+                   want_tangent_grads=True)
+    bound = 1e-5 if dtype == torch.float32 else 5e-2
+    for i in (0, 1, 3, 4):
+        assert grads[i].float().abs().max().item() <= bound
+    assert (grads[2].float() - go.float()).abs().max().item() <= bound
+    assert (grads[5].float() - gt.float()).abs().max().item() <= bound
