@@ -2,6 +2,7 @@
 //   -DJVPFA_T=<__bf16|_Float16|float> -DJVPFA_D=<32|64|128> -DJVPFA_NAME=<symbol>
 // and exporting  int JVPFA_NAME(const FwdParams&, bool dual, int mask_kind, hipStream_t).
 #include "fwd_kernel.hpp"
+#include "fwd_kernel_v2.hpp"
 #include "launch.hpp"
 
 namespace jvpfa {
@@ -19,14 +20,37 @@ static int launch_fwd_one(const FwdParams &p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }
 
+// 16-bit element types with D >= 64 take the direct-to-LDS, double-buffered kernel.
+template <typename T, int D, bool DUAL, int MASK>
+static int launch_fwd2_one(const FwdParams &p, hipStream_t stream) {
+  using Cfg = Fwd2Cfg<T, D, DUAL>;
+  auto kern = fwd2_kernel<T, D, DUAL, MASK>;
+  int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
+  if (rc != 0) return rc;
+  const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
+  const long long blocks = (long long)nqb * p.pr.Z * p.pr.H;
+  if (blocks > 0x7fffffffLL) return -2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : -6;
+}
+
 template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
-  switch (mask) {
-    case MASK_NONE: return launch_fwd_one<T, D, BN, DUAL, MASK_NONE>(p, stream);
-    case MASK_BOOL: return launch_fwd_one<T, D, BN, DUAL, MASK_BOOL>(p, stream);
-    case MASK_ADD: return launch_fwd_one<T, D, BN, DUAL, MASK_ADD>(p, stream);
+  if constexpr (sizeof(T) == 2 && D >= 64) {
+    switch (mask) {
+      case MASK_NONE: return launch_fwd2_one<T, D, DUAL, MASK_NONE>(p, stream);
+      case MASK_BOOL: return launch_fwd2_one<T, D, DUAL, MASK_BOOL>(p, stream);
+      case MASK_ADD: return launch_fwd2_one<T, D, DUAL, MASK_ADD>(p, stream);
+    }
+    return -3;
+  } else {
+    switch (mask) {
+      case MASK_NONE: return launch_fwd_one<T, D, BN, DUAL, MASK_NONE>(p, stream);
+      case MASK_BOOL: return launch_fwd_one<T, D, BN, DUAL, MASK_BOOL>(p, stream);
+      case MASK_ADD: return launch_fwd_one<T, D, BN, DUAL, MASK_ADD>(p, stream);
+    }
+    return -3;
   }
-  return -3;
 }
 
 int JVPFA_NAME(const FwdParams &p, bool dual, int mask, hipStream_t stream) {

@@ -1,0 +1,332 @@
+// Fused dual forward for 16-bit element types (bf16 / fp16), D in {64, 128}: the headline kernel.
+//
+// Same mathematics and register layout as fwd_kernel.hpp (one workgroup = 4 waves = 128 query
+// rows, scores formed transposed so that a lane owns a query column), with the memory side
+// rebuilt for gfx950:
+//   * K, K', V, V' tiles (64 keys) go global -> LDS with direct-to-LDS loads (no registers, no
+//     VALU), double buffered: the loads of tile j+1 are in flight while tile j is computed, and
+//     there is one workgroup barrier per tile.
+//   * every tile is stored row-major; 16-byte chunks are XOR-swizzled on the global-address side
+//     so that both read patterns below are bank-conflict free without padding.
+//   * K / K' fragments (contraction over d) are read with ds_read_b128; V / V' fragments
+//     (contraction over keys) with the transposing ds_read_b64_tr_b16, so V is never transposed
+//     in memory.
+#pragma once
+#include "common.hpp"
+#include "mask.hpp"
+#include "params.hpp"
+
+namespace jvpfa {
+
+#define JVPFA_LDS(T) __attribute__((address_space(3))) T *
+#define JVPFA_GLB(T) __attribute__((address_space(1))) T *
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <typename T, int D, bool DUAL> struct Fwd2Cfg {
+  static constexpr int NW = 4;
+  static constexpr int NT = NW * WAVE;
+  static constexpr int BM = NW * 32;
+  static constexpr int BN = 64;
+  static constexpr int CH = D * sizeof(T) / 16;       // 16-byte chunks per row
+  static constexpr int ROWB = D * sizeof(T);          // bytes per row
+  static constexpr int TILEB = BN * ROWB;             // bytes per tile
+  static constexpr int NTILE = DUAL ? 4 : 2;          // K, V (, K', V')
+  static constexpr int STAGEB = NTILE * TILEB;
+  static constexpr size_t LDS_BYTES = 2 * (size_t)STAGEB;
+  static constexpr int IPW = TILEB / 1024 / NW;       // direct-load instructions per wave per tile
+};
+
+// chunk swizzles (row -> xor value applied to the 16-byte chunk index)
+template <int CH> __device__ __forceinline__ int swz_k(int row) { return CH == 16 ? (row & 15) : ((row >> 1) & 7); }
+template <int CH> __device__ __forceinline__ int swz_v(int row) { return CH == 16 ? ((row & 7) << 1) : (((row >> 1) & 3) << 1); }
+
+template <typename T, int D, bool DUAL, int MASK>
+__global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
+  using Cfg = Fwd2Cfg<T, D, DUAL>;
+  constexpr int BN = Cfg::BN, CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW;
+  constexpr int NB = BN / 32, KK = D / 16, DB = D / 32;
+  constexpr float NEG_INF = -__builtin_inff();
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+  // stage s: [K | V | K' | V'] each TILEB bytes
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem_raw;
+
+  const Problem &pr = p.pr;
+  const int L = pr.L;
+  const int nqb = (L + Cfg::BM - 1) / Cfg::BM;
+  const int total = nqb * pr.Z * pr.H;
+  const int id = xcd_remap(blockIdx.x, total);
+  const int zh = id / nqb;
+  const int qb = pr.causal ? nqb - 1 - id % nqb : id % nqb;
+  const int z = zh / pr.H, h = zh % pr.H;
+
+  const int tid = threadIdx.x;
+  const int wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 32, g = lane / 32;
+  const int pr32 = perm32(r);
+
+  const size_t head = (size_t)zh * L * D;
+  const T *Qg = reinterpret_cast<const T *>(p.q) + head;
+  const T *Kg = reinterpret_cast<const T *>(p.k) + head;
+  const T *Vg = reinterpret_cast<const T *>(p.v) + head;
+  const T *Qtg = DUAL ? reinterpret_cast<const T *>(p.qt) + head : nullptr;
+  const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + head : nullptr;
+  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + head : nullptr;
+
+  const int q0 = qb * Cfg::BM;
+  const int qrow = q0 + wave * 32 + r;
+  const int qld = qrow < L ? qrow : L - 1;
+
+  // ---- per-lane constants of the direct loads: instruction i of this wave fills LDS chunks
+  // 64*(wave*IPW+i) .. +63 of a tile; this lane's chunk holds (row, logical chunk c).
+  int ld_row[IPW], ld_ck[IPW], ld_cv[IPW];
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) {
+    const int lc = 64 * (wave * IPW + i) + lane;
+    const int row = lc / CH, cp = lc % CH;
+    ld_row[i] = row;
+    ld_ck[i] = (cp ^ swz_k<CH>(row)) * 8;  // element offset within the row, K-type tiles
+    ld_cv[i] = (cp ^ swz_v<CH>(row)) * 8;  // V-type tiles
+  }
+  auto issue_loads = [&](int stage, int j0) {
+    const uint32_t sbase = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
+#pragma unroll
+    for (int i = 0; i < IPW; ++i) {
+      int grow = j0 + ld_row[i];
+      grow = grow < L ? grow : L - 1;  // rows past the end re-read the last row; their scores are masked
+      const size_t ok = (size_t)grow * D + ld_ck[i], ov = (size_t)grow * D + ld_cv[i];
+      const uint32_t dst = sbase + i * 1024;
+      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(Kg + ok), (JVPFA_LDS(void))(uintptr_t)(dst), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(Vg + ov), (JVPFA_LDS(void))(uintptr_t)(dst + TILEB), 16, 0, 0);
+      if constexpr (DUAL) {
+        __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(Ktg + ok), (JVPFA_LDS(void))(uintptr_t)(dst + 2 * TILEB), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(Vtg + ov), (JVPFA_LDS(void))(uintptr_t)(dst + 3 * TILEB), 16, 0, 0);
+      }
+    }
+  };
+
+  // ---- per-lane LDS read offsets (bytes within a tile)
+  // K-type: row 32nb + perm32(r), logical chunk 2kk + g
+  uint32_t koff[KK];
+  {
+    const int x = swz_k<CH>(pr32);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) koff[kk] = pr32 * ROWB + (((2 * kk + g) ^ x) * 16);
+  }
+  // V-type (transposing read): lane = 32g + 16a + j; it addresses key row 8g + 4hh + j/4 (+16c) and
+  // the 8-byte half (j>>1)&1 of logical chunk 4db + 2a + (j&1); it receives keys 16c+8g+4hh+(0..3)
+  // at d = 32db + perm32(16a + j).
+  uint32_t voff[DB][2];
+  {
+    const int a = (lane >> 4) & 1, j = lane & 15;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int row = 8 * g + 4 * hh + (j >> 2);
+        const int ch = (4 * db + 2 * a + (j & 1)) ^ swz_v<CH>(row);
+        voff[db][hh] = row * ROWB + ch * 16 + 8 * ((j >> 1) & 1);
+      }
+    }
+  }
+
+  Frag<T> Qf[KK], Qtf[DUAL ? KK : 1];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    Qf[kk] = ld8<T>(Qg + (size_t)qld * D + 16 * kk + 8 * g);
+    if constexpr (DUAL) Qtf[kk] = ld8<T>(Qtg + (size_t)qld * D + 16 * kk + 8 * g);
+  }
+
+  f32x16 Oacc[DB], Tacc[DUAL ? DB : 1];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      Oacc[db][e] = 0.f;
+      if constexpr (DUAL) Tacc[db][e] = 0.f;
+    }
+  }
+  float m_i = NEG_INF, l_i = 0.f, mu_i = 0.f;
+
+  const float sl2 = pr.scale * LOG2E;
+  const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
+
+  int kend = L;
+  if (pr.causal) kend = min(L, q0 + Cfg::BM);
+  const int ntiles = (kend + BN - 1) / BN;
+
+  issue_loads(0, 0);
+  for (int t = 0; t < ntiles; ++t) {
+    const int j0 = t * BN;
+    const int stage = t & 1;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
+    __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
+    if (t + 1 < ntiles) issue_loads(stage ^ 1, j0 + BN);
+
+    const uint32_t sK = lds0 + stage * Cfg::STAGEB, sV = sK + TILEB, sKt = sK + 2 * TILEB, sVt = sK + 3 * TILEB;
+
+    // ---- S^T = K Q^T and S'^T = K Q'^T + K' Q^T -------------------------------------------
+    f32x16 S[NB], Sp[DUAL ? NB : 1];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        S[nb][e] = 0.f;
+        if constexpr (DUAL) Sp[nb][e] = 0.f;
+      }
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        const uint32_t o = nb * 32 * ROWB + koff[kk];
+        Frag<T> a = *(JVPFA_LDS(const Frag<T>))(uintptr_t)(sK + o);
+        mma(S[nb], a, Qf[kk]);
+        if constexpr (DUAL) {
+          mma(Sp[nb], a, Qtf[kk]);
+          Frag<T> a2 = *(JVPFA_LDS(const Frag<T>))(uintptr_t)(sKt + o);
+          mma(Sp[nb], a2, Qf[kk]);
+        }
+      }
+    }
+
+    // ---- online softmax (log2 domain) -------------------------------------------------------
+    const bool diag = pr.causal && (j0 + BN - 1 > q0 + wave * 32);
+    const bool ragged = j0 + BN > L;
+    float m_new, m_use;
+    if (MASK != MASK_NONE || diag || ragged) {
+      float mx = NEG_INF;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          const int key0 = j0 + 32 * nb + 16 * hf + 8 * g;
+          float bias[8];
+          bool keep[8];
+          if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
+          if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float s = S[nb][8 * hf + e] * sl2;
+            if constexpr (MASK == MASK_ADD) s += bias[e];
+            if constexpr (MASK == MASK_BOOL) s = keep[e] ? s : NEG_INF;
+            if (diag) s = (key0 + e <= qrow) ? s : NEG_INF;
+            if (ragged) s = (key0 + e < L) ? s : NEG_INF;
+            S[nb][8 * hf + e] = s;
+            mx = fmaxf(mx, s);
+          }
+        }
+      }
+      mx = fmaxf(mx, xor32(mx));
+      m_new = fmaxf(m_i, mx);
+      m_use = (m_new == NEG_INF) ? 0.f : m_new;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[nb][e] = fast_exp2(S[nb][e] - m_use);
+      }
+    } else {
+      float mx = S[0][0];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, S[nb][e]);
+      }
+      mx = fmaxf(mx, xor32(mx));
+      m_new = fmaxf(m_i, mx * sl2);  // sl2 > 0 is not assumed: fall back below if it is not
+      if (sl2 < 0.f) {
+        float mn = S[0][0];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) mn = fminf(mn, S[nb][e]);
+        }
+        mn = fminf(mn, xor32(mn));
+        m_new = fmaxf(m_i, mn * sl2);
+      }
+      m_use = m_new;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[nb][e] = fast_exp2(__builtin_fmaf(S[nb][e], sl2, -m_use));
+      }
+    }
+    const float alpha = fast_exp2(m_i - m_use);
+    float rs = 0.f, rmu = 0.f;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        rs += S[nb][e];
+        if constexpr (DUAL) {
+          const float ps = S[nb][e] * (Sp[nb][e] * pr.scale);
+          Sp[nb][e] = ps;
+          rmu += ps;
+        }
+      }
+    }
+    l_i = l_i * alpha + rs;
+    m_i = m_new;
+    if constexpr (DUAL) mu_i = mu_i * alpha + rmu;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        Oacc[db][e] *= alpha;
+        if constexpr (DUAL) Tacc[db][e] *= alpha;
+      }
+    }
+
+    // ---- O^T += V^T P^T,  T^T += V^T (P*S')^T + V'^T P^T -----------------------------------
+#pragma unroll
+    for (int c = 0; c < BN / 16; ++c) {
+      Frag<T> pf = to_frag<T>(S[c / 2], c % 2);
+      Frag<T> psf;
+      if constexpr (DUAL) psf = to_frag<T>(Sp[c / 2], c % 2);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        union { s16x4 h[2]; Frag<T> f; } va, vb;
+        const uint32_t o0 = c * 16 * ROWB + voff[db][0], o1 = c * 16 * ROWB + voff[db][1];
+        va.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sV + o0));
+        va.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sV + o1));
+        mma(Oacc[db], va.f, pf);
+        if constexpr (DUAL) {
+          mma(Tacc[db], va.f, psf);
+          vb.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sVt + o0));
+          vb.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sVt + o1));
+          mma(Tacc[db], vb.f, pf);
+        }
+      }
+    }
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------
+  l_i += xor32(l_i);
+  if constexpr (DUAL) mu_i += xor32(mu_i);
+  const bool dead = !(l_i > 0.f);
+  const float inv = dead ? 0.f : 1.f / l_i;
+  const float mu_n = mu_i * inv;
+  if (qrow < L) {
+    T *Og = reinterpret_cast<T *>(p.o) + head + (size_t)qrow * D;
+    T *Otg = DUAL ? reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D : nullptr;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        float o8[8], t8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          o8[e] = Oacc[db][8 * hf + e] * inv;
+          if constexpr (DUAL) t8[e] = Tacc[db][8 * hf + e] * inv - mu_n * o8[e];
+        }
+        const int d0 = 32 * db + 16 * hf + 8 * g;
+        store8<T>(Og + d0, o8);
+        if constexpr (DUAL) store8<T>(Otg + d0, t8);
+      }
+    }
+    if (g == 0) {
+      p.M[(size_t)zh * L + qrow] = dead ? __builtin_inff() : m_i + __builtin_amdgcn_logf(l_i);
+      if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = mu_n;
+    }
+  }
+}
+
+}  // namespace jvpfa
