@@ -61,6 +61,16 @@ template <typename T> __device__ __forceinline__ Frag<T> to_frag(const f32x16 &x
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+// Combine a value with the one held by the lane 32 away (the other half of a query column):
+// v_permlane32_swap of x with itself returns (lower half broadcast, upper half broadcast).
+__device__ __forceinline__ float pair_max(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 // Eight consecutive elements from a 16-byte aligned address (LDS or global).
 template <typename T> __device__ __forceinline__ Frag<T> ld8(const T *p) {

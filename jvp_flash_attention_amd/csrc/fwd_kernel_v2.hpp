@@ -156,135 +156,104 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   if (pr.causal) kend = min(L, q0 + Cfg::BM);
   const int ntiles = (kend + BN - 1) / BN;
 
-  issue_loads(0, 0);
-  for (int t = 0; t < ntiles; ++t) {
-    const int j0 = t * BN;
-    const int stage = t & 1;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
-    __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
-    if (t + 1 < ntiles) issue_loads(stage ^ 1, j0 + BN);
-
-    const uint32_t sK = lds0 + stage * Cfg::STAGEB, sV = sK + TILEB, sKt = sK + 2 * TILEB, sVt = sK + 3 * TILEB;
-
-    // ---- S^T = K Q^T and S'^T = K Q'^T + K' Q^T -------------------------------------------
-    f32x16 S[NB], Sp[DUAL ? NB : 1];
+  // Half-tile body: 32 keys starting at key index jh, read from the tile at LDS byte address sK
+  // (K-type tiles) / sV (V-type tiles) with row offset hb*32 inside the tile.
+  //
+  // Rescaling is lazy: the reference point m_i of the exponentials only moves when some row's new
+  // maximum exceeds it by more than RESCALE_TAU (log2 units), so p <= 2^TAU and the accumulators,
+  // which live in the matrix-core accumulation registers, are touched by VALU code only on the few
+  // tiles where the running maximum really grows.  O = acc / l is unchanged by the choice of m_i.
+  constexpr float RESCALE_TAU = 8.f;
+  auto half_tile = [&](uint32_t sK, uint32_t sV, uint32_t sKt, uint32_t sVt, int hb, int jh) {
+    f32x16 S, Sp;
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
+    for (int e = 0; e < 16; ++e) {
+      S[e] = 0.f;
+      Sp[e] = 0.f;
+    }
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        S[nb][e] = 0.f;
-        if constexpr (DUAL) Sp[nb][e] = 0.f;
-      }
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        const uint32_t o = nb * 32 * ROWB + koff[kk];
-        Frag<T> a = *(JVPFA_LDS(const Frag<T>))(uintptr_t)(sK + o);
-        mma(S[nb], a, Qf[kk]);
-        if constexpr (DUAL) {
-          mma(Sp[nb], a, Qtf[kk]);
-          Frag<T> a2 = *(JVPFA_LDS(const Frag<T>))(uintptr_t)(sKt + o);
-          mma(Sp[nb], a2, Qf[kk]);
-        }
+    for (int kk = 0; kk < KK; ++kk) {
+      const uint32_t o = hb * 32 * ROWB + koff[kk];
+      Frag<T> a = *(JVPFA_LDS(const Frag<T>))(uintptr_t)(sK + o);
+      mma(S, a, Qf[kk]);
+      if constexpr (DUAL) {
+        mma(Sp, a, Qtf[kk]);
+        Frag<T> a2 = *(JVPFA_LDS(const Frag<T>))(uintptr_t)(sKt + o);
+        mma(Sp, a2, Qf[kk]);
       }
     }
 
-    // ---- online softmax (log2 domain) -------------------------------------------------------
-    const bool diag = pr.causal && (j0 + BN - 1 > q0 + wave * 32);
-    const bool ragged = j0 + BN > L;
-    float m_new, m_use;
-    if (MASK != MASK_NONE || diag || ragged) {
-      float mx = NEG_INF;
+    const bool diag = pr.causal && (jh + 31 > q0 + wave * 32);
+    const bool ragged = jh + 32 > L;
+    float mx;
+    const bool general = MASK != MASK_NONE || diag || ragged || !(sl2 > 0.f);
+    if (general) {
+      mx = NEG_INF;
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
+      for (int hf = 0; hf < 2; ++hf) {
+        const int key0 = jh + 16 * hf + 8 * g;
+        float bias[8];
+        bool keep[8];
+        if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
+        if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-          const int key0 = j0 + 32 * nb + 16 * hf + 8 * g;
-          float bias[8];
-          bool keep[8];
-          if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
-          if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            float s = S[nb][8 * hf + e] * sl2;
-            if constexpr (MASK == MASK_ADD) s += bias[e];
-            if constexpr (MASK == MASK_BOOL) s = keep[e] ? s : NEG_INF;
-            if (diag) s = (key0 + e <= qrow) ? s : NEG_INF;
-            if (ragged) s = (key0 + e < L) ? s : NEG_INF;
-            S[nb][8 * hf + e] = s;
-            mx = fmaxf(mx, s);
-          }
+        for (int e = 0; e < 8; ++e) {
+          float s = S[8 * hf + e] * sl2;
+          if constexpr (MASK == MASK_ADD) s += bias[e];
+          if constexpr (MASK == MASK_BOOL) s = keep[e] ? s : NEG_INF;
+          if (diag) s = (key0 + e <= qrow) ? s : NEG_INF;
+          if (ragged) s = (key0 + e < L) ? s : NEG_INF;
+          S[8 * hf + e] = s;
+          mx = fmaxf(mx, s);
         }
       }
-      mx = fmaxf(mx, xor32(mx));
-      m_new = fmaxf(m_i, mx);
-      m_use = (m_new == NEG_INF) ? 0.f : m_new;
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) S[nb][e] = fast_exp2(S[nb][e] - m_use);
-      }
+      mx = pair_max(mx);
     } else {
-      float mx = S[0][0];
+      mx = S[0];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
+      for (int e = 1; e < 16; ++e) mx = fmaxf(mx, S[e]);
+      mx = pair_max(mx) * sl2;
+    }
+    if (__any(mx > m_i + RESCALE_TAU)) {
+      const float m_new = fmaxf(m_i, mx);
+      const float alpha = fast_exp2(m_i - ((m_new == NEG_INF) ? 0.f : m_new));
+      m_i = m_new;
+      l_i *= alpha;
+      if constexpr (DUAL) mu_i *= alpha;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, S[nb][e]);
-      }
-      mx = fmaxf(mx, xor32(mx));
-      m_new = fmaxf(m_i, mx * sl2);  // sl2 > 0 is not assumed: fall back below if it is not
-      if (sl2 < 0.f) {
-        float mn = S[0][0];
+      for (int db = 0; db < DB; ++db) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-          for (int e = 0; e < 16; ++e) mn = fminf(mn, S[nb][e]);
+        for (int e = 0; e < 16; ++e) {
+          Oacc[db][e] *= alpha;
+          if constexpr (DUAL) Tacc[db][e] *= alpha;
         }
-        mn = fminf(mn, xor32(mn));
-        m_new = fmaxf(m_i, mn * sl2);
-      }
-      m_use = m_new;
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) S[nb][e] = fast_exp2(__builtin_fmaf(S[nb][e], sl2, -m_use));
       }
     }
-    const float alpha = fast_exp2(m_i - m_use);
+    const float m_use = (m_i == NEG_INF) ? 0.f : m_i;
     float rs = 0.f, rmu = 0.f;
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        rs += S[nb][e];
-        if constexpr (DUAL) {
-          const float ps = S[nb][e] * (Sp[nb][e] * pr.scale);
-          Sp[nb][e] = ps;
-          rmu += ps;
-        }
+    for (int e = 0; e < 16; ++e) {
+      const float pv = general ? fast_exp2(S[e] - m_use) : fast_exp2(__builtin_fmaf(S[e], sl2, -m_use));
+      S[e] = pv;
+      rs += pv;
+      if constexpr (DUAL) {
+        const float ps = pv * (Sp[e] * pr.scale);
+        Sp[e] = ps;
+        rmu += ps;
       }
     }
-    l_i = l_i * alpha + rs;
-    m_i = m_new;
-    if constexpr (DUAL) mu_i = mu_i * alpha + rmu;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        Oacc[db][e] *= alpha;
-        if constexpr (DUAL) Tacc[db][e] *= alpha;
-      }
-    }
+    l_i += rs;
+    if constexpr (DUAL) mu_i += rmu;
 
-    // ---- O^T += V^T P^T,  T^T += V^T (P*S')^T + V'^T P^T -----------------------------------
 #pragma unroll
-    for (int c = 0; c < BN / 16; ++c) {
-      Frag<T> pf = to_frag<T>(S[c / 2], c % 2);
+    for (int c = 0; c < 2; ++c) {
+      Frag<T> pf = to_frag<T>(S, c);
       Frag<T> psf;
-      if constexpr (DUAL) psf = to_frag<T>(Sp[c / 2], c % 2);
+      if constexpr (DUAL) psf = to_frag<T>(Sp, c);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         union { s16x4 h[2]; Frag<T> f; } va, vb;
-        const uint32_t o0 = c * 16 * ROWB + voff[db][0], o1 = c * 16 * ROWB + voff[db][1];
+        const uint32_t o0 = (hb * 32 + c * 16) * ROWB + voff[db][0], o1 = (hb * 32 + c * 16) * ROWB + voff[db][1];
         va.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sV + o0));
         va.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sV + o1));
         mma(Oacc[db], va.f, pf);
@@ -296,6 +265,18 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
         }
       }
     }
+  };
+
+  issue_loads(0, 0);
+  for (int t = 0; t < ntiles; ++t) {
+    const int j0 = t * BN;
+    const int stage = t & 1;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
+    __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
+    if (t + 1 < ntiles) issue_loads(stage ^ 1, j0 + BN);
+    const uint32_t sK = lds0 + stage * Cfg::STAGEB, sV = sK + TILEB, sKt = sK + 2 * TILEB, sVt = sK + 3 * TILEB;
+    half_tile(sK, sV, sKt, sVt, 0, j0);
+    if (j0 + 32 < kend) half_tile(sK, sV, sKt, sVt, 1, j0 + 32);
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------
