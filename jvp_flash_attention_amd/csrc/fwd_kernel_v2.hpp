@@ -12,6 +12,8 @@
 //     (contraction over keys) with the transposing ds_read_b64_tr_b16, so V is never transposed
 //     in memory.
 #pragma once
+#include <utility>
+
 #include "common.hpp"
 #include "mask.hpp"
 #include "params.hpp"
@@ -22,6 +24,41 @@ namespace jvpfa {
 #define JVPFA_GLB(T) __attribute__((address_space(1))) T *
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <int... Is, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F &&f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), fully unrolled
+template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F &&>(f));
+}
+
+// LDS reads whose issue point is fixed by the program text (not by the scheduler).  The data is
+// valid only after an lds_wait<N>() on the same registers, N = number of such reads issued after
+// the one waited for (LDS reads complete in issue order).
+template <int OFF> __device__ __forceinline__ u32x4 lds_b128(uint32_t addr) {
+  u32x4 d;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(d) : "v"(addr), "n"(OFF));
+  return d;
+}
+template <int OFF> __device__ __forceinline__ u32x2 lds_tr64(uint32_t addr) {
+  u32x2 d;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(d) : "v"(addr), "n"(OFF));
+  return d;
+}
+template <int N> __device__ __forceinline__ void lds_wait(u32x4 &a) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait(u32x4 &a, u32x4 &b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait(u32x2 &a, u32x2 &b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait(u32x2 &a, u32x2 &b, u32x2 &c, u32x2 &d) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
 
 template <typename T, int D, bool DUAL> struct Fwd2Cfg {
   static constexpr int NW = 4;
@@ -156,32 +193,68 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   if (pr.causal) kend = min(L, q0 + Cfg::BM);
   const int ntiles = (kend + BN - 1) / BN;
 
-  // Half-tile body: 32 keys starting at key index jh, read from the tile at LDS byte address sK
-  // (K-type tiles) / sV (V-type tiles) with row offset hb*32 inside the tile.
+  // Half-tile body: the 32 keys HB*32 .. HB*32+31 of the tile staged at LDS byte address sbase
+  // (layout [K | V | K' | V']); jh is the index of its first key.
+  //
+  // LDS fragment reads are issued two steps ahead of the matrix products that consume them (a ring
+  // of three fragment buffers), through inline asm so that their order and the waits are exactly
+  // the ones written here.
   //
   // Rescaling is lazy: the reference point m_i of the exponentials only moves when some row's new
   // maximum exceeds it by more than RESCALE_TAU (log2 units), so p <= 2^TAU and the accumulators,
   // which live in the matrix-core accumulation registers, are touched by VALU code only on the few
   // tiles where the running maximum really grows.  O = acc / l is unchanged by the choice of m_i.
   constexpr float RESCALE_TAU = 8.f;
-  auto half_tile = [&](uint32_t sK, uint32_t sV, uint32_t sKt, uint32_t sVt, int hb, int jh) {
+  auto half_tile = [&](auto HBc, uint32_t sbase, int jh) {
+    constexpr int HB = decltype(HBc)::value;
+    constexpr int KO = HB * 32 * ROWB;  // K at +0, K' at +2*TILEB, V at +TILEB, V' at +3*TILEB
+    constexpr int NRS = DUAL ? 2 : 1;   // LDS reads per S step
+    constexpr int NRV = DUAL ? 4 : 2;   // LDS reads per PV step
+    constexpr int NPV = 2 * DB;         // PV steps: (16-key chunk c, d-block db)
+
+    u32x4 ka[3], kb[3];
+    auto issue_k = [&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value;
+      const uint32_t ad = sbase + koff[kk];
+      ka[kk % 3] = lds_b128<KO>(ad);
+      if constexpr (DUAL) kb[kk % 3] = lds_b128<KO + 2 * TILEB>(ad);
+    };
+    u32x2 va[3][2], vb[3][2];
+    auto issue_v = [&](auto ic) {
+      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB;
+      constexpr int VO = TILEB + (HB * 32 + c * 16) * ROWB;
+      const uint32_t a0 = sbase + voff[db][0], a1 = sbase + voff[db][1];
+      va[i % 3][0] = lds_tr64<VO>(a0);
+      va[i % 3][1] = lds_tr64<VO>(a1);
+      if constexpr (DUAL) {
+        vb[i % 3][0] = lds_tr64<VO + 2 * TILEB>(a0);
+        vb[i % 3][1] = lds_tr64<VO + 2 * TILEB>(a1);
+      }
+    };
+
     f32x16 S, Sp;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       S[e] = 0.f;
       Sp[e] = 0.f;
     }
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      const uint32_t o = hb * 32 * ROWB + koff[kk];
-      Frag<T> a = *(JVPFA_LDS(const Frag<T>))(uintptr_t)(sK + o);
+    issue_k(std::integral_constant<int, 0>{});
+    issue_k(std::integral_constant<int, 1>{});
+    static_for<KK>([&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value;
+      if constexpr (DUAL) lds_wait<(kk + 1 < KK) ? NRS : 0>(ka[kk % 3], kb[kk % 3]);
+      else lds_wait<(kk + 1 < KK) ? NRS : 0>(ka[kk % 3]);
+      if constexpr (kk + 2 < KK) issue_k(std::integral_constant<int, kk + 2>{});
+      const Frag<T> a = __builtin_bit_cast(Frag<T>, ka[kk % 3]);
       mma(S, a, Qf[kk]);
       if constexpr (DUAL) {
         mma(Sp, a, Qtf[kk]);
-        Frag<T> a2 = *(JVPFA_LDS(const Frag<T>))(uintptr_t)(sKt + o);
-        mma(Sp, a2, Qf[kk]);
+        mma(Sp, __builtin_bit_cast(Frag<T>, kb[kk % 3]), Qf[kk]);
       }
-    }
+    });
+    // V fragments of the first two PV steps travel while the softmax runs
+    issue_v(std::integral_constant<int, 0>{});
+    issue_v(std::integral_constant<int, 1>{});
 
     const bool diag = pr.causal && (jh + 31 > q0 + wave * 32);
     const bool ragged = jh + 32 > L;
@@ -245,26 +318,26 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     l_i += rs;
     if constexpr (DUAL) mu_i += rmu;
 
+    Frag<T> pf[2], psf[2];
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
-      Frag<T> pf = to_frag<T>(S, c);
-      Frag<T> psf;
-      if constexpr (DUAL) psf = to_frag<T>(Sp, c);
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        union { s16x4 h[2]; Frag<T> f; } va, vb;
-        const uint32_t o0 = (hb * 32 + c * 16) * ROWB + voff[db][0], o1 = (hb * 32 + c * 16) * ROWB + voff[db][1];
-        va.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sV + o0));
-        va.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sV + o1));
-        mma(Oacc[db], va.f, pf);
-        if constexpr (DUAL) {
-          mma(Tacc[db], va.f, psf);
-          vb.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sVt + o0));
-          vb.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((JVPFA_LDS(s16x4))(uintptr_t)(sVt + o1));
-          mma(Tacc[db], vb.f, pf);
-        }
-      }
+      pf[c] = to_frag<T>(S, c);
+      if constexpr (DUAL) psf[c] = to_frag<T>(Sp, c);
     }
+    static_for<NPV>([&](auto ic) {
+      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % 3;
+      if constexpr (DUAL) lds_wait<(i + 1 < NPV) ? NRV : 0>(va[sl][0], va[sl][1], vb[sl][0], vb[sl][1]);
+      else lds_wait<(i + 1 < NPV) ? NRV : 0>(va[sl][0], va[sl][1]);
+      if constexpr (i + 2 < NPV) issue_v(std::integral_constant<int, i + 2>{});
+      const u32x4 av = {va[sl][0][0], va[sl][0][1], va[sl][1][0], va[sl][1][1]};
+      const Frag<T> a = __builtin_bit_cast(Frag<T>, av);
+      mma(Oacc[db], a, pf[c]);
+      if constexpr (DUAL) {
+        mma(Tacc[db], a, psf[c]);
+        const u32x4 bv = {vb[sl][0][0], vb[sl][0][1], vb[sl][1][0], vb[sl][1][1]};
+        mma(Tacc[db], __builtin_bit_cast(Frag<T>, bv), pf[c]);
+      }
+    });
   };
 
   issue_loads(0, 0);
@@ -274,9 +347,9 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
     if (t + 1 < ntiles) issue_loads(stage ^ 1, j0 + BN);
-    const uint32_t sK = lds0 + stage * Cfg::STAGEB, sV = sK + TILEB, sKt = sK + 2 * TILEB, sVt = sK + 3 * TILEB;
-    half_tile(sK, sV, sKt, sVt, 0, j0);
-    if (j0 + 32 < kend) half_tile(sK, sV, sKt, sVt, 1, j0 + 32);
+    const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
+    half_tile(std::integral_constant<int, 0>{}, sbase, j0);
+    if (j0 + 32 < kend) half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------
