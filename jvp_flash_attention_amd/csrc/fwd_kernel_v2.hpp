@@ -47,6 +47,15 @@ template <int OFF> __device__ __forceinline__ u32x2 lds_tr64(uint32_t addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(d) : "v"(addr), "n"(OFF));
   return d;
 }
+// x * alpha for a value that lives in a matrix-core accumulation register, done where it stands:
+// the value never changes register class, so code paths that do not rescale carry no copies.
+__device__ __forceinline__ float acc_scale(float x, float alpha) {
+  float t;
+  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 1"
+               : "+a"(x), "=&v"(t)
+               : "v"(alpha));
+  return x;
+}
 template <int N> __device__ __forceinline__ void lds_wait(u32x4 &a) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
 }
@@ -117,28 +126,41 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
 
   // ---- per-lane constants of the direct loads: instruction i of this wave fills LDS chunks
   // 64*(wave*IPW+i) .. +63 of a tile; this lane's chunk holds (row, logical chunk c).
-  int ld_row[IPW], ld_ck[IPW], ld_cv[IPW];
+  // Byte offsets inside a full tile are per-lane constants, so a load is "uniform tile pointer +
+  // 32-bit lane offset"; only a ragged last tile recomputes them with the row clamped to L-1.
+  int ld_row[IPW];
+  uint32_t ld_ck[IPW], ld_cv[IPW], ld_bk[IPW], ld_bv[IPW];
 #pragma unroll
   for (int i = 0; i < IPW; ++i) {
     const int lc = 64 * (wave * IPW + i) + lane;
     const int row = lc / CH, cp = lc % CH;
     ld_row[i] = row;
-    ld_ck[i] = (cp ^ swz_k<CH>(row)) * 8;  // element offset within the row, K-type tiles
-    ld_cv[i] = (cp ^ swz_v<CH>(row)) * 8;  // V-type tiles
+    ld_ck[i] = (cp ^ swz_k<CH>(row)) * 16;  // byte offset within the row, K-type tiles
+    ld_cv[i] = (cp ^ swz_v<CH>(row)) * 16;  // V-type tiles
+    ld_bk[i] = row * ROWB + ld_ck[i];
+    ld_bv[i] = row * ROWB + ld_cv[i];
   }
   auto issue_loads = [&](int stage, int j0) {
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
+    const size_t tb = (size_t)j0 * ROWB;
+    const char *kp = reinterpret_cast<const char *>(Kg) + tb, *vp = reinterpret_cast<const char *>(Vg) + tb;
+    const char *ktp = DUAL ? reinterpret_cast<const char *>(Ktg) + tb : nullptr;
+    const char *vtp = DUAL ? reinterpret_cast<const char *>(Vtg) + tb : nullptr;
+    const bool ragged_tile = j0 + BN > L;
 #pragma unroll
     for (int i = 0; i < IPW; ++i) {
-      int grow = j0 + ld_row[i];
-      grow = grow < L ? grow : L - 1;  // rows past the end re-read the last row; their scores are masked
-      const size_t ok = (size_t)grow * D + ld_ck[i], ov = (size_t)grow * D + ld_cv[i];
+      uint32_t ok = ld_bk[i], ov = ld_bv[i];
+      if (ragged_tile) {  // rows past the end re-read the last row; their scores are masked
+        const int row = min(ld_row[i], L - 1 - j0);
+        ok = row * ROWB + ld_ck[i];
+        ov = row * ROWB + ld_cv[i];
+      }
       const uint32_t dst = sbase + i * 1024;
-      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(Kg + ok), (JVPFA_LDS(void))(uintptr_t)(dst), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(Vg + ov), (JVPFA_LDS(void))(uintptr_t)(dst + TILEB), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(kp + ok), (JVPFA_LDS(void))(uintptr_t)(dst), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(vp + ov), (JVPFA_LDS(void))(uintptr_t)(dst + TILEB), 16, 0, 0);
       if constexpr (DUAL) {
-        __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(Ktg + ok), (JVPFA_LDS(void))(uintptr_t)(dst + 2 * TILEB), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(Vtg + ov), (JVPFA_LDS(void))(uintptr_t)(dst + 3 * TILEB), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(ktp + ok), (JVPFA_LDS(void))(uintptr_t)(dst + 2 * TILEB), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(vtp + ov), (JVPFA_LDS(void))(uintptr_t)(dst + 3 * TILEB), 16, 0, 0);
       }
     }
   };
@@ -252,10 +274,6 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
         mma(Sp, __builtin_bit_cast(Frag<T>, kb[kk % 3]), Qf[kk]);
       }
     });
-    // V fragments of the first two PV steps travel while the softmax runs
-    issue_v(std::integral_constant<int, 0>{});
-    issue_v(std::integral_constant<int, 1>{});
-
     const bool diag = pr.causal && (jh + 31 > q0 + wave * 32);
     const bool ragged = jh + 32 > L;
     float mx;
@@ -297,20 +315,29 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       for (int db = 0; db < DB; ++db) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          Oacc[db][e] *= alpha;
-          if constexpr (DUAL) Tacc[db][e] *= alpha;
+          Oacc[db][e] = acc_scale(Oacc[db][e], alpha);
+          if constexpr (DUAL) Tacc[db][e] = acc_scale(Tacc[db][e], alpha);
         }
       }
     }
+    // V fragments of the first two PV steps travel while the softmax runs
+    issue_v(std::integral_constant<int, 0>{});
+    issue_v(std::integral_constant<int, 1>{});
+
     const float m_use = (m_i == NEG_INF) ? 0.f : m_i;
     float rs = 0.f, rmu = 0.f;
+    if (general) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) S[e] = fast_exp2(S[e] - m_use);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) S[e] = fast_exp2(__builtin_fmaf(S[e], sl2, -m_use));
+    }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const float pv = general ? fast_exp2(S[e] - m_use) : fast_exp2(__builtin_fmaf(S[e], sl2, -m_use));
-      S[e] = pv;
-      rs += pv;
+      rs += S[e];
       if constexpr (DUAL) {
-        const float ps = pv * (Sp[e] * pr.scale);
+        const float ps = S[e] * (Sp[e] * pr.scale);
         Sp[e] = ps;
         rmu += ps;
       }
