@@ -20,6 +20,16 @@
 
 namespace jvpfa {
 
+#ifdef JVPFA_TRACE
+__device__ long long *g_trace = nullptr;  // debugging aid: time stamps of one wave
+#define JVPFA_STAMP(slot)                                                        \
+  do {                                                                           \
+    if (g_trace && blockIdx.x == 0 && threadIdx.x == 0 && trace_n < 4096) g_trace[trace_n++] = ((long long)(slot) << 48) | (clock64() & 0xffffffffffffLL); \
+  } while (0)
+#else
+#define JVPFA_STAMP(slot) do {} while (0)
+#endif
+
 #define JVPFA_LDS(T) __attribute__((address_space(3))) T *
 #define JVPFA_GLB(T) __attribute__((address_space(1))) T *
 
@@ -94,6 +104,8 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   constexpr int NB = BN / 32, KK = D / 16, DB = D / 32;
   constexpr float NEG_INF = -__builtin_inff();
 
+  int trace_n = 0;
+  (void)trace_n;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   // stage s: [K | V | K' | V'] each TILEB bytes
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem_raw;
@@ -215,6 +227,44 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   if (pr.causal) kend = min(L, q0 + Cfg::BM);
   const int ntiles = (kend + BN - 1) / BN;
 
+  // The loads of the next tile are not issued in one burst (the vector-memory queue would back up
+  // and stall this wave for longer than a whole GEMM phase) but one instruction at a time, spread
+  // over the steps of the current tile's matrix products.
+  constexpr int NLOAD = IPW * Cfg::NTILE;      // direct-load instructions per wave per tile
+  constexpr int NSTEP = 2 * (KK + 2 * DB);     // S and PV steps of the two half tiles
+  bool ld_on = false, ld_rag = false;
+  int ld_rows = 0;
+  uint32_t ld_dst = 0;
+  const char *ld_p[4] = {nullptr, nullptr, nullptr, nullptr};
+  auto prepare_loads = [&](int stage, int j0, bool on) {
+    ld_on = on;
+    ld_rag = j0 + BN > L;
+    ld_rows = L - 1 - j0;
+    ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
+    const size_t tb = (size_t)j0 * ROWB;
+    ld_p[0] = reinterpret_cast<const char *>(Kg) + tb;
+    ld_p[1] = reinterpret_cast<const char *>(Vg) + tb;
+    if constexpr (DUAL) {
+      ld_p[2] = reinterpret_cast<const char *>(Ktg) + tb;
+      ld_p[3] = reinterpret_cast<const char *>(Vtg) + tb;
+    }
+  };
+  auto load_piece = [&](auto pc) {
+    constexpr int pi = decltype(pc)::value, i = pi / Cfg::NTILE, ts = pi % Cfg::NTILE;
+    if (ld_on) {
+      uint32_t off = (ts & 1) ? ld_bv[i] : ld_bk[i];
+      if (ld_rag) off = min(ld_row[i], ld_rows) * ROWB + ((ts & 1) ? ld_cv[i] : ld_ck[i]);
+      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(ld_p[ts] + off),
+                                       (JVPFA_LDS(void))(uintptr_t)(ld_dst + i * 1024 + ts * TILEB), 16, 0, 0);
+    }
+  };
+  // pieces [ceil(g*NLOAD/NSTEP), ceil((g+1)*NLOAD/NSTEP)) belong to step g
+  auto load_step = [&](auto gc) {
+    constexpr int g = decltype(gc)::value;
+    constexpr int lo = (g * NLOAD + NSTEP - 1) / NSTEP, hi = ((g + 1) * NLOAD + NSTEP - 1) / NSTEP;
+    static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+  };
+
   // Half-tile body: the 32 keys HB*32 .. HB*32+31 of the tile staged at LDS byte address sbase
   // (layout [K | V | K' | V']); jh is the index of its first key.
   //
@@ -267,6 +317,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       if constexpr (DUAL) lds_wait<(kk + 1 < KK) ? NRS : 0>(ka[kk % 3], kb[kk % 3]);
       else lds_wait<(kk + 1 < KK) ? NRS : 0>(ka[kk % 3]);
       if constexpr (kk + 2 < KK) issue_k(std::integral_constant<int, kk + 2>{});
+      load_step(std::integral_constant<int, HB * (KK + NPV) + kk>{});
       const Frag<T> a = __builtin_bit_cast(Frag<T>, ka[kk % 3]);
       mma(S, a, Qf[kk]);
       if constexpr (DUAL) {
@@ -274,6 +325,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
         mma(Sp, __builtin_bit_cast(Frag<T>, kb[kk % 3]), Qf[kk]);
       }
     });
+    JVPFA_STAMP(5);
     const bool diag = pr.causal && (jh + 31 > q0 + wave * 32);
     const bool ragged = jh + 32 > L;
     float mx;
@@ -345,6 +397,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     l_i += rs;
     if constexpr (DUAL) mu_i += rmu;
 
+    JVPFA_STAMP(6);
     Frag<T> pf[2], psf[2];
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
@@ -356,6 +409,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       if constexpr (DUAL) lds_wait<(i + 1 < NPV) ? NRV : 0>(va[sl][0], va[sl][1], vb[sl][0], vb[sl][1]);
       else lds_wait<(i + 1 < NPV) ? NRV : 0>(va[sl][0], va[sl][1]);
       if constexpr (i + 2 < NPV) issue_v(std::integral_constant<int, i + 2>{});
+      load_step(std::integral_constant<int, HB * (KK + NPV) + KK + i>{});
       const u32x4 av = {va[sl][0][0], va[sl][0][1], va[sl][1][0], va[sl][1][1]};
       const Frag<T> a = __builtin_bit_cast(Frag<T>, av);
       mma(Oacc[db], a, pf[c]);
@@ -365,18 +419,26 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
         mma(Tacc[db], __builtin_bit_cast(Frag<T>, bv), pf[c]);
       }
     });
+    JVPFA_STAMP(7);
   };
 
   issue_loads(0, 0);
   for (int t = 0; t < ntiles; ++t) {
     const int j0 = t * BN;
     const int stage = t & 1;
+    JVPFA_STAMP(1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
+    JVPFA_STAMP(2);
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
-    if (t + 1 < ntiles) issue_loads(stage ^ 1, j0 + BN);
+    JVPFA_STAMP(3);
+    prepare_loads(stage ^ 1, j0 + BN, t + 1 < ntiles);
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
     half_tile(std::integral_constant<int, 0>{}, sbase, j0);
-    if (j0 + 32 < kend) half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
+    if (j0 + 32 < kend) {
+      half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
+    } else {  // second half skipped (end of a ragged or causal row block): issue its share of the loads
+      static_for<NSTEP / 2>([&](auto gc) { load_step(std::integral_constant<int, NSTEP / 2 + decltype(gc)::value>{}); });
+    }
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------
