@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   const int z = zh / pr.H, h = zh % pr.H;
 
   const int tid = threadIdx.x;
-  const int wave = tid / WAVE, lane = tid % WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;  // wave index is uniform
   const int r = lane % 32, g = lane / 32;
   const int pr32 = perm32(r);
 
@@ -232,14 +232,14 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   // over the steps of the current tile's matrix products.
   constexpr int NLOAD = IPW * Cfg::NTILE;      // direct-load instructions per wave per tile
   constexpr int NSTEP = 2 * (KK + 2 * DB);     // S and PV steps of the two half tiles
-  bool ld_on = false, ld_rag = false;
   int ld_rows = 0;
   uint32_t ld_dst = 0;
   const char *ld_p[4] = {nullptr, nullptr, nullptr, nullptr};
+  // Past the last tile the loads are pointed at tile 0 again (never read) instead of being
+  // predicated off, which keeps every step of the tile loop one straight-line block.
   auto prepare_loads = [&](int stage, int j0, bool on) {
-    ld_on = on;
-    ld_rag = j0 + BN > L;
-    ld_rows = L - 1 - j0;
+    j0 = on ? j0 : 0;
+    ld_rows = L - 1 - j0;  // rows past the end re-read the last row; their scores are masked
     ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
     const size_t tb = (size_t)j0 * ROWB;
     ld_p[0] = reinterpret_cast<const char *>(Kg) + tb;
@@ -251,12 +251,9 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   };
   auto load_piece = [&](auto pc) {
     constexpr int pi = decltype(pc)::value, i = pi / Cfg::NTILE, ts = pi % Cfg::NTILE;
-    if (ld_on) {
-      uint32_t off = (ts & 1) ? ld_bv[i] : ld_bk[i];
-      if (ld_rag) off = min(ld_row[i], ld_rows) * ROWB + ((ts & 1) ? ld_cv[i] : ld_ck[i]);
-      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(ld_p[ts] + off),
-                                       (JVPFA_LDS(void))(uintptr_t)(ld_dst + i * 1024 + ts * TILEB), 16, 0, 0);
-    }
+    const uint32_t off = min(ld_row[i], ld_rows) * ROWB + ((ts & 1) ? ld_cv[i] : ld_ck[i]);
+    __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(ld_p[ts] + off),
+                                     (JVPFA_LDS(void))(uintptr_t)(ld_dst + i * 1024 + ts * TILEB), 16, 0, 0);
   };
   // pieces [ceil(g*NLOAD/NSTEP), ceil((g+1)*NLOAD/NSTEP)) belong to step g
   auto load_step = [&](auto gc) {
