@@ -1,0 +1,129 @@
+"""The C ABI without a GPU: the library loads, exports every function ``include/jvpfa.h`` declares,
+its structs have the layout the ctypes binding assumes (checked against gcc compiling the header),
+and argument validation returns the documented codes before any HIP call is made."""
+import ctypes as C
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+from jvp_flash_attention_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "jvpfa.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(jvpfa_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_function():
+    lib = _lib.load()
+    names = _declared_functions()
+    assert set(names) == set(_lib.EXPORTS)
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert lib.jvpfa_abi_version() == _lib.ABI_VERSION
+
+
+def test_struct_layout_matches_the_header(tmp_path):
+    src = tmp_path / "layout.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "jvpfa.h"\n'
+        "int main(void){\n"
+        'printf("%zu %zu %zu\\n", sizeof(jvpfa_problem), sizeof(jvpfa_fwd_args), sizeof(jvpfa_bwd_args));\n'
+        'printf("%zu %zu %zu %zu\\n", offsetof(jvpfa_problem, sm_scale), offsetof(jvpfa_problem, mask), '
+        "offsetof(jvpfa_problem, mask_stride), offsetof(jvpfa_fwd_args, q));\n"
+        'printf("%zu %zu %zu\\n", offsetof(jvpfa_fwd_args, mu), offsetof(jvpfa_bwd_args, go), offsetof(jvpfa_bwd_args, workspace));\n'
+        "return 0;}\n"
+    )
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    got = [int(x) for x in out]
+    want = [
+        C.sizeof(_lib.Problem), C.sizeof(_lib.FwdArgs), C.sizeof(_lib.BwdArgs),
+        _lib.Problem.sm_scale.offset, _lib.Problem.mask.offset, _lib.Problem.mask_stride.offset, _lib.FwdArgs.q.offset,
+        _lib.FwdArgs.mu.offset, _lib.BwdArgs.go.offset, _lib.BwdArgs.workspace.offset,
+    ]
+    assert got == want
+
+
+def _fwd_args(**kw):
+    a = _lib.FwdArgs()
+    a.struct_size = C.sizeof(_lib.FwdArgs)
+    a.p.Z, a.p.H, a.p.L, a.p.D = 1, 1, 32, 64
+    a.p.dtype, a.p.causal, a.p.mask_kind, a.p.sm_scale = 0, 0, 0, 0.125
+    for name in ("q", "k", "v", "o", "M"):
+        setattr(a, name, 0x1000)
+    for k, v in kw.items():
+        if k.startswith("p_"):
+            setattr(a.p, k[2:], v)
+        else:
+            setattr(a, k, v)
+    return a
+
+
+@pytest.mark.parametrize(
+    "kw,code",
+    [
+        (dict(struct_size=4), -7),
+        (dict(q=None), -1),
+        (dict(p_D=48), -2),
+        (dict(p_L=0), -2),
+        (dict(p_dtype=5), -3),
+        (dict(p_mask_kind=1), -1),          # mask kind set, mask pointer NULL
+        (dict(p_mask_kind=1, p_mask=0x1000, p_causal=1), -5),
+        (dict(qt=0x1000), -1),              # tangents must come as a full set
+        (dict(qt=0x1000, kt=0x1000, vt=0x1000), -1),  # dual without ot / mu
+        (dict(q=0x1004), -4),
+    ],
+)
+def test_forward_argument_validation_codes(kw, code):
+    lib = _lib.load()
+    assert lib.jvpfa_fwd(C.byref(_fwd_args(**kw)), None) == code
+    assert lib.jvpfa_error_string(code).decode() not in ("ok", "unknown status")
+
+
+def test_backward_argument_validation_codes():
+    lib = _lib.load()
+    a = _lib.BwdArgs()
+    a.struct_size = C.sizeof(_lib.BwdArgs)
+    a.p.Z, a.p.H, a.p.L, a.p.D = 1, 1, 32, 64
+    a.p.sm_scale = 0.125
+    assert lib.jvpfa_bwd(C.byref(a), None) == -1
+    for name in ("q", "k", "v", "o", "M", "dq", "dk", "dv", "workspace"):
+        setattr(a, name, 0x1000)
+    assert lib.jvpfa_bwd(C.byref(a), None) == -1  # neither go nor gt
+    a.gt = 0x1000
+    assert lib.jvpfa_bwd(C.byref(a), None) == -1  # gt needs the tangent tensors, ot and mu
+    a.gt = None
+    a.go = 0x1000
+    a.dqt = 0x1000
+    assert lib.jvpfa_bwd(C.byref(a), None) == -1  # tangent gradients need gt (and all three)
+    a.dqt = None
+    a.struct_size = 8
+    assert lib.jvpfa_bwd(C.byref(a), None) == -7
+    assert lib.jvpfa_bwd(None, None) == -1
+    assert lib.jvpfa_bwd_workspace_bytes(2, 3, 5) == 3 * 32 * 4  # 30 rows padded to 32 floats per statistic
+    assert lib.jvpfa_bwd_workspace_bytes(0, 3, 5) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libjvpfa.so")
+    with pytest.raises(RuntimeError, match="no non-HIP fallback"):
+        _lib.load()
+
+
+def test_product_does_not_import_the_oracle():
+    code = "import sys, jvp_flash_attention_amd; sys.exit(1 if any(m == 'oracle' or m.startswith('oracle.') for m in sys.modules) else 0)"
+    assert subprocess.run([sys.executable, "-c", code], cwd=ROOT).returncode == 0
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "jvp_flash_attention_amd")):
+        for f in files:
+            if f.endswith(".py"):
+                assert "oracle" not in open(os.path.join(dirpath, f)).read().replace("oracle_backend", "")

@@ -1,0 +1,216 @@
+"""GPU tests of the Python surface (``attention``, ``JVPAttn.fwd_dual``) and of the BASELINE
+configurations at their full sizes.
+
+Small shapes are compared with the fp64 oracle directly.  At full size one (z, h) slab is compared
+with the oracle and the rest is covered by properties that do not depend on size: O' is linear in
+the tangents, a V'-only tangent gives O' = softmax(S) V', key order does not matter without a
+mask, causal rows do not see later keys (bit-exact against a run on the truncated sequence), and
+the different backward modes agree where the mathematics says they must.
+"""
+from functools import partial
+
+import numpy as np
+import pytest
+import torch
+import torch.autograd.forward_ad as fwAD
+
+from oracle import dense
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(got, ref):
+    got = got.detach().double().cpu().numpy() if isinstance(got, torch.Tensor) else got
+    ref = ref.detach().double().cpu().numpy() if isinstance(ref, torch.Tensor) else ref
+    assert np.isfinite(got).all()
+    return np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30)
+
+
+def _randn(shape, dtype, seed, std=1.0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return (torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * std).to(dtype)
+
+
+@pytest.mark.parametrize("dt,tol", [(torch.float32, None), (torch.bfloat16, 2e-2), (torch.float16, 2e-2)])
+@pytest.mark.parametrize("mode", ["none", "causal", "keypad", "bias"])
+def test_surface_three_way_and_gradients(dt, tol, mode):
+    """fwAD route, torch.func.jvp route and autograd, all through the public functions."""
+    from jvp_flash_attention_amd import JVPAttn
+
+    Z, H, L, D = 2, 2, 128, 64
+    q, k, v, qt, kt, vt, go, gt = [_randn((Z, H, L, D), dt, 10 + i) for i in range(8)]
+    mask, causal = None, mode == "causal"
+    if mode == "keypad":
+        lens = torch.tensor([80, 128], device="cuda")
+        mask = (torch.arange(L, device="cuda")[None, :] < lens[:, None]).view(Z, 1, 1, L)
+    if mode == "bias":
+        mask = _randn((Z, H, L, L), dt, 99)
+    npm = None if mask is None else (mask.cpu().numpy() if mask.dtype == torch.bool else mask.double().cpu().numpy())
+    f64 = [x.double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    ref = dense.forward(*f64[:6], mask=npm, causal=causal)
+    rb = dense.backward(*f64, mask=npm, causal=causal)
+    fn = partial(JVPAttn.fwd_dual, attn_mask=mask, causal=causal)
+
+    leaves = [x.clone().requires_grad_() for x in (q, k, v, qt, kt, vt)]
+    with fwAD.dual_level():
+        out = fn(*(fwAD.make_dual(p, t) for p, t in zip(leaves[:3], leaves[3:])))
+        o1, ot1 = fwAD.unpack_dual(out)
+        loss = (o1.float() * go.float()).sum() + (ot1.float() * gt.float()).sum()
+        grads = torch.autograd.grad(loss, leaves)
+    o2, ot2 = torch.func.jvp(fn, (q, k, v), (qt, kt, vt))
+    assert torch.equal(o1, o2) and torch.equal(ot1, ot2)
+
+    def check(name, got, want):
+        if dt == torch.float32:
+            err = np.abs(got.detach().double().cpu().numpy() - want).max()
+            assert err <= 1e-4, f"{name}: {err:.3e}"
+        else:
+            assert _rel(got, want) <= tol, f"{name}: {_rel(got, want):.3e}"
+
+    check("O", o1, ref["O"])
+    check("O'", ot1, ref["Ot"])
+    for n, g in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        check(n, g, rb[n])
+
+
+def test_plain_attention_autograd_and_apply_tuple():
+    from jvp_flash_attention_amd import JVPAttn, attention
+
+    Z, H, L, D = 1, 3, 96, 128
+    q, k, v, go = [_randn((Z, H, L, D), torch.bfloat16, 20 + i) for i in range(4)]
+    f64 = [x.double().cpu().numpy() for x in (q, k, v, go)]
+    qq, kk, vv = [x.clone().requires_grad_() for x in (q, k, v)]
+    o = attention(qq, kk, vv, causal=True)
+    (o.float() * go.float()).sum().backward()
+    ref = dense.forward(*f64[:3], causal=True)
+    rb = dense.backward(*f64[:3], None, None, None, f64[3], None, causal=True)
+    assert _rel(o, ref["O"]) <= 2e-2
+    for n, g in (("dq", qq.grad), ("dk", kk.grad), ("dv", vv.grad)):
+        assert _rel(g, rb[n]) <= 2e-2, n
+    o2, ctx = JVPAttn.apply(q, k, v, None, None, None, None, 0.0, True, None, True, True)
+    assert torch.equal(o2, o.detach()) and ctx.o_t is None and ctx.M.shape == (Z, H, L)
+    # log2-domain log-sum-exp
+    assert np.abs(ctx.M.double().cpu().numpy() - ref["M"]).max() < 2e-2
+
+
+def test_config2_dense_bf16_full_size_properties():
+    """BASELINE config 2: bf16 B4 H16 L2048 D64, tangents ~ N(0, 0.1^2), no mask."""
+    from jvp_flash_attention_amd import _lib, attention
+
+    be = _lib.backend()
+    Z, H, L, D = 4, 16, 2048, 64
+    dt = torch.bfloat16
+    q, k, v = [_randn((Z, H, L, D), dt, 30 + i) for i in range(3)]
+    qt, kt, vt = [_randn((Z, H, L, D), dt, 40 + i, std=0.1) for i in range(3)]
+    go, gt = [_randn((Z, H, L, D), dt, 50 + i) for i in range(2)]
+    scale = D**-0.5
+    o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, 0, False, scale)
+    # one slab against the oracle
+    f64 = [x[1, 5:6][None].double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    ref = dense.forward(*f64[:6])
+    assert _rel(o[1, 5], ref["O"][0, 0]) <= 2e-2 and _rel(ot[1, 5], ref["Ot"][0, 0]) <= 2e-2
+    dq, dk, dv, dqt, dkt, dvt = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, 0, False, scale,
+                                       want_tangent_grads=True)
+    rb = dense.backward(*f64)
+    for n, g in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), (dq, dk, dv, dqt, dkt, dvt)):
+        assert _rel(g[1, 5], rb[n][0, 0]) <= 2e-2, n
+    # V'-only tangent: O' = softmax(S) V', the plain attention output with V := V'
+    zero = torch.zeros_like(q)
+    _, ot_v, _, _ = be.fwd(q, k, v, zero, zero, vt, None, 0, False, scale)
+    assert _rel(ot_v, attention(q, k, vt)) <= 1e-2
+    # linearity in the tangents
+    _, ot_q, _, _ = be.fwd(q, k, v, qt, zero, zero, None, 0, False, scale)
+    _, ot_k, _, _ = be.fwd(q, k, v, zero, kt, zero, None, 0, False, scale)
+    assert _rel(ot_q.float() + ot_k.float() + ot_v.float(), ot.float()) <= 2e-2
+    # without a mask the order of the keys does not matter
+    perm = torch.randperm(L, device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
+    o_p, ot_p, _, _ = be.fwd(q, k[:, :, perm].contiguous(), v[:, :, perm].contiguous(), qt,
+                             kt[:, :, perm].contiguous(), vt[:, :, perm].contiguous(), None, 0, False, scale)
+    assert _rel(o_p, o) <= 1e-2 and _rel(ot_p, ot) <= 2e-2
+    # dV' = P^T gT in tangent mode equals dV = P^T gO of the first-order backward when gO := gT
+    g1 = be.bwd(q, k, v, None, None, None, o, None, M, None, gt, None, None, 0, False, scale)
+    assert _rel(dvt, g1[2]) <= 1e-2
+
+
+def test_config3_causal_long_full_size_properties():
+    """BASELINE config 3: fp16 B2 H32 L4096 D128 causal, and the headline bf16 B4 H16 L4096 D128."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    for dt, (Z, H) in ((torch.float16, (2, 32)), (torch.bfloat16, (4, 16))):
+        L, D = 4096, 128
+        scale = D**-0.5
+        q, k, v, qt, kt, vt, go, gt = [_randn((Z, H, L, D), dt, 60 + i) for i in range(8)]
+        o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, 0, True, scale)
+        assert torch.isfinite(o).all() and torch.isfinite(ot).all()
+        # causal rows never see later keys: the first half equals a run on the truncated sequence, bit for bit
+        h = L // 2
+        cut = [x[:, :, :h].contiguous() for x in (q, k, v, qt, kt, vt)]
+        o_h, ot_h, M_h, mu_h = be.fwd(*cut, None, 0, True, scale)
+        assert torch.equal(o[:, :, :h], o_h) and torch.equal(ot[:, :, :h], ot_h) and torch.equal(M[:, :, :h], M_h)
+        # one slab against the oracle (forward and the tangent-path backward)
+        z, hh = Z - 1, 3
+        f64 = [x[z, hh:hh + 1][None].double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+        ref = dense.forward(*f64[:6], causal=True)
+        assert _rel(o[z, hh], ref["O"][0, 0]) <= 2e-2 and _rel(ot[z, hh], ref["Ot"][0, 0]) <= 2e-2
+        dq, dk, dv, *_ = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, 0, True, scale)
+        rb = dense.backward(*f64, causal=True)
+        for n, g in zip(("dq", "dk", "dv"), (dq, dk, dv)):
+            assert _rel(g[z, hh], rb[n][0, 0]) <= 2e-2, n
+        # gradients are causal too: dk, dv of the second half do not depend on queries of the first half
+        del o_h, ot_h, dq, dk, dv
+        torch.cuda.empty_cache()
+
+
+def test_config4_mask_modes_fp32_full_size():
+    """BASELINE config 4: fp32 B4 H8 L1024 D64; (a) key padding [B,1,1,L], (b) additive bias [B,H,L,L]."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    Z, H, L, D = 4, 8, 1024, 64
+    dt = torch.float32
+    scale = D**-0.5
+    q, k, v, qt, kt, vt, go, gt = [_randn((Z, H, L, D), dt, 70 + i) for i in range(8)]
+    g = torch.Generator().manual_seed(7)
+    lens = torch.randint(L // 2, L + 1, (Z,), generator=g)
+    keypad = (torch.arange(L)[None, :] < lens[:, None]).view(Z, 1, 1, L).cuda()
+    bias = _randn((Z, H, L, L), dt, 79)
+    for mask, kind in ((keypad, _lib.MASK_BOOL), (bias, _lib.MASK_ADD)):
+        o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, mask, kind, False, scale)
+        grads = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, kind, False, scale, want_tangent_grads=True)
+        for z, h in ((0, 0), (3, 7)):
+            f64 = [x[z, h:h + 1][None].double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+            m = mask[z:z + 1, 0:1] if kind == _lib.MASK_BOOL else mask[z:z + 1, h:h + 1]
+            npm = m.cpu().numpy() if kind == _lib.MASK_BOOL else m.double().cpu().numpy()
+            ref = dense.forward(*f64[:6], mask=npm)
+            rb = dense.backward(*f64, mask=npm)
+            assert np.abs(o[z, h].double().cpu().numpy() - ref["O"][0, 0]).max() <= 1e-4
+            assert np.abs(ot[z, h].double().cpu().numpy() - ref["Ot"][0, 0]).max() <= 1e-4
+            for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+                assert np.abs(t[z, h].double().cpu().numpy() - rb[n][0, 0]).max() <= 1e-4, n
+        if kind == _lib.MASK_BOOL:
+            # masked keys receive no gradient and contribute nothing
+            for zz in range(Z):
+                n = int(lens[zz])
+                if n < L:
+                    assert torch.all(grads[1][zz, :, n:] == 0) and torch.all(grads[2][zz, :, n:] == 0)
+
+
+def test_config5_hvp_memory_is_linear_in_sequence_length():
+    """BASELINE config 5 at two lengths: peak memory of fwd_dual + backward grows like L, not L^2."""
+    from jvp_flash_attention_amd import JVPAttn
+
+    def peak(L):
+        torch.cuda.empty_cache()
+        Z, H, D = 1, 16, 128
+        q, k, v, qt, kt, vt, gt = [_randn((Z, H, L, D), torch.bfloat16, 80 + i) for i in range(7)]
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        leaves = [x.requires_grad_() for x in (q, k, v)]
+        _, ot = torch.func.jvp(partial(JVPAttn.fwd_dual, causal=True), tuple(leaves), (qt, kt, vt))
+        grads = torch.autograd.grad((ot.float() * gt.float()).sum(), leaves)
+        assert all(torch.isfinite(g).all() for g in grads)
+        return torch.cuda.max_memory_allocated() - base
+
+    p1, p2 = peak(4096), peak(16384)
+    assert p2 <= 4.5 * p1, (p1, p2)  # 4x the length: ~4x the memory (16x if anything were O(L^2))

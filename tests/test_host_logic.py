@@ -1,0 +1,197 @@
+"""Host-side logic on CPU: argument checks, mask classification and the autograd / forward-mode
+wiring of ``JVPAttn``, with the device work replaced by the oracle's tile-loop restatement
+(``tests/fake_backend.py``).  What is checked here is the plumbing, against the SDPA route."""
+from functools import partial
+
+import pytest
+import torch
+import torch.autograd.forward_ad as fwAD
+
+from jvp_flash_attention_amd import MASK_CONST, JVPAttn, attention
+from jvp_flash_attention_amd import _lib
+from oracle import sdpa_jvp
+from tests.fake_backend import oracle_backend
+
+
+def _inputs(Z=1, H=2, L=32, D=32, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(Z, H, L, D, generator=g) for _ in range(8)]
+
+
+def _close(a, b, tol=2e-5):
+    assert (a - b).abs().max().item() <= tol * max(1.0, b.abs().max().item())
+
+
+def test_import_path_alias_matches_reference_import_line():
+    from jvp_flash_attention.jvp_attention import JVPAttn as J2, attention as a2, MASK_CONST as m2
+
+    assert J2 is JVPAttn and a2 is attention and m2 == MASK_CONST == -100.0
+
+
+def test_plain_attention_and_first_order_backward():
+    q, k, v, qt, kt, vt, go, _ = _inputs()
+    _, _, ref = sdpa_jvp.forward_backward(q, k, v, qt, kt, vt, go, None)
+    o_ref, _ = sdpa_jvp.forward(q, k, v, qt, kt, vt)
+    with oracle_backend() as be:
+        qq, kk, vv = [x.clone().requires_grad_() for x in (q, k, v)]
+        o = attention(qq, kk, vv)
+        (o * go).sum().backward()
+        assert be.calls[0][:2] == ("fwd", False) and be.calls[1][:2] == ("bwd", False)
+    _close(o, o_ref)
+    for got, want in zip((qq.grad, kk.grad, vv.grad), ref[:3]):
+        _close(got, want)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_fwd_dual_three_way_like_reference_tests(causal):
+    """SDPA under fwAD vs fwd_dual under fwAD vs torch.func.jvp(fwd_dual): the reference's own
+    three-way comparison (tests/test_jvp_attention.py:572-617)."""
+    q, k, v, qt, kt, vt, _, _ = _inputs()
+    o_ref, ot_ref = sdpa_jvp.forward(q, k, v, qt, kt, vt, causal=causal)
+    with oracle_backend():
+        with fwAD.dual_level():
+            out = JVPAttn.fwd_dual(fwAD.make_dual(q, qt), fwAD.make_dual(k, kt), fwAD.make_dual(v, vt), causal=causal)
+            o1, ot1 = fwAD.unpack_dual(out)
+            o1, ot1 = o1.clone(), ot1.clone()
+        o2, ot2 = torch.func.jvp(partial(JVPAttn.fwd_dual, causal=causal), (q, k, v), (qt, kt, vt))
+    for o, ot in ((o1, ot1), (o2, ot2)):
+        _close(o, o_ref)
+        _close(ot, ot_ref)
+
+
+def test_gradients_through_the_tangent_reach_all_six_inputs():
+    q, k, v, qt, kt, vt, go, gt = _inputs()
+    _, _, ref = sdpa_jvp.forward_backward(q, k, v, qt, kt, vt, go, gt)
+    with oracle_backend() as be:
+        leaves = [x.clone().requires_grad_() for x in (q, k, v, qt, kt, vt)]
+        with fwAD.dual_level():
+            out = JVPAttn.fwd_dual(*(fwAD.make_dual(p, t) for p, t in zip(leaves[:3], leaves[3:])))
+            o, ot = fwAD.unpack_dual(out)
+            grads = torch.autograd.grad((o * go).sum() + (ot * gt).sum(), leaves)
+        assert ("bwd", True, 0, False, True) in be.calls  # tangent grads requested
+    for got, want in zip(grads, ref):
+        _close(got, want)
+
+
+def test_hvp_style_gradient_of_tangent_only_under_func_jvp():
+    q, k, v, qt, kt, vt, _, gt = _inputs()
+    _, _, ref = sdpa_jvp.forward_backward(q, k, v, qt, kt, vt, torch.zeros_like(q), gt)
+    with oracle_backend() as be:
+        leaves = [x.clone().requires_grad_() for x in (q, k, v)]
+        _, ot = torch.func.jvp(JVPAttn.fwd_dual, tuple(leaves), (qt, kt, vt))
+        grads = torch.autograd.grad((ot * gt).sum(), leaves)
+        assert be.calls[-1][:2] == ("bwd", True) and be.calls[-1][-1] is False  # primal grads only
+    for got, want in zip(grads, ref[:3]):
+        _close(got, want)
+
+
+def test_apply_returns_output_and_context_tuple_and_13_slot_backward():
+    q, k, v, qt, kt, vt, go, _ = _inputs()
+    _, ot_ref = sdpa_jvp.forward(q, k, v, qt, kt, vt)
+    with oracle_backend():
+        qq = q.clone().requires_grad_()
+        out = JVPAttn.apply(qq, k, v, qt, kt, vt, None, 0.0, False, None, True, True)
+        o, ctx = out
+        o_t, M, grid, head_dim, sm_scale, mask_tensor, mask_type, dropout_p, seed, drop = ctx
+        _close(o_t, ot_ref)
+        assert M.shape == q.shape[:3] and M.dtype == torch.float32
+        assert tuple(grid) == (1, 2, 1) and head_dim == 32 and mask_type == 0 and dropout_p == 0.0 and not drop
+        assert abs(sm_scale - 32**-0.5) < 1e-12 and mask_tensor.numel() == 0
+        (o * go).sum().backward()
+        assert qq.grad is not None
+    assert len(JVPAttn.BwdOut._fields) == 13
+
+    class Ctx:
+        pass
+
+    with oracle_backend():
+        o, ctx = JVPAttn.forward(q, k, v, None, None, None)
+        c = Ctx()
+        c.saved_tensors = (q, k, v, o, ctx.M)
+        c.mask_tensor, c.MASK_TYPE, c.causal, c.sm_scale = ctx.mask_tensor, 0, False, ctx.sm_scale
+        res = JVPAttn.backward(c, go, None)
+    assert isinstance(res, JVPAttn.BwdOut) and all(x is None for x in res[3:]) and all(x is not None for x in res[:3])
+
+
+def test_argument_errors_match_the_reference():
+    q, k, v, *_ = _inputs()
+    with oracle_backend():
+        with pytest.raises(NotImplementedError):
+            attention(q, k, v, dropout_p=0.1)
+        with pytest.raises(ValueError):
+            attention(q, k, v, attn_mask=torch.ones(1, 2, 32, 32, dtype=torch.bool), causal=True)
+        with pytest.raises(AssertionError):
+            attention(q, k, v[..., :16])
+        with pytest.raises(AssertionError):
+            attention(q[..., :24], k[..., :24], v[..., :24])  # head dim not supported
+        with pytest.raises(AssertionError):
+            attention(q, k, v, attn_mask=torch.ones(1, 2, 32, 16, dtype=torch.bool))
+        with pytest.raises(AssertionError):
+            attention(q, k, v, attn_mask=torch.zeros(1, 2, 32, 32, dtype=torch.float64))
+        bad = torch.ones(1, 2, 32, 32, dtype=torch.bool)
+        bad[0, 1] = False
+        with pytest.raises(AssertionError):
+            attention(q, k, v, attn_mask=bad)  # a head with every key masked
+        nanmask = torch.zeros(1, 2, 32, 32)
+        nanmask[0, 0, 0, 0] = float("nan")
+        with pytest.raises(AssertionError):
+            attention(q, k, v, attn_mask=nanmask)
+        # a float mask without MASK_CONST is fine here (the reference raises UserWarning)
+        attention(q, k, v, attn_mask=torch.zeros(1, 2, 32, 32))
+
+
+@pytest.mark.parametrize("kind", ["keypad", "bias", "mask_const"])
+def test_masks_follow_sdpa_semantics(kind):
+    q, k, v, qt, kt, vt, go, gt = _inputs(Z=2)
+    if kind == "keypad":
+        mask = (torch.arange(32)[None, :] < torch.tensor([20, 32])[:, None]).view(2, 1, 1, 32)
+        sdpa_mask = mask
+    elif kind == "bias":
+        mask = torch.randn(2, 2, 32, 32, generator=torch.Generator().manual_seed(3))
+        sdpa_mask = mask
+    else:  # the reference's float-mask convention: MASK_CONST marks masked entries
+        keep = torch.rand(2, 2, 32, 32, generator=torch.Generator().manual_seed(4)) > 0.5
+        keep[..., 0] = True
+        mask = torch.where(keep, 0.0, MASK_CONST)
+        sdpa_mask = keep
+    o_ref, ot_ref, ref = sdpa_jvp.forward_backward(q, k, v, qt, kt, vt, go, gt, attn_mask=sdpa_mask)
+    with oracle_backend() as be:
+        leaves = [x.clone().requires_grad_() for x in (q, k, v)]
+        o, ot = torch.func.jvp(partial(JVPAttn.fwd_dual, attn_mask=mask), tuple(leaves), (qt, kt, vt))
+        grads = torch.autograd.grad((o * go).sum() + (ot * gt).sum(), leaves)
+        expect = _lib.MASK_BOOL if mask.dtype == torch.bool else _lib.MASK_ADD
+        assert be.calls[0][2] == expect
+    tol = 2e-5 if kind != "mask_const" else 1e-4  # exp(-100) is not exactly 0
+    _close(o, o_ref, tol)
+    _close(ot, ot_ref, tol)
+    for got, want in zip(grads, ref[:3]):
+        _close(got, want, tol)
+
+
+def test_broadcast_mask_strides_are_zero_on_size_one_axes():
+    q = torch.zeros(2, 3, 8, 32)
+    mask = torch.ones(2, 1, 1, 8, dtype=torch.bool)
+    p = _lib.make_problem(q, mask, _lib.MASK_BOOL, False, 0.5)
+    assert list(p.mask_stride) == [8, 0, 0, 1] and p.mask_kind == _lib.MASK_BOOL
+    assert (p.Z, p.H, p.L, p.D, p.dtype, p.causal) == (2, 3, 8, 32, 2, 0)
+
+
+def test_non_contiguous_inputs_are_copied_and_missing_tangents_are_zero():
+    q, k, v, qt, kt, vt, _, _ = _inputs()
+    qn = q.transpose(1, 2).contiguous().transpose(1, 2)
+    assert not qn.is_contiguous()
+    o_ref, ot_ref = sdpa_jvp.forward(q, k, v, qt, torch.zeros_like(k), torch.zeros_like(v))
+    with oracle_backend():
+        with fwAD.dual_level():
+            out = JVPAttn.fwd_dual(fwAD.make_dual(qn, qt), k, v)  # only q carries a tangent
+            o, ot = fwAD.unpack_dual(out)
+            _close(o, o_ref)
+            _close(ot, ot_ref)
+        # no tangents at all: plain forward
+        _close(JVPAttn.fwd_dual(q, k, v), o_ref)
+
+
+def test_product_has_no_cpu_path():
+    q, k, v, *_ = _inputs()
+    with pytest.raises(RuntimeError, match="no CPU path|There is no CPU path"):
+        attention(q, k, v)
