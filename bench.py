@@ -26,9 +26,10 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
 Z, H, L, D = 4, 16, 4096, 128
 
-# HBM bytes per forward launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
-# profiles/); None until measured.
-MEASURED_FWD_TRAFFIC_BYTES = None
+# HBM bytes per forward launch measured with rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a plain
+# copy of known size gives) and WRITE_SIZE (x1.0): 407.0 MB read + 136.3 MB written; the figures
+# and commands are in profiles/fwd2_kernel_bf16_B4_H16_L4096_D128.md.
+MEASURED_FWD_TRAFFIC_BYTES = 543.3e6
 
 
 def timed(fn, steps, warmup):
@@ -56,13 +57,23 @@ def cpu_baseline():
 
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
     cores = torch.get_num_threads()
-    zb, hb = 1, 2
     g = torch.Generator().manual_seed(0)
-    q, k, v, qt, kt, vt = [torch.randn(zb, hb, L, D, generator=g) for _ in range(6)]
-    sdpa_jvp.forward(q[:, :1, :512], k[:, :1, :512], v[:, :1, :512], qt[:, :1, :512], kt[:, :1, :512], vt[:, :1, :512])
-    t0 = time.perf_counter()
-    sdpa_jvp.forward(q, k, v, qt, kt, vt)
-    dt = time.perf_counter() - t0
+
+    def run(zb, hb):
+        q, k, v, qt, kt, vt = [torch.randn(zb, hb, L, D, generator=g) for _ in range(6)]
+        t0 = time.perf_counter()
+        sdpa_jvp.forward(q, k, v, qt, kt, vt)
+        return time.perf_counter() - t0
+
+    run(1, 1)  # warm-up
+    t2 = run(1, 2)
+    # size the sample for roughly 15 s of CPU work, at most the whole B*H = 64 heads
+    zb, hb = 1, 2
+    dt = t2
+    heads = int(min(Z * H, max(2, 15.0 / max(t2 / 2, 1e-3))))
+    if heads > 2:
+        zb, hb = (1, heads) if heads <= H else (heads // H, H)
+        dt = run(zb, hb)
     flops = 12.0 * zb * hb * L * L * D
     return {
         "value": flops / dt / 1e12,
@@ -74,6 +85,36 @@ def cpu_baseline():
     }
 
 
+def hvp_sweep(be, _lib):
+    """BASELINE config 5: bf16 B1 H16 D128 causal, L swept; fused dual forward + the backward of
+    sum(O' * gO') w.r.t. q, k, v (the Hessian-vector-product pattern): time and peak HBM vs L."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    rows = []
+    for Ls in (1024, 4096, 16384, 32768):
+        torch.cuda.empty_cache()
+        g = torch.Generator(device=dev).manual_seed(Ls)
+        q, k, v, qt, kt, vt, gt = [
+            torch.randn(1, 16, Ls, 128, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(7)
+        ]
+        scale = 128**-0.5
+
+        def step():
+            o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, True, scale)
+            return be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, None, gt, None, _lib.MASK_NONE, True, scale)
+
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        ms, _ = timed(step, 3, 1)
+        peak = torch.cuda.max_memory_allocated() - base
+        n = 16.0 * Ls * Ls * 128
+        rows.append({"L": Ls, "ms": ms, "tflops": (12 + 24) * n / 2 / (ms * 1e-3) / 1e12,
+                     "peak_extra_hbm_mb": peak / 2**20, "inputs_mb": 7 * q.numel() * 2 / 2**20,
+                     "one_fp32_score_tensor_mb_if_materialised": 16.0 * Ls * Ls * 4 / 2**20})
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -81,6 +122,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--fwd-only", action="store_true", help="time only the headline forward (for profiling)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy, whose known traffic scales the rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE readings of the forward kernel")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (B*H shards trivially); use --gpus 1")
@@ -111,6 +155,12 @@ def main():
         o, ot, M, mu = fwd(causal)
         state["g"] = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, causal, scale)
 
+    if args.calibrate_copy:
+        src = torch.empty(256 * 2**20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     ms_fwd, wall_fwd = timed(fwd, args.steps, args.warmup)
     out = {
         "metric": "fused JVP dual-forward throughput, bf16 B4 H16 L4096 D128 (non-causal)",
@@ -154,6 +204,7 @@ def main():
             "fwd_tflops_reference_flop_convention": tf(ref_conv_flops, ms_fwd),
             "peak_hbm_allocated_mb": torch.cuda.max_memory_allocated() / 2**20,
         }
+        out["extra"]["hvp_sweep_bf16_B1_H16_D128_causal"] = hvp_sweep(be, _lib)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)
