@@ -80,8 +80,9 @@ def cpu_baseline():
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"math SDPA + torch.func.jvp fp32 dual forward on a B={zb},H={hb},L={L},D={D} slab "
-                  f"({dt:.1f} s); full shape would take ~{dt * Z * H / (zb * hb):.0f} s (extrapolated)",
+        "sample": f"math SDPA + torch.func.jvp fp32 dual forward on B={zb},H={hb},L={L},D={D} ({dt:.1f} s)"
+                  + ("; the whole headline shape" if zb * hb == Z * H
+                     else f"; {zb * hb} of {Z * H} heads, the whole shape would take ~{dt * Z * H / (zb * hb):.0f} s"),
     }
 
 
