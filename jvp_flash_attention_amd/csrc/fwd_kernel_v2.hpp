@@ -17,6 +17,7 @@
 #include "common.hpp"
 #include "mask.hpp"
 #include "params.hpp"
+#include "pipeline.hpp"
 
 namespace jvpfa {
 
@@ -29,55 +30,6 @@ __device__ long long *g_trace = nullptr;  // debugging aid: time stamps of one w
 #else
 #define JVPFA_STAMP(slot) do {} while (0)
 #endif
-
-#define JVPFA_LDS(T) __attribute__((address_space(3))) T *
-#define JVPFA_GLB(T) __attribute__((address_space(1))) T *
-
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-
-template <int... Is, typename F>
-__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F &&f) {
-  (f(std::integral_constant<int, Is>{}), ...);
-}
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), fully unrolled
-template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
-  static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F &&>(f));
-}
-
-// LDS reads whose issue point is fixed by the program text (not by the scheduler).  The data is
-// valid only after an lds_wait<N>() on the same registers, N = number of such reads issued after
-// the one waited for (LDS reads complete in issue order).
-template <int OFF> __device__ __forceinline__ u32x4 lds_b128(uint32_t addr) {
-  u32x4 d;
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(d) : "v"(addr), "n"(OFF));
-  return d;
-}
-template <int OFF> __device__ __forceinline__ u32x2 lds_tr64(uint32_t addr) {
-  u32x2 d;
-  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(d) : "v"(addr), "n"(OFF));
-  return d;
-}
-// x * alpha for a value that lives in a matrix-core accumulation register, done where it stands:
-// the value never changes register class, so code paths that do not rescale carry no copies.
-__device__ __forceinline__ float acc_scale(float x, float alpha) {
-  float t;
-  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1\n\ts_nop 1"
-               : "+a"(x), "=&v"(t)
-               : "v"(alpha));
-  return x;
-}
-template <int N> __device__ __forceinline__ void lds_wait(u32x4 &a) {
-  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
-}
-template <int N> __device__ __forceinline__ void lds_wait(u32x4 &a, u32x4 &b) {
-  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
-}
-template <int N> __device__ __forceinline__ void lds_wait(u32x2 &a, u32x2 &b) {
-  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
-}
-template <int N> __device__ __forceinline__ void lds_wait(u32x2 &a, u32x2 &b, u32x2 &c, u32x2 &d) {
-  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
-}
 
 template <typename T, int D, bool DUAL> struct Fwd2Cfg {
   static constexpr int NW = 4;
@@ -92,10 +44,6 @@ template <typename T, int D, bool DUAL> struct Fwd2Cfg {
   static constexpr size_t LDS_BYTES = 2 * (size_t)STAGEB;
   static constexpr int IPW = TILEB / 1024 / NW;       // direct-load instructions per wave per tile
 };
-
-// chunk swizzles (row -> xor value applied to the 16-byte chunk index)
-template <int CH> __device__ __forceinline__ int swz_k(int row) { return CH == 16 ? (row & 15) : ((row >> 1) & 7); }
-template <int CH> __device__ __forceinline__ int swz_v(int row) { return CH == 16 ? ((row & 7) << 1) : (((row >> 1) & 3) << 1); }
 
 template <typename T, int D, bool DUAL, int MASK>
 __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
