@@ -3,6 +3,7 @@
 // and exporting  int JVPFA_NAME(const BwdParams&, int mask_kind, bool dual, bool tangent_grads,
 // hipStream_t): pre-pass, then the dq and dk/dv kernels of every requested mode.
 #include "bwd_kernel.hpp"
+#include "bwd_kernel_v2.hpp"
 #include "launch.hpp"
 
 namespace jvpfa {
@@ -13,14 +14,26 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
   const int nb = (p.pr.L + BWD_BLK - 1) / BWD_BLK;
   const long long blocks = (long long)nb * p.pr.Z * p.pr.H;
   if (blocks > 0x7fffffffLL) return -2;
-  auto kq = bwd_dq_kernel<T, D, MODE, MASK>;
-  auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK>;
-  int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);
-  if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg::DKV_LDS);
-  if (rc != 0) return rc;
-  hipLaunchKernelGGL(kkv, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
-  hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DQ_LDS, stream, p);
-  return hipGetLastError() == hipSuccess ? 0 : -6;
+  if constexpr (sizeof(T) == 2 && D >= 64) {  // direct-to-LDS, double-buffered kernels
+    using Cfg2 = Bwd2Cfg<T, D, MODE>;
+    auto kq = bwd2_dq_kernel<T, D, MODE, MASK>;
+    auto kkv = bwd2_dkdv_kernel<T, D, MODE, MASK>;
+    int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
+    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);
+    if (rc != 0) return rc;
+    hipLaunchKernelGGL(kkv, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
+    hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
+    return hipGetLastError() == hipSuccess ? 0 : -6;
+  } else {
+    auto kq = bwd_dq_kernel<T, D, MODE, MASK>;
+    auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK>;
+    int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);
+    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg::DKV_LDS);
+    if (rc != 0) return rc;
+    hipLaunchKernelGGL(kkv, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+    hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DQ_LDS, stream, p);
+    return hipGetLastError() == hipSuccess ? 0 : -6;
+  }
 }
 
 template <typename T, int D, int MASK>

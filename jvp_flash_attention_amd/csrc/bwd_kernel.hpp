@@ -1,7 +1,7 @@
 // Backward kernels for  Loss = <gO, O> + <gT, O'>  with P recomputed from the saved
 // log-sum-exp M (and mu for the tangent path).
 //
-//   prepass   d1 = rowsum(gO*O), a = rowsum(gT*O), d2 = rowsum(gT*O') - a*mu
+//   prepass   d1 = rowsum(gO*O), a = rowsum(gT*O), d2 = d1 + rowsum(gT*O') - a*mu
 //   dq        one workgroup per 128 query rows, loop over key tiles
 //   dkdv      one workgroup per 128 key rows, loop over query tiles
 //
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void bwd_prepass_kernel(const BwdParams p, lon
     p.d1[row] = s1;
     if (dual) {
       p.a[row] = sa;
-      p.d2[row] = s2 - sa * p.mu[row];
+      p.d2[row] = s1 + s2 - sa * p.mu[row];  // BWD_DUAL uses d1 + d2 only, kept in one statistic
     }
   }
 }
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
   if constexpr (DUAL || TAN) load_row_frags<KK>(gTf, reinterpret_cast<const T *>(p.gt) + head + (size_t)qld * D, g);
 
   const float Mq = qrow < L ? p.M[srow + qld] : __builtin_inff();
-  const float d1 = (!TAN && has_go) ? p.d1[srow + qld] : 0.f;
+  const float d1 = (MODE == BWD_PLAIN) ? p.d1[srow + qld] : 0.f;  // BWD_DUAL: d2 already holds d1 + d2
   const float mu = (DUAL) ? p.mu[srow + qld] : 0.f;
   const float av = (DUAL || TAN) ? p.a[srow + qld] : 0.f;
   const float d2 = (DUAL) ? p.d2[srow + qld] : 0.f;
@@ -331,7 +331,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
       const bool ok = i0 + tid < L;
       const size_t si = srow + (ok ? i0 + tid : 0);
       sM[tid] = ok ? p.M[si] : __builtin_inff();
-      sd1[tid] = (ok && !TAN && has_go) ? p.d1[si] : 0.f;
+      sd1[tid] = (ok && MODE == BWD_PLAIN) ? p.d1[si] : 0.f;  // BWD_DUAL: d2 already holds d1 + d2
       smu[tid] = (ok && DUAL) ? p.mu[si] : 0.f;
       sa[tid] = (ok && (DUAL || TAN)) ? p.a[si] : 0.f;
       sd2[tid] = (ok && DUAL) ? p.d2[si] : 0.f;

@@ -1,0 +1,588 @@
+// Backward kernels for 16-bit element types (bf16 / fp16), D in {64, 128}, on the forward's memory
+// pipeline: 64-row tiles of the streamed tensors go global -> LDS with direct-to-LDS loads, double
+// buffered and issued one instruction at a time between the matrix products of the current tile;
+// tiles stay row-major (XOR-swizzled 16-byte chunks) and are read both ways from that one copy:
+// ds_read_b128 gives the operand of the recomputed products (contraction over d), the transposing
+// ds_read_b64_tr_b16 gives the operand of the gradient accumulations (contraction over the
+// streamed index).  LDS reads are issued one step ahead of their matrix products.
+//
+// Mathematics, modes and the reference lines it replaces: see bwd_kernel.hpp.  In BWD_DUAL the
+// pre-pass statistic d2 already contains d1 (d2 := d1 + rowsum(gT*O') - a*mu).
+#pragma once
+#include "common.hpp"
+#include "mask.hpp"
+#include "params.hpp"
+#include "pipeline.hpp"
+
+namespace jvpfa {
+
+template <typename T, int D, int MODE> struct Bwd2Cfg {
+  static constexpr int NW = 4;
+  static constexpr int NT = NW * WAVE;
+  static constexpr int BLK = NW * 32;                 // rows owned by a workgroup
+  static constexpr int BT = 64;                       // rows of a streamed tile
+  static constexpr int CH = D * sizeof(T) / 16;
+  static constexpr int ROWB = D * sizeof(T);
+  static constexpr int TILEB = BT * ROWB;
+  static constexpr int NTILE = MODE == BWD_DUAL ? 4 : 2;
+  static constexpr int STAGEB = NTILE * TILEB;
+  static constexpr int IPW = TILEB / 1024 / NW;
+  static constexpr int NSTAT = MODE == BWD_DUAL ? 4 : 2;
+  static constexpr int STATB = NSTAT * BT * 4;        // row statistics of a query tile (dk/dv only)
+  static constexpr size_t DQ_LDS = 2 * (size_t)STAGEB;
+  static constexpr size_t DKV_LDS = 2 * (size_t)STAGEB + 2 * (size_t)STATB;
+};
+
+// One LDS fragment (8 elements per lane) read ahead with lds_b128 / two lds_tr64.
+struct FragN { u32x4 v; };
+struct FragT { u32x2 lo, hi; };
+template <typename T> __device__ __forceinline__ Frag<T> as_frag(const FragN &f) { return __builtin_bit_cast(Frag<T>, f.v); }
+template <typename T> __device__ __forceinline__ Frag<T> as_frag(const FragT &f) {
+  const u32x4 v = {f.lo[0], f.lo[1], f.hi[0], f.hi[1]};
+  return __builtin_bit_cast(Frag<T>, v);
+}
+template <int N> __device__ __forceinline__ void lds_wait(FragN &a, FragN &b) { lds_wait<N>(a.v, b.v); }
+template <int N> __device__ __forceinline__ void lds_wait(FragN &a, FragN &b, FragN &c, FragN &d) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a.v), "+v"(b.v), "+v"(c.v), "+v"(d.v) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait(FragT &a, FragT &b) { lds_wait<N>(a.lo, a.hi, b.lo, b.hi); }
+template <int N> __device__ __forceinline__ void lds_wait(FragT &a, FragT &b, FragT &c, FragT &d) {
+  asm volatile("s_waitcnt lgkmcnt(%8)"
+               : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi), "+v"(c.lo), "+v"(c.hi), "+v"(d.lo), "+v"(d.hi)
+               : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait4(u32x4 &a, u32x4 &b, u32x4 &c, u32x4 &d) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+
+// Everything the two kernels share: tile geometry, direct loads spread over steps, fragment reads.
+// SLOTn are LDS tile slots inside a stage; a tile is BT rows, row-major, chunks swizzled by swz_u.
+#define JVPFA_BWD2_COMMON(Cfg)                                                                                      \
+  constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT;                   \
+  constexpr int KK = D / 16, DB = D / 32;                                                                           \
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];                                        \
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem_raw;                                                              \
+  const Problem &pr = p.pr;                                                                                         \
+  const int L = pr.L;                                                                                               \
+  const int nblk = (L + Cfg::BLK - 1) / Cfg::BLK;                                                                   \
+  const int total = nblk * pr.Z * pr.H;                                                                             \
+  const int id = xcd_remap(blockIdx.x, total);                                                                      \
+  const int zh = id / nblk;                                                                                         \
+  const int z = zh / pr.H, h = zh % pr.H;                                                                           \
+  const int tid = threadIdx.x;                                                                                      \
+  const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;                                   \
+  const int r = lane % 32, g = lane / 32, pr32 = perm32(r);                                                         \
+  const size_t head = (size_t)zh * L * D;                                                                           \
+  const size_t srow = (size_t)zh * L;                                                                               \
+  (void)z; (void)h; (void)srow;                                                                                     \
+  /* direct loads: instruction i of this wave fills LDS chunks 64*(wave*IPW+i) .. +63 of a tile */                   \
+  int ld_row[IPW];                                                                                                  \
+  uint32_t ld_c[IPW];                                                                                               \
+  _Pragma("unroll") for (int i = 0; i < IPW; ++i) {                                                                 \
+    const int lc = 64 * (wave * IPW + i) + lane;                                                                    \
+    ld_row[i] = lc / CH;                                                                                            \
+    ld_c[i] = ((lc % CH) ^ swz_u<CH>(lc / CH)) * 16;                                                                \
+  }                                                                                                                 \
+  int ld_rows = 0;                                                                                                  \
+  uint32_t ld_dst = 0;                                                                                              \
+  const char *ld_p[4] = {nullptr, nullptr, nullptr, nullptr};                                                       \
+  auto load_piece = [&](auto pc) {                                                                                  \
+    constexpr int pi = decltype(pc)::value, i = pi / Cfg::NTILE, ts = pi % Cfg::NTILE;                              \
+    const uint32_t off = min(ld_row[i], ld_rows) * ROWB + ld_c[i];                                                  \
+    __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(ld_p[ts] + off),                                       \
+                                     (JVPFA_LDS(void))(uintptr_t)(ld_dst + i * 1024 + ts * TILEB), 16, 0, 0);       \
+  };                                                                                                                \
+  /* row-major fragment (rows = streamed index, contraction over d): row 32hb + perm32(r), chunk 2kk+g */           \
+  uint32_t noff[KK];                                                                                                \
+  {                                                                                                                 \
+    const int x = swz_u<CH>(pr32);                                                                                  \
+    _Pragma("unroll") for (int kk = 0; kk < KK; ++kk) noff[kk] = pr32 * ROWB + (((2 * kk + g) ^ x) * 16);           \
+  }                                                                                                                 \
+  /* transposed fragment (rows = d, contraction over the streamed index), see fwd_kernel_v2.hpp */                  \
+  uint32_t toff[DB][2];                                                                                             \
+  {                                                                                                                 \
+    const int a_ = (lane >> 4) & 1, j_ = lane & 15;                                                                 \
+    _Pragma("unroll") for (int db = 0; db < DB; ++db) {                                                             \
+      _Pragma("unroll") for (int hh = 0; hh < 2; ++hh) {                                                            \
+        const int row = 8 * g + 4 * hh + (j_ >> 2);                                                                 \
+        const int ch = (4 * db + 2 * a_ + (j_ & 1)) ^ swz_u<CH>(row);                                               \
+        toff[db][hh] = row * ROWB + ch * 16 + 8 * ((j_ >> 1) & 1);                                                  \
+      }                                                                                                             \
+    }                                                                                                               \
+  }
+
+template <int KK, typename T>
+__device__ __forceinline__ void load_bfrags(Frag<T> *f, const T *row, int g) {
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) f[kk] = ld8<T>(row + 16 * kk + 8 * g);
+}
+
+__device__ __forceinline__ void zero_acc(f32x16 &x) {
+#pragma unroll
+  for (int e = 0; e < 16; ++e) x[e] = 0.f;
+}
+
+// ------------------------------------------------------------------------------------------------
+// dq (PLAIN / DUAL) or dq' (TANGENT): workgroup = 128 query rows, loop over 64-key tiles of
+// K, V (, K', V').  Scores are transposed (lane = query) so dS is the B operand of dQ^T += K^T dS^T.
+template <typename T, int D, int MODE, int MASK>
+__global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
+  using Cfg = Bwd2Cfg<T, D, MODE>;
+  constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
+  JVPFA_BWD2_COMMON(Cfg)
+  const int qb = pr.causal ? nblk - 1 - id % nblk : id % nblk;
+  const int q0 = qb * Cfg::BLK;
+  const int qrow = q0 + wave * 32 + r;
+  const int qld = qrow < L ? qrow : L - 1;
+  const bool has_go = p.go != nullptr;
+
+  Frag<T> Qf[KK], gOf[TAN ? 1 : KK], Qtf[DUAL ? KK : 1], gTf[(DUAL || TAN) ? KK : 1];
+  load_bfrags<KK>(Qf, reinterpret_cast<const T *>(p.q) + head + (size_t)qld * D, g);
+  if constexpr (!TAN) {
+    if (has_go) load_bfrags<KK>(gOf, reinterpret_cast<const T *>(p.go) + head + (size_t)qld * D, g);
+  }
+  if constexpr (DUAL) load_bfrags<KK>(Qtf, reinterpret_cast<const T *>(p.qt) + head + (size_t)qld * D, g);
+  if constexpr (DUAL || TAN) load_bfrags<KK>(gTf, reinterpret_cast<const T *>(p.gt) + head + (size_t)qld * D, g);
+
+  const float Mq = qrow < L ? p.M[srow + qld] : __builtin_inff();
+  const float d1 = (MODE == BWD_PLAIN) ? p.d1[srow + qld] : 0.f;
+  const float mu = DUAL ? p.mu[srow + qld] : 0.f;
+  const float av = (DUAL || TAN) ? p.a[srow + qld] : 0.f;
+  const float dsum = DUAL ? p.d2[srow + qld] : 0.f;
+
+  f32x16 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) zero_acc(acc[db]);
+
+  const float sl2 = pr.scale * LOG2E;
+  const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
+  const char *Kb = reinterpret_cast<const char *>(p.k) + head * sizeof(T);
+  const char *Vb = reinterpret_cast<const char *>(p.v) + head * sizeof(T);
+  const char *Ktb = DUAL ? reinterpret_cast<const char *>(p.kt) + head * sizeof(T) : nullptr;
+  const char *Vtb = DUAL ? reinterpret_cast<const char *>(p.vt) + head * sizeof(T) : nullptr;
+
+  const int kend = pr.causal ? min(L, q0 + Cfg::BLK) : L;
+  const int ntiles = (kend + BT - 1) / BT;
+  // tile slots in a stage: 0 K, 1 V, 2 K', 3 V'
+  constexpr int NLOAD = IPW * Cfg::NTILE;
+  constexpr int NACC = DUAL ? 2 : 1;            // operand tensors of the accumulation (K, K')
+  constexpr int NPV = 2 * DB / 2;               // accumulation steps of a half: (chunk c, pair of d-blocks)
+  constexpr int NSTEP = 2 * (KK + NPV);
+  auto prepare_loads = [&](int stage, int j0, bool on) {
+    j0 = on ? j0 : 0;
+    ld_rows = L - 1 - j0;
+    ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
+    const size_t tb = (size_t)j0 * ROWB;
+    ld_p[0] = Kb + tb;
+    ld_p[1] = Vb + tb;
+    if constexpr (DUAL) {
+      ld_p[2] = Ktb + tb;
+      ld_p[3] = Vtb + tb;
+    }
+  };
+  auto load_step = [&](auto gc) {
+    constexpr int gi = decltype(gc)::value;
+    constexpr int lo = (gi * NLOAD + NSTEP - 1) / NSTEP, hi = ((gi + 1) * NLOAD + NSTEP - 1) / NSTEP;
+    static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+  };
+
+  auto half_tile = [&](auto HBc, uint32_t sbase, int jh) {
+    constexpr int HB = decltype(HBc)::value;
+    constexpr int RO = HB * 32 * ROWB;
+    // ---- recompute: S, (S', dP, A, B) --------------------------------------------------------
+    FragN fk[2], fv[2], fkt[2], fvt[2];
+    auto issue_n = [&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value, sl = kk % 2;
+      const uint32_t ad = sbase + noff[kk];
+      fk[sl].v = lds_b128<RO>(ad);
+      fv[sl].v = lds_b128<RO + TILEB>(ad);
+      if constexpr (DUAL) {
+        fkt[sl].v = lds_b128<RO + 2 * TILEB>(ad);
+        fvt[sl].v = lds_b128<RO + 3 * TILEB>(ad);
+      }
+    };
+    constexpr int NRN = DUAL ? 4 : 2;
+    f32x16 S, dP, Sp, At, Bt;
+    zero_acc(S);
+    zero_acc(dP);
+    zero_acc(Sp);
+    zero_acc(At);
+    zero_acc(Bt);
+    issue_n(std::integral_constant<int, 0>{});
+    static_for<KK>([&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value, sl = kk % 2;
+      if constexpr (kk + 1 < KK) issue_n(std::integral_constant<int, kk + 1>{});
+      if constexpr (DUAL) lds_wait<(kk + 1 < KK) ? NRN : 0>(fk[sl], fv[sl], fkt[sl], fvt[sl]);
+      else lds_wait<(kk + 1 < KK) ? NRN : 0>(fk[sl], fv[sl]);
+      load_step(std::integral_constant<int, HB * KK + kk>{});
+      const Frag<T> k_ = as_frag<T>(fk[sl]), v_ = as_frag<T>(fv[sl]);
+      mma(S, k_, Qf[kk]);
+      if constexpr (MODE == BWD_PLAIN) mma(dP, v_, gOf[kk]);
+      if constexpr (TAN) mma(At, v_, gTf[kk]);
+      if constexpr (DUAL) {
+        if (has_go) mma(dP, v_, gOf[kk]);
+        mma(Sp, k_, Qtf[kk]);
+        mma(At, v_, gTf[kk]);
+        mma(Sp, as_frag<T>(fkt[sl]), Qf[kk]);
+        mma(Bt, as_frag<T>(fvt[sl]), gTf[kk]);
+      }
+    });
+
+    // ---- P and the score gradients -------------------------------------------------------------
+    const bool diag = pr.causal && (jh + 31 > q0 + wave * 32);
+    const bool ragged = jh + 32 > L;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int key0 = jh + 16 * hf + 8 * g;
+      float bias[8];
+      bool keep[8];
+      if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
+      if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int i = 8 * hf + e;
+        float s = S[i] * sl2;
+        if constexpr (MASK == MASK_ADD) s += bias[e];
+        float pv = fast_exp2(s - Mq);
+        if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
+        if (diag) pv = (key0 + e <= qrow) ? pv : 0.f;
+        if (ragged) pv = (key0 + e < L) ? pv : 0.f;
+        if constexpr (MODE == BWD_PLAIN) {
+          S[i] = pv * (dP[i] - d1);
+        } else if constexpr (DUAL) {
+          const float sp = Sp[i] * pr.scale, am = At[i] - av;
+          Sp[i] = pv * am;
+          S[i] = pv * (dP[i] + Bt[i] + am * sp - At[i] * mu - dsum);
+        } else {
+          S[i] = pv * (At[i] - av);
+        }
+      }
+    }
+    Frag<T> dsf[2], dspf[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      dsf[c] = to_frag<T>(S, c);
+      if constexpr (DUAL) dspf[c] = to_frag<T>(Sp, c);
+    }
+
+    // ---- dQ^T += K^T dS^T (+ K'^T dS'^T): steps over (key chunk c, pair of d-blocks) -------------
+    FragT tk[2][2], tkt[2][2];  // [ring slot][d-block of the pair]
+    auto issue_t = [&](auto ic) {
+      constexpr int i = decltype(ic)::value, c = i / (DB / 2), dp = i % (DB / 2), sl = i % 2;
+      constexpr int TO = (HB * 32 + c * 16) * ROWB;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const uint32_t a0 = sbase + toff[2 * dp + u][0], a1 = sbase + toff[2 * dp + u][1];
+        tk[sl][u].lo = lds_tr64<TO>(a0);
+        tk[sl][u].hi = lds_tr64<TO>(a1);
+        if constexpr (DUAL) {
+          tkt[sl][u].lo = lds_tr64<TO + 2 * TILEB>(a0);
+          tkt[sl][u].hi = lds_tr64<TO + 2 * TILEB>(a1);
+        }
+      }
+    };
+    constexpr int NRT = 4 * NACC;
+    issue_t(std::integral_constant<int, 0>{});
+    static_for<NPV>([&](auto ic) {
+      constexpr int i = decltype(ic)::value, c = i / (DB / 2), dp = i % (DB / 2), sl = i % 2;
+      if constexpr (i + 1 < NPV) issue_t(std::integral_constant<int, i + 1>{});
+      if constexpr (DUAL) lds_wait<(i + 1 < NPV) ? NRT : 0>(tk[sl][0], tk[sl][1], tkt[sl][0], tkt[sl][1]);
+      else lds_wait<(i + 1 < NPV) ? NRT : 0>(tk[sl][0], tk[sl][1]);
+      load_step(std::integral_constant<int, 2 * KK + HB * NPV + i>{});
+      mma(acc[2 * dp], as_frag<T>(tk[sl][0]), dsf[c]);
+      mma(acc[2 * dp + 1], as_frag<T>(tk[sl][1]), dsf[c]);
+      if constexpr (DUAL) {
+        mma(acc[2 * dp], as_frag<T>(tkt[sl][0]), dspf[c]);
+        mma(acc[2 * dp + 1], as_frag<T>(tkt[sl][1]), dspf[c]);
+      }
+    });
+  };
+
+  prepare_loads(0, 0, true);
+  static_for<NLOAD>([&](auto pc) { load_piece(pc); });
+  for (int t = 0; t < ntiles; ++t) {
+    const int j0 = t * BT;
+    const int stage = t & 1;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
+    __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
+    prepare_loads(stage ^ 1, j0 + BT, t + 1 < ntiles);
+    const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
+    half_tile(std::integral_constant<int, 0>{}, sbase, j0);
+    if (j0 + 32 < kend) {
+      half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
+    } else {
+      static_for<KK>([&](auto gc) { load_step(std::integral_constant<int, KK + decltype(gc)::value>{}); });
+      static_for<NPV>([&](auto gc) { load_step(std::integral_constant<int, 2 * KK + NPV + decltype(gc)::value>{}); });
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the redirected loads of the last iteration must not outlive the kernel
+
+  if (qrow < L) {
+    T *out = reinterpret_cast<T *>(TAN ? p.dqt : p.dq) + head + (size_t)qrow * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = acc[db][8 * hf + e] * pr.scale;
+        store8<T>(out + 32 * db + 16 * hf + 8 * g, x);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// dk, dv (PLAIN / DUAL) or dk', dv' (TANGENT): workgroup = 128 key rows, loop over 64-query tiles
+// of Q, G (, Q', gT), G = gO (gT in TANGENT).  Scores are S = Q K^T (lane = key, registers =
+// queries) so P, dS are the B operands of dV^T += G^T P and dK^T += Q^T dS.
+template <typename T, int D, int MODE, int MASK>
+__global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
+  using Cfg = Bwd2Cfg<T, D, MODE>;
+  constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
+  JVPFA_BWD2_COMMON(Cfg)
+  const int kb = id % nblk;  // causal: the first key blocks have the longest query loops
+  const int k0 = kb * Cfg::BLK;
+  const int krow = k0 + wave * 32 + r;
+  const int kld = krow < L ? krow : L - 1;
+  const bool has_go = p.go != nullptr;
+  const uint32_t stat0 = lds0 + 2 * Cfg::STAGEB;  // row statistics, two stages of NSTAT x 64 floats
+
+  Frag<T> Kf[KK], Vf[KK], Ktf[DUAL ? KK : 1], Vtf[DUAL ? KK : 1];
+  load_bfrags<KK>(Kf, reinterpret_cast<const T *>(p.k) + head + (size_t)kld * D, g);
+  load_bfrags<KK>(Vf, reinterpret_cast<const T *>(p.v) + head + (size_t)kld * D, g);
+  if constexpr (DUAL) {
+    load_bfrags<KK>(Ktf, reinterpret_cast<const T *>(p.kt) + head + (size_t)kld * D, g);
+    load_bfrags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + head + (size_t)kld * D, g);
+  }
+
+  f32x16 dK[DB], dV[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    zero_acc(dK[db]);
+    zero_acc(dV[db]);
+  }
+
+  const float sl2 = pr.scale * LOG2E;
+  // tile slots: 0 Q, 1 G (gO; gT in TANGENT; gT again in DUAL without gO), 2 Q', 3 gT
+  const char *Qb = reinterpret_cast<const char *>(p.q) + head * sizeof(T);
+  const char *gTb = (DUAL || TAN) ? reinterpret_cast<const char *>(p.gt) + head * sizeof(T) : nullptr;
+  const char *Gb = TAN ? gTb : (has_go ? reinterpret_cast<const char *>(p.go) + head * sizeof(T) : gTb);
+  const char *Qtb = DUAL ? reinterpret_cast<const char *>(p.qt) + head * sizeof(T) : nullptr;
+  // statistics slots: PLAIN M, d1 | DUAL M, mu, a, d2 (= d1 + d2) | TANGENT M, a
+  const float *st_p[4] = {p.M + srow, MODE == BWD_PLAIN ? p.d1 + srow : (DUAL ? p.mu + srow : p.a + srow),
+                          DUAL ? p.a + srow : nullptr, DUAL ? p.d2 + srow : nullptr};
+
+  const int istart = pr.causal ? (k0 / BT) * BT : 0;
+  const int ntiles = (L - istart + BT - 1) / BT;
+  constexpr int NLOAD = IPW * Cfg::NTILE;
+  constexpr int NPV = 2 * DB;  // accumulation steps of a half: (query chunk c, d-block db)
+  constexpr int NSTEP = 2 * (KK + NPV);
+  int st_row = 0;
+  uint32_t st_dst = 0;
+  auto prepare_loads = [&](int stage, int i0, bool on) {
+    i0 = on ? i0 : istart;
+    ld_rows = L - 1 - i0;
+    ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
+    const size_t tb = (size_t)i0 * ROWB;
+    ld_p[0] = Qb + tb;
+    ld_p[1] = Gb + tb;
+    if constexpr (DUAL) {
+      ld_p[2] = Qtb + tb;
+      ld_p[3] = gTb + tb;
+    }
+    st_row = min(i0 + lane, L - 1);
+    st_dst = stat0 + stage * Cfg::STATB;
+  };
+  // one 4-byte-per-lane direct load per statistic (64 rows); wave s loads statistic s
+  auto load_stats = [&]() {
+    if (wave < Cfg::NSTAT) {
+      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(st_p[wave] + st_row),
+                                       (JVPFA_LDS(void))(uintptr_t)(st_dst + wave * BT * 4), 4, 0, 0);
+    }
+  };
+  auto load_step = [&](auto gc) {
+    constexpr int gi = decltype(gc)::value;
+    constexpr int lo = (gi * NLOAD + NSTEP - 1) / NSTEP, hi = ((gi + 1) * NLOAD + NSTEP - 1) / NSTEP;
+    static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+  };
+
+  auto half_tile = [&](auto HBc, uint32_t sbase, uint32_t sstat, int ih) {
+    constexpr int HB = decltype(HBc)::value;
+    constexpr int RO = HB * 32 * ROWB;
+    // ---- recompute ------------------------------------------------------------------------------
+    FragN fq[2], fg[2], fqt[2], fgt[2];
+    auto issue_n = [&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value, sl = kk % 2;
+      const uint32_t ad = sbase + noff[kk];
+      fq[sl].v = lds_b128<RO>(ad);
+      fg[sl].v = lds_b128<RO + TILEB>(ad);
+      if constexpr (DUAL) {
+        fqt[sl].v = lds_b128<RO + 2 * TILEB>(ad);
+        fgt[sl].v = lds_b128<RO + 3 * TILEB>(ad);
+      }
+    };
+    constexpr int NRN = DUAL ? 4 : 2;
+    f32x16 S, dP, Sp, At, Bt;
+    zero_acc(S);
+    zero_acc(dP);
+    zero_acc(Sp);
+    zero_acc(At);
+    zero_acc(Bt);
+    issue_n(std::integral_constant<int, 0>{});
+    static_for<KK>([&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value, sl = kk % 2;
+      if constexpr (kk + 1 < KK) issue_n(std::integral_constant<int, kk + 1>{});
+      if constexpr (DUAL) lds_wait<(kk + 1 < KK) ? NRN : 0>(fq[sl], fg[sl], fqt[sl], fgt[sl]);
+      else lds_wait<(kk + 1 < KK) ? NRN : 0>(fq[sl], fg[sl]);
+      load_step(std::integral_constant<int, HB * KK + kk>{});
+      const Frag<T> q_ = as_frag<T>(fq[sl]), g_ = as_frag<T>(fg[sl]);
+      mma(S, q_, Kf[kk]);
+      if constexpr (MODE == BWD_PLAIN) mma(dP, g_, Vf[kk]);
+      if constexpr (TAN) mma(At, g_, Vf[kk]);
+      if constexpr (DUAL) {
+        const Frag<T> gt_ = as_frag<T>(fgt[sl]);
+        if (has_go) mma(dP, g_, Vf[kk]);
+        mma(Sp, as_frag<T>(fqt[sl]), Kf[kk]);
+        mma(At, gt_, Vf[kk]);
+        mma(Sp, q_, Ktf[kk]);
+        mma(Bt, gt_, Vtf[kk]);
+      }
+    });
+
+    // ---- row statistics of the 32 queries: register e belongs to query 16(e/8) + 8g + e%8 ------
+    // read as four quads per statistic (quad c4 holds registers 4*c4 .. 4*c4+3)
+    u32x4 stq[Cfg::NSTAT][4];
+    const uint32_t sad = sstat + (HB * 32 + 8 * g) * 4;
+#pragma unroll
+    for (int s = 0; s < Cfg::NSTAT; ++s) {
+      stq[s][0] = lds_b128<0>(sad + s * BT * 4);
+      stq[s][1] = lds_b128<16>(sad + s * BT * 4);
+      stq[s][2] = lds_b128<64>(sad + s * BT * 4);
+      stq[s][3] = lds_b128<80>(sad + s * BT * 4);
+    }
+#pragma unroll
+    for (int s = 0; s < Cfg::NSTAT; ++s) lds_wait4<0>(stq[s][0], stq[s][1], stq[s][2], stq[s][3]);
+    auto stat = [&](int s, int e) { return __uint_as_float(stq[s][e / 4][e % 4]); };
+
+    const bool diag = pr.causal && (ih < k0 + wave * 32 + 31);
+    const bool ragged = ih + 32 > L;
+    f32x16 Pp;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
+      float s = S[e] * sl2;
+      bool keep = true;
+      if constexpr (MASK != MASK_NONE) {
+        const int qc = qi < L ? qi : L - 1;
+        const int64_t off = z * pr.ms[0] + h * pr.ms[1] + (int64_t)qc * pr.ms[2] + (int64_t)kld * pr.ms[3];
+        if constexpr (MASK == MASK_ADD) s += (float)reinterpret_cast<const T *>(pr.mask)[off] * LOG2E;
+        if constexpr (MASK == MASK_BOOL) keep = reinterpret_cast<const uint8_t *>(pr.mask)[off] != 0;
+      }
+      float pv = fast_exp2(s - stat(0, e));
+      if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
+      if (diag) pv = (krow <= qi) ? pv : 0.f;
+      if (ragged) pv = (qi < L) ? pv : 0.f;
+      S[e] = pv;
+      if constexpr (MODE == BWD_PLAIN) {
+        dP[e] = pv * (dP[e] - stat(1, e));
+      } else if constexpr (DUAL) {
+        const float sp = Sp[e] * pr.scale, m_ = stat(1, e), am = At[e] - stat(2, e);
+        Pp[e] = pv * (sp - m_);
+        Sp[e] = pv * am;
+        dP[e] = pv * (dP[e] + Bt[e] + am * sp - At[e] * m_ - stat(3, e));
+      } else {
+        Sp[e] = pv * (At[e] - stat(1, e));
+      }
+    }
+    Frag<T> pf[2], dsf[2], dspf[2], ppf[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      pf[c] = to_frag<T>(S, c);
+      if constexpr (!TAN) dsf[c] = to_frag<T>(dP, c);
+      if constexpr (DUAL || TAN) dspf[c] = to_frag<T>(Sp, c);
+      if constexpr (DUAL) ppf[c] = to_frag<T>(Pp, c);
+    }
+
+    // ---- dK^T += Q^T dS (+ Q'^T dS'), dV^T += G^T P (+ gT^T P'): steps over (query chunk, d-block) -
+    FragT tq[2], tg[2], tqt[2], tgt[2];
+    auto issue_t = [&](auto ic) {
+      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % 2;
+      constexpr int TO = (HB * 32 + c * 16) * ROWB;
+      const uint32_t a0 = sbase + toff[db][0], a1 = sbase + toff[db][1];
+      tq[sl].lo = lds_tr64<TO>(a0);
+      tq[sl].hi = lds_tr64<TO>(a1);
+      tg[sl].lo = lds_tr64<TO + TILEB>(a0);
+      tg[sl].hi = lds_tr64<TO + TILEB>(a1);
+      if constexpr (DUAL) {
+        tqt[sl].lo = lds_tr64<TO + 2 * TILEB>(a0);
+        tqt[sl].hi = lds_tr64<TO + 2 * TILEB>(a1);
+        tgt[sl].lo = lds_tr64<TO + 3 * TILEB>(a0);
+        tgt[sl].hi = lds_tr64<TO + 3 * TILEB>(a1);
+      }
+    };
+    constexpr int NRT = DUAL ? 8 : 4;
+    issue_t(std::integral_constant<int, 0>{});
+    static_for<NPV>([&](auto ic) {
+      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % 2;
+      if constexpr (i + 1 < NPV) issue_t(std::integral_constant<int, i + 1>{});
+      if constexpr (DUAL) lds_wait<(i + 1 < NPV) ? NRT : 0>(tq[sl], tg[sl], tqt[sl], tgt[sl]);
+      else lds_wait<(i + 1 < NPV) ? NRT : 0>(tq[sl], tg[sl]);
+      load_step(std::integral_constant<int, 2 * KK + HB * NPV + i>{});
+      if constexpr (MODE == BWD_PLAIN) {
+        mma(dK[db], as_frag<T>(tq[sl]), dsf[c]);
+        mma(dV[db], as_frag<T>(tg[sl]), pf[c]);
+      } else if constexpr (DUAL) {
+        mma(dK[db], as_frag<T>(tq[sl]), dsf[c]);
+        if (has_go) mma(dV[db], as_frag<T>(tg[sl]), pf[c]);
+        mma(dK[db], as_frag<T>(tqt[sl]), dspf[c]);
+        mma(dV[db], as_frag<T>(tgt[sl]), ppf[c]);
+      } else {
+        mma(dK[db], as_frag<T>(tq[sl]), dspf[c]);
+        mma(dV[db], as_frag<T>(tg[sl]), pf[c]);
+      }
+    });
+  };
+
+  prepare_loads(0, istart, true);
+  static_for<NLOAD>([&](auto pc) { load_piece(pc); });
+  load_stats();
+  for (int t = 0; t < ntiles; ++t) {
+    const int i0 = istart + t * BT;
+    const int stage = t & 1;
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    prepare_loads(stage ^ 1, i0 + BT, t + 1 < ntiles);
+    load_stats();
+    const uint32_t sbase = lds0 + stage * Cfg::STAGEB, sstat = stat0 + stage * Cfg::STATB;
+    half_tile(std::integral_constant<int, 0>{}, sbase, sstat, i0);
+    if (i0 + 32 < L) {
+      half_tile(std::integral_constant<int, 1>{}, sbase, sstat, i0 + 32);
+    } else {
+      static_for<KK>([&](auto gc) { load_step(std::integral_constant<int, KK + decltype(gc)::value>{}); });
+      static_for<NPV>([&](auto gc) { load_step(std::integral_constant<int, 2 * KK + NPV + decltype(gc)::value>{}); });
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+
+  if (krow < L) {
+    T *outk = reinterpret_cast<T *>(TAN ? p.dkt : p.dk) + head + (size_t)krow * D;
+    T *outv = reinterpret_cast<T *>(TAN ? p.dvt : p.dv) + head + (size_t)krow * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        float xk[8], xv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xk[e] = dK[db][8 * hf + e] * pr.scale;
+          xv[e] = dV[db][8 * hf + e];
+        }
+        store8<T>(outk + 32 * db + 16 * hf + 8 * g, xk);
+        store8<T>(outv + 32 * db + 16 * hf + 8 * g, xv);
+      }
+    }
+  }
+}
+
+}  // namespace jvpfa
