@@ -451,60 +451,21 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
     });
 
     // ---- row statistics of the 32 queries: register e belongs to query 16(e/8) + 8g + e%8 ------
-    // read as four quads per statistic (quad c4 holds registers 4*c4 .. 4*c4+3)
-    u32x4 stq[Cfg::NSTAT][4];
+    // read one quad of registers at a time (quad c4 = registers 4*c4 .. 4*c4+3), one quad ahead
+    u32x4 stq[2][Cfg::NSTAT];
     const uint32_t sad = sstat + (HB * 32 + 8 * g) * 4;
-#pragma unroll
-    for (int s = 0; s < Cfg::NSTAT; ++s) {
-      stq[s][0] = lds_b128<0>(sad + s * BT * 4);
-      stq[s][1] = lds_b128<16>(sad + s * BT * 4);
-      stq[s][2] = lds_b128<64>(sad + s * BT * 4);
-      stq[s][3] = lds_b128<80>(sad + s * BT * 4);
-    }
-#pragma unroll
-    for (int s = 0; s < Cfg::NSTAT; ++s) lds_wait4<0>(stq[s][0], stq[s][1], stq[s][2], stq[s][3]);
-    auto stat = [&](int s, int e) { return __uint_as_float(stq[s][e / 4][e % 4]); };
-
+    auto issue_s = [&](auto c4c) {
+      constexpr int c4 = decltype(c4c)::value;
+      static_for<Cfg::NSTAT>([&](auto sc) {
+        constexpr int s_ = decltype(sc)::value;
+        stq[c4 % 2][s_] = lds_b128<s_ * BT * 4 + (c4 / 2) * 64 + (c4 % 2) * 16>(sad);
+      });
+    };
     const bool diag = pr.causal && (ih < k0 + wave * 32 + 31);
     const bool ragged = ih + 32 > L;
-    f32x16 Pp;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
-      float s = S[e] * sl2;
-      bool keep = true;
-      if constexpr (MASK != MASK_NONE) {
-        const int qc = qi < L ? qi : L - 1;
-        const int64_t off = z * pr.ms[0] + h * pr.ms[1] + (int64_t)qc * pr.ms[2] + (int64_t)kld * pr.ms[3];
-        if constexpr (MASK == MASK_ADD) s += (float)reinterpret_cast<const T *>(pr.mask)[off] * LOG2E;
-        if constexpr (MASK == MASK_BOOL) keep = reinterpret_cast<const uint8_t *>(pr.mask)[off] != 0;
-      }
-      float pv = fast_exp2(s - stat(0, e));
-      if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
-      if (diag) pv = (krow <= qi) ? pv : 0.f;
-      if (ragged) pv = (qi < L) ? pv : 0.f;
-      S[e] = pv;
-      if constexpr (MODE == BWD_PLAIN) {
-        dP[e] = pv * (dP[e] - stat(1, e));
-      } else if constexpr (DUAL) {
-        const float sp = Sp[e] * pr.scale, m_ = stat(1, e), am = At[e] - stat(2, e);
-        Pp[e] = pv * (sp - m_);
-        Sp[e] = pv * am;
-        dP[e] = pv * (dP[e] + Bt[e] + am * sp - At[e] * m_ - stat(3, e));
-      } else {
-        Sp[e] = pv * (At[e] - stat(1, e));
-      }
-    }
-    Frag<T> pf[2], dsf[2], dspf[2], ppf[2];
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      pf[c] = to_frag<T>(S, c);
-      if constexpr (!TAN) dsf[c] = to_frag<T>(dP, c);
-      if constexpr (DUAL || TAN) dspf[c] = to_frag<T>(Sp, c);
-      if constexpr (DUAL) ppf[c] = to_frag<T>(Pp, c);
-    }
-
-    // ---- dK^T += Q^T dS (+ Q'^T dS'), dV^T += G^T P (+ gT^T P'): steps over (query chunk, d-block) -
+    // The 32 queries are handled as two chunks of 16 (registers 8c .. 8c+7): score gradients of a
+    // chunk, then its share of dK^T += Q^T dS (+ Q'^T dS'), dV^T += G^T P (+ gT^T P'), one step per
+    // d-block; the transposed fragments of a step are read one step ahead.
     FragT tq[2], tg[2], tqt[2], tgt[2];
     auto issue_t = [&](auto ic) {
       constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % 2;
@@ -522,25 +483,74 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
       }
     };
     constexpr int NRT = DUAL ? 8 : 4;
-    issue_t(std::integral_constant<int, 0>{});
-    static_for<NPV>([&](auto ic) {
-      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % 2;
-      if constexpr (i + 1 < NPV) issue_t(std::integral_constant<int, i + 1>{});
-      if constexpr (DUAL) lds_wait<(i + 1 < NPV) ? NRT : 0>(tq[sl], tg[sl], tqt[sl], tgt[sl]);
-      else lds_wait<(i + 1 < NPV) ? NRT : 0>(tq[sl], tg[sl]);
-      load_step(std::integral_constant<int, 2 * KK + HB * NPV + i>{});
-      if constexpr (MODE == BWD_PLAIN) {
-        mma(dK[db], as_frag<T>(tq[sl]), dsf[c]);
-        mma(dV[db], as_frag<T>(tg[sl]), pf[c]);
-      } else if constexpr (DUAL) {
-        mma(dK[db], as_frag<T>(tq[sl]), dsf[c]);
-        if (has_go) mma(dV[db], as_frag<T>(tg[sl]), pf[c]);
-        mma(dK[db], as_frag<T>(tqt[sl]), dspf[c]);
-        mma(dV[db], as_frag<T>(tgt[sl]), ppf[c]);
-      } else {
-        mma(dK[db], as_frag<T>(tq[sl]), dspf[c]);
-        mma(dV[db], as_frag<T>(tg[sl]), pf[c]);
+    issue_s(std::integral_constant<int, 0>{});
+    static_for<2>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      f32x8 Pp;  // P * (S' - mu) of this chunk
+      static_for<2>([&](auto hc) {
+        constexpr int c4 = 2 * c + decltype(hc)::value, sl = c4 % 2;
+        if constexpr (c4 + 1 < 4) issue_s(std::integral_constant<int, c4 + 1>{});
+        // waits also cover the transposed fragments issued before (LDS reads complete in order)
+        if constexpr (Cfg::NSTAT == 4) lds_wait4<(c4 + 1 < 4) ? 4 : 0>(stq[sl][0], stq[sl][1], stq[sl][2], stq[sl][3]);
+        else lds_wait<(c4 + 1 < 4) ? 2 : 0>(stq[sl][0], stq[sl][1]);
+        auto stat = [&](int s_, int e) { return __uint_as_float(stq[sl][s_][e % 4]); };
+#pragma unroll
+        for (int e = 4 * c4; e < 4 * c4 + 4; ++e) {
+          const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
+          float s = S[e] * sl2;
+          bool keep = true;
+          if constexpr (MASK != MASK_NONE) {
+            const int qc = qi < L ? qi : L - 1;
+            const int64_t off = z * pr.ms[0] + h * pr.ms[1] + (int64_t)qc * pr.ms[2] + (int64_t)kld * pr.ms[3];
+            if constexpr (MASK == MASK_ADD) s += (float)reinterpret_cast<const T *>(pr.mask)[off] * LOG2E;
+            if constexpr (MASK == MASK_BOOL) keep = reinterpret_cast<const uint8_t *>(pr.mask)[off] != 0;
+          }
+          float pv = fast_exp2(s - stat(0, e));
+          if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
+          if (diag) pv = (krow <= qi) ? pv : 0.f;
+          if (ragged) pv = (qi < L) ? pv : 0.f;
+          S[e] = pv;
+          if constexpr (MODE == BWD_PLAIN) {
+            dP[e] = pv * (dP[e] - stat(1, e));
+          } else if constexpr (DUAL) {
+            const float sp = Sp[e] * pr.scale, m_ = stat(1, e), am = At[e] - stat(2, e);
+            Pp[e - 8 * c] = pv * (sp - m_);
+            Sp[e] = pv * am;
+            dP[e] = pv * (dP[e] + Bt[e] + am * sp - At[e] * m_ - stat(3, e));
+          } else {
+            Sp[e] = pv * (At[e] - stat(1, e));
+          }
+        }
+      });
+      const Frag<T> pf = to_frag<T>(S, c);
+      Frag<T> dsf, dspf, ppf;
+      if constexpr (!TAN) dsf = to_frag<T>(dP, c);
+      if constexpr (DUAL || TAN) dspf = to_frag<T>(Sp, c);
+      if constexpr (DUAL) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ppf[e] = (T)Pp[e];
       }
+      // the next quad of statistics (if any) was issued above, before these fragment reads
+      issue_t(std::integral_constant<int, c * DB>{});
+      static_for<DB>([&](auto dbc) {
+        constexpr int db = decltype(dbc)::value, i = c * DB + db, sl = i % 2;
+        if constexpr (db + 1 < DB) issue_t(std::integral_constant<int, i + 1>{});
+        if constexpr (DUAL) lds_wait<(db + 1 < DB) ? NRT : 0>(tq[sl], tg[sl], tqt[sl], tgt[sl]);
+        else lds_wait<(db + 1 < DB) ? NRT : 0>(tq[sl], tg[sl]);
+        load_step(std::integral_constant<int, 2 * KK + HB * NPV + i>{});
+        if constexpr (MODE == BWD_PLAIN) {
+          mma(dK[db], as_frag<T>(tq[sl]), dsf);
+          mma(dV[db], as_frag<T>(tg[sl]), pf);
+        } else if constexpr (DUAL) {
+          mma(dK[db], as_frag<T>(tq[sl]), dsf);
+          if (has_go) mma(dV[db], as_frag<T>(tg[sl]), pf);
+          mma(dK[db], as_frag<T>(tqt[sl]), dspf);
+          mma(dV[db], as_frag<T>(tgt[sl]), ppf);
+        } else {
+          mma(dK[db], as_frag<T>(tq[sl]), dspf);
+          mma(dV[db], as_frag<T>(tg[sl]), pf);
+        }
+      });
     });
   };
 
