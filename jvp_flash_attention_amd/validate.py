@@ -1,0 +1,161 @@
+"""Accuracy and speed report for JVP attention on the current GPU.
+
+    python -m jvp_flash_attention_amd.validate --dtype bfloat16 [--seq-lengths 32 64 ... 2048]
+                                               [--no-masks] [--json out.json]
+
+Counterpart of the reference's script ``tests/test_jvp_attention.py`` (run as a program there,
+README.md:111-113): for every sequence length, mask type (none / boolean / additive) and causal
+flag it (1) compares ``JVPAttn.fwd_dual`` under ``fwAD.dual_level()`` and under ``torch.func.jvp``
+with PyTorch's math SDPA under forward-mode AD (the reference's oracle, test file lines 548-617):
+primal, tangent, the loss ``mean((out - target)^2)`` and its q/k/v gradients; (2) times the dual
+forward the way the reference does (10 warm-up + 100 calls, input clones and ``make_dual``
+included, lines 129-143 and 770-780) next to math SDPA; (3) records the peak memory of one call.
+Shapes default to the reference's (batch 2, 12 heads, head dim 64, lines 225-230); masks are its
+random masks with keep-probability 0.1 (lines 334-394).  TFLOP/s uses the reference's FLOP
+convention ``2 * (4 B H L^2 D + 5 B H L^2)``, halved when causal (lines 49-83).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import time
+from functools import partial
+
+import torch
+import torch.autograd.forward_ad as fwAD
+import torch.nn.functional as F
+from torch.nn.attention import SDPBackend, sdpa_kernel
+
+from . import MASK_CONST, JVPAttn
+
+TOLERANCE = {"float16": 4e-3, "float32": 2.35e-2, "bfloat16": 3.2e-2}  # reference lines 688-693
+DTYPES = {"float16": torch.float16, "float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def flop_count(B, H, L, D, causal):
+    f = 2.0 * (4.0 * B * H * L * L * D + 5.0 * B * H * L * L)
+    return f / 2 if causal else f
+
+
+def make_mask(kind, B, H, L, dtype, device):
+    if kind == "none":
+        return None
+    g = torch.Generator(device=device).manual_seed(1042)
+    keep = torch.rand(B, H, L, L, generator=g, device=device) > 0.9
+    keep[..., 0] |= ~keep.any(-1)  # no fully masked row
+    if kind == "boolean":
+        return keep
+    return torch.where(keep, 0.0, MASK_CONST).to(dtype)
+
+
+def sdpa_dual(q, k, v, qt, kt, vt, mask, causal):
+    sdpa_mask = mask
+    if mask is not None and mask.dtype != torch.bool:
+        sdpa_mask = mask != MASK_CONST  # the reference's float masks mark masked entries with MASK_CONST
+    with sdpa_kernel(SDPBackend.MATH), fwAD.dual_level():
+        out = F.scaled_dot_product_attention(fwAD.make_dual(q, qt), fwAD.make_dual(k, kt), fwAD.make_dual(v, vt),
+                                             attn_mask=sdpa_mask, is_causal=causal)
+        o, ot = fwAD.unpack_dual(out)
+        return o.clone(), ot.clone()
+
+
+def grads_of_mse(fn, q, k, v, target):
+    leaves = [x.clone().requires_grad_() for x in (q, k, v)]
+    loss = ((fn(*leaves).float() - target.float()) ** 2).mean()
+    return loss.detach(), torch.autograd.grad(loss, leaves)
+
+
+def timed(fn, warmup=10, iters=100):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / iters
+
+
+def peak_mb(fn):
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    fn()
+    torch.cuda.synchronize()
+    return (torch.cuda.max_memory_allocated() - base) / 2**20
+
+
+def run(args):
+    dev = torch.device("cuda")
+    dtype = DTYPES[args.dtype]
+    B, H, D = args.bsz, args.model_dim // args.head_dim, args.head_dim
+    rows = []
+    for L in args.seq_lengths:
+        g = torch.Generator(device=dev).manual_seed(42)
+        q, qt, k, kt, v, vt, target = [torch.randn(B, H, L, D, generator=g, device=dev, dtype=dtype) for _ in range(7)]
+        for kind in (["none"] if args.no_masks else ["none", "boolean", "additive"]):
+            mask = make_mask(kind, B, H, L, dtype, dev)
+            for causal in (False, True):
+                if causal and kind != "none":
+                    continue
+                fn = partial(JVPAttn.fwd_dual, attn_mask=mask, causal=causal)
+                o_ref, ot_ref = sdpa_dual(q, k, v, qt, kt, vt, mask, causal)
+                with fwAD.dual_level():
+                    o1, ot1 = (t.clone() for t in fwAD.unpack_dual(fn(fwAD.make_dual(q, qt), fwAD.make_dual(k, kt), fwAD.make_dual(v, vt))))
+                o2, ot2 = torch.func.jvp(fn, (q, k, v), (qt, kt, vt))
+                sdpa_mask = mask if (mask is None or mask.dtype == torch.bool) else mask != MASK_CONST
+                with sdpa_kernel(SDPBackend.MATH):
+                    loss_ref, g_ref = grads_of_mse(
+                        lambda a, b, c: F.scaled_dot_product_attention(a, b, c, attn_mask=sdpa_mask, is_causal=causal),
+                        q, k, v, target)
+                loss, g_ours = grads_of_mse(lambda a, b, c: JVPAttn.fwd(a, b, c, attn_mask=mask, causal=causal), q, k, v, target)
+                err = lambda a, b: (a.float() - b.float()).abs().max().item()  # noqa: E731
+                acc = {
+                    "primal": max(err(o1, o_ref), err(o2, o_ref)), "tangent": max(err(ot1, ot_ref), err(ot2, ot_ref)),
+                    "loss": abs(loss.item() - loss_ref.item()),
+                    "dq": err(g_ours[0], g_ref[0]), "dk": err(g_ours[1], g_ref[1]), "dv": err(g_ours[2], g_ref[2]),
+                }
+                ok = max(acc["primal"], acc["tangent"]) < TOLERANCE[args.dtype] and max(acc["loss"], acc["dq"], acc["dk"], acc["dv"]) < 5e-4
+
+                def ours():
+                    with fwAD.dual_level():
+                        return fn(fwAD.make_dual(q.clone(), qt.clone()), fwAD.make_dual(k.clone(), kt.clone()),
+                                  fwAD.make_dual(v.clone(), vt.clone()))
+
+                def ours_kernel_only():
+                    return JVPAttn.forward(q, k, v, qt, kt, vt, mask, 0.0, causal, None, True, True, False)
+
+                ms, ms_k = timed(ours), timed(ours_kernel_only)
+                ms_sdpa = timed(lambda: sdpa_dual(q, k, v, qt, kt, vt, mask, causal), 2, 10)
+                fl = 2 * flop_count(B, H, L, D, causal) / 2  # the convention already counts the JVP (x2 inside)
+                row = {"L": L, "mask": kind, "causal": causal, "ok": ok, **acc, "ms": ms, "ms_kernel_only": ms_k,
+                       "ms_sdpa_math": ms_sdpa, "speedup": ms_sdpa / ms, "tflops": fl / (ms * 1e-3) / 1e12,
+                       "tflops_kernel_only": fl / (ms_k * 1e-3) / 1e12, "mem_mb": peak_mb(ours),
+                       "mem_mb_sdpa": peak_mb(lambda: sdpa_dual(q, k, v, qt, kt, vt, mask, causal))}
+                rows.append(row)
+                print(f"L={L:5d} mask={kind:9s} causal={str(causal):5s} {'ok ' if ok else 'FAIL'} "
+                      f"primal {acc['primal']:.2e} tangent {acc['tangent']:.2e} grads {max(acc['dq'], acc['dk'], acc['dv']):.2e} | "
+                      f"{ms:7.3f} ms ({ms_k:7.3f} kernel only) sdpa {ms_sdpa:8.3f} ms x{ms_sdpa / ms:5.1f} | "
+                      f"{row['tflops']:6.1f} TFLOP/s | {row['mem_mb']:7.1f} MB vs {row['mem_mb_sdpa']:8.1f} MB", flush=True)
+    n_ok = sum(r["ok"] for r in rows)
+    print(f"\naccuracy: {n_ok}/{len(rows)} passed; mean speed-up over math SDPA {sum(r['speedup'] for r in rows) / len(rows):.2f}x")
+    if args.json:
+        with open(args.json, "w") as f:
+            json.dump({"dtype": args.dtype, "bsz": B, "heads": H, "head_dim": D, "rows": rows}, f, indent=1)
+    return rows
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--dtype", default="bfloat16", choices=list(DTYPES))
+    ap.add_argument("--bsz", type=int, default=2)
+    ap.add_argument("--model-dim", type=int, default=768)
+    ap.add_argument("--head-dim", type=int, default=64)
+    ap.add_argument("--seq-lengths", type=int, nargs="+", default=[32, 64, 128, 256, 512, 1024, 2048])
+    ap.add_argument("--no-masks", action="store_true")
+    ap.add_argument("--json", default=None)
+    run(ap.parse_args())
+
+
+if __name__ == "__main__":
+    main()
