@@ -200,3 +200,98 @@ def test_single_key(dt):
         assert grads[i].float().abs().max().item() <= bound
     assert (grads[2].float() - go.float()).abs().max().item() <= bound
     assert (grads[5].float() - gt.float()).abs().max().item() <= bound
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_growing_row_maximum_exercises_the_rescale_path(dt, causal):
+    """Keys whose scores grow along the sequence: the running maximum keeps rising past the lazy
+    rescale threshold, so the accumulators are rescaled on many tiles (not only the first)."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    dtype = DTYPES[dt]
+    Z, H, L, D = 1, 2, 512, 128
+    q, k, v, qt, kt, vt, go, gt = _make(Z, H, L, D, dtype, 21)
+    ramp = torch.linspace(0.2, 6.0, L).view(1, 1, L, 1)
+    k = (k.float() * ramp).to(dtype)
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    scale = D**-0.5
+    ref = dense.forward(*f64[:6], causal=causal, scale=scale)
+    rb = dense.backward(*f64, causal=causal, scale=scale)
+    o, ot, M, mu = be.fwd(*dev[:6], None, _lib.MASK_NONE, causal, scale)
+    # fp32 bound relative to the size of the outputs here (scores reach +-60, O' reaches ~1e2)
+    for name, got, want in (("O", o, ref["O"]), ("O'", ot, ref["Ot"])):
+        got = got.double().cpu().numpy()
+        rel = np.abs(got - want).max() / np.abs(want).max()
+        assert np.isfinite(got).all() and rel <= (2e-5 if dtype == torch.float32 else 2e-2), (name, rel)
+    assert np.abs(M.double().cpu().numpy() - ref["M"]).max() < (1e-3 if dtype == torch.float32 else 0.25)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], None, _lib.MASK_NONE, causal, scale, want_tangent_grads=True)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        got = t.double().cpu().numpy()
+        rel = np.abs(got - rb[n]).max() / np.abs(rb[n]).max()
+        assert np.isfinite(got).all() and rel <= (5e-5 if dtype == torch.float32 else 3e-2), (n, rel)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+@pytest.mark.parametrize("scale", [0.05, 1.0, -0.3])
+def test_custom_softmax_scale_including_negative(dt, scale):
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    dtype = DTYPES[dt]
+    Z, H, L, D = 1, 2, 192, 64
+    xs = _make(Z, H, L, D, dtype, 33)
+    if abs(scale) >= 1.0:
+        xs[0] = (xs[0].float() * 0.3).to(dtype)
+    f64 = [x.double().numpy() for x in xs]
+    dev = [x.cuda() for x in xs]
+    ref = dense.forward(*f64[:6], scale=scale)
+    rb = dense.backward(*f64, scale=scale)
+    o, ot, M, mu = be.fwd(*dev[:6], None, _lib.MASK_NONE, False, scale)
+
+    def check(name, got, want):
+        # with |scale| = 1 the gradients reach ~50, so the fp32 bound is taken relative to that size
+        if dtype == torch.float32:
+            err = np.abs(got.double().cpu().numpy() - want).max()
+            assert err <= 1e-4 * max(1.0, np.abs(want).max() / 8), f"{name}: {err:.3e}"
+        else:
+            _tol_check(name, got, want, dtype)
+
+    check("O", o, ref["O"])
+    check("O'", ot, ref["Ot"])
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], None, _lib.MASK_NONE, False, scale)
+    for n, t in zip(("dq", "dk", "dv"), grads[:3]):
+        check(n, t, rb[n])
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+def test_additive_mask_with_minus_infinity_entries(dt):
+    """SDPA-style float masks use -inf for masked entries; whole tiles and whole rows of -inf included."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    dtype = DTYPES[dt]
+    Z, H, L, D = 1, 2, 160, 64
+    xs = _make(Z, H, L, D, dtype, 35)
+    g = torch.Generator().manual_seed(5)
+    bias = torch.randn(Z, H, L, L, generator=g)
+    bias[torch.rand(Z, H, L, L, generator=g) < 0.5] = -float("inf")
+    bias[..., :, 64:128] = -float("inf")   # a whole 64-key tile masked for every row
+    bias[..., 0] = 0.0                      # every row keeps key 0 ...
+    bias[0, 1, 17, :] = -float("inf")      # ... except one fully masked row
+    bias = bias.to(dtype)
+    f64 = [x.double().numpy() for x in xs]
+    dev = [x.cuda() for x in xs]
+    scale = D**-0.5
+    ref = dense.forward(*f64[:6], mask=bias.double().numpy(), scale=scale)
+    rb = dense.backward(*f64, mask=bias.double().numpy(), scale=scale)
+    o, ot, M, mu = be.fwd(*dev[:6], bias.cuda(), _lib.MASK_ADD, False, scale)
+    assert torch.all(o[0, 1, 17] == 0) and torch.all(ot[0, 1, 17] == 0) and torch.isposinf(M[0, 1, 17])
+    _tol_check("O", o, ref["O"], dtype)
+    _tol_check("O'", ot, ref["Ot"], dtype)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], bias.cuda(), _lib.MASK_ADD, False, scale,
+                   want_tangent_grads=True)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        _tol_check(n, t, rb[n], dtype)
