@@ -47,28 +47,30 @@ def units():
 
 
 def _compile(unit):
-    name, src, defs = unit
-    obj = os.path.join(OBJ, name + ".o")
-    cmd = [HIPCC, *FLAGS, *defs, "-c", src, "-o", obj]
+    name, src, defs, objdir, extra = unit
+    obj = os.path.join(objdir, name + ".o")
+    cmd = [HIPCC, *FLAGS, *extra, *defs, "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {name}:\n{' '.join(cmd)}\n{r.stderr[-4000:]}")
     return obj
 
 
-def build(jobs: int | None = None, verbose: bool = True) -> str:
-    os.makedirs(OBJ, exist_ok=True)
+def build(jobs: int | None = None, verbose: bool = True, extra_flags=(), lib: str = LIB, objdir: str = OBJ) -> str:
+    """Compile and link.  ``extra_flags`` / ``lib`` / ``objdir`` build a variant next to the default
+    library (used to compare kernel tuning constants, e.g. ``-DJVPFA_RING=4``)."""
+    os.makedirs(objdir, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
-    us = units()
+    us = [(*u, objdir, list(extra_flags)) for u in units()]
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(_compile, us))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", lib]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
     if verbose:
-        print(f"built {LIB} from {len(objs)} objects", flush=True)
-    return LIB
+        print(f"built {lib} from {len(objs)} objects", flush=True)
+    return lib
 
 
 if __name__ == "__main__":

@@ -19,6 +19,10 @@
 #include "params.hpp"
 #include "pipeline.hpp"
 
+#ifndef JVPFA_RING
+#define JVPFA_RING 5
+#endif
+
 namespace jvpfa {
 
 #ifdef JVPFA_TRACE
@@ -229,23 +233,25 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     constexpr int NRV = DUAL ? 4 : 2;   // LDS reads per PV step
     constexpr int NPV = 2 * DB;         // PV steps: (16-key chunk c, d-block db)
 
-    u32x4 ka[3], kb[3];
+    constexpr int RD = JVPFA_RING;  // fragment ring slots; reads run RD-1 steps ahead
+    constexpr int PD = RD - 1;
+    u32x4 ka[RD], kb[RD];
     auto issue_k = [&](auto kkc) {
       constexpr int kk = decltype(kkc)::value;
       const uint32_t ad = sbase + koff[kk];
-      ka[kk % 3] = lds_b128<KO>(ad);
-      if constexpr (DUAL) kb[kk % 3] = lds_b128<KO + 2 * TILEB>(ad);
+      ka[kk % RD] = lds_b128<KO>(ad);
+      if constexpr (DUAL) kb[kk % RD] = lds_b128<KO + 2 * TILEB>(ad);
     };
-    u32x2 va[3][2], vb[3][2];
+    u32x2 va[RD][2], vb[RD][2];
     auto issue_v = [&](auto ic) {
       constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB;
       constexpr int VO = TILEB + (HB * 32 + c * 16) * ROWB;
       const uint32_t a0 = sbase + voff[db][0], a1 = sbase + voff[db][1];
-      va[i % 3][0] = lds_tr64<VO>(a0);
-      va[i % 3][1] = lds_tr64<VO>(a1);
+      va[i % RD][0] = lds_tr64<VO>(a0);
+      va[i % RD][1] = lds_tr64<VO>(a1);
       if constexpr (DUAL) {
-        vb[i % 3][0] = lds_tr64<VO + 2 * TILEB>(a0);
-        vb[i % 3][1] = lds_tr64<VO + 2 * TILEB>(a1);
+        vb[i % RD][0] = lds_tr64<VO + 2 * TILEB>(a0);
+        vb[i % RD][1] = lds_tr64<VO + 2 * TILEB>(a1);
       }
     };
 
@@ -255,19 +261,19 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       S[e] = 0.f;
       Sp[e] = 0.f;
     }
-    issue_k(std::integral_constant<int, 0>{});
-    issue_k(std::integral_constant<int, 1>{});
+    static_for<(PD < KK ? PD : KK)>([&](auto kkc) { issue_k(kkc); });
     static_for<KK>([&](auto kkc) {
       constexpr int kk = decltype(kkc)::value;
-      if constexpr (DUAL) lds_wait<(kk + 1 < KK) ? NRS : 0>(ka[kk % 3], kb[kk % 3]);
-      else lds_wait<(kk + 1 < KK) ? NRS : 0>(ka[kk % 3]);
-      if constexpr (kk + 2 < KK) issue_k(std::integral_constant<int, kk + 2>{});
+      constexpr int younger = (KK - 1 - kk < PD - 1) ? KK - 1 - kk : PD - 1;  // read groups issued after this one
+      if constexpr (DUAL) lds_wait<younger * NRS>(ka[kk % RD], kb[kk % RD]);
+      else lds_wait<younger * NRS>(ka[kk % RD]);
+      if constexpr (kk + PD < KK) issue_k(std::integral_constant<int, kk + PD>{});
       load_step(std::integral_constant<int, HB * (KK + NPV) + kk>{});
-      const Frag<T> a = __builtin_bit_cast(Frag<T>, ka[kk % 3]);
+      const Frag<T> a = __builtin_bit_cast(Frag<T>, ka[kk % RD]);
       mma(S, a, Qf[kk]);
       if constexpr (DUAL) {
         mma(Sp, a, Qtf[kk]);
-        mma(Sp, __builtin_bit_cast(Frag<T>, kb[kk % 3]), Qf[kk]);
+        mma(Sp, __builtin_bit_cast(Frag<T>, kb[kk % RD]), Qf[kk]);
       }
     });
     JVPFA_STAMP(5);
@@ -317,9 +323,8 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
         }
       }
     }
-    // V fragments of the first two PV steps travel while the softmax runs
-    issue_v(std::integral_constant<int, 0>{});
-    issue_v(std::integral_constant<int, 1>{});
+    // V fragments of the first PV steps travel while the softmax runs
+    static_for<(PD < NPV ? PD : NPV)>([&](auto ic) { issue_v(ic); });
 
     const float m_use = (m_i == NEG_INF) ? 0.f : m_i;
     float rs = 0.f, rmu = 0.f;
@@ -350,10 +355,11 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       if constexpr (DUAL) psf[c] = to_frag<T>(Sp, c);
     }
     static_for<NPV>([&](auto ic) {
-      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % 3;
-      if constexpr (DUAL) lds_wait<(i + 1 < NPV) ? NRV : 0>(va[sl][0], va[sl][1], vb[sl][0], vb[sl][1]);
-      else lds_wait<(i + 1 < NPV) ? NRV : 0>(va[sl][0], va[sl][1]);
-      if constexpr (i + 2 < NPV) issue_v(std::integral_constant<int, i + 2>{});
+      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % RD;
+      constexpr int younger = (NPV - 1 - i < PD - 1) ? NPV - 1 - i : PD - 1;
+      if constexpr (DUAL) lds_wait<younger * NRV>(va[sl][0], va[sl][1], vb[sl][0], vb[sl][1]);
+      else lds_wait<younger * NRV>(va[sl][0], va[sl][1]);
+      if constexpr (i + PD < NPV) issue_v(std::integral_constant<int, i + PD>{});
       load_step(std::integral_constant<int, HB * (KK + NPV) + KK + i>{});
       const u32x4 av = {va[sl][0][0], va[sl][0][1], va[sl][1][0], va[sl][1][1]};
       const Frag<T> a = __builtin_bit_cast(Frag<T>, av);
