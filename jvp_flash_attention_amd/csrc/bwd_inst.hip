@@ -16,8 +16,10 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
   if (blocks > 0x7fffffffLL) return -2;
   if constexpr (sizeof(T) == 2 && D >= 64) {  // direct-to-LDS, double-buffered kernels
     using Cfg2 = Bwd2Cfg<T, D, MODE>;
-    auto kq = bwd2_dq_kernel<T, D, MODE, MASK>;
-    auto kkv = bwd2_dkdv_kernel<T, D, MODE, MASK>;
+    // gO may be absent only in the dual mode (loss depends on O' alone)
+    const bool no_go = MODE == BWD_DUAL && p.go == nullptr;
+    auto kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, MODE != BWD_DUAL> : bwd2_dq_kernel<T, D, MODE, MASK, true>;
+    auto kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, MODE != BWD_DUAL> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
     int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
     if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);
     if (rc != 0) return rc;

@@ -125,7 +125,7 @@ __device__ __forceinline__ void zero_acc(f32x16 &x) {
 // ------------------------------------------------------------------------------------------------
 // dq (PLAIN / DUAL) or dq' (TANGENT): workgroup = 128 query rows, loop over 64-key tiles of
 // K, V (, K', V').  Scores are transposed (lane = query) so dS is the B operand of dQ^T += K^T dS^T.
-template <typename T, int D, int MODE, int MASK>
+template <typename T, int D, int MODE, int MASK, bool GO>
 __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
@@ -134,15 +134,23 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
   const int q0 = qb * Cfg::BLK;
   const int qrow = q0 + wave * 32 + r;
   const int qld = qrow < L ? qrow : L - 1;
-  const bool has_go = p.go != nullptr;
+  constexpr bool has_go = GO;  // compile-time: a run-time test here would split every step into its own block
 
   Frag<T> Qf[KK], gOf[TAN ? 1 : KK], Qtf[DUAL ? KK : 1], gTf[(DUAL || TAN) ? KK : 1];
   load_bfrags<KK>(Qf, reinterpret_cast<const T *>(p.q) + head + (size_t)qld * D, g);
   if constexpr (!TAN) {
-    if (has_go) load_bfrags<KK>(gOf, reinterpret_cast<const T *>(p.go) + head + (size_t)qld * D, g);
+    if constexpr (has_go) load_bfrags<KK>(gOf, reinterpret_cast<const T *>(p.go) + head + (size_t)qld * D, g);
   }
   if constexpr (DUAL) load_bfrags<KK>(Qtf, reinterpret_cast<const T *>(p.qt) + head + (size_t)qld * D, g);
   if constexpr (DUAL || TAN) load_bfrags<KK>(gTf, reinterpret_cast<const T *>(p.gt) + head + (size_t)qld * D, g);
+  // the resident operands live in the accumulation register file from here on
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    pin_acc(Qf[kk]);
+    if constexpr (!TAN && has_go) pin_acc(gOf[kk]);
+    if constexpr (DUAL) pin_acc(Qtf[kk]);
+    if constexpr (DUAL || TAN) pin_acc(gTf[kk]);
+  }
 
   const float Mq = qrow < L ? p.M[srow + qld] : __builtin_inff();
   const float d1 = (MODE == BWD_PLAIN) ? p.d1[srow + qld] : 0.f;
@@ -202,31 +210,31 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
       }
     };
     constexpr int NRN = DUAL ? 4 : 2;
-    f32x16 S, dP, Sp, At, Bt;
-    zero_acc(S);
-    zero_acc(dP);
-    zero_acc(Sp);
-    zero_acc(At);
-    zero_acc(Bt);
+    // tiles in ordinary vector registers; in DUAL, dP also collects V' gT^T (the B term)
+    f32x16 S, dP, Sp, At;
     issue_n(std::integral_constant<int, 0>{});
     static_for<KK>([&](auto kkc) {
       constexpr int kk = decltype(kkc)::value, sl = kk % 2;
+      constexpr bool F = kk == 0;
       if constexpr (kk + 1 < KK) issue_n(std::integral_constant<int, kk + 1>{});
       if constexpr (DUAL) lds_wait<(kk + 1 < KK) ? NRN : 0>(fk[sl], fv[sl], fkt[sl], fvt[sl]);
       else lds_wait<(kk + 1 < KK) ? NRN : 0>(fk[sl], fv[sl]);
       load_step(std::integral_constant<int, HB * KK + kk>{});
       const Frag<T> k_ = as_frag<T>(fk[sl]), v_ = as_frag<T>(fv[sl]);
-      mma(S, k_, Qf[kk]);
-      if constexpr (MODE == BWD_PLAIN) mma(dP, v_, gOf[kk]);
-      if constexpr (TAN) mma(At, v_, gTf[kk]);
+      mma_vra<F>(S, k_, Qf[kk]);
+      if constexpr (MODE == BWD_PLAIN) mma_vra<F>(dP, v_, gOf[kk]);
+      if constexpr (TAN) mma_vra<F>(At, v_, gTf[kk]);
       if constexpr (DUAL) {
-        if (has_go) mma(dP, v_, gOf[kk]);
-        mma(Sp, k_, Qtf[kk]);
-        mma(At, v_, gTf[kk]);
-        mma(Sp, as_frag<T>(fkt[sl]), Qf[kk]);
-        mma(Bt, as_frag<T>(fvt[sl]), gTf[kk]);
+        if constexpr (has_go) mma_vra<F>(dP, v_, gOf[kk]);
+        mma_vra<F>(Sp, k_, Qtf[kk]);
+        mma_vra<F>(At, v_, gTf[kk]);
+        mma_vra<false>(Sp, as_frag<T>(fkt[sl]), Qf[kk]);
+        mma_vra<F && !has_go>(dP, as_frag<T>(fvt[sl]), gTf[kk]);
       }
     });
+    if constexpr (DUAL) tiles_ready(S, dP, Sp, At);
+    else if constexpr (TAN) tiles_ready(S, At);
+    else tiles_ready(S, dP);
 
     // ---- P and the score gradients -------------------------------------------------------------
     const bool diag = pr.causal && (jh + 31 > q0 + wave * 32);
@@ -252,7 +260,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
         } else if constexpr (DUAL) {
           const float sp = Sp[i] * pr.scale, am = At[i] - av;
           Sp[i] = pv * am;
-          S[i] = pv * (dP[i] + Bt[i] + am * sp - At[i] * mu - dsum);
+          S[i] = pv * (dP[i] + am * sp - At[i] * mu - dsum);
         } else {
           S[i] = pv * (At[i] - av);
         }
@@ -308,12 +316,9 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
     prepare_loads(stage ^ 1, j0 + BT, t + 1 < ntiles);
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
     half_tile(std::integral_constant<int, 0>{}, sbase, j0);
-    if (j0 + 32 < kend) {
-      half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
-    } else {
-      static_for<KK>([&](auto gc) { load_step(std::integral_constant<int, KK + decltype(gc)::value>{}); });
-      static_for<NPV>([&](auto gc) { load_step(std::integral_constant<int, 2 * KK + NPV + decltype(gc)::value>{}); });
-    }
+    // always both halves: a half past the last key or past the diagonal contributes exact zeros, and a
+    // branch here would make the accumulators change register file around it
+    half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the redirected loads of the last iteration must not outlive the kernel
 
@@ -336,7 +341,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
 // dk, dv (PLAIN / DUAL) or dk', dv' (TANGENT): workgroup = 128 key rows, loop over 64-query tiles
 // of Q, G (, Q', gT), G = gO (gT in TANGENT).  Scores are S = Q K^T (lane = key, registers =
 // queries) so P, dS are the B operands of dV^T += G^T P and dK^T += Q^T dS.
-template <typename T, int D, int MODE, int MASK>
+template <typename T, int D, int MODE, int MASK, bool GO>
 __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
@@ -345,7 +350,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
   const int k0 = kb * Cfg::BLK;
   const int krow = k0 + wave * 32 + r;
   const int kld = krow < L ? krow : L - 1;
-  const bool has_go = p.go != nullptr;
+  constexpr bool has_go = GO;  // compile-time: a run-time test here would split every step into its own block
   const uint32_t stat0 = lds0 + 2 * Cfg::STAGEB;  // row statistics, two stages of NSTAT x 64 floats
 
   Frag<T> Kf[KK], Vf[KK], Ktf[DUAL ? KK : 1], Vtf[DUAL ? KK : 1];
@@ -354,6 +359,15 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
   if constexpr (DUAL) {
     load_bfrags<KK>(Ktf, reinterpret_cast<const T *>(p.kt) + head + (size_t)kld * D, g);
     load_bfrags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + head + (size_t)kld * D, g);
+  }
+  // the resident operands live in the accumulation register file from here on
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    pin_acc(Kf[kk]);
+    pin_acc(Vf[kk]);
+    if constexpr (DUAL) {
+      pin_acc(Ktf[kk]);  // V' stays in vector registers: the accumulation file also holds dK, dV
+    }
   }
 
   f32x16 dK[DB], dV[DB];
@@ -423,32 +437,32 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
       }
     };
     constexpr int NRN = DUAL ? 4 : 2;
-    f32x16 S, dP, Sp, At, Bt;
-    zero_acc(S);
-    zero_acc(dP);
-    zero_acc(Sp);
-    zero_acc(At);
-    zero_acc(Bt);
+    // tiles in ordinary vector registers; in DUAL, dP also collects gT V'^T (the B term)
+    f32x16 S, dP, Sp, At;
     issue_n(std::integral_constant<int, 0>{});
     static_for<KK>([&](auto kkc) {
       constexpr int kk = decltype(kkc)::value, sl = kk % 2;
+      constexpr bool F = kk == 0;
       if constexpr (kk + 1 < KK) issue_n(std::integral_constant<int, kk + 1>{});
       if constexpr (DUAL) lds_wait<(kk + 1 < KK) ? NRN : 0>(fq[sl], fg[sl], fqt[sl], fgt[sl]);
       else lds_wait<(kk + 1 < KK) ? NRN : 0>(fq[sl], fg[sl]);
       load_step(std::integral_constant<int, HB * KK + kk>{});
       const Frag<T> q_ = as_frag<T>(fq[sl]), g_ = as_frag<T>(fg[sl]);
-      mma(S, q_, Kf[kk]);
-      if constexpr (MODE == BWD_PLAIN) mma(dP, g_, Vf[kk]);
-      if constexpr (TAN) mma(At, g_, Vf[kk]);
+      mma_vra<F>(S, q_, Kf[kk]);
+      if constexpr (MODE == BWD_PLAIN) mma_vra<F>(dP, g_, Vf[kk]);
+      if constexpr (TAN) mma_vra<F>(At, g_, Vf[kk]);
       if constexpr (DUAL) {
         const Frag<T> gt_ = as_frag<T>(fgt[sl]);
-        if (has_go) mma(dP, g_, Vf[kk]);
-        mma(Sp, as_frag<T>(fqt[sl]), Kf[kk]);
-        mma(At, gt_, Vf[kk]);
-        mma(Sp, q_, Ktf[kk]);
-        mma(Bt, gt_, Vtf[kk]);
+        if constexpr (has_go) mma_vra<F>(dP, g_, Vf[kk]);
+        mma_vra<F>(Sp, as_frag<T>(fqt[sl]), Kf[kk]);
+        mma_vra<F>(At, gt_, Vf[kk]);
+        mma_vra<false>(Sp, q_, Ktf[kk]);
+        mma_vrv<F && !has_go>(dP, gt_, Vtf[kk]);
       }
     });
+    if constexpr (DUAL) tiles_ready(S, dP, Sp, At);
+    else if constexpr (TAN) tiles_ready(S, At);
+    else tiles_ready(S, dP);
 
     // ---- row statistics of the 32 queries: register e belongs to query 16(e/8) + 8g + e%8 ------
     // read one quad of registers at a time (quad c4 = registers 4*c4 .. 4*c4+3), one quad ahead
@@ -516,7 +530,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
             const float sp = Sp[e] * pr.scale, m_ = stat(1, e), am = At[e] - stat(2, e);
             Pp[e - 8 * c] = pv * (sp - m_);
             Sp[e] = pv * am;
-            dP[e] = pv * (dP[e] + Bt[e] + am * sp - At[e] * m_ - stat(3, e));
+            dP[e] = pv * (dP[e] + am * sp - At[e] * m_ - stat(3, e));
           } else {
             Sp[e] = pv * (At[e] - stat(1, e));
           }
@@ -543,7 +557,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
           mma(dV[db], as_frag<T>(tg[sl]), pf);
         } else if constexpr (DUAL) {
           mma(dK[db], as_frag<T>(tq[sl]), dsf);
-          if (has_go) mma(dV[db], as_frag<T>(tg[sl]), pf);
+          if constexpr (has_go) mma(dV[db], as_frag<T>(tg[sl]), pf);
           mma(dK[db], as_frag<T>(tqt[sl]), dspf);
           mma(dV[db], as_frag<T>(tgt[sl]), ppf);
         } else {
@@ -566,12 +580,9 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
     load_stats();
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB, sstat = stat0 + stage * Cfg::STATB;
     half_tile(std::integral_constant<int, 0>{}, sbase, sstat, i0);
-    if (i0 + 32 < L) {
-      half_tile(std::integral_constant<int, 1>{}, sbase, sstat, i0 + 32);
-    } else {
-      static_for<KK>([&](auto gc) { load_step(std::integral_constant<int, KK + decltype(gc)::value>{}); });
-      static_for<NPV>([&](auto gc) { load_step(std::integral_constant<int, 2 * KK + NPV + decltype(gc)::value>{}); });
-    }
+    // always both halves: a half past the last query contributes exact zeros, and a branch here would
+    // make the accumulators change register file around it
+    half_tile(std::integral_constant<int, 1>{}, sbase, sstat, i0 + 32);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);
 

@@ -44,6 +44,35 @@ __device__ __forceinline__ float acc_scale(float x, float alpha) {
                : "v"(alpha));
   return x;
 }
+// Products whose B operand stays resident in the accumulation register file for the whole kernel
+// while the result tile lives in ordinary vector registers: c = a*b (FIRST) or c += a*b.  The
+// result may only be read by other instruction kinds after tiles_ready().
+__device__ __forceinline__ void pin_acc(bf16x8 &f) { asm volatile("" : "+a"(f)); }
+__device__ __forceinline__ void pin_acc(f16x8 &f) { asm volatile("" : "+a"(f)); }
+template <bool FIRST> __device__ __forceinline__ void mma_vra(f32x16 &c, const bf16x8 &a, const bf16x8 &b) {
+  if constexpr (FIRST) asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+  else asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+}
+template <bool FIRST> __device__ __forceinline__ void mma_vra(f32x16 &c, const f16x8 &a, const f16x8 &b) {
+  if constexpr (FIRST) asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+  else asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+}
+// the same with the B operand in ordinary vector registers
+template <bool FIRST> __device__ __forceinline__ void mma_vrv(f32x16 &c, const bf16x8 &a, const bf16x8 &b) {
+  if constexpr (FIRST) asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  else asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+template <bool FIRST> __device__ __forceinline__ void mma_vrv(f32x16 &c, const f16x8 &a, const f16x8 &b) {
+  if constexpr (FIRST) asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  else asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+// 16 + 4 idle issue slots: the last matrix-core pass has written its registers when this returns
+__device__ __forceinline__ void tiles_ready(f32x16 &a, f32x16 &b) {
+  asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void tiles_ready(f32x16 &a, f32x16 &b, f32x16 &c, f32x16 &d) {
+  asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
 template <int N> __device__ __forceinline__ void lds_wait(u32x4 &a) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
 }
