@@ -119,10 +119,12 @@ def hvp_sweep(be, _lib):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--fwd-only", action="store_true", help="time only the headline forward (for profiling)")
+    ap.add_argument("--bwd-only", action="store_true",
+                    help="run one forward, then time only the headline backward (for profiling); prints its own line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, whose known traffic scales the rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings of the forward kernel")
@@ -156,6 +158,13 @@ def main():
         o, ot, M, mu = fwd(causal)
         state["g"] = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, causal, scale)
 
+    if args.bwd_only:
+        o, ot, M, mu = fwd()
+        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, False, scale),
+                        args.steps, args.warmup)
+        print(json.dumps({"workload": "bf16 B4 H16 L4096 D128 backward of (gO, gT) -> dq, dk, dv", "ms_per_step": ms_b,
+                          "tflops_algorithmic": bwd_flops / (ms_b * 1e-3) / 1e12}), flush=True)
+        return
     if args.calibrate_copy:
         src = torch.empty(256 * 2**20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
@@ -192,8 +201,8 @@ def main():
     }
     if not args.fwd_only:
         ms_fc, _ = timed(lambda: fwd(True), args.steps, args.warmup)
-        ms_fb, _ = timed(fwd_bwd, max(1, args.steps // 2), 1)
-        ms_fbc, _ = timed(lambda: fwd_bwd(True), max(1, args.steps // 2), 1)
+        ms_fb, _ = timed(fwd_bwd, max(1, args.steps // 2), 2)
+        ms_fbc, _ = timed(lambda: fwd_bwd(True), max(1, args.steps // 2), 2)
         tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12  # noqa: E731
         out["extra"] = {
             "fwd_causal": {"ms": ms_fc, "tflops": tf(fwd_flops / 2, ms_fc),
