@@ -3,6 +3,7 @@
 // and exporting  int JVPFA_NAME(const FwdParams&, bool dual, int mask_kind, hipStream_t).
 #include "fwd_kernel.hpp"
 #include "fwd_kernel_v2.hpp"
+#include "fwd_kernel_v3.hpp"
 #include "launch.hpp"
 
 namespace jvpfa {
@@ -34,11 +35,28 @@ static int launch_fwd2_one(const FwdParams &p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }
 
+// ... and, without an explicit mask, its software-pipelined form.
+template <typename T, int D, bool DUAL>
+static int launch_fwd3_one(const FwdParams &p, hipStream_t stream) {
+  using Cfg = Fwd2Cfg<T, D, DUAL>;
+  auto kern = fwd3_kernel<T, D, DUAL>;
+  int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
+  if (rc != 0) return rc;
+  const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
+  const long long blocks = (long long)nqb * p.pr.Z * p.pr.H;
+  if (blocks > 0x7fffffffLL) return -2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : -6;
+}
+
 template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
   if constexpr (sizeof(T) == 2 && D >= 64) {
     switch (mask) {
-      case MASK_NONE: return launch_fwd2_one<T, D, DUAL, MASK_NONE>(p, stream);
+      case MASK_NONE:
+        // the pipelined kernel pays off where a slot has enough matrix work to hide the softmax behind
+        if constexpr (D >= 128) return launch_fwd3_one<T, D, DUAL>(p, stream);
+        else return launch_fwd2_one<T, D, DUAL, MASK_NONE>(p, stream);
       case MASK_BOOL: return launch_fwd2_one<T, D, DUAL, MASK_BOOL>(p, stream);
       case MASK_ADD: return launch_fwd2_one<T, D, DUAL, MASK_ADD>(p, stream);
     }

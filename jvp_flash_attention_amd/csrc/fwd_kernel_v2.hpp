@@ -160,6 +160,12 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     Qf[kk] = ld8<T>(Qg + (size_t)qld * D + 16 * kk + 8 * g);
     if constexpr (DUAL) Qtf[kk] = ld8<T>(Qtg + (size_t)qld * D + 16 * kk + 8 * g);
   }
+  // the resident operands live in the accumulation register file from here on
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    pin_acc(Qf[kk]);
+    if constexpr (DUAL) pin_acc(Qtf[kk]);
+  }
 
   f32x16 Oacc[DB], Tacc[DUAL ? DB : 1];
 #pragma unroll
@@ -255,12 +261,9 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       }
     };
 
+    // score tiles in ordinary vector registers, written by matrix instructions whose B operand (Q, Q')
+    // is resident in the accumulation register file
     f32x16 S, Sp;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      S[e] = 0.f;
-      Sp[e] = 0.f;
-    }
     static_for<(PD < KK ? PD : KK)>([&](auto kkc) { issue_k(kkc); });
     static_for<KK>([&](auto kkc) {
       constexpr int kk = decltype(kkc)::value;
@@ -270,12 +273,12 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       if constexpr (kk + PD < KK) issue_k(std::integral_constant<int, kk + PD>{});
       load_step(std::integral_constant<int, HB * (KK + NPV) + kk>{});
       const Frag<T> a = __builtin_bit_cast(Frag<T>, ka[kk % RD]);
-      mma(S, a, Qf[kk]);
-      if constexpr (DUAL) {
-        mma(Sp, a, Qtf[kk]);
-        mma(Sp, __builtin_bit_cast(Frag<T>, kb[kk % RD]), Qf[kk]);
-      }
+      if constexpr (DUAL) mma_vra<kk == 0>(Sp, a, Qtf[kk]);
+      mma_vra<kk == 0>(S, a, Qf[kk]);
+      if constexpr (DUAL) mma_vra<false>(Sp, __builtin_bit_cast(Frag<T>, kb[kk % RD]), Qf[kk]);
     });
+    if constexpr (DUAL) tiles_ready(S, Sp);
+    else tiles_ready(S);
     JVPFA_STAMP(5);
     const bool diag = pr.causal && (jh + 31 > q0 + wave * 32);
     const bool ragged = jh + 32 > L;
@@ -385,11 +388,9 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     prepare_loads(stage ^ 1, j0 + BN, t + 1 < ntiles);
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
     half_tile(std::integral_constant<int, 0>{}, sbase, j0);
-    if (j0 + 32 < kend) {
-      half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
-    } else {  // second half skipped (end of a ragged or causal row block): issue its share of the loads
-      static_for<NSTEP / 2>([&](auto gc) { load_step(std::integral_constant<int, NSTEP / 2 + decltype(gc)::value>{}); });
-    }
+    // always both halves: a half past the last key is fully masked and contributes exact zeros, and a
+    // branch here would make the accumulators change register file around it
+    half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------

@@ -1,0 +1,512 @@
+// Software-pipelined fused dual forward for 16-bit element types, D in {64, 128}, no explicit mask
+// (causal and ragged sequence ends are handled).  Same tiles, swizzles, fragment layouts and
+// mathematics as fwd_kernel_v2.hpp; what changes is the order of work inside a wave.
+//
+// A wave issues instructions in order, but a matrix instruction occupies the issue port for a
+// fraction of the time the matrix pipe needs to execute it, so independent vector instructions
+// placed between two matrix instructions run for free.  The unit of work here is a *slot*, one per
+// 32-key half tile h, whose instruction stream interleaves three independent pieces:
+//     matrix:  S(h+1) = K Q^T, S'(h+1)            (scores of the next half tile)
+//     matrix:  O, T += V^T P(h-1), ...            (accumulation of the previous half tile)
+//     vector:  softmax of half tile h             (S(h), S'(h) -> P(h), P(h)S'(h), row sums)
+// The vector work is cut into small units and one unit is placed after each matrix instruction.
+// K tiles are consumed one slot earlier than V tiles, so the K half and the V half of an LDS stage
+// hold different tiles: at the top of iteration t (one workgroup barrier), K(t) and V(t-1) have
+// landed and the loads of K(t+1) and V(t) are started.
+#pragma once
+#include "fwd_kernel_v2.hpp"
+
+namespace jvpfa {
+
+// matrix instructions in program order: score tile in vector registers (B operand resident in the
+// accumulation file), and output accumulators in the accumulation file
+template <bool FIRST> __device__ __forceinline__ void mfma_s(f32x16 &c, const bf16x8 &a, const bf16x8 &b) {
+  if constexpr (FIRST) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+  else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+}
+template <bool FIRST> __device__ __forceinline__ void mfma_s(f32x16 &c, const f16x8 &a, const f16x8 &b) {
+  if constexpr (FIRST) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+  else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+}
+__device__ __forceinline__ void mfma_acc(f32x16 &c, const bf16x8 &a, const bf16x8 &b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_acc(f32x16 &c, const f16x8 &a, const f16x8 &b) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void pin_acc(f32x16 &c) { asm volatile("" : "+a"(c)); }
+
+__device__ __forceinline__ void anchor(float &x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void anchor(bf16x8 &x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void anchor(f16x8 &x) { asm volatile("" : "+v"(x)); }
+
+template <int N>
+__device__ __forceinline__ void lds_wait6(u32x4 &a, u32x4 &b, u32x2 &c, u32x2 &d, u32x2 &e, u32x2 &f) {
+  asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait3(u32x4 &a, u32x2 &c, u32x2 &d) {
+  asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a), "+v"(c), "+v"(d) : "n"(N));
+}
+
+template <typename T, int D, bool DUAL>
+__global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
+  using Cfg = Fwd2Cfg<T, D, DUAL>;
+  constexpr int BN = Cfg::BN, CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW;
+  constexpr int KK = D / 16, DB = D / 32;
+  constexpr int NSS = KK;  // super-steps of a slot: one contraction step of the scores + one (chunk, d-block) of PV
+  static_assert(2 * DB == KK, "a slot pairs score step kk with accumulation step kk");
+  constexpr float NEG_INF = -__builtin_inff();
+  int trace_n = 0;
+  (void)trace_n;
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+  // stage s: [K | V | K' | V'] each TILEB bytes; the K-type and V-type halves hold different tiles
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem_raw;
+
+  const Problem &pr = p.pr;
+  const int L = pr.L;
+  const int nqb = (L + Cfg::BM - 1) / Cfg::BM;
+  const int total = nqb * pr.Z * pr.H;
+  const int id = xcd_remap(blockIdx.x, total);
+  const int zh = id / nqb;
+  const int qb = pr.causal ? nqb - 1 - id % nqb : id % nqb;
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
+  const int r = lane % 32, g = lane / 32;
+  const int pr32 = perm32(r);
+
+  const size_t head = (size_t)zh * L * D;
+  const T *Qg = reinterpret_cast<const T *>(p.q) + head;
+  const char *Kg = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.k) + head);
+  const char *Vg = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.v) + head);
+  const T *Qtg = DUAL ? reinterpret_cast<const T *>(p.qt) + head : nullptr;
+  const char *Ktg = DUAL ? reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.kt) + head) : nullptr;
+  const char *Vtg = DUAL ? reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.vt) + head) : nullptr;
+
+  const int q0 = qb * Cfg::BM;
+  const int qrow = q0 + wave * 32 + r;
+  const int qld = qrow < L ? qrow : L - 1;
+
+  // ---- direct loads (see fwd_kernel_v2.hpp): instruction i of this wave fills chunks 64*(wave*IPW+i)..+63
+  int ld_row[IPW];
+  uint32_t ld_ck[IPW], ld_cv[IPW];
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) {
+    const int lc = 64 * (wave * IPW + i) + lane;
+    const int row = lc / CH, cp = lc % CH;
+    ld_row[i] = row;
+    ld_ck[i] = (cp ^ swz_k<CH>(row)) * 16;
+    ld_cv[i] = (cp ^ swz_v<CH>(row)) * 16;
+  }
+  uint32_t koff[KK];
+  {
+    const int x = swz_k<CH>(pr32);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) koff[kk] = pr32 * ROWB + (((2 * kk + g) ^ x) * 16);
+  }
+  uint32_t voff[DB][2];
+  {
+    const int a = (lane >> 4) & 1, j = lane & 15;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int row = 8 * g + 4 * hh + (j >> 2);
+        const int ch = (4 * db + 2 * a + (j & 1)) ^ swz_v<CH>(row);
+        voff[db][hh] = row * ROWB + ch * 16 + 8 * ((j >> 1) & 1);
+      }
+    }
+  }
+
+  Frag<T> Qf[KK], Qtf[DUAL ? KK : 1];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    Qf[kk] = ld8<T>(Qg + (size_t)qld * D + 16 * kk + 8 * g);
+    if constexpr (DUAL) Qtf[kk] = ld8<T>(Qtg + (size_t)qld * D + 16 * kk + 8 * g);
+  }
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    pin_acc(Qf[kk]);
+    if constexpr (DUAL) pin_acc(Qtf[kk]);
+  }
+
+  f32x16 Oacc[DB], Tacc[DUAL ? DB : 1];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      Oacc[db][e] = 0.f;
+      if constexpr (DUAL) Tacc[db][e] = 0.f;
+    }
+    pin_acc(Oacc[db]);
+    if constexpr (DUAL) pin_acc(Tacc[db]);
+  }
+  float m_i = NEG_INF, l_i = 0.f, mu_i = 0.f;
+
+  const float sl2 = pr.scale * LOG2E;
+  const bool neg_scale = !(sl2 > 0.f);
+  const int kend = pr.causal ? min(L, q0 + Cfg::BM) : L;
+  const int ntiles = (kend + BN - 1) / BN;
+  const int qlim = pr.causal ? qrow : 0x7fffffff;  // keys above this index are masked
+
+  // ---- next-tile loads, one instruction per super-step -------------------------------------------
+  constexpr int NLOAD = IPW * Cfg::NTILE;
+  constexpr int NSTEP = 2 * NSS;
+  int ld_rows_k = 0, ld_rows_v = 0;
+  uint32_t ld_dst_k = 0, ld_dst_v = 0;
+  const char *ld_p[4] = {nullptr, nullptr, nullptr, nullptr};
+  // iteration t loads K(t+1) into the K half of stage (t+1)&1 and V(t) into the V half of stage t&1;
+  // a tile that does not exist is replaced by tile 0 (never read), which keeps the stream branch-free
+  auto prepare_loads = [&](int t) {
+    const int jk = (t + 1 < ntiles) ? (t + 1) * BN : 0, jv = (t < ntiles) ? t * BN : 0;
+    ld_rows_k = L - 1 - jk;
+    ld_rows_v = L - 1 - jv;
+    ld_dst_k = lds0 + ((t + 1) & 1) * Cfg::STAGEB + (wave * IPW) * 1024;
+    ld_dst_v = lds0 + (t & 1) * Cfg::STAGEB + (wave * IPW) * 1024;
+    ld_p[0] = Kg + (size_t)jk * ROWB;
+    ld_p[1] = Vg + (size_t)jv * ROWB;
+    if constexpr (DUAL) {
+      ld_p[2] = Ktg + (size_t)jk * ROWB;
+      ld_p[3] = Vtg + (size_t)jv * ROWB;
+    }
+  };
+  auto load_piece = [&](auto pc) {
+    constexpr int pi = decltype(pc)::value, i = pi / Cfg::NTILE, ts = pi % Cfg::NTILE;
+    constexpr bool vt = (ts & 1) != 0;
+    const uint32_t off = min(ld_row[i], vt ? ld_rows_v : ld_rows_k) * ROWB + (vt ? ld_cv[i] : ld_ck[i]);
+    __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(ld_p[ts] + off),
+                                     (JVPFA_LDS(void))(uintptr_t)((vt ? ld_dst_v : ld_dst_k) + i * 1024 + ts * TILEB), 16, 0, 0);
+  };
+  auto load_step = [&](auto gc) {
+    constexpr int gi = decltype(gc)::value;
+    constexpr int lo = (gi * NLOAD + NSTEP - 1) / NSTEP, hi = ((gi + 1) * NLOAD + NSTEP - 1) / NSTEP;
+    static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+  };
+
+  constexpr float RESCALE_TAU = 8.f;
+  constexpr int NQ = DUAL ? 3 : 1, NP = DUAL ? 3 : 1;  // matrix instructions per super-step: scores, accumulation
+  constexpr int NRS = DUAL ? 2 : 1, NRV = DUAL ? 4 : 2;  // LDS reads per super-step
+  constexpr int NU = 38;                                 // vector units of one softmax
+  constexpr int NU0 = 5;                                 // ... of which this many form its front
+#ifndef JVPFA_F3_RD
+#define JVPFA_F3_RD 4
+#endif
+  constexpr int RD = JVPFA_F3_RD, PD = RD - 1;           // fragment ring slots; reads run PD super-steps ahead
+
+  // One slot.  QK: scores of a half tile (K rows at LDS address kaddr) into Sn, Spn.  PV: accumulate
+  // the half tile whose V rows are at vaddr, with fragments pfp, psfp.  SM: softmax of Sc, Spc (first
+  // key jh) into pfn, psfn.  GEN: the softmax applies the causal / sequence-end limits.  LB: index of
+  // the first load step of this slot, or -1.
+  u32x4 ka[RD], kb[RD];
+  u32x2 va[RD][2], vb[RD][2];
+  auto slot = [&](auto QKc, auto PVc, auto SMc, auto GENc, auto LBc, auto PREc, auto NEXTc, uint32_t kaddr, uint32_t vaddr, f32x16 &Sc,
+                  f32x16 &Spc, f32x16 &Sn, f32x16 &Spn, Frag<T>(&pfp)[2], Frag<T>(&psfp)[2], Frag<T>(&pfn)[2],
+                  Frag<T>(&psfn)[2], int jh) {
+    constexpr bool QK = decltype(QKc)::value, PV = decltype(PVc)::value, SM = decltype(SMc)::value;
+    constexpr bool GEN = decltype(GENc)::value;
+    constexpr int LB = decltype(LBc)::value;
+    // PRE: the reads of the first PD super-steps were issued by the previous slot; NEXT: issue those of
+    // the next slot, which works on the other half of the same two tiles
+    constexpr bool PRE = decltype(PREc)::value, NEXT = decltype(NEXTc)::value;
+    constexpr int MPS = (QK ? NQ : 0) + (PV ? NP : 0);  // matrix instructions per super-step
+    constexpr int NG = NSS * MPS;                       // gaps of the slot
+    constexpr int UPG = SM ? (NU - NU0 + NG - 1) / NG : 0;  // vector units per gap
+    constexpr int RPS = (QK ? NRS : 0) + (PV ? NRV : 0);
+    static_assert((PD - 1) * RPS <= 15, "lgkmcnt is a 4-bit counter");
+    static_assert(!NEXT || (NSS % RD == 0 && QK && PV), "the fragment ring continues into the next slot");
+
+    // ---- softmax state and units ----------------------------------------------------------------
+    float mxa = NEG_INF, mxb = NEG_INF, mx = NEG_INF, alpha = 1.f, m_use = 0.f, rs = 0.f, rmu = 0.f;
+    float pv[16], sv[16];
+    bool any_up = false;
+    auto unit = [&](auto uc) {
+      constexpr int u = decltype(uc)::value;
+      if constexpr (u == 0 || u == 1) {  // row maximum over registers 8u .. 8u+7
+        float m8 = NEG_INF;
+#pragma unroll
+        for (int e = 8 * u; e < 8 * u + 8; ++e) {
+          if constexpr (GEN) {
+            const int key = jh + 16 * (e / 8) + 8 * g + (e % 8);
+            float s = Sc[e] * sl2;
+            s = (key <= qlim) ? s : NEG_INF;
+            s = (key < L) ? s : NEG_INF;
+            Sc[e] = s;
+            m8 = fmaxf(m8, s);
+          } else {
+            m8 = (e == 8 * u) ? Sc[e] : fmaxf(m8, Sc[e]);
+          }
+        }
+        if constexpr (u == 0) mxa = m8;
+        else mxb = m8;
+        anchor(m8);
+      } else if constexpr (u == 2) {
+        mx = pair_max(fmaxf(mxa, mxb));
+        if constexpr (!GEN) mx *= sl2;
+        anchor(mx);
+      } else if constexpr (u == 3) {
+        // lazy rescale, decided per query row: the reference point only moves when the row maximum
+        // exceeds it by more than RESCALE_TAU (log2 units)
+        const bool up = mx > m_i + RESCALE_TAU;
+        any_up = __any(up);
+        alpha = up ? fast_exp2(m_i - mx) : 1.f;
+        m_i = up ? mx : m_i;
+        anchor(alpha);
+      } else if constexpr (u == 4) {
+        m_use = (m_i == NEG_INF) ? 0.f : m_i;
+      } else if constexpr (u < 37) {
+        constexpr int e = (u - 5) / 2;
+        if constexpr ((u - 5) % 2 == 0) {
+          if constexpr (GEN) pv[e] = fast_exp2(Sc[e] - m_use);
+          else pv[e] = fast_exp2(__builtin_fmaf(Sc[e], sl2, -m_use));
+          if constexpr (DUAL) sv[e] = Spc[e] * pr.scale;
+          anchor(pv[e]);
+        } else {
+          rs += pv[e];
+          if constexpr (DUAL) {
+            sv[e] *= pv[e];
+            rmu += sv[e];
+          }
+          if constexpr (e % 2 == 1) {
+            constexpr int c = e / 8, j = e % 8;
+            pfn[c][j - 1] = (T)pv[e - 1];
+            pfn[c][j] = (T)pv[e];
+            if constexpr (DUAL) {
+              psfn[c][j - 1] = (T)sv[e - 1];
+              psfn[c][j] = (T)sv[e];
+            }
+            if constexpr (j == 7) {
+              anchor(pfn[c]);
+              if constexpr (DUAL) anchor(psfn[c]);
+            }
+          }
+          anchor(rs);
+        }
+      } else {
+        l_i = __builtin_fmaf(l_i, alpha, rs);
+        if constexpr (DUAL) mu_i = __builtin_fmaf(mu_i, alpha, rmu);
+      }
+    };
+    // (anchor(): an empty asm statement that consumes a value; it keeps the unit that produced the value
+    // at its place in the instruction stream, between the matrix instructions written around it)
+    // the vector work that follows matrix instruction number gi of the slot
+    auto gap = [&](auto gc) {
+      constexpr int gi = decltype(gc)::value;
+      if constexpr (SM) {
+        static_for<UPG>([&](auto uc) {
+          constexpr int u = NU0 + gi * UPG + decltype(uc)::value;
+          if constexpr (u < NU) unit(std::integral_constant<int, u>{});
+        });
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // ---- fragment reads --------------------------------------------------------------------------
+    // step NSS + j is step j of the next slot (rows 32 further down in the same tiles)
+    auto issue = [&](auto ic) {
+      constexpr int i = decltype(ic)::value % NSS, sl = i % RD;
+      constexpr int HO = (decltype(ic)::value / NSS) * 32 * ROWB;
+      if constexpr (QK) {
+        const uint32_t ad = kaddr + koff[i];
+        ka[sl] = lds_b128<HO>(ad);
+        if constexpr (DUAL) kb[sl] = lds_b128<HO + 2 * TILEB>(ad);
+      }
+      if constexpr (PV) {
+        constexpr int c = i / DB, db = i % DB;
+        constexpr int VO = HO + TILEB + c * 16 * ROWB;
+        const uint32_t a0 = vaddr + voff[db][0], a1 = vaddr + voff[db][1];
+        va[sl][0] = lds_tr64<VO>(a0);
+        va[sl][1] = lds_tr64<VO>(a1);
+        if constexpr (DUAL) {
+          vb[sl][0] = lds_tr64<VO + 2 * TILEB>(a0);
+          vb[sl][1] = lds_tr64<VO + 2 * TILEB>(a1);
+        }
+      }
+    };
+
+    if constexpr (SM) {
+      if constexpr (DUAL) tiles_ready(Sc, Spc);
+      else tiles_ready(Sc);
+    }
+    JVPFA_STAMP(4);
+    if constexpr (!PRE) static_for<(PD < NSS ? PD : NSS)>([&](auto ic) { issue(ic); });
+    // the front of the softmax (row maximum, reference point) runs while the first fragments travel
+    if constexpr (SM) static_for<NU0>([&](auto uc) { unit(uc); });
+    static_for<NSS>([&](auto ic) {
+      constexpr int i = decltype(ic)::value, sl = i % RD;
+      constexpr int younger = (NEXT ? PD - 1 : ((NSS - 1 - i < PD - 1) ? NSS - 1 - i : PD - 1)) * RPS;
+      if constexpr (QK && PV) {
+        if constexpr (DUAL) lds_wait6<younger>(ka[sl], kb[sl], va[sl][0], va[sl][1], vb[sl][0], vb[sl][1]);
+        else lds_wait3<younger>(ka[sl], va[sl][0], va[sl][1]);
+      } else if constexpr (QK) {
+        if constexpr (DUAL) lds_wait<younger>(ka[sl], kb[sl]);
+        else lds_wait<younger>(ka[sl]);
+      } else {
+        if constexpr (DUAL) lds_wait<younger>(va[sl][0], va[sl][1], vb[sl][0], vb[sl][1]);
+        else lds_wait<younger>(va[sl][0], va[sl][1]);
+      }
+      if constexpr (i == 0) JVPFA_STAMP(5);
+      if constexpr (i + PD < NSS || NEXT) issue(std::integral_constant<int, i + PD>{});
+      if constexpr (LB >= 0) load_step(std::integral_constant<int, (LB >= 0 ? LB : 0) + i>{});
+      constexpr int c = i / DB, db = i % DB;
+      constexpr int G0 = i * MPS;
+      Frag<T> fa, fb, fv, fw;
+      if constexpr (QK) {
+        fa = __builtin_bit_cast(Frag<T>, ka[sl]);
+        if constexpr (DUAL) fb = __builtin_bit_cast(Frag<T>, kb[sl]);
+      }
+      if constexpr (PV) {
+        const u32x4 av = {va[sl][0][0], va[sl][0][1], va[sl][1][0], va[sl][1][1]};
+        fv = __builtin_bit_cast(Frag<T>, av);
+        if constexpr (DUAL) {
+          const u32x4 bv = {vb[sl][0][0], vb[sl][0][1], vb[sl][1][0], vb[sl][1][1]};
+          fw = __builtin_bit_cast(Frag<T>, bv);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (DUAL) {
+        // order: no two consecutive matrix instructions update the same tile
+        if constexpr (QK && PV) {
+          mfma_s<i == 0>(Spn, fa, Qtf[i]);
+          gap(std::integral_constant<int, G0 + 0>{});
+          mfma_acc(Oacc[db], fv, pfp[c]);
+          gap(std::integral_constant<int, G0 + 1>{});
+          mfma_s<i == 0>(Sn, fa, Qf[i]);
+          gap(std::integral_constant<int, G0 + 2>{});
+          mfma_acc(Tacc[db], fv, psfp[c]);
+          gap(std::integral_constant<int, G0 + 3>{});
+          mfma_s<false>(Spn, fb, Qf[i]);
+          gap(std::integral_constant<int, G0 + 4>{});
+          mfma_acc(Tacc[db], fw, pfp[c]);
+          gap(std::integral_constant<int, G0 + 5>{});
+        } else if constexpr (QK) {
+          mfma_s<i == 0>(Spn, fa, Qtf[i]);
+          gap(std::integral_constant<int, G0 + 0>{});
+          mfma_s<i == 0>(Sn, fa, Qf[i]);
+          gap(std::integral_constant<int, G0 + 1>{});
+          mfma_s<false>(Spn, fb, Qf[i]);
+          gap(std::integral_constant<int, G0 + 2>{});
+        } else {
+          mfma_acc(Tacc[db], fv, psfp[c]);
+          gap(std::integral_constant<int, G0 + 0>{});
+          mfma_acc(Oacc[db], fv, pfp[c]);
+          gap(std::integral_constant<int, G0 + 1>{});
+          mfma_acc(Tacc[db], fw, pfp[c]);
+          gap(std::integral_constant<int, G0 + 2>{});
+        }
+      } else {
+        if constexpr (QK) {
+          mfma_s<i == 0>(Sn, fa, Qf[i]);
+          gap(std::integral_constant<int, G0 + 0>{});
+        }
+        if constexpr (PV) {
+          mfma_acc(Oacc[db], fv, pfp[c]);
+          gap(std::integral_constant<int, G0 + (QK ? 1 : 0)>{});
+        }
+      }
+    });
+    JVPFA_STAMP(6);
+    if constexpr (SM) {
+      if (any_up) {  // rare: some row's reference point moved; the accumulators follow it
+        asm volatile("s_nop 15\n\ts_nop 15");  // the last accumulation above has written its registers
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            Oacc[db][e] = acc_scale(Oacc[db][e], alpha);
+            if constexpr (DUAL) Tacc[db][e] = acc_scale(Tacc[db][e], alpha);
+          }
+        }
+      }
+    }
+  };
+
+  using B0 = std::false_type;
+  using B1 = std::true_type;
+  using XP = std::integral_constant<bool, NSS % RD == 0>;  // fragment prefetch across the two slots of an iteration
+  f32x16 SX, SpX, SY, SpY;
+  Frag<T> pfA[2], psfA[2], pfB[2], psfB[2];
+
+  // ---- prologue: K(0) in one burst ---------------------------------------------------------------
+  {
+    ld_rows_k = L - 1;
+    ld_dst_k = lds0 + (wave * IPW) * 1024;
+    ld_p[0] = Kg;
+    if constexpr (DUAL) ld_p[2] = Ktg;
+    static_for<NLOAD>([&](auto pc) {
+      if constexpr (decltype(pc)::value % 2 == 0) load_piece(pc);
+    });
+  }
+  auto kad = [&](int t, int hb) { return lds0 + (t & 1) * Cfg::STAGEB + hb * 32 * ROWB; };
+
+  // iteration 0: scores of half tiles 0 and 1, softmax of half tile 0
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  prepare_loads(0);
+  slot(B1{}, B0{}, B0{}, B1{}, std::integral_constant<int, 0>{}, B0{}, B0{}, kad(0, 0), 0u, SX, SpX, SY, SpY, pfA, psfA, pfB, psfB, 0);
+  slot(B1{}, B0{}, B1{}, B1{}, std::integral_constant<int, NSS>{}, B0{}, B0{}, kad(0, 1), 0u, SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0);
+  // Iterations whose softmax needs the causal / sequence-end limits form the tail of the loop; they
+  // get a loop of their own so that the common iteration is one straight-line block.
+  int t_gen = (L >= 32) ? (L - 32) / BN + 1 : 0;
+  if (pr.causal) t_gen = min(t_gen, (q0 + 32) / BN);
+  t_gen = neg_scale ? 1 : max(1, t_gen);
+  int t = 1;
+  for (; t < min(t_gen, ntiles); ++t) {
+    JVPFA_STAMP(1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of K(t), V(t-1) has landed
+    JVPFA_STAMP(2);
+    __syncthreads();                      // ... everyone's has, and K(t-1), V(t-2) are no longer read
+    JVPFA_STAMP(3);
+    prepare_loads(t);
+    slot(B1{}, B1{}, B1{}, B0{}, std::integral_constant<int, 0>{}, B0{}, XP{}, kad(t, 0), kad(t - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB, 0);
+    slot(B1{}, B1{}, B1{}, B0{}, std::integral_constant<int, NSS>{}, XP{}, B0{}, kad(t, 1), kad(t - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0);
+  }
+  for (; t < ntiles; ++t) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    prepare_loads(t);
+    slot(B1{}, B1{}, B1{}, B1{}, std::integral_constant<int, 0>{}, B0{}, XP{}, kad(t, 0), kad(t - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
+         (t - 1) * BN + 32);
+    slot(B1{}, B1{}, B1{}, B1{}, std::integral_constant<int, NSS>{}, XP{}, B0{}, kad(t, 1), kad(t - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA,
+         t * BN);
+  }
+  // drain: softmax of the last half tile, accumulation of the last two
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  slot(B0{}, B1{}, B1{}, B1{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
+       (ntiles - 1) * BN + 32);
+  slot(B0{}, B1{}, B0{}, B1{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0);
+  asm volatile("s_nop 15\n\ts_nop 15");  // the last accumulation has written its registers
+
+  // ---- epilogue ---------------------------------------------------------------------------------
+  l_i += xor32(l_i);
+  if constexpr (DUAL) mu_i += xor32(mu_i);
+  const bool dead = !(l_i > 0.f);
+  const float inv = dead ? 0.f : 1.f / l_i;
+  const float mu_n = mu_i * inv;
+  if (qrow < L) {
+    T *Og = reinterpret_cast<T *>(p.o) + head + (size_t)qrow * D;
+    T *Otg = DUAL ? reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D : nullptr;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        float o8[8], t8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          o8[e] = Oacc[db][8 * hf + e] * inv;
+          if constexpr (DUAL) t8[e] = Tacc[db][8 * hf + e] * inv - mu_n * o8[e];
+        }
+        const int d0 = 32 * db + 16 * hf + 8 * g;
+        store8<T>(Og + d0, o8);
+        if constexpr (DUAL) store8<T>(Otg + d0, t8);
+      }
+    }
+    if (g == 0) {
+      p.M[(size_t)zh * L + qrow] = dead ? __builtin_inff() : m_i + __builtin_amdgcn_logf(l_i);
+      if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = mu_n;
+    }
+  }
+}
+
+}  // namespace jvpfa

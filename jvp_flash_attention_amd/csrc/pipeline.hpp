@@ -67,6 +67,7 @@ template <bool FIRST> __device__ __forceinline__ void mma_vrv(f32x16 &c, const f
   else asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
 // 16 + 4 idle issue slots: the last matrix-core pass has written its registers when this returns
+__device__ __forceinline__ void tiles_ready(f32x16 &a) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a)); }
 __device__ __forceinline__ void tiles_ready(f32x16 &a, f32x16 &b) {
   asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a), "+v"(b));
 }
