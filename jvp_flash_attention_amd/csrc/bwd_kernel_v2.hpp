@@ -57,6 +57,9 @@ template <int N> __device__ __forceinline__ void lds_wait4(u32x4 &a, u32x4 &b, u
 
 // Everything the two kernels share: tile geometry, direct loads spread over steps, fragment reads.
 // SLOTn are LDS tile slots inside a stage; a tile is BT rows, row-major, chunks swizzled by swz_u.
+#ifndef JVPFA_BWD_SPREAD
+#define JVPFA_BWD_SPREAD(n) (3 * (n) / 4)
+#endif
 #define JVPFA_BWD2_COMMON(Cfg)                                                                                      \
   constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT;                   \
   constexpr int KK = D / 16, DB = D / 32;                                                                           \
@@ -190,8 +193,12 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
   };
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
-    constexpr int lo = (gi * NLOAD + NSTEP - 1) / NSTEP, hi = ((gi + 1) * NLOAD + NSTEP - 1) / NSTEP;
-    static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+    // spread over the first NSPREAD steps only: the last load then has time to land before the barrier
+    constexpr int NSPREAD = JVPFA_BWD_SPREAD(NSTEP);
+    if constexpr (gi < NSPREAD) {
+      constexpr int lo = (gi * NLOAD + NSPREAD - 1) / NSPREAD, hi = ((gi + 1) * NLOAD + NSPREAD - 1) / NSPREAD;
+      static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+    }
   };
 
   auto half_tile = [&](auto HBc, uint32_t sbase, int jh) {
@@ -417,8 +424,12 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
   };
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
-    constexpr int lo = (gi * NLOAD + NSTEP - 1) / NSTEP, hi = ((gi + 1) * NLOAD + NSTEP - 1) / NSTEP;
-    static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+    // spread over the first NSPREAD steps only: the last load then has time to land before the barrier
+    constexpr int NSPREAD = JVPFA_BWD_SPREAD(NSTEP);
+    if constexpr (gi < NSPREAD) {
+      constexpr int lo = (gi * NLOAD + NSPREAD - 1) / NSPREAD, hi = ((gi + 1) * NLOAD + NSPREAD - 1) / NSPREAD;
+      static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+    }
   };
 
   auto half_tile = [&](auto HBc, uint32_t sbase, uint32_t sstat, int ih) {

@@ -152,7 +152,9 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
 
   // ---- next-tile loads, one instruction per super-step -------------------------------------------
   constexpr int NLOAD = IPW * Cfg::NTILE;
-  constexpr int NSTEP = 2 * NSS;
+  // the loads of an iteration are spread over its first NSTEP super-steps, not all 2*NSS of them: the
+  // last load then has half a slot to land before the barrier that waits for it
+  constexpr int NSTEP = 3 * NSS / 2;
   int ld_rows_k = 0, ld_rows_v = 0;
   uint32_t ld_dst_k = 0, ld_dst_v = 0;
   const char *ld_p[4] = {nullptr, nullptr, nullptr, nullptr};
@@ -180,8 +182,10 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   };
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
-    constexpr int lo = (gi * NLOAD + NSTEP - 1) / NSTEP, hi = ((gi + 1) * NLOAD + NSTEP - 1) / NSTEP;
-    static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+    if constexpr (gi < NSTEP) {
+      constexpr int lo = (gi * NLOAD + NSTEP - 1) / NSTEP, hi = ((gi + 1) * NLOAD + NSTEP - 1) / NSTEP;
+      static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+    }
   };
 
   constexpr float RESCALE_TAU = 8.f;
