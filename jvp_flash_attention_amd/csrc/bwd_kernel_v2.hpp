@@ -201,8 +201,10 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
     }
   };
 
-  auto half_tile = [&](auto HBc, uint32_t sbase, int jh) {
+  // EDGE: the half tile may cross the causal diagonal or the end of the sequence
+  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, int jh) {
     constexpr int HB = decltype(HBc)::value;
+    constexpr bool EDGE = decltype(EDGEc)::value;
     constexpr int RO = HB * 32 * ROWB;
     // ---- recompute: S, (S', dP, A, B) --------------------------------------------------------
     FragN fk[2], fv[2], fkt[2], fvt[2];
@@ -244,8 +246,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
     else tiles_ready(S, dP);
 
     // ---- P and the score gradients -------------------------------------------------------------
-    const bool diag = pr.causal && (jh + 31 > q0 + wave * 32);
-    const bool ragged = jh + 32 > L;
+    const int klim = min(pr.causal ? qrow : 0x7fffffff, L - 1);  // keys above this index are masked
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
       const int key0 = jh + 16 * hf + 8 * g;
@@ -260,8 +261,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
         if constexpr (MASK == MASK_ADD) s += bias[e];
         float pv = fast_exp2(s - Mq);
         if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
-        if (diag) pv = (key0 + e <= qrow) ? pv : 0.f;
-        if (ragged) pv = (key0 + e < L) ? pv : 0.f;
+        if constexpr (EDGE) pv = (key0 + e <= klim) ? pv : 0.f;
         if constexpr (MODE == BWD_PLAIN) {
           S[i] = pv * (dP[i] - d1);
         } else if constexpr (DUAL) {
@@ -315,18 +315,25 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
 
   prepare_loads(0, 0, true);
   static_for<NLOAD>([&](auto pc) { load_piece(pc); });
-  for (int t = 0; t < ntiles; ++t) {
+  auto tile = [&](int t, auto EDGEc) {
     const int j0 = t * BT;
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
     prepare_loads(stage ^ 1, j0 + BT, t + 1 < ntiles);
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
-    half_tile(std::integral_constant<int, 0>{}, sbase, j0);
+    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, j0);
     // always both halves: a half past the last key or past the diagonal contributes exact zeros, and a
     // branch here would make the accumulators change register file around it
-    half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
-  }
+    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, j0 + 32);
+  };
+  // Tiles that cross the diagonal or the end of the sequence are the last ones; they get a loop of their
+  // own so that the common tile carries no limit tests.  (q0 is a multiple of the tile size.)
+  int t_edge = L / BT;
+  if (pr.causal) t_edge = min(t_edge, q0 / BT);
+  int t = 0;
+  for (; t < min(t_edge, ntiles); ++t) tile(t, std::false_type{});
+  for (; t < ntiles; ++t) tile(t, std::true_type{});
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the redirected loads of the last iteration must not outlive the kernel
 
   if (qrow < L) {
@@ -432,8 +439,10 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
     }
   };
 
-  auto half_tile = [&](auto HBc, uint32_t sbase, uint32_t sstat, int ih) {
+  // EDGE: the half tile may cross the causal diagonal or the end of the sequence
+  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih) {
     constexpr int HB = decltype(HBc)::value;
+    constexpr bool EDGE = decltype(EDGEc)::value;
     constexpr int RO = HB * 32 * ROWB;
     // ---- recompute ------------------------------------------------------------------------------
     FragN fq[2], fg[2], fqt[2], fgt[2];
@@ -486,8 +495,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
         stq[c4 % 2][s_] = lds_b128<s_ * BT * 4 + (c4 / 2) * 64 + (c4 % 2) * 16>(sad);
       });
     };
-    const bool diag = pr.causal && (ih < k0 + wave * 32 + 31);
-    const bool ragged = ih + 32 > L;
+    const int qmin = pr.causal ? krow : 0;  // queries below this index do not see this key
     // The 32 queries are handled as two chunks of 16 (registers 8c .. 8c+7): score gradients of a
     // chunk, then its share of dK^T += Q^T dS (+ Q'^T dS'), dV^T += G^T P (+ gT^T P'), one step per
     // d-block; the transposed fragments of a step are read one step ahead.
@@ -532,8 +540,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
           }
           float pv = fast_exp2(s - stat(0, e));
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
-          if (diag) pv = (krow <= qi) ? pv : 0.f;
-          if (ragged) pv = (qi < L) ? pv : 0.f;
+          if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
           S[e] = pv;
           if constexpr (MODE == BWD_PLAIN) {
             dP[e] = pv * (dP[e] - stat(1, e));
@@ -582,7 +589,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
   prepare_loads(0, istart, true);
   static_for<NLOAD>([&](auto pc) { load_piece(pc); });
   load_stats();
-  for (int t = 0; t < ntiles; ++t) {
+  auto tile = [&](int t, auto EDGEc) {
     const int i0 = istart + t * BT;
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -590,11 +597,19 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
     prepare_loads(stage ^ 1, i0 + BT, t + 1 < ntiles);
     load_stats();
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB, sstat = stat0 + stage * Cfg::STATB;
-    half_tile(std::integral_constant<int, 0>{}, sbase, sstat, i0);
+    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, sstat, i0);
     // always both halves: a half past the last query contributes exact zeros, and a branch here would
     // make the accumulators change register file around it
-    half_tile(std::integral_constant<int, 1>{}, sbase, sstat, i0 + 32);
-  }
+    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32);
+  };
+  // Query tiles that cross the diagonal come first (causal), those that cross the end of the sequence
+  // last; the tiles in between run without limit tests.
+  const int t_diag = pr.causal ? min(ntiles, (k0 + Cfg::BLK - istart + BT - 1) / BT) : 0;
+  const int t_end = max(t_diag, min(ntiles, (L - istart) / BT));
+  int t = 0;
+  for (; t < t_diag; ++t) tile(t, std::true_type{});
+  for (; t < t_end; ++t) tile(t, std::false_type{});
+  for (; t < ntiles; ++t) tile(t, std::true_type{});
   __builtin_amdgcn_s_waitcnt(0x0F70);
 
   if (krow < L) {
