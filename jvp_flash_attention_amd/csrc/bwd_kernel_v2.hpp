@@ -167,6 +167,8 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
+  bool mask_al = false;  // mask rows can be fetched with aligned vector loads
+  if constexpr (MASK != MASK_NONE) mask_al = mask_rows_aligned<T, MASK>(pr);
   const char *Kb = reinterpret_cast<const char *>(p.k) + head * sizeof(T);
   const char *Vb = reinterpret_cast<const char *>(p.v) + head * sizeof(T);
   const char *Ktb = DUAL ? reinterpret_cast<const char *>(p.kt) + head * sizeof(T) : nullptr;
@@ -219,6 +221,15 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
       }
     };
     constexpr int NRN = DUAL ? 4 : 2;
+    // mask values of this half tile, fetched before the products that hide their latency
+    MaskAhead<T, MASK> mah[2];
+    const bool mask_ahead = MASK != MASK_NONE && mask_al && jh + 32 <= L;
+    if constexpr (MASK != MASK_NONE) {
+      if (mask_ahead) {
+        mah[0] = mask_fetch8<T, MASK>(pr, mrow, jh + 8 * g);
+        mah[1] = mask_fetch8<T, MASK>(pr, mrow, jh + 16 + 8 * g);
+      }
+    }
     // tiles in ordinary vector registers; in DUAL, dP also collects V' gT^T (the B term)
     f32x16 S, dP, Sp, At;
     issue_n(std::integral_constant<int, 0>{});
@@ -252,8 +263,18 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
       const int key0 = jh + 16 * hf + 8 * g;
       float bias[8];
       bool keep[8];
-      if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
-      if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
+      if constexpr (MASK != MASK_NONE) {
+        if (mask_ahead) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            if constexpr (MASK == MASK_ADD) bias[e] = mask_bias_of<T, MASK>(mah[hf], e);
+            if constexpr (MASK == MASK_BOOL) keep[e] = mask_keep_of<T, MASK>(mah[hf], e);
+          }
+        } else {
+          if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
+          if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
+        }
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int i = 8 * hf + e;
@@ -457,6 +478,20 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
       }
     };
     constexpr int NRN = DUAL ? 4 : 2;
+    // mask values of this lane's key for the 32 queries of the half tile (register e <-> query
+    // 16(e/8) + 8g + e%8), fetched before the products that hide their latency
+    T mraw_a[MASK == MASK_ADD ? 16 : 1];
+    uint8_t mraw_b[MASK == MASK_BOOL ? 16 : 1];
+    if constexpr (MASK != MASK_NONE) {
+      const int64_t mcol = z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
+        const int64_t off = mcol + (int64_t)min(qi, L - 1) * pr.ms[2];
+        if constexpr (MASK == MASK_ADD) mraw_a[e] = reinterpret_cast<const T *>(pr.mask)[off];
+        if constexpr (MASK == MASK_BOOL) mraw_b[e] = reinterpret_cast<const uint8_t *>(pr.mask)[off];
+      }
+    }
     // tiles in ordinary vector registers; in DUAL, dP also collects gT V'^T (the B term)
     f32x16 S, dP, Sp, At;
     issue_n(std::integral_constant<int, 0>{});
@@ -532,12 +567,8 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
           const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
           float s = S[e] * sl2;
           bool keep = true;
-          if constexpr (MASK != MASK_NONE) {
-            const int qc = qi < L ? qi : L - 1;
-            const int64_t off = z * pr.ms[0] + h * pr.ms[1] + (int64_t)qc * pr.ms[2] + (int64_t)kld * pr.ms[3];
-            if constexpr (MASK == MASK_ADD) s += (float)reinterpret_cast<const T *>(pr.mask)[off] * LOG2E;
-            if constexpr (MASK == MASK_BOOL) keep = reinterpret_cast<const uint8_t *>(pr.mask)[off] != 0;
-          }
+          if constexpr (MASK == MASK_ADD) s += (float)mraw_a[e] * LOG2E;
+          if constexpr (MASK == MASK_BOOL) keep = mraw_b[e] != 0;
           float pv = fast_exp2(s - stat(0, e));
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
           if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;

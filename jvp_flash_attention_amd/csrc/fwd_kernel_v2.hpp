@@ -180,6 +180,8 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
+  bool mask_al = false;  // mask rows can be fetched with aligned vector loads
+  if constexpr (MASK != MASK_NONE) mask_al = mask_rows_aligned<T, MASK>(pr);
 
   int kend = L;
   if (pr.causal) kend = min(L, q0 + Cfg::BM);
@@ -232,14 +234,18 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   // which live in the matrix-core accumulation registers, are touched by VALU code only on the few
   // tiles where the running maximum really grows.  O = acc / l is unchanged by the choice of m_i.
   constexpr float RESCALE_TAU = 8.f;
-  auto half_tile = [&](auto HBc, uint32_t sbase, int jh) {
+  const int klim = min(pr.causal ? qrow : 0x7fffffff, L - 1);  // keys above this index are masked
+  // EDGE: the half tile may cross the causal diagonal or the end of the sequence, the scale may be
+  // negative, or the mask rows are not aligned for vector fetches
+  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, int jh) {
     constexpr int HB = decltype(HBc)::value;
+    constexpr bool EDGE = decltype(EDGEc)::value;
     constexpr int KO = HB * 32 * ROWB;  // K at +0, K' at +2*TILEB, V at +TILEB, V' at +3*TILEB
     constexpr int NRS = DUAL ? 2 : 1;   // LDS reads per S step
     constexpr int NRV = DUAL ? 4 : 2;   // LDS reads per PV step
     constexpr int NPV = 2 * DB;         // PV steps: (16-key chunk c, d-block db)
 
-    constexpr int RD = JVPFA_RING;  // fragment ring slots; reads run RD-1 steps ahead
+    constexpr int RD = MASK != MASK_NONE ? 4 : JVPFA_RING;  // fragment ring slots (reads run RD-1 steps ahead); the masked kernels need the registers
     constexpr int PD = RD - 1;
     u32x4 ka[RD], kb[RD];
     auto issue_k = [&](auto kkc) {
@@ -264,6 +270,15 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     // score tiles in ordinary vector registers, written by matrix instructions whose B operand (Q, Q')
     // is resident in the accumulation register file
     f32x16 S, Sp;
+    // mask values of this half tile, fetched before the score products that hide their latency
+    MaskAhead<T, MASK> mah[2];
+    const bool mask_ahead = MASK != MASK_NONE && (!EDGE || (mask_al && jh + 32 <= L));
+    if constexpr (MASK != MASK_NONE) {
+      if (mask_ahead) {
+        mah[0] = mask_fetch8<T, MASK>(pr, mrow, jh + 8 * g);
+        mah[1] = mask_fetch8<T, MASK>(pr, mrow, jh + 16 + 8 * g);
+      }
+    }
     static_for<(PD < KK ? PD : KK)>([&](auto kkc) { issue_k(kkc); });
     static_for<KK>([&](auto kkc) {
       constexpr int kk = decltype(kkc)::value;
@@ -280,26 +295,33 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     if constexpr (DUAL) tiles_ready(S, Sp);
     else tiles_ready(S);
     JVPFA_STAMP(5);
-    const bool diag = pr.causal && (jh + 31 > q0 + wave * 32);
-    const bool ragged = jh + 32 > L;
     float mx;
-    const bool general = MASK != MASK_NONE || diag || ragged || !(sl2 > 0.f);
-    if (general) {
+    constexpr bool general = MASK != MASK_NONE || EDGE;
+    if constexpr (general) {
       mx = NEG_INF;
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf) {
         const int key0 = jh + 16 * hf + 8 * g;
         float bias[8];
         bool keep[8];
-        if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
-        if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
+        if constexpr (MASK != MASK_NONE) {
+          if (mask_ahead) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              if constexpr (MASK == MASK_ADD) bias[e] = mask_bias_of<T, MASK>(mah[hf], e);
+              if constexpr (MASK == MASK_BOOL) keep[e] = mask_keep_of<T, MASK>(mah[hf], e);
+            }
+          } else {
+            if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
+            if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
+          }
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           float s = S[8 * hf + e] * sl2;
           if constexpr (MASK == MASK_ADD) s += bias[e];
           if constexpr (MASK == MASK_BOOL) s = keep[e] ? s : NEG_INF;
-          if (diag) s = (key0 + e <= qrow) ? s : NEG_INF;
-          if (ragged) s = (key0 + e < L) ? s : NEG_INF;
+          if constexpr (EDGE) s = (key0 + e <= klim) ? s : NEG_INF;
           S[8 * hf + e] = s;
           mx = fmaxf(mx, s);
         }
@@ -331,7 +353,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
 
     const float m_use = (m_i == NEG_INF) ? 0.f : m_i;
     float rs = 0.f, rmu = 0.f;
-    if (general) {
+    if constexpr (general) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) S[e] = fast_exp2(S[e] - m_use);
     } else {
@@ -377,7 +399,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   };
 
   issue_loads(0, 0);
-  for (int t = 0; t < ntiles; ++t) {
+  auto tile = [&](int t, auto EDGEc) {
     const int j0 = t * BN;
     const int stage = t & 1;
     JVPFA_STAMP(1);
@@ -387,11 +409,19 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     JVPFA_STAMP(3);
     prepare_loads(stage ^ 1, j0 + BN, t + 1 < ntiles);
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
-    half_tile(std::integral_constant<int, 0>{}, sbase, j0);
+    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, j0);
     // always both halves: a half past the last key is fully masked and contributes exact zeros, and a
     // branch here would make the accumulators change register file around it
-    half_tile(std::integral_constant<int, 1>{}, sbase, j0 + 32);
-  }
+    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, j0 + 32);
+  };
+  // Tiles that need the general treatment are the last ones; they get a loop of their own so that the
+  // common tile carries no limit tests.  (q0 is a multiple of the tile size.)
+  int t_edge = L / BN;
+  if (pr.causal) t_edge = min(t_edge, q0 / BN);
+  if (!(sl2 > 0.f) || (MASK != MASK_NONE && !mask_al)) t_edge = 0;
+  int t = 0;
+  for (; t < min(t_edge, ntiles); ++t) tile(t, std::false_type{});
+  for (; t < ntiles; ++t) tile(t, std::true_type{});
 
   // ---- epilogue ---------------------------------------------------------------------------------
   l_i += xor32(l_i);

@@ -12,7 +12,7 @@ __device__ __forceinline__ void mask_keep8(const Problem &pr, int64_t rowoff, in
   if (pr.ms[3] == 1 && key0 + 8 <= pr.L && ((reinterpret_cast<uintptr_t>(base + key0) & 7) == 0)) {
     uint64_t w = *reinterpret_cast<const uint64_t *>(base + key0);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) keep[e] = ((w >> (8 * e)) & 0xff) != 0;
+    for (int e = 0; e < 8; ++e) keep[e] = ((e < 4 ? (uint32_t)w : (uint32_t)(w >> 32)) & (0xffu << (8 * (e & 3)))) != 0;
   } else {
 #pragma unroll
     for (int e = 0; e < 8; ++e) keep[e] = (key0 + e < pr.L) ? base[(int64_t)(key0 + e) * pr.ms[3]] != 0 : false;
@@ -32,6 +32,36 @@ __device__ __forceinline__ void mask_bias8(const Problem &pr, int64_t rowoff, in
     for (int e = 0; e < 8; ++e)
       bias[e] = (key0 + e < pr.L) ? (float)base[(int64_t)(key0 + e) * pr.ms[3]] * LOG2E : 0.f;
   }
+}
+
+// ---- mask data fetched ahead of its use -----------------------------------------------------------
+// The loads above sit right where their values are needed, so their latency is exposed.  When the
+// key stride is 1 and every row start is aligned, the eight keys of a lane are one vector load that
+// can be issued a whole phase of matrix instructions earlier and decoded later.
+template <typename T, int MASK> struct MaskAhead {
+  uint64_t w;   // MASK_BOOL: eight bytes
+  Frag<T> f;    // MASK_ADD: eight elements
+};
+template <typename T, int MASK> __device__ __forceinline__ bool mask_rows_aligned(const Problem &pr) {
+  constexpr int64_t AL = MASK == MASK_BOOL ? 8 : (int64_t)(16 / sizeof(T));  // in elements
+  const uintptr_t base = reinterpret_cast<uintptr_t>(pr.mask);
+  return pr.ms[3] == 1 && (pr.ms[0] % AL) == 0 && (pr.ms[1] % AL) == 0 && (pr.ms[2] % AL) == 0 &&
+         (base % (MASK == MASK_BOOL ? 8 : 16)) == 0;
+}
+// keys key0 .. key0+7 must exist (key0 + 8 <= L) and key0 must be a multiple of 8
+template <typename T, int MASK>
+__device__ __forceinline__ MaskAhead<T, MASK> mask_fetch8(const Problem &pr, int64_t rowoff, int key0) {
+  MaskAhead<T, MASK> m;
+  if constexpr (MASK == MASK_BOOL) m.w = *reinterpret_cast<const uint64_t *>(reinterpret_cast<const uint8_t *>(pr.mask) + rowoff + key0);
+  else m.f = ld8<T>(reinterpret_cast<const T *>(pr.mask) + rowoff + key0);
+  return m;
+}
+template <typename T, int MASK> __device__ __forceinline__ bool mask_keep_of(const MaskAhead<T, MASK> &m, int e) {
+  const uint32_t half = e < 4 ? (uint32_t)m.w : (uint32_t)(m.w >> 32);  // 32-bit tests: 64-bit shifts are slow
+  return (half & (0xffu << (8 * (e & 3)))) != 0;
+}
+template <typename T, int MASK> __device__ __forceinline__ float mask_bias_of(const MaskAhead<T, MASK> &m, int e) {
+  return (float)m.f[e] * LOG2E;
 }
 
 }  // namespace jvpfa

@@ -6,7 +6,7 @@
 Counterpart of the reference's script ``tests/test_jvp_attention.py`` (run as a program there,
 README.md:111-113): for every sequence length, mask type (none / boolean / additive) and causal
 flag it (1) compares ``JVPAttn.fwd_dual`` under ``fwAD.dual_level()`` and under ``torch.func.jvp``
-with PyTorch's math SDPA under forward-mode AD (the reference's oracle, test file lines 548-617):
+with PyTorch's math SDPA under forward-mode AD (what the reference's own tests compare with, test file lines 548-617):
 primal, tangent, the loss ``mean((out - target)^2)`` and its q/k/v gradients; (2) times the dual
 forward the way the reference does (10 warm-up + 100 calls, input clones and ``make_dual``
 included, lines 129-143 and 770-780) next to math SDPA; (3) records the peak memory of one call.
