@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
     constexpr int NRN = DUAL ? 4 : 2;
     // mask values of this half tile, fetched before the products that hide their latency
     MaskAhead<T, MASK> mah[2];
-    const bool mask_ahead = MASK != MASK_NONE && mask_al && jh + 32 <= L;
+    const bool mask_ahead = MASK != MASK_NONE && (!EDGE || (mask_al && jh + 32 <= L));
     if constexpr (MASK != MASK_NONE) {
       if (mask_ahead) {
         mah[0] = mask_fetch8<T, MASK>(pr, mrow, jh + 8 * g);
@@ -352,6 +352,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
   // own so that the common tile carries no limit tests.  (q0 is a multiple of the tile size.)
   int t_edge = L / BT;
   if (pr.causal) t_edge = min(t_edge, q0 / BT);
+  if (MASK != MASK_NONE && !mask_al) t_edge = 0;  // interior tiles fetch mask rows with aligned vector loads
   int t = 0;
   for (; t < min(t_edge, ntiles); ++t) tile(t, std::false_type{});
   for (; t < ntiles; ++t) tile(t, std::true_type{});
@@ -413,6 +414,14 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
   }
 
   const float sl2 = pr.scale * LOG2E;
+  // mask element of (query 8g, this lane's key) relative to a row pointer, as a 32-bit offset
+  bool mask_small = true;
+  uint32_t mlane = 0;
+  if constexpr (MASK != MASK_NONE) {
+    const int64_t lim = (int64_t)1 << 31;
+    mask_small = pr.ms[2] >= 0 && pr.ms[3] >= 0 && 8 * pr.ms[2] + (int64_t)L * pr.ms[3] < lim;
+    mlane = (uint32_t)(8 * g * pr.ms[2] + (int64_t)kld * pr.ms[3]);
+  }
   // tile slots: 0 Q, 1 G (gO; gT in TANGENT; gT again in DUAL without gO), 2 Q', 3 gT
   const char *Qb = reinterpret_cast<const char *>(p.q) + head * sizeof(T);
   const char *gTb = (DUAL || TAN) ? reinterpret_cast<const char *>(p.gt) + head * sizeof(T) : nullptr;
@@ -483,13 +492,25 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
     T mraw_a[MASK == MASK_ADD ? 16 : 1];
     uint8_t mraw_b[MASK == MASK_BOOL ? 16 : 1];
     if constexpr (MASK != MASK_NONE) {
-      const int64_t mcol = z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3];
+      if constexpr (!EDGE) {
+        // uniform 64-bit row pointer + 32-bit lane offset: no per-lane address arithmetic per element
+        // (interior tiles only run when the lane offsets fit 32 bits, see mask_small below)
+        const int64_t mrow0 = z * pr.ms[0] + h * pr.ms[1];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
-        const int64_t off = mcol + (int64_t)min(qi, L - 1) * pr.ms[2];
-        if constexpr (MASK == MASK_ADD) mraw_a[e] = reinterpret_cast<const T *>(pr.mask)[off];
-        if constexpr (MASK == MASK_BOOL) mraw_b[e] = reinterpret_cast<const uint8_t *>(pr.mask)[off];
+        for (int e = 0; e < 16; ++e) {
+          const int64_t urow = mrow0 + (int64_t)(ih + 16 * (e / 8) + (e % 8)) * pr.ms[2];
+          if constexpr (MASK == MASK_ADD) mraw_a[e] = (reinterpret_cast<const T *>(pr.mask) + urow)[mlane];
+          if constexpr (MASK == MASK_BOOL) mraw_b[e] = (reinterpret_cast<const uint8_t *>(pr.mask) + urow)[mlane];
+        }
+      } else {
+        const int64_t mcol = z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
+          const int64_t off = mcol + (int64_t)min(qi, L - 1) * pr.ms[2];
+          if constexpr (MASK == MASK_ADD) mraw_a[e] = reinterpret_cast<const T *>(pr.mask)[off];
+          if constexpr (MASK == MASK_BOOL) mraw_b[e] = reinterpret_cast<const uint8_t *>(pr.mask)[off];
+        }
       }
     }
     // tiles in ordinary vector registers; in DUAL, dP also collects gT V'^T (the B term)
@@ -636,7 +657,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
   // Query tiles that cross the diagonal come first (causal), those that cross the end of the sequence
   // last; the tiles in between run without limit tests.
   const int t_diag = pr.causal ? min(ntiles, (k0 + Cfg::BLK - istart + BT - 1) / BT) : 0;
-  const int t_end = max(t_diag, min(ntiles, (L - istart) / BT));
+  const int t_end = mask_small ? max(t_diag, min(ntiles, (L - istart) / BT)) : t_diag;
   int t = 0;
   for (; t < t_diag; ++t) tile(t, std::true_type{});
   for (; t < t_end; ++t) tile(t, std::false_type{});
