@@ -475,9 +475,12 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
     constexpr bool EDGE = decltype(EDGEc)::value;
     constexpr int RO = HB * 32 * ROWB;
     // ---- recompute ------------------------------------------------------------------------------
+    // D = 64 reads fragments and statistics when it needs them instead of one step ahead: the
+    // registers saved let two workgroups share a compute unit, and the second one covers the waits
+    constexpr bool SAHEAD = D > 64;
     FragN fq[2], fg[2], fqt[2], fgt[2];
     auto issue_n = [&](auto kkc) {
-      constexpr int kk = decltype(kkc)::value, sl = kk % 2;
+      constexpr int kk = decltype(kkc)::value, sl = SAHEAD ? kk % 2 : 0;
       const uint32_t ad = sbase + noff[kk];
       fq[sl].v = lds_b128<RO>(ad);
       fg[sl].v = lds_b128<RO + TILEB>(ad);
@@ -515,13 +518,15 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
     }
     // tiles in ordinary vector registers; in DUAL, dP also collects gT V'^T (the B term)
     f32x16 S, dP, Sp, At;
-    issue_n(std::integral_constant<int, 0>{});
+    if constexpr (SAHEAD) issue_n(std::integral_constant<int, 0>{});
     static_for<KK>([&](auto kkc) {
-      constexpr int kk = decltype(kkc)::value, sl = kk % 2;
+      constexpr int kk = decltype(kkc)::value, sl = SAHEAD ? kk % 2 : 0;
       constexpr bool F = kk == 0;
-      if constexpr (kk + 1 < KK) issue_n(std::integral_constant<int, kk + 1>{});
-      if constexpr (DUAL) lds_wait<(kk + 1 < KK) ? NRN : 0>(fq[sl], fg[sl], fqt[sl], fgt[sl]);
-      else lds_wait<(kk + 1 < KK) ? NRN : 0>(fq[sl], fg[sl]);
+      if constexpr (!SAHEAD) issue_n(std::integral_constant<int, kk>{});
+      else if constexpr (kk + 1 < KK) issue_n(std::integral_constant<int, kk + 1>{});
+      constexpr int younger_n = (SAHEAD && kk + 1 < KK) ? NRN : 0;
+      if constexpr (DUAL) lds_wait<younger_n>(fq[sl], fg[sl], fqt[sl], fgt[sl]);
+      else lds_wait<younger_n>(fq[sl], fg[sl]);
       load_step(std::integral_constant<int, HB * KK + kk>{});
       const Frag<T> q_ = as_frag<T>(fq[sl]), g_ = as_frag<T>(fg[sl]);
       mma_vra<F>(S, q_, Kf[kk]);
@@ -557,7 +562,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
     // d-block; the transposed fragments of a step are read one step ahead.
     FragT tq[2], tg[2], tqt[2], tgt[2];
     auto issue_t = [&](auto ic) {
-      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % 2;
+      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = (D > 64) ? i % 2 : 0;
       constexpr int TO = (HB * 32 + c * 16) * ROWB;
       const uint32_t a0 = sbase + toff[db][0], a1 = sbase + toff[db][1];
       tq[sl].lo = lds_tr64<TO>(a0);
@@ -572,16 +577,18 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
       }
     };
     constexpr int NRT = DUAL ? 8 : 4;
-    issue_s(std::integral_constant<int, 0>{});
+    if constexpr (SAHEAD) issue_s(std::integral_constant<int, 0>{});
     static_for<2>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
       f32x8 Pp;  // P * (S' - mu) of this chunk
       static_for<2>([&](auto hc) {
         constexpr int c4 = 2 * c + decltype(hc)::value, sl = c4 % 2;
-        if constexpr (c4 + 1 < 4) issue_s(std::integral_constant<int, c4 + 1>{});
+        if constexpr (!SAHEAD) issue_s(std::integral_constant<int, c4>{});
+        else if constexpr (c4 + 1 < 4) issue_s(std::integral_constant<int, c4 + 1>{});
         // waits also cover the transposed fragments issued before (LDS reads complete in order)
-        if constexpr (Cfg::NSTAT == 4) lds_wait4<(c4 + 1 < 4) ? 4 : 0>(stq[sl][0], stq[sl][1], stq[sl][2], stq[sl][3]);
-        else lds_wait<(c4 + 1 < 4) ? 2 : 0>(stq[sl][0], stq[sl][1]);
+        constexpr int younger = (SAHEAD && c4 + 1 < 4) ? Cfg::NSTAT : 0;
+        if constexpr (Cfg::NSTAT == 4) lds_wait4<younger>(stq[sl][0], stq[sl][1], stq[sl][2], stq[sl][3]);
+        else lds_wait<younger>(stq[sl][0], stq[sl][1]);
         auto stat = [&](int s_, int e) { return __uint_as_float(stq[sl][s_][e % 4]); };
 #pragma unroll
         for (int e = 4 * c4; e < 4 * c4 + 4; ++e) {
@@ -615,12 +622,14 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
         for (int e = 0; e < 8; ++e) ppf[e] = (T)Pp[e];
       }
       // the next quad of statistics (if any) was issued above, before these fragment reads
-      issue_t(std::integral_constant<int, c * DB>{});
+      if constexpr (SAHEAD) issue_t(std::integral_constant<int, c * DB>{});
       static_for<DB>([&](auto dbc) {
-        constexpr int db = decltype(dbc)::value, i = c * DB + db, sl = i % 2;
-        if constexpr (db + 1 < DB) issue_t(std::integral_constant<int, i + 1>{});
-        if constexpr (DUAL) lds_wait<(db + 1 < DB) ? NRT : 0>(tq[sl], tg[sl], tqt[sl], tgt[sl]);
-        else lds_wait<(db + 1 < DB) ? NRT : 0>(tq[sl], tg[sl]);
+        constexpr int db = decltype(dbc)::value, i = c * DB + db, sl = SAHEAD ? i % 2 : 0;
+        if constexpr (!SAHEAD) issue_t(std::integral_constant<int, i>{});
+        else if constexpr (db + 1 < DB) issue_t(std::integral_constant<int, i + 1>{});
+        constexpr int younger = (SAHEAD && db + 1 < DB) ? NRT : 0;
+        if constexpr (DUAL) lds_wait<younger>(tq[sl], tg[sl], tqt[sl], tgt[sl]);
+        else lds_wait<younger>(tq[sl], tg[sl]);
         load_step(std::integral_constant<int, 2 * KK + HB * NPV + i>{});
         if constexpr (MODE == BWD_PLAIN) {
           mma(dK[db], as_frag<T>(tq[sl]), dsf);
