@@ -86,14 +86,20 @@ template <int N> __device__ __forceinline__ void lds_wait4(u32x4 &a, u32x4 &b, u
     ld_row[i] = lc / CH;                                                                                            \
     ld_c[i] = ((lc % CH) ^ swz_u<CH>(lc / CH)) * 16;                                                                \
   }                                                                                                                 \
-  int ld_rows = 0;                                                                                                  \
+  /* buffer loads: descriptor = (start of the tile, bytes left in the head), per-lane offset constant; rows */      \
+  /* past the end of the sequence and tiles that do not exist are out of range and read as zeros */                \
+  uint32_t ld_o[IPW];                                                                                               \
+  _Pragma("unroll") for (int i = 0; i < IPW; ++i) ld_o[i] = ld_row[i] * ROWB + ld_c[i];                            \
   uint32_t ld_dst = 0;                                                                                              \
-  const char *ld_p[4] = {nullptr, nullptr, nullptr, nullptr};                                                       \
+  __amdgpu_buffer_rsrc_t ld_rs[4];                                                                                  \
+  auto tile_rsrc = [&](const char *base, int j, bool exists) {                                                      \
+    const int rows = exists ? max(L - j, 0) : 0;                                                                    \
+    return __builtin_amdgcn_make_buffer_rsrc((void *)(base + (size_t)j * ROWB), 0, rows * ROWB, 0x00020000);       \
+  };                                                                                                                \
   auto load_piece = [&](auto pc) {                                                                                  \
     constexpr int pi = decltype(pc)::value, i = pi / Cfg::NTILE, ts = pi % Cfg::NTILE;                              \
-    const uint32_t off = min(ld_row[i], ld_rows) * ROWB + ld_c[i];                                                  \
-    __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(ld_p[ts] + off),                                       \
-                                     (JVPFA_LDS(void))(uintptr_t)(ld_dst + i * 1024 + ts * TILEB), 16, 0, 0);       \
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ld_rs[ts], (JVPFA_LDS(void))(uintptr_t)(ld_dst + i * 1024 + ts * TILEB),  \
+                                             16, ld_o[i], 0, 0, 0);                                                 \
   };                                                                                                                \
   /* row-major fragment (rows = streamed index, contraction over d): row 32hb + perm32(r), chunk 2kk+g */           \
   uint32_t noff[KK];                                                                                                \
@@ -130,6 +136,7 @@ __device__ __forceinline__ void zero_acc(f32x16 &x) {
 // K, V (, K', V').  Scores are transposed (lane = query) so dS is the B operand of dQ^T += K^T dS^T.
 template <typename T, int D, int MODE, int MASK, bool GO>
 __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (and has no buffer descriptor type)
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
   JVPFA_BWD2_COMMON(Cfg)
@@ -182,15 +189,12 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
   constexpr int NPV = 2 * DB / 2;               // accumulation steps of a half: (chunk c, pair of d-blocks)
   constexpr int NSTEP = 2 * (KK + NPV);
   auto prepare_loads = [&](int stage, int j0, bool on) {
-    j0 = on ? j0 : 0;
-    ld_rows = L - 1 - j0;
     ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
-    const size_t tb = (size_t)j0 * ROWB;
-    ld_p[0] = Kb + tb;
-    ld_p[1] = Vb + tb;
+    ld_rs[0] = tile_rsrc(Kb, j0, on);
+    ld_rs[1] = tile_rsrc(Vb, j0, on);
     if constexpr (DUAL) {
-      ld_p[2] = Ktb + tb;
-      ld_p[3] = Vtb + tb;
+      ld_rs[2] = tile_rsrc(Ktb, j0, on);
+      ld_rs[3] = tile_rsrc(Vtb, j0, on);
     }
   };
   auto load_step = [&](auto gc) {
@@ -371,6 +375,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
       }
     }
   }
+#endif
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -379,6 +384,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
 // queries) so P, dS are the B operands of dV^T += G^T P and dK^T += Q^T dS.
 template <typename T, int D, int MODE, int MASK, bool GO>
 __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (and has no buffer descriptor type)
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
   JVPFA_BWD2_COMMON(Cfg)
@@ -439,16 +445,14 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
   int st_row = 0;
   uint32_t st_dst = 0;
   auto prepare_loads = [&](int stage, int i0, bool on) {
-    i0 = on ? i0 : istart;
-    ld_rows = L - 1 - i0;
     ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
-    const size_t tb = (size_t)i0 * ROWB;
-    ld_p[0] = Qb + tb;
-    ld_p[1] = Gb + tb;
+    ld_rs[0] = tile_rsrc(Qb, i0, on);
+    ld_rs[1] = tile_rsrc(Gb, i0, on);
     if constexpr (DUAL) {
-      ld_p[2] = Qtb + tb;
-      ld_p[3] = gTb + tb;
+      ld_rs[2] = tile_rsrc(Qtb, i0, on);
+      ld_rs[3] = tile_rsrc(gTb, i0, on);
     }
+    i0 = on ? i0 : istart;
     st_row = min(i0 + lane, L - 1);
     st_dst = stat0 + stage * Cfg::STATB;
   };
@@ -691,6 +695,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
       }
     }
   }
+#endif
 }
 
 }  // namespace jvpfa

@@ -50,6 +50,7 @@ template <int N> __device__ __forceinline__ void lds_wait3(u32x4 &a, u32x2 &c, u
 
 template <typename T, int D, bool DUAL>
 __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (and has no buffer descriptor type)
   using Cfg = Fwd2Cfg<T, D, DUAL>;
   constexpr int BN = Cfg::BN, CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW;
   constexpr int KK = D / 16, DB = D / 32;
@@ -155,30 +156,42 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   // the loads of an iteration are spread over its first NSTEP super-steps, not all 2*NSS of them: the
   // last load then has half a slot to land before the barrier that waits for it
   constexpr int NSTEP = 3 * NSS / 2;
-  int ld_rows_k = 0, ld_rows_v = 0;
   uint32_t ld_dst_k = 0, ld_dst_v = 0;
-  const char *ld_p[4] = {nullptr, nullptr, nullptr, nullptr};
-  // iteration t loads K(t+1) into the K half of stage (t+1)&1 and V(t) into the V half of stage t&1;
-  // a tile that does not exist is replaced by tile 0 (never read), which keeps the stream branch-free
+  // Buffer loads: the descriptor of a tensor holds (start of the tile, bytes left in the head) and the
+  // per-lane offset is a constant of the kernel, so a load needs no vector arithmetic; rows past the
+  // end of the sequence, and tiles that do not exist, are out of range and read as zeros.
+  __amdgpu_buffer_rsrc_t ld_rs[4];
+  uint32_t ldo_k[IPW], ldo_v[IPW];
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) {
+    ldo_k[i] = ld_row[i] * ROWB + ld_ck[i];
+    ldo_v[i] = ld_row[i] * ROWB + ld_cv[i];
+  }
+  auto tile_rsrc = [&](const char *base, int j, bool exists) {
+    const int rows = exists ? max(L - j, 0) : 0;
+    return __builtin_amdgcn_make_buffer_rsrc((void *)(base + (size_t)j * ROWB), 0, rows * ROWB, 0x00020000);
+  };
+  // iteration t loads K(t+1) into the K half of stage (t+1)&1 and V(t) into the V half of stage t&1
   auto prepare_loads = [&](int t) {
-    const int jk = (t + 1 < ntiles) ? (t + 1) * BN : 0, jv = (t < ntiles) ? t * BN : 0;
-    ld_rows_k = L - 1 - jk;
-    ld_rows_v = L - 1 - jv;
     ld_dst_k = lds0 + ((t + 1) & 1) * Cfg::STAGEB + (wave * IPW) * 1024;
     ld_dst_v = lds0 + (t & 1) * Cfg::STAGEB + (wave * IPW) * 1024;
-    ld_p[0] = Kg + (size_t)jk * ROWB;
-    ld_p[1] = Vg + (size_t)jv * ROWB;
+    ld_rs[0] = tile_rsrc(Kg, (t + 1) * BN, t + 1 < ntiles);
+    ld_rs[1] = tile_rsrc(Vg, t * BN, t < ntiles);
     if constexpr (DUAL) {
-      ld_p[2] = Ktg + (size_t)jk * ROWB;
-      ld_p[3] = Vtg + (size_t)jv * ROWB;
+      ld_rs[2] = tile_rsrc(Ktg, (t + 1) * BN, t + 1 < ntiles);
+      ld_rs[3] = tile_rsrc(Vtg, t * BN, t < ntiles);
     }
+  };
+  auto prepare_first = [&]() {
+    ld_dst_k = lds0 + (wave * IPW) * 1024;
+    ld_rs[0] = tile_rsrc(Kg, 0, true);
+    if constexpr (DUAL) ld_rs[2] = tile_rsrc(Ktg, 0, true);
   };
   auto load_piece = [&](auto pc) {
     constexpr int pi = decltype(pc)::value, i = pi / Cfg::NTILE, ts = pi % Cfg::NTILE;
     constexpr bool vt = (ts & 1) != 0;
-    const uint32_t off = min(ld_row[i], vt ? ld_rows_v : ld_rows_k) * ROWB + (vt ? ld_cv[i] : ld_ck[i]);
-    __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(ld_p[ts] + off),
-                                     (JVPFA_LDS(void))(uintptr_t)((vt ? ld_dst_v : ld_dst_k) + i * 1024 + ts * TILEB), 16, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ld_rs[ts], (JVPFA_LDS(void))(uintptr_t)((vt ? ld_dst_v : ld_dst_k) + i * 1024 + ts * TILEB),
+                                             16, vt ? ldo_v[i] : ldo_k[i], 0, 0, 0);
   };
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
@@ -432,15 +445,10 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   Frag<T> pfA[2], psfA[2], pfB[2], psfB[2];
 
   // ---- prologue: K(0) in one burst ---------------------------------------------------------------
-  {
-    ld_rows_k = L - 1;
-    ld_dst_k = lds0 + (wave * IPW) * 1024;
-    ld_p[0] = Kg;
-    if constexpr (DUAL) ld_p[2] = Ktg;
-    static_for<NLOAD>([&](auto pc) {
-      if constexpr (decltype(pc)::value % 2 == 0) load_piece(pc);
-    });
-  }
+  prepare_first();
+  static_for<NLOAD>([&](auto pc) {
+    if constexpr (decltype(pc)::value % 2 == 0) load_piece(pc);
+  });
   auto kad = [&](int t, int hb) { return lds0 + (t & 1) * Cfg::STAGEB + hb * 32 * ROWB; };
 
   // iteration 0: scores of half tiles 0 and 1, softmax of half tile 0
@@ -511,6 +519,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
       if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = mu_n;
     }
   }
+#endif
 }
 
 }  // namespace jvpfa
