@@ -53,13 +53,13 @@ def _mask(mode, Z, H, L, dtype, seed=1):
     raise ValueError(mode)
 
 
-def _run_case(Z, H, L, D, dtype, mode, seed=0, tangent_std=1.0, plain=False, tangent_grads=True):
+def _run_case(Z, H, L, D, dtype, mode, seed=0, tangent_std=1.0, plain=False, tangent_grads=True, causal=None):
     from jvp_flash_attention_amd import _lib
 
     be = _lib.backend()
     q, k, v, qt, kt, vt, go, gt = _make(Z, H, L, D, dtype, seed, tangent_std)
     mask = _mask(mode, Z, H, L, dtype)
-    causal = mode == "causal"
+    causal = (mode == "causal") if causal is None else causal
     kind = _lib.MASK_NONE if mask is None else (_lib.MASK_BOOL if mask.dtype == torch.bool else _lib.MASK_ADD)
     scale = D**-0.5
     npm = None if mask is None else (mask.numpy() if mask.dtype == torch.bool else mask.double().numpy())
@@ -124,6 +124,27 @@ def test_masks_d128(dt, mode):
 @pytest.mark.parametrize("mode", ["none", "causal", "keypad"])
 def test_ragged_lengths(dt, L, mode):
     _run_case(1, 2, L, 64, DTYPES[dt], mode)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+@pytest.mark.parametrize("L", [100, 333])
+@pytest.mark.parametrize("mode", ["bool_full", "bias"])
+def test_dense_masks_with_unaligned_rows(dt, L, mode):
+    # a row of the mask starts at a multiple of L elements: not aligned for vector fetches when L is odd-ish
+    _run_case(1, 2, L, 64, DTYPES[dt], mode, seed=11)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("mode", ["bool_full", "bias", "keypad"])
+def test_masks_over_several_tiles_interior_and_edge(D, mode):
+    # L = 328: five key tiles, the last one ragged; aligned rows, so interior tiles take the fetch-ahead path
+    _run_case(1, 2, 328, D, torch.bfloat16, mode, seed=12)
+
+
+def test_mask_combined_with_causal_is_refused():
+    # as in the reference, causal attention takes no explicit mask: the library reports it instead of guessing
+    with pytest.raises(RuntimeError, match="causal"):
+        _run_case(1, 2, 128, 64, torch.bfloat16, "keypad", causal=True)
 
 
 @pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
