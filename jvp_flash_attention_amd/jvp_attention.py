@@ -19,6 +19,8 @@ Differences from the reference, all deliberate:
   reference's tangent is a constant (JA:2399, JA:2828) and its backward ignores it (JA:2831).
 * Any sequence length L >= 1 and head dims {32, 64, 128} (the reference: L a multiple of 32,
   D in {32, 64, 128, 256}, JA:2371-2378, JA:2892).
+* ``attention`` notices dual inputs and then behaves like ``fwd_dual`` (the reference's ``attention``
+  is ``JVPAttn.fwd`` and drops the tangent, its README.md:65-67).
 """
 from __future__ import annotations
 
@@ -364,4 +366,19 @@ class JVPAttn(Function):
         return JVPAttn.BwdOut(dq, dk, dv, None, None, None, None, None, None, None, None, None, None)
 
 
-attention = JVPAttn.fwd
+def attention(
+    q: Tensor,
+    k: Tensor,
+    v: Tensor,
+    attn_mask: Tensor | None = None,
+    dropout_p: float = 0.0,
+    causal: bool = False,
+    sm_scale: float | None = None,
+    warp_specialize: bool = True,
+    USE_TMA: bool = True,
+) -> Tensor:
+    """The reference's ``attention`` (JA:2981, an alias of ``JVPAttn.fwd``), except that dual inputs are
+    noticed: inside ``fwAD.dual_level()`` or ``torch.func.jvp`` the tangent O' is propagated, which in
+    the reference needs an explicit ``JVPAttn.fwd_dual`` call (its README.md:65-67).  Without tangents
+    this is exactly ``JVPAttn.fwd``."""
+    return JVPAttn.fwd_dual(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)

@@ -59,6 +59,22 @@ def test_fwd_dual_three_way_like_reference_tests(causal):
         _close(ot, ot_ref)
 
 
+def test_attention_notices_dual_inputs():
+    """attention() under forward-mode AD returns the tangent too (the reference needs fwd_dual for that)."""
+    q, k, v, qt, kt, vt, _, _ = _inputs(seed=3)
+    o_ref, ot_ref = sdpa_jvp.forward(q, k, v, qt, kt, vt)
+    with oracle_backend() as be:
+        o2, ot2 = torch.func.jvp(attention, (q, k, v), (qt, kt, vt))
+        assert be.calls[0][:2] == ("fwd", True)
+        with fwAD.dual_level():
+            o1, ot1 = fwAD.unpack_dual(attention(fwAD.make_dual(q, qt), k, v))  # k, v without tangents
+            o1, ot1 = o1.clone(), ot1.clone()
+    _close(o2, o_ref)
+    _close(ot2, ot_ref)
+    _close(o1, o_ref)
+    _close(ot1, sdpa_jvp.forward(q, k, v, qt, torch.zeros_like(kt), torch.zeros_like(vt))[1])
+
+
 def test_gradients_through_the_tangent_reach_all_six_inputs():
     q, k, v, qt, kt, vt, go, gt = _inputs()
     _, _, ref = sdpa_jvp.forward_backward(q, k, v, qt, kt, vt, go, gt)
