@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define JVPFA_ABI_VERSION 1
+#define JVPFA_ABI_VERSION 2
 
 enum jvpfa_dtype { JVPFA_BF16 = 0, JVPFA_FP16 = 1, JVPFA_FP32 = 2 };
 
@@ -41,7 +41,7 @@ enum jvpfa_status {
   JVPFA_E_ALIGN = -4,     /* a tensor pointer is not 16-byte aligned */
   JVPFA_E_CONFLICT = -5,  /* causal together with a mask (JA:2380-2381 raises ValueError) */
   JVPFA_E_LAUNCH = -6,    /* hipGetLastError() reported a launch failure */
-  JVPFA_E_ABI = -7        /* struct_size does not match this library */
+  JVPFA_E_ABI = -7        /* struct_size is neither this version's nor version 1's */
 };
 
 /* Shape, numeric type and masking shared by forward and backward. */
@@ -74,6 +74,12 @@ typedef struct jvpfa_fwd_args {
   const void *qt, *kt, *vt; /* all three NULL, or all three set */
   void *o, *ot;
   float *M, *mu;
+  /* since version 2 (a caller may pass the version-1 size, which ends before this field):
+   * optional hint for padded batches, Z int32 values on the device or NULL.  The caller promises
+   * that the mask itself masks every key index >= key_limit[z] for all heads and queries of batch
+   * z; key tiles past the limit are then skipped instead of read and masked.  No counterpart in the
+   * reference, which reads the full (Z,H,L,L) mask (JA:2383-2388).  Ignored without a mask. */
+  const int32_t *key_limit;
 } jvpfa_fwd_args;
 
 int jvpfa_fwd(const jvpfa_fwd_args *args, void *hip_stream);
@@ -104,6 +110,7 @@ typedef struct jvpfa_bwd_args {
   void *dq, *dk, *dv;
   void *dqt, *dkt, *dvt;
   void *workspace;
+  const int32_t *key_limit; /* since version 2: as in jvpfa_fwd_args */
 } jvpfa_bwd_args;
 
 int jvpfa_bwd(const jvpfa_bwd_args *args, void *hip_stream);

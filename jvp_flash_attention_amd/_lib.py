@@ -14,7 +14,7 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libjvpfa.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
 EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_bwd_workspace_bytes", "jvpfa_abi_version", "jvpfa_error_string")
@@ -38,6 +38,7 @@ class FwdArgs(C.Structure):
         ("qt", C.c_void_p), ("kt", C.c_void_p), ("vt", C.c_void_p),
         ("o", C.c_void_p), ("ot", C.c_void_p),
         ("M", C.c_void_p), ("mu", C.c_void_p),
+        ("key_limit", C.c_void_p),
     ]
 
 
@@ -53,6 +54,7 @@ class BwdArgs(C.Structure):
         ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
         ("dqt", C.c_void_p), ("dkt", C.c_void_p), ("dvt", C.c_void_p),
         ("workspace", C.c_void_p),
+        ("key_limit", C.c_void_p),
     ]
 
 
@@ -114,6 +116,31 @@ def make_problem(q, mask, mask_kind, causal, sm_scale) -> Problem:
     return p
 
 
+KEY_LIMIT_MIN_L = 512  # below this the two small reductions cost more than the skipped tiles save
+
+
+def key_limit_hint(mask, mask_kind, Z, L):
+    """For a key-padding mask (one row of L keys per batch entry, shared by heads and queries): the
+    index after the last key that is not masked, per batch entry, as Z int32 values on the mask's
+    device; None for any other mask.  The kernels skip the key tiles past it.  Cached on the mask
+    tensor so that the backward reuses what the forward computed."""
+    if mask is None or mask_kind == MASK_NONE or L < KEY_LIMIT_MIN_L:
+        return None
+    if mask.dim() != 4 or mask.shape[1] != 1 or mask.shape[2] != 1 or mask.shape[3] != L:
+        return None
+    cached = getattr(mask, "_jvpfa_key_limit", None)
+    if cached is not None and cached[0] == mask._version:
+        return cached[1]
+    alive = mask if mask.dtype == torch.bool else mask > float("-inf")
+    idx = torch.arange(1, L + 1, device=mask.device, dtype=torch.int32)
+    lim = (alive.view(mask.shape[0], L) * idx).amax(dim=1).to(torch.int32).expand(Z).contiguous()
+    try:
+        mask._jvpfa_key_limit = (mask._version, lim)
+    except (AttributeError, RuntimeError):
+        pass
+    return lim
+
+
 def _require_gpu(*tensors):
     for t in tensors:
         if t is not None and not t.is_cuda:
@@ -149,6 +176,8 @@ class HipBackend:
         a.qt, a.kt, a.vt = _ptr(qt), _ptr(kt), _ptr(vt)
         a.o, a.ot, a.M, a.mu = _ptr(o), _ptr(ot), _ptr(M), _ptr(mu)
         with torch.cuda.device(q.device):
+            lim = key_limit_hint(mask, mask_kind, Z, L)
+            a.key_limit = _ptr(lim)
             check(lib.jvpfa_fwd(C.byref(a), _stream(q)))
         return o, ot, M, mu
 
@@ -174,6 +203,8 @@ class HipBackend:
         a.dqt, a.dkt, a.dvt = _ptr(dqt), _ptr(dkt), _ptr(dvt)
         a.workspace = _ptr(ws)
         with torch.cuda.device(q.device):
+            lim = key_limit_hint(mask, mask_kind, Z, L)
+            a.key_limit = _ptr(lim)
             check(lib.jvpfa_bwd(C.byref(a), _stream(q)))
         return dq, dk, dv, dqt, dkt, dvt
 

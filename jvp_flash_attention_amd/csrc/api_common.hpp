@@ -23,8 +23,9 @@ inline int check_problem(const jvpfa_problem &p) {
   return JVPFA_OK;
 }
 
-inline Problem to_problem(const jvpfa_problem &p) {
+inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit) {
   Problem r;
+  r.klimit = p.mask_kind == JVPFA_MASK_NONE ? nullptr : key_limit;
   r.Z = p.Z;
   r.H = p.H;
   r.L = p.L;

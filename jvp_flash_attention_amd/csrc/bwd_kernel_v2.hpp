@@ -181,7 +181,10 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
   const char *Ktb = DUAL ? reinterpret_cast<const char *>(p.kt) + head * sizeof(T) : nullptr;
   const char *Vtb = DUAL ? reinterpret_cast<const char *>(p.vt) + head * sizeof(T) : nullptr;
 
-  const int kend = pr.causal ? min(L, q0 + Cfg::BLK) : L;
+  int kend = pr.causal ? min(L, q0 + Cfg::BLK) : L;
+  if constexpr (MASK != MASK_NONE) {  // key tiles that the caller's hint declares fully masked are not visited
+    if (pr.klimit) kend = min(kend, max(pr.klimit[z], 1));
+  }
   const int ntiles = (kend + BT - 1) / BT;
   // tile slots in a stage: 0 K, 1 V, 2 K', 3 V'
   constexpr int NLOAD = IPW * Cfg::NTILE;
@@ -392,6 +395,22 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
   const int k0 = kb * Cfg::BLK;
   const int krow = k0 + wave * 32 + r;
   const int kld = krow < L ? krow : L - 1;
+  if constexpr (MASK != MASK_NONE) {
+    // a key block that the caller's hint declares fully masked has zero gradients
+    if (pr.klimit && k0 >= pr.klimit[z]) {
+      if (krow < L) {
+        T *outk = reinterpret_cast<T *>(MODE == BWD_TANGENT ? p.dkt : p.dk) + head + (size_t)krow * D;
+        T *outv = reinterpret_cast<T *>(MODE == BWD_TANGENT ? p.dvt : p.dv) + head + (size_t)krow * D;
+        float zero8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int d0 = 8 * g; d0 < D; d0 += 16) {
+          store8<T>(outk + d0, zero8);
+          store8<T>(outv + d0, zero8);
+        }
+      }
+      return;
+    }
+  }
   constexpr bool has_go = GO;  // compile-time: a run-time test here would split every step into its own block
   const uint32_t stat0 = lds0 + 2 * Cfg::STAGEB;  // row statistics, two stages of NSTAT x 64 floats
 

@@ -184,6 +184,11 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   if constexpr (MASK != MASK_NONE) mask_al = mask_rows_aligned<T, MASK>(pr);
 
   int kend = L;
+  // padded batches: the caller's hint says the mask hides every key from klimit[z] on, so those tiles
+  // need not be visited (at least one tile is, which keeps rows without any key well defined)
+  if constexpr (MASK != MASK_NONE) {
+    if (pr.klimit) kend = min(L, max(pr.klimit[z], 1));
+  }
   if (pr.causal) kend = min(L, q0 + Cfg::BM);
   const int ntiles = (kend + BN - 1) / BN;
 

@@ -12,6 +12,7 @@ struct Problem {
   float scale;
   const void *mask;
   int64_t ms[4];  // element strides (z, h, query, key)
+  const int *klimit;  // per batch entry: keys at or past this index are masked by the mask (hint), or null
 };
 
 struct FwdParams {

@@ -89,6 +89,44 @@ def test_forward_argument_validation_codes(kw, code):
     assert lib.jvpfa_error_string(code).decode() not in ("ok", "unknown status")
 
 
+def test_version_1_struct_sizes_are_still_accepted():
+    """A caller built against version 1 passes structs that end before key_limit."""
+    lib = _lib.load()
+    a = _fwd_args(q=None)
+    a.struct_size = _lib.FwdArgs.key_limit.offset
+    assert lib.jvpfa_fwd(C.byref(a), None) == -1  # got past the size check, to the NULL pointer check
+    a.struct_size = _lib.FwdArgs.key_limit.offset - 8
+    assert lib.jvpfa_fwd(C.byref(a), None) == -7
+    b = _lib.BwdArgs()
+    b.struct_size = _lib.BwdArgs.key_limit.offset
+    b.p.Z, b.p.H, b.p.L, b.p.D = 1, 1, 32, 64
+    assert lib.jvpfa_bwd(C.byref(b), None) == -1
+
+
+def test_key_limit_hint_of_key_padding_masks():
+    import torch
+
+    L = _lib.KEY_LIMIT_MIN_L
+    m = torch.zeros(3, 1, 1, L, dtype=torch.bool)
+    m[0, ..., :100] = True
+    m[1, ..., :L] = True
+    m[2, ..., 5] = True  # last attended key at index 5; earlier ones masked: still a valid limit
+    assert _lib.key_limit_hint(m, _lib.MASK_BOOL, 3, L).tolist() == [100, L, 6]
+    assert m._jvpfa_key_limit[1].tolist() == [100, L, 6]  # cached for the backward
+    m[0, ..., 200] = True  # an in-place change invalidates the cache
+    assert _lib.key_limit_hint(m, _lib.MASK_BOOL, 3, L).tolist() == [201, L, 6]
+    one = torch.ones(1, 1, 1, L, dtype=torch.bool)
+    one[..., L // 2:] = False
+    assert _lib.key_limit_hint(one, _lib.MASK_BOOL, 4, L).tolist() == [L // 2] * 4  # broadcast over the batch
+    bias = torch.zeros(2, 1, 1, L)
+    bias[0, ..., 300:] = float("-inf")
+    assert _lib.key_limit_hint(bias, _lib.MASK_ADD, 2, L).tolist() == [300, L]
+    # anything that is not one row of keys per batch entry gives no hint; neither do short sequences
+    assert _lib.key_limit_hint(torch.ones(2, 1, L, L, dtype=torch.bool), _lib.MASK_BOOL, 2, L) is None
+    assert _lib.key_limit_hint(torch.ones(2, 1, 1, 64, dtype=torch.bool), _lib.MASK_BOOL, 2, 64) is None
+    assert _lib.key_limit_hint(None, _lib.MASK_NONE, 2, L) is None
+
+
 def test_backward_argument_validation_codes():
     lib = _lib.load()
     a = _lib.BwdArgs()

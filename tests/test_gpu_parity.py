@@ -141,6 +141,38 @@ def test_masks_over_several_tiles_interior_and_edge(D, mode):
     _run_case(1, 2, 328, D, torch.bfloat16, mode, seed=12)
 
 
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("kind", ["bool", "bias"])
+def test_key_padding_with_skipped_tiles(D, kind):
+    """Long enough for the host to pass the key-limit hint: key tiles past the longest valid length of a
+    batch entry are skipped (forward, dq) and fully padded key blocks return zero gradients (dk/dv)."""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H, L = 3, 2, 640
+    dtype = torch.bfloat16
+    q, k, v, qt, kt, vt, go, gt = _make(Z, H, L, D, dtype, 21)
+    lens = [640, 200, 65]
+    keep = torch.arange(L)[None, :] < torch.tensor(lens)[:, None]
+    mask = keep.view(Z, 1, 1, L) if kind == "bool" else torch.where(keep, 0.0, float("-inf")).view(Z, 1, 1, L).to(dtype)
+    mk = _lib.MASK_BOOL if kind == "bool" else _lib.MASK_ADD
+    npm = keep.view(Z, 1, 1, L).numpy()
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dmask = mask.cuda()
+    be = _lib.backend()
+    scale = D**-0.5
+    assert _lib.key_limit_hint(dmask, mk, Z, L).tolist() == lens
+    ref = dense.forward(*f64[:6], mask=npm, causal=False, scale=scale)
+    o, ot, M, mu = be.fwd(*dev[:6], dmask, mk, False, scale)
+    _tol_check("O", o, ref["O"], dtype)
+    _tol_check("O'", ot, ref["Ot"], dtype)
+    rb = dense.backward(*f64, mask=npm, causal=False, scale=scale)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, mk, False, scale, want_tangent_grads=True)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        _tol_check(n, t, rb[n], dtype)
+    assert grads[1][1, :, 256:].abs().max().item() == 0.0 and grads[2][2, :, 128:].abs().max().item() == 0.0
+
+
 def test_mask_combined_with_causal_is_refused():
     # as in the reference, causal attention takes no explicit mask: the library reports it instead of guessing
     with pytest.raises(RuntimeError, match="causal"):
