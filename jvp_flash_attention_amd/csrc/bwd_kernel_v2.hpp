@@ -230,11 +230,13 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
     constexpr int NRN = DUAL ? 4 : 2;
     // mask values of this half tile, fetched before the products that hide their latency
     MaskAhead<T, MASK> mah[2];
-    const bool mask_ahead = MASK != MASK_NONE && (!EDGE || (mask_al && jh + 32 <= L));
     if constexpr (MASK != MASK_NONE) {
-      if (mask_ahead) {
+      if (!EDGE || (mask_al && jh + 32 <= L)) {  // aligned rows, all 32 keys exist: one vector load per 8 keys
         mah[0] = mask_fetch8<T, MASK>(pr, mrow, jh + 8 * g);
         mah[1] = mask_fetch8<T, MASK>(pr, mrow, jh + 16 + 8 * g);
+      } else {
+        mah[0] = mask_fetch8_any<T, MASK>(pr, mrow, jh + 8 * g);
+        mah[1] = mask_fetch8_any<T, MASK>(pr, mrow, jh + 16 + 8 * g);
       }
     }
     // tiles in ordinary vector registers; in DUAL, dP also collects V' gT^T (the B term)
@@ -271,15 +273,10 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
       float bias[8];
       bool keep[8];
       if constexpr (MASK != MASK_NONE) {
-        if (mask_ahead) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            if constexpr (MASK == MASK_ADD) bias[e] = mask_bias_of<T, MASK>(mah[hf], e);
-            if constexpr (MASK == MASK_BOOL) keep[e] = mask_keep_of<T, MASK>(mah[hf], e);
-          }
-        } else {
-          if constexpr (MASK == MASK_ADD) mask_bias8<T>(pr, mrow, key0, bias);
-          if constexpr (MASK == MASK_BOOL) mask_keep8(pr, mrow, key0, keep);
+        for (int e = 0; e < 8; ++e) {
+          if constexpr (MASK == MASK_ADD) bias[e] = mask_bias_of<T, MASK>(mah[hf], e);
+          if constexpr (MASK == MASK_BOOL) keep[e] = mask_keep_of<T, MASK>(mah[hf], e);
         }
       }
 #pragma unroll

@@ -56,6 +56,28 @@ __device__ __forceinline__ MaskAhead<T, MASK> mask_fetch8(const Problem &pr, int
   else m.f = ld8<T>(reinterpret_cast<const T *>(pr.mask) + rowoff + key0);
   return m;
 }
+// The same for any strides and alignment: eight element loads, packed into the same form.  Keys past
+// the end are read from the last key instead (callers mask them by index).
+template <typename T, int MASK>
+__device__ __forceinline__ MaskAhead<T, MASK> mask_fetch8_any(const Problem &pr, int64_t rowoff, int key0) {
+  MaskAhead<T, MASK> m;
+  if constexpr (MASK == MASK_BOOL) {
+    const uint8_t *base = reinterpret_cast<const uint8_t *>(pr.mask) + rowoff;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t b = base[(int64_t)min(key0 + e, pr.L - 1) * pr.ms[3]] != 0 ? 0xffu : 0u;
+      if (e < 4) lo |= b << (8 * e);
+      else hi |= b << (8 * (e - 4));
+    }
+    m.w = (uint64_t)lo | ((uint64_t)hi << 32);
+  } else {
+    const T *base = reinterpret_cast<const T *>(pr.mask) + rowoff;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) m.f[e] = base[(int64_t)min(key0 + e, pr.L - 1) * pr.ms[3]];
+  }
+  return m;
+}
 template <typename T, int MASK> __device__ __forceinline__ bool mask_keep_of(const MaskAhead<T, MASK> &m, int e) {
   const uint32_t half = e < 4 ? (uint32_t)m.w : (uint32_t)(m.w >> 32);  // 32-bit tests: 64-bit shifts are slow
   return (half & (0xffu << (8 * (e & 3)))) != 0;
