@@ -18,8 +18,18 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
     using Cfg2 = Bwd2Cfg<T, D, MODE>;
     // gO may be absent only in the dual mode (loss depends on O' alone)
     const bool no_go = MODE == BWD_DUAL && p.go == nullptr;
-    auto kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, MODE != BWD_DUAL> : bwd2_dq_kernel<T, D, MODE, MASK, true>;
-    auto kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, MODE != BWD_DUAL> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
+    constexpr bool NG = MODE != BWD_DUAL;  // the GO template argument of the kernels without gO
+    void (*kq)(const BwdParams), (*kkv)(const BwdParams);
+    if constexpr (D <= 64) {  // the register-capped twins: two workgroups per compute unit
+      kq = no_go ? bwd2_dq_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dq_kernel_2wg<T, D, MODE, MASK, true>;
+      if constexpr (MASK == MASK_NONE || MODE != BWD_DUAL)
+        kkv = no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, true>;
+      else  // the masked dual dk/dv kernel needs a few registers more than the cap leaves
+        kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
+    } else {
+      kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG> : bwd2_dq_kernel<T, D, MODE, MASK, true>;
+      kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
+    }
     int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
     if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);
     if (rc != 0) return rc;

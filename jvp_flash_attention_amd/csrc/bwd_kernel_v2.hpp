@@ -134,9 +134,9 @@ __device__ __forceinline__ void zero_acc(f32x16 &x) {
 // ------------------------------------------------------------------------------------------------
 // dq (PLAIN / DUAL) or dq' (TANGENT): workgroup = 128 query rows, loop over 64-key tiles of
 // K, V (, K', V').  Scores are transposed (lane = query) so dS is the B operand of dQ^T += K^T dS^T.
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stubs (and has no buffer descriptor type)
 template <typename T, int D, int MODE, int MASK, bool GO>
-__global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
-#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (and has no buffer descriptor type)
+__device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
   JVPFA_BWD2_COMMON(Cfg)
@@ -375,6 +375,20 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
       }
     }
   }
+}
+#endif
+template <typename T, int D, int MODE, int MASK, bool GO>
+__global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  bwd2_dq_body<T, D, MODE, MASK, GO>(p);
+#endif
+}
+// The same code with the vector registers capped, for D = 64: together with the accumulation registers
+// the kernel then needs at most 256 registers and two workgroups share a compute unit.
+template <typename T, int D, int MODE, int MASK, bool GO>
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(160))) void bwd2_dq_kernel_2wg(const BwdParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  bwd2_dq_body<T, D, MODE, MASK, GO>(p);
 #endif
 }
 
@@ -382,9 +396,9 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
 // dk, dv (PLAIN / DUAL) or dk', dv' (TANGENT): workgroup = 128 key rows, loop over 64-query tiles
 // of Q, G (, Q', gT), G = gO (gT in TANGENT).  Scores are S = Q K^T (lane = key, registers =
 // queries) so P, dS are the B operands of dV^T += G^T P and dK^T += Q^T dS.
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stubs (and has no buffer descriptor type)
 template <typename T, int D, int MODE, int MASK, bool GO>
-__global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
-#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (and has no buffer descriptor type)
+__device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
   JVPFA_BWD2_COMMON(Cfg)
@@ -514,7 +528,11 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
     // 16(e/8) + 8g + e%8), fetched before the products that hide their latency
     T mraw_a[MASK == MASK_ADD ? 16 : 1];
     uint8_t mraw_b[MASK == MASK_BOOL ? 16 : 1];
-    if constexpr (MASK != MASK_NONE) {
+    // (where two workgroups share a compute unit, D = 64 outside the dual mode, each value is fetched where
+    // it is used: the other workgroup covers the wait and the registers stay within the cap)
+    constexpr bool MAHEAD = D > 64 || MODE == BWD_DUAL;
+    const int64_t mcol_use = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3] : 0;
+    if constexpr (MASK != MASK_NONE && MAHEAD) {
       if constexpr (!EDGE) {
         // uniform 64-bit row pointer + 32-bit lane offset: no per-lane address arithmetic per element
         // (interior tiles only run when the lane offsets fit 32 bits, see mask_small below)
@@ -615,8 +633,19 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
           const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
           float s = S[e] * sl2;
           bool keep = true;
-          if constexpr (MASK == MASK_ADD) s += (float)mraw_a[e] * LOG2E;
-          if constexpr (MASK == MASK_BOOL) keep = mraw_b[e] != 0;
+          if constexpr (MASK != MASK_NONE && !MAHEAD) {
+            if constexpr (!EDGE) {  // uniform row pointer + 32-bit lane offset, as above
+              const int64_t urow = z * pr.ms[0] + h * pr.ms[1] + (int64_t)(ih + 16 * (e / 8) + (e % 8)) * pr.ms[2];
+              if constexpr (MASK == MASK_ADD) mraw_a[0] = (reinterpret_cast<const T *>(pr.mask) + urow)[mlane];
+              if constexpr (MASK == MASK_BOOL) mraw_b[0] = (reinterpret_cast<const uint8_t *>(pr.mask) + urow)[mlane];
+            } else {
+              const int64_t off = mcol_use + (int64_t)min(qi, L - 1) * pr.ms[2];
+              if constexpr (MASK == MASK_ADD) mraw_a[0] = reinterpret_cast<const T *>(pr.mask)[off];
+              if constexpr (MASK == MASK_BOOL) mraw_b[0] = reinterpret_cast<const uint8_t *>(pr.mask)[off];
+            }
+          }
+          if constexpr (MASK == MASK_ADD) s += (float)mraw_a[MAHEAD ? e : 0] * LOG2E;
+          if constexpr (MASK == MASK_BOOL) keep = mraw_b[MAHEAD ? e : 0] != 0;
           float pv = fast_exp2(s - stat(0, e));
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
           if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
@@ -711,6 +740,20 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
       }
     }
   }
+}
+#endif
+template <typename T, int D, int MODE, int MASK, bool GO>
+__global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  bwd2_dkdv_body<T, D, MODE, MASK, GO>(p);
+#endif
+}
+// The same code with the vector registers capped, for D = 64: together with the accumulation registers
+// the kernel then needs at most 256 registers and two workgroups share a compute unit.
+template <typename T, int D, int MODE, int MASK, bool GO>
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(144))) void bwd2_dkdv_kernel_2wg(const BwdParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  bwd2_dkdv_body<T, D, MODE, MASK, GO>(p);
 #endif
 }
 
