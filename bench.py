@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
-Workload (BASELINE.json headline): bf16, B=4, H=16, L=4096, D=128, synthetic N(0,1) inputs that
+Workload (the headline benchmark configuration): bf16, B=4, H=16, L=4096, D=128, synthetic N(0,1) inputs that
 are resident in HBM before the timed region.  A step is one fused dual forward (O and O' in
 one kernel).  ``value`` is its throughput in TFLOP/s with the algorithmic FLOP count
 12 * B*H*L^2*D (six GEMM-shaped products, 2 FLOPs per multiply-add).  The same JSON line also
@@ -87,7 +87,7 @@ def cpu_baseline():
 
 
 def hvp_sweep(be, _lib):
-    """BASELINE config 5: bf16 B1 H16 D128 causal, L swept; fused dual forward + the backward of
+    """benchmark configuration 5: bf16 B1 H16 D128 causal, L swept; fused dual forward + the backward of
     sum(O' * gO') w.r.t. q, k, v (the Hessian-vector-product pattern): time and peak HBM vs L."""
     import torch
 

@@ -1,6 +1,6 @@
 """GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle.
 
-Tolerances (BASELINE north star): fp32 max-abs <= 1e-4; bf16 / fp16 relative error
+Tolerances (the stated target): fp32 max-abs <= 1e-4; bf16 / fp16 relative error
 ``max|x - ref| / max|ref| <= 2e-2``.  The oracle is the dense fp64 closed form evaluated on the
 same, already rounded, inputs (it is itself pinned against PyTorch's math SDPA under
 ``torch.func.jvp`` in ``test_oracle.py``).
@@ -39,10 +39,10 @@ def _mask(mode, Z, H, L, dtype, seed=1):
     g = torch.Generator().manual_seed(seed)
     if mode in ("none", "causal"):
         return None
-    if mode == "keypad":  # BASELINE config 4(a): per-batch valid length uniform in [L/2, L]
+    if mode == "keypad":  # benchmark configuration 4(a): per-batch valid length uniform in [L/2, L]
         lens = torch.randint(L // 2, L + 1, (Z,), generator=g)
         return (torch.arange(L)[None, :] < lens[:, None]).view(Z, 1, 1, L)
-    if mode == "bias":  # BASELINE config 4(b)
+    if mode == "bias":  # benchmark configuration 4(b)
         return torch.randn(Z, H, L, L, generator=g).to(dtype)
     if mode == "bool_full":  # the reference's test masks: random, keep-probability 0.1 (test file :334-363)
         m = torch.rand(Z, H, L, L, generator=g) > 0.9
@@ -187,7 +187,7 @@ def test_plain_forward_and_first_order_backward(dt, mode):
 
 
 def test_small_tangents_config2_shape_slice():
-    # BASELINE config 2 statistics (tangents ~ N(0, 0.1^2)) on a slice of its shape
+    # benchmark configuration 2 statistics (tangents ~ N(0, 0.1^2)) on a slice of its shape
     _run_case(1, 4, 512, 64, torch.bfloat16, "none", tangent_std=0.1)
 
 

@@ -1,4 +1,4 @@
-"""GPU tests of the Python surface (``attention``, ``JVPAttn.fwd_dual``) and of the BASELINE
+"""GPU tests of the Python surface (``attention``, ``JVPAttn.fwd_dual``) and of the benchmark
 configurations at their full sizes.
 
 Small shapes are compared with the fp64 oracle directly.  At full size one (z, h) slab is compared
@@ -94,7 +94,7 @@ def test_plain_attention_autograd_and_apply_tuple():
 
 
 def test_config2_dense_bf16_full_size_properties():
-    """BASELINE config 2: bf16 B4 H16 L2048 D64, tangents ~ N(0, 0.1^2), no mask."""
+    """benchmark configuration 2: bf16 B4 H16 L2048 D64, tangents ~ N(0, 0.1^2), no mask."""
     from jvp_flash_attention_amd import _lib, attention
 
     be = _lib.backend()
@@ -133,7 +133,7 @@ def test_config2_dense_bf16_full_size_properties():
 
 
 def test_config3_causal_long_full_size_properties():
-    """BASELINE config 3: fp16 B2 H32 L4096 D128 causal, and the headline bf16 B4 H16 L4096 D128."""
+    """benchmark configuration 3: fp16 B2 H32 L4096 D128 causal, and the headline bf16 B4 H16 L4096 D128."""
     from jvp_flash_attention_amd import _lib
 
     be = _lib.backend()
@@ -163,7 +163,7 @@ def test_config3_causal_long_full_size_properties():
 
 
 def test_config4_mask_modes_fp32_full_size():
-    """BASELINE config 4: fp32 B4 H8 L1024 D64; (a) key padding [B,1,1,L], (b) additive bias [B,H,L,L]."""
+    """benchmark configuration 4: fp32 B4 H8 L1024 D64; (a) key padding [B,1,1,L], (b) additive bias [B,H,L,L]."""
     from jvp_flash_attention_amd import _lib
 
     be = _lib.backend()
@@ -197,7 +197,7 @@ def test_config4_mask_modes_fp32_full_size():
 
 
 def test_config5_hvp_memory_is_linear_in_sequence_length():
-    """BASELINE config 5 at two lengths: peak memory of fwd_dual + backward grows like L, not L^2."""
+    """benchmark configuration 5 at two lengths: peak memory of fwd_dual + backward grows like L, not L^2."""
     from jvp_flash_attention_amd import JVPAttn
 
     def peak(L):

@@ -177,7 +177,7 @@ def test_tiled_matches_dense(mode, L, bm, bn):
 
 
 def test_config1_cpu_plumbing_fp32():
-    """BASELINE config 1: fp32 B2 H4 L128 D64, seed 0, N(0,1); SDPA route vs tiled restatement."""
+    """benchmark configuration 1: fp32 B2 H4 L128 D64, seed 0, N(0,1); SDPA route vs tiled restatement."""
     g = torch.Generator().manual_seed(0)
     q, k, v, qt, kt, vt, go, gt = [torch.randn(2, 4, 128, 64, generator=g) for _ in range(8)]
     o_ref, ot_ref, grads = sdpa_jvp.forward_backward(q, k, v, qt, kt, vt, go, gt)
