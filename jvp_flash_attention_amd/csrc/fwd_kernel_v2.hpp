@@ -239,6 +239,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   // which live in the matrix-core accumulation registers, are touched by VALU code only on the few
   // tiles where the running maximum really grows.  O = acc / l is unchanged by the choice of m_i.
   constexpr float RESCALE_TAU = 8.f;
+  MaskAhead<T, MASK> mcur[2][2], mnext[2][2];  // mask values of this tile and the next: [half tile][16-key group]
   const int klim = min(pr.causal ? qrow : 0x7fffffff, L - 1);  // keys above this index are masked
   // EDGE: the half tile may cross the causal diagonal or the end of the sequence, the scale may be
   // negative, or the mask rows are not aligned for vector fetches
@@ -275,16 +276,11 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     // score tiles in ordinary vector registers, written by matrix instructions whose B operand (Q, Q')
     // is resident in the accumulation register file
     f32x16 S, Sp;
-    // mask values of this half tile, fetched before the score products that hide their latency
+    // mask values of this half tile: fetched a whole tile earlier (see tile() below)
     MaskAhead<T, MASK> mah[2];
     if constexpr (MASK != MASK_NONE) {
-      if (!EDGE || (mask_al && jh + 32 <= L)) {  // aligned rows, all 32 keys exist: one vector load per 8 keys
-        mah[0] = mask_fetch8<T, MASK>(pr, mrow, jh + 8 * g);
-        mah[1] = mask_fetch8<T, MASK>(pr, mrow, jh + 16 + 8 * g);
-      } else {
-        mah[0] = mask_fetch8_any<T, MASK>(pr, mrow, jh + 8 * g);
-        mah[1] = mask_fetch8_any<T, MASK>(pr, mrow, jh + 16 + 8 * g);
-      }
+      mah[0] = mcur[HB][0];
+      mah[1] = mcur[HB][1];
     }
     static_for<(PD < KK ? PD : KK)>([&](auto kkc) { issue_k(kkc); });
     static_for<KK>([&](auto kkc) {
@@ -400,6 +396,21 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     JVPFA_STAMP(7);
   };
 
+  // Mask values travel from HBM or the far caches, further than one phase of matrix products hides:
+  // those of tile t+1 are requested at the top of tile t.  [half tile][16-key group] of a tile.
+  auto fetch_masks = [&](int tn) {
+    if constexpr (MASK != MASK_NONE) {
+      const int jn = tn * BN;
+      if (mask_al && jn + BN <= L) {  // aligned rows, all 64 keys exist: one vector load per 8 keys
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mnext[i / 2][i % 2] = mask_fetch8<T, MASK>(pr, mrow, jn + 16 * i + 8 * g);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mnext[i / 2][i % 2] = mask_fetch8_any<T, MASK>(pr, mrow, jn + 16 * i + 8 * g);
+      }
+    }
+  };
+  fetch_masks(0);
   issue_loads(0, 0);
   auto tile = [&](int t, auto EDGEc) {
     const int j0 = t * BN;
@@ -409,6 +420,11 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     JVPFA_STAMP(2);
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
     JVPFA_STAMP(3);
+    if constexpr (MASK != MASK_NONE) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mcur[i / 2][i % 2] = mnext[i / 2][i % 2];
+      fetch_masks(min(t + 1, ntiles - 1));
+    }
     prepare_loads(stage ^ 1, j0 + BN, t + 1 < ntiles);
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
     half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, j0);
