@@ -210,6 +210,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
     }
   };
 
+  MaskAhead<T, MASK> mcur[2][2], mnext[2][2];  // mask values of this tile and the next: [half tile][16-key group]
   // EDGE: the half tile may cross the causal diagonal or the end of the sequence
   auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, int jh) {
     constexpr int HB = decltype(HBc)::value;
@@ -228,16 +229,11 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
       }
     };
     constexpr int NRN = DUAL ? 4 : 2;
-    // mask values of this half tile, fetched before the products that hide their latency
+    // mask values of this half tile: requested a whole tile earlier (see tile() below)
     MaskAhead<T, MASK> mah[2];
     if constexpr (MASK != MASK_NONE) {
-      if (!EDGE || (mask_al && jh + 32 <= L)) {  // aligned rows, all 32 keys exist: one vector load per 8 keys
-        mah[0] = mask_fetch8<T, MASK>(pr, mrow, jh + 8 * g);
-        mah[1] = mask_fetch8<T, MASK>(pr, mrow, jh + 16 + 8 * g);
-      } else {
-        mah[0] = mask_fetch8_any<T, MASK>(pr, mrow, jh + 8 * g);
-        mah[1] = mask_fetch8_any<T, MASK>(pr, mrow, jh + 16 + 8 * g);
-      }
+      mah[0] = mcur[HB][0];
+      mah[1] = mcur[HB][1];
     }
     // tiles in ordinary vector registers; in DUAL, dP also collects V' gT^T (the B term)
     f32x16 S, dP, Sp, At;
@@ -338,6 +334,21 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
     });
   };
 
+  // Mask values travel from HBM or the far caches, further than one phase of matrix products hides:
+  // those of tile t+1 are requested at the top of tile t.
+  auto fetch_masks = [&](int tn) {
+    if constexpr (MASK != MASK_NONE) {
+      const int jn = tn * BT;
+      if (mask_al && jn + BT <= L) {  // aligned rows, all 64 keys exist: one vector load per 8 keys
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mnext[i / 2][i % 2] = mask_fetch8<T, MASK>(pr, mrow, jn + 16 * i + 8 * g);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mnext[i / 2][i % 2] = mask_fetch8_any<T, MASK>(pr, mrow, jn + 16 * i + 8 * g);
+      }
+    }
+  };
+  fetch_masks(0);
   prepare_loads(0, 0, true);
   static_for<NLOAD>([&](auto pc) { load_piece(pc); });
   auto tile = [&](int t, auto EDGEc) {
@@ -345,6 +356,11 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
+    if constexpr (MASK != MASK_NONE) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mcur[i / 2][i % 2] = mnext[i / 2][i % 2];
+      fetch_masks(min(t + 1, ntiles - 1));
+    }
     prepare_loads(stage ^ 1, j0 + BT, t + 1 < ntiles);
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
     half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, j0);
@@ -504,6 +520,36 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   };
 
   // EDGE: the half tile may cross the causal diagonal or the end of the sequence
+  // Mask values of the half tile that starts at query ihn, for this lane's key.  They travel from HBM or
+  // the far caches, so they are requested a whole half tile before their use.  (Where two workgroups
+  // share a compute unit, D = 64 outside the dual mode, each value is instead fetched where it is used:
+  // the other workgroup covers the wait and the registers stay within the cap.)
+  constexpr bool MAHEAD = D > 64 || MODE == BWD_DUAL;
+  T mnext_a[MASK == MASK_ADD ? 16 : 1];
+  uint8_t mnext_b[MASK == MASK_BOOL ? 16 : 1];
+  auto fetch_mask_half = [&](int ihn) {
+    if constexpr (MASK != MASK_NONE) {
+      if (mask_small && ihn + 32 <= L) {
+        // uniform 64-bit row pointer + 32-bit lane offset: no per-lane address arithmetic per element
+        const int64_t mrow0 = z * pr.ms[0] + h * pr.ms[1];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int64_t urow = mrow0 + (int64_t)(ihn + 16 * (e / 8) + (e % 8)) * pr.ms[2];
+          if constexpr (MASK == MASK_ADD) mnext_a[e] = (reinterpret_cast<const T *>(pr.mask) + urow)[mlane];
+          if constexpr (MASK == MASK_BOOL) mnext_b[e] = (reinterpret_cast<const uint8_t *>(pr.mask) + urow)[mlane];
+        }
+      } else {  // rows past the end are read from the last row (their scores are masked by index)
+        const int64_t mcol = z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int qi = ihn + 16 * (e / 8) + 8 * g + (e % 8);
+          const int64_t off = mcol + (int64_t)min(qi, L - 1) * pr.ms[2];
+          if constexpr (MASK == MASK_ADD) mnext_a[e] = reinterpret_cast<const T *>(pr.mask)[off];
+          if constexpr (MASK == MASK_BOOL) mnext_b[e] = reinterpret_cast<const uint8_t *>(pr.mask)[off];
+        }
+      }
+    }
+  };
   auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih) {
     constexpr int HB = decltype(HBc)::value;
     constexpr bool EDGE = decltype(EDGEc)::value;
@@ -525,34 +571,17 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
     };
     constexpr int NRN = DUAL ? 4 : 2;
     // mask values of this lane's key for the 32 queries of the half tile (register e <-> query
-    // 16(e/8) + 8g + e%8), fetched before the products that hide their latency
+    // 16(e/8) + 8g + e%8): requested one half tile earlier (see fetch_mask_half), taken over here
     T mraw_a[MASK == MASK_ADD ? 16 : 1];
     uint8_t mraw_b[MASK == MASK_BOOL ? 16 : 1];
-    // (where two workgroups share a compute unit, D = 64 outside the dual mode, each value is fetched where
-    // it is used: the other workgroup covers the wait and the registers stay within the cap)
-    constexpr bool MAHEAD = D > 64 || MODE == BWD_DUAL;
     const int64_t mcol_use = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3] : 0;
     if constexpr (MASK != MASK_NONE && MAHEAD) {
-      if constexpr (!EDGE) {
-        // uniform 64-bit row pointer + 32-bit lane offset: no per-lane address arithmetic per element
-        // (interior tiles only run when the lane offsets fit 32 bits, see mask_small below)
-        const int64_t mrow0 = z * pr.ms[0] + h * pr.ms[1];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int64_t urow = mrow0 + (int64_t)(ih + 16 * (e / 8) + (e % 8)) * pr.ms[2];
-          if constexpr (MASK == MASK_ADD) mraw_a[e] = (reinterpret_cast<const T *>(pr.mask) + urow)[mlane];
-          if constexpr (MASK == MASK_BOOL) mraw_b[e] = (reinterpret_cast<const uint8_t *>(pr.mask) + urow)[mlane];
-        }
-      } else {
-        const int64_t mcol = z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3];
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
-          const int64_t off = mcol + (int64_t)min(qi, L - 1) * pr.ms[2];
-          if constexpr (MASK == MASK_ADD) mraw_a[e] = reinterpret_cast<const T *>(pr.mask)[off];
-          if constexpr (MASK == MASK_BOOL) mraw_b[e] = reinterpret_cast<const uint8_t *>(pr.mask)[off];
-        }
+      for (int e = 0; e < 16; ++e) {
+        if constexpr (MASK == MASK_ADD) mraw_a[e] = mnext_a[e];
+        if constexpr (MASK == MASK_BOOL) mraw_b[e] = mnext_b[e];
       }
+      fetch_mask_half(ih + 32);
     }
     // tiles in ordinary vector registers; in DUAL, dP also collects gT V'^T (the B term)
     f32x16 S, dP, Sp, At;
@@ -696,6 +725,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
     });
   };
 
+  if constexpr (MASK != MASK_NONE && MAHEAD) fetch_mask_half(istart);
   prepare_loads(0, istart, true);
   static_for<NLOAD>([&](auto pc) { load_piece(pc); });
   load_stats();
