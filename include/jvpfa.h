@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define JVPFA_ABI_VERSION 2
+#define JVPFA_ABI_VERSION 3
 
 enum jvpfa_dtype { JVPFA_BF16 = 0, JVPFA_FP16 = 1, JVPFA_FP32 = 2 };
 
@@ -41,7 +41,7 @@ enum jvpfa_status {
   JVPFA_E_ALIGN = -4,     /* a tensor pointer is not 16-byte aligned */
   JVPFA_E_CONFLICT = -5,  /* causal together with a mask (JA:2380-2381 raises ValueError) */
   JVPFA_E_LAUNCH = -6,    /* hipGetLastError() reported a launch failure */
-  JVPFA_E_ABI = -7        /* struct_size is neither this version's nor version 1's */
+  JVPFA_E_ABI = -7        /* struct_size is neither this version's nor an earlier version's */
 };
 
 /* Shape, numeric type and masking shared by forward and backward. */
@@ -80,6 +80,11 @@ typedef struct jvpfa_fwd_args {
    * z; key tiles past the limit are then skipped instead of read and masked.  No counterpart in the
    * reference, which reads the full (Z,H,L,L) mask (JA:2383-2388).  Ignored without a mask. */
   const int32_t *key_limit;
+  /* since version 3 (a caller may pass the version-2 size, which ends before this field):
+   * optional lists of the key tiles that hold an attended entry, written by jvpfa_mask_tiles() for
+   * this same mask, or NULL.  Tiles not listed are skipped instead of read and masked.  When set,
+   * key_limit is ignored.  Ignored without a mask. */
+  const int32_t *tiles_q;
 } jvpfa_fwd_args;
 
 int jvpfa_fwd(const jvpfa_fwd_args *args, void *hip_stream);
@@ -111,11 +116,31 @@ typedef struct jvpfa_bwd_args {
   void *dqt, *dkt, *dvt;
   void *workspace;
   const int32_t *key_limit; /* since version 2: as in jvpfa_fwd_args */
+  const int32_t *tiles_q;   /* since version 3: as in jvpfa_fwd_args (used by the dq kernels) */
+  const int32_t *tiles_k;   /* since version 3: the other list of jvpfa_mask_tiles() (dk/dv kernels);
+                               tiles_q and tiles_k are both NULL or both set */
 } jvpfa_bwd_args;
 
 int jvpfa_bwd(const jvpfa_bwd_args *args, void *hip_stream);
 
 size_t jvpfa_bwd_workspace_bytes(int32_t Z, int32_t H, int32_t L);
+
+/*
+ * Tile lists of a mask: which 64-wide tiles hold at least one attended entry (boolean: nonzero;
+ * additive: anything but -inf).  The kernels then visit only those; a mask that is block-diagonal,
+ * banded or padded on both axes costs time in proportion to its attended area.  No counterpart in
+ * the reference, which visits every tile of the materialised (Z,H,L,L) mask (JA:2383-2388).
+ *   tiles_q  for every mask plane and block of 128 query rows: the 64-key tiles to visit
+ *   tiles_k  for every mask plane and block of 128 keys: the 64-query tiles to visit
+ * Either may be NULL (not both): the forward needs tiles_q only.
+ * A mask plane is a (z, h) pair, with one plane along an axis whose mask stride is 0.  Each list
+ * is 1 + ceil(L/64) int32 values: the count (at least 1), then the tile indices in ascending
+ * order.  Both buffers are jvpfa_mask_tiles_bytes(p) bytes of device memory, 4-byte aligned.  The
+ * lists describe the mask's contents: rebuild them when those change.  Only p->Z, H, L, dtype,
+ * mask_kind, mask and mask_stride are read.
+ */
+size_t jvpfa_mask_tiles_bytes(const jvpfa_problem *p);
+int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t *tiles_q, int32_t *tiles_k, void *hip_stream);
 
 /* JVPFA_ABI_VERSION of the loaded library. */
 int jvpfa_abi_version(void);

@@ -14,10 +14,11 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libjvpfa.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
-EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_bwd_workspace_bytes", "jvpfa_abi_version", "jvpfa_error_string")
+EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_bwd_workspace_bytes", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
+           "jvpfa_abi_version", "jvpfa_error_string")
 
 
 class Problem(C.Structure):
@@ -39,6 +40,7 @@ class FwdArgs(C.Structure):
         ("o", C.c_void_p), ("ot", C.c_void_p),
         ("M", C.c_void_p), ("mu", C.c_void_p),
         ("key_limit", C.c_void_p),
+        ("tiles_q", C.c_void_p),
     ]
 
 
@@ -55,6 +57,7 @@ class BwdArgs(C.Structure):
         ("dqt", C.c_void_p), ("dkt", C.c_void_p), ("dvt", C.c_void_p),
         ("workspace", C.c_void_p),
         ("key_limit", C.c_void_p),
+        ("tiles_q", C.c_void_p), ("tiles_k", C.c_void_p),
     ]
 
 
@@ -77,6 +80,10 @@ def load() -> C.CDLL:
         lib.jvpfa_bwd.restype = C.c_int
         lib.jvpfa_bwd_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         lib.jvpfa_bwd_workspace_bytes.restype = C.c_size_t
+        lib.jvpfa_mask_tiles_bytes.argtypes = [C.POINTER(Problem)]
+        lib.jvpfa_mask_tiles_bytes.restype = C.c_size_t
+        lib.jvpfa_mask_tiles.argtypes = [C.POINTER(Problem), C.c_void_p, C.c_void_p, C.c_void_p]
+        lib.jvpfa_mask_tiles.restype = C.c_int
         lib.jvpfa_abi_version.argtypes = []
         lib.jvpfa_abi_version.restype = C.c_int
         lib.jvpfa_error_string.argtypes = [C.c_int]
@@ -141,6 +148,51 @@ def key_limit_hint(mask, mask_kind, Z, L):
     return lim
 
 
+TILE_LISTS_MIN_L = 512  # below this a mask has too few tiles for skipping some to pay for the scan
+_tile_lists_enabled = True
+
+
+def set_tile_lists(enabled: bool) -> None:
+    """Switch the scan of two-dimensional masks for skippable tiles on or off (default on)."""
+    global _tile_lists_enabled
+    _tile_lists_enabled = bool(enabled)
+
+
+def tile_lists(q, mask, mask_kind, want_k):
+    """For a mask with a row per query (shape [*, *, L, L]): the lists of 64-wide tiles that hold an
+    attended entry, made on the device by ``jvpfa_mask_tiles`` -- (tiles_q, tiles_k) int32 tensors,
+    tiles_k only if ``want_k`` (the backward).  The kernels visit the listed tiles only, so block
+    diagonal, banded or doubly padded masks cost time in proportion to their attended area.
+    (None, None) for masks that are not two-dimensional, short sequences, and the element types /
+    head dims whose kernels visit every tile.  Cached on the mask tensor, keyed by its version
+    counter, so that layers and the backward reuse one scan."""
+    Z, H, L, D = q.shape
+    if (not _tile_lists_enabled or mask is None or mask_kind == MASK_NONE or L < TILE_LISTS_MIN_L
+            or q.dtype == torch.float32 or D < 64):
+        return None, None
+    if mask.dim() != 4 or mask.shape[2] != L or mask.shape[3] != L:
+        return None, None
+    cached = getattr(mask, "_jvpfa_tiles", None)
+    if cached is None or cached[0] != mask._version:
+        cached = [mask._version, None, None]
+    tq, tk = cached[1], cached[2]
+    if tq is None or (want_k and tk is None):
+        lib = load()
+        prob = make_problem(q, mask, mask_kind, False, 1.0)
+        n = lib.jvpfa_mask_tiles_bytes(C.byref(prob)) // 4
+        new_q = torch.empty(n, device=q.device, dtype=torch.int32) if tq is None else None
+        new_k = torch.empty(n, device=q.device, dtype=torch.int32) if (want_k and tk is None) else None
+        check(lib.jvpfa_mask_tiles(C.byref(prob), _ptr(new_q), _ptr(new_k), _stream(q)))
+        tq = new_q if tq is None else tq
+        tk = new_k if new_k is not None else tk
+        cached[1], cached[2] = tq, tk
+        try:
+            mask._jvpfa_tiles = cached
+        except (AttributeError, RuntimeError):
+            pass
+    return tq, (tk if want_k else None)
+
+
 def _require_gpu(*tensors):
     for t in tensors:
         if t is not None and not t.is_cuda:
@@ -178,6 +230,8 @@ class HipBackend:
         with torch.cuda.device(q.device):
             lim = key_limit_hint(mask, mask_kind, Z, L)
             a.key_limit = _ptr(lim)
+            tq, _ = tile_lists(q, mask, mask_kind, False)
+            a.tiles_q = _ptr(tq)
             check(lib.jvpfa_fwd(C.byref(a), _stream(q)))
         return o, ot, M, mu
 
@@ -205,6 +259,8 @@ class HipBackend:
         with torch.cuda.device(q.device):
             lim = key_limit_hint(mask, mask_kind, Z, L)
             a.key_limit = _ptr(lim)
+            tq, tk = tile_lists(q, mask, mask_kind, True)
+            a.tiles_q, a.tiles_k = _ptr(tq), _ptr(tk)
             check(lib.jvpfa_bwd(C.byref(a), _stream(q)))
         return dq, dk, dv, dqt, dkt, dvt
 

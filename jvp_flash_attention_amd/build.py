@@ -39,7 +39,7 @@ def units():
             for d in DIMS:
                 name = f"{kind}_{tag}_{d}"
                 out.append((name, src, [f"-DJVPFA_T={ctype}", f"-DJVPFA_D={d}", f"-DJVPFA_NAME={name}"]))
-    for api in ("api_fwd", "api_bwd"):
+    for api in ("api_fwd", "api_bwd", "mask_tiles"):
         src = os.path.join(CSRC, f"{api}.hip")
         if os.path.exists(src):
             out.append((api, src, []))

@@ -23,9 +23,13 @@ inline int check_problem(const jvpfa_problem &p) {
   return JVPFA_OK;
 }
 
-inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit) {
+inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit, const int32_t *tiles_q,
+                          const int32_t *tiles_k) {
   Problem r;
-  r.klimit = p.mask_kind == JVPFA_MASK_NONE ? nullptr : key_limit;
+  const bool masked = p.mask_kind != JVPFA_MASK_NONE;
+  r.tiles_q = masked ? tiles_q : nullptr;
+  r.tiles_k = masked ? tiles_k : nullptr;
+  r.klimit = (masked && !r.tiles_q && !r.tiles_k) ? key_limit : nullptr;
   r.Z = p.Z;
   r.H = p.H;
   r.L = p.L;

@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
   const int L = pr.L;
   const int nqb = (L + BWD_BLK - 1) / BWD_BLK;
   const int total = nqb * pr.Z * pr.H;
-  const int id = xcd_remap(blockIdx.x, total);
+  const int id = xcd_remap(blockIdx.x, nqb, pr.Z * pr.H);
   const int zh = id / nqb;
   const int qb = pr.causal ? nqb - 1 - id % nqb : id % nqb;
   const int z = zh / pr.H, h = zh % pr.H;
@@ -275,7 +275,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
   const int L = pr.L;
   const int nkb = (L + BWD_BLK - 1) / BWD_BLK;
   const int total = nkb * pr.Z * pr.H;
-  const int id = xcd_remap(blockIdx.x, total);
+  const int id = xcd_remap(blockIdx.x, nkb, pr.Z * pr.H);
   const int zh = id / nkb;
   const int kb = id % nkb;  // causal: the first key blocks have the longest query loops
   const int z = zh / pr.H, h = zh % pr.H;

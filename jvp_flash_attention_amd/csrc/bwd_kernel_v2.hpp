@@ -69,7 +69,7 @@ template <int N> __device__ __forceinline__ void lds_wait4(u32x4 &a, u32x4 &b, u
   const int L = pr.L;                                                                                               \
   const int nblk = (L + Cfg::BLK - 1) / Cfg::BLK;                                                                   \
   const int total = nblk * pr.Z * pr.H;                                                                             \
-  const int id = xcd_remap(blockIdx.x, total);                                                                      \
+  const int id = xcd_remap(blockIdx.x, nblk, pr.Z * pr.H);                                                                      \
   const int zh = id / nblk;                                                                                         \
   const int z = zh / pr.H, h = zh % pr.H;                                                                           \
   const int tid = threadIdx.x;                                                                                      \
@@ -185,7 +185,16 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   if constexpr (MASK != MASK_NONE) {  // key tiles that the caller's hint declares fully masked are not visited
     if (pr.klimit) kend = min(kend, max(pr.klimit[z], 1));
   }
-  const int ntiles = (kend + BT - 1) / BT;
+  // Key tiles visited: 0 .. ceil(kend/BT)-1, or the caller's list of the tiles of this query block
+  // that hold an attended entry (ascending); tile_at(i) is the i-th one.
+  const int *tlist = nullptr;
+  if constexpr (MASK != MASK_NONE) {
+    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
+  }
+  const int ntiles = tlist ? tlist[0] : (kend + BT - 1) / BT;
+  // List elements are requested a tile ahead, unconditionally (from a harmless address when there is
+  // no list: a branch around the read would split the tile loop's straight-line body).
+  auto list_slot = [&](int i) { return tlist ? tlist + 1 + i : reinterpret_cast<const int *>(p.q); };
   // tile slots in a stage: 0 K, 1 V, 2 K', 3 V'
   constexpr int NLOAD = IPW * Cfg::NTILE;
   constexpr int NACC = DUAL ? 2 : 1;            // operand tensors of the accumulation (K, K')
@@ -348,25 +357,35 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
       }
     }
   };
-  fetch_masks(0);
-  prepare_loads(0, 0, true);
+  // the tile of this step and of the next
+  int tcur = tlist ? tlist[1] : 0, tnext = tlist ? tlist[1 + min(1, ntiles - 1)] : min(1, ntiles - 1);
+  fetch_masks(tcur);
+  prepare_loads(0, tcur * BT, true);
   static_for<NLOAD>([&](auto pc) { load_piece(pc); });
   auto tile = [&](int t, auto EDGEc) {
-    const int j0 = t * BT;
+    const int j0 = tcur * BT;
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
+    int tnext2 = min(t + 2, ntiles - 1), tahead = 0;
     if constexpr (MASK != MASK_NONE) {
+      tahead = list_request(list_slot(tnext2));
 #pragma unroll
       for (int i = 0; i < 4; ++i) mcur[i / 2][i % 2] = mnext[i / 2][i % 2];
-      fetch_masks(min(t + 1, ntiles - 1));
+      fetch_masks(tnext);
     }
-    prepare_loads(stage ^ 1, j0 + BT, t + 1 < ntiles);
+    prepare_loads(stage ^ 1, tnext * BT, t + 1 < ntiles);
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
     half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, j0);
     // always both halves: a half past the last key or past the diagonal contributes exact zeros, and a
     // branch here would make the accumulators change register file around it
     half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, j0 + 32);
+    if constexpr (MASK != MASK_NONE) {
+      const int listed = list_take(tahead);
+      tnext2 = tlist ? listed : tnext2;
+    }
+    tcur = tnext;
+    tnext = tnext2;
   };
   // Tiles that cross the diagonal or the end of the sequence are the last ones; they get a loop of their
   // own so that the common tile carries no limit tests.  (q0 is a multiple of the tile size.)
@@ -374,7 +393,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   if (pr.causal) t_edge = min(t_edge, q0 / BT);
   if (MASK != MASK_NONE && !mask_al) t_edge = 0;  // interior tiles fetch mask rows with aligned vector loads
   int t = 0;
-  for (; t < min(t_edge, ntiles); ++t) tile(t, std::false_type{});
+  for (; t < ntiles && tcur < t_edge; ++t) tile(t, std::false_type{});
   for (; t < ntiles; ++t) tile(t, std::true_type{});
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the redirected loads of the last iteration must not outlive the kernel
 
@@ -484,7 +503,17 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
                           DUAL ? p.a + srow : nullptr, DUAL ? p.d2 + srow : nullptr};
 
   const int istart = pr.causal ? (k0 / BT) * BT : 0;
-  const int ntiles = (L - istart + BT - 1) / BT;
+  // Query tiles visited, counted from istart: 0 .. ntiles-1, or the caller's list of the tiles of this
+  // key block that hold an attended entry (ascending; only with a mask, where istart is 0);
+  // tile_at(i) is the i-th one.
+  const int *tlist = nullptr;
+  if constexpr (MASK != MASK_NONE) {
+    if (pr.tiles_k) tlist = pr.tiles_k + tile_list_offset(pr, z, h, kb);
+  }
+  const int ntiles = tlist ? tlist[0] : (L - istart + BT - 1) / BT;
+  // List elements are requested a tile ahead, unconditionally (from a harmless address when there is
+  // no list: a branch around the read would split the tile loop's straight-line body).
+  auto list_slot = [&](int i) { return tlist ? tlist + 1 + i : reinterpret_cast<const int *>(p.q); };
   constexpr int NLOAD = IPW * Cfg::NTILE;
   constexpr int NPV = 2 * DB;  // accumulation steps of a half: (query chunk c, d-block db)
   constexpr int NSTEP = 2 * (KK + NPV);
@@ -550,7 +579,8 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
       }
     }
   };
-  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih) {
+  // ih: first query of this half tile; ihn: of the half tile that follows it
+  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn) {
     constexpr int HB = decltype(HBc)::value;
     constexpr bool EDGE = decltype(EDGEc)::value;
     constexpr int RO = HB * 32 * ROWB;
@@ -581,7 +611,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
         if constexpr (MASK == MASK_ADD) mraw_a[e] = mnext_a[e];
         if constexpr (MASK == MASK_BOOL) mraw_b[e] = mnext_b[e];
       }
-      fetch_mask_half(ih + 32);
+      fetch_mask_half(ihn);
     }
     // tiles in ordinary vector registers; in DUAL, dP also collects gT V'^T (the B term)
     f32x16 S, dP, Sp, At;
@@ -725,30 +755,40 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
     });
   };
 
-  if constexpr (MASK != MASK_NONE && MAHEAD) fetch_mask_half(istart);
-  prepare_loads(0, istart, true);
+  // the tile of this step and of the next
+  int tcur = tlist ? tlist[1] : 0, tnext = tlist ? tlist[1 + min(1, ntiles - 1)] : min(1, ntiles - 1);
+  if constexpr (MASK != MASK_NONE && MAHEAD) fetch_mask_half(istart + tcur * BT);
+  prepare_loads(0, istart + tcur * BT, true);
   static_for<NLOAD>([&](auto pc) { load_piece(pc); });
   load_stats();
   auto tile = [&](int t, auto EDGEc) {
-    const int i0 = istart + t * BT;
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    prepare_loads(stage ^ 1, i0 + BT, t + 1 < ntiles);
+    int tnext2 = min(t + 2, ntiles - 1), tahead = 0;
+    if constexpr (MASK != MASK_NONE) tahead = list_request(list_slot(tnext2));
+    const int i0 = istart + tcur * BT, i0n = istart + tnext * BT;
+    prepare_loads(stage ^ 1, i0n, t + 1 < ntiles);
     load_stats();
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB, sstat = stat0 + stage * Cfg::STATB;
-    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, sstat, i0);
+    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, sstat, i0, i0 + 32);
     // always both halves: a half past the last query contributes exact zeros, and a branch here would
     // make the accumulators change register file around it
-    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32);
+    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32, i0n);
+    if constexpr (MASK != MASK_NONE) {
+      const int listed = list_take(tahead);
+      tnext2 = tlist ? listed : tnext2;
+    }
+    tcur = tnext;
+    tnext = tnext2;
   };
   // Query tiles that cross the diagonal come first (causal), those that cross the end of the sequence
   // last; the tiles in between run without limit tests.
   const int t_diag = pr.causal ? min(ntiles, (k0 + Cfg::BLK - istart + BT - 1) / BT) : 0;
-  const int t_end = mask_small ? max(t_diag, min(ntiles, (L - istart) / BT)) : t_diag;
+  const int t_end = mask_small ? max(t_diag, (L - istart) / BT) : t_diag;  // first tile that crosses the end
   int t = 0;
   for (; t < t_diag; ++t) tile(t, std::true_type{});
-  for (; t < t_end; ++t) tile(t, std::false_type{});
+  for (; t < ntiles && tcur < t_end; ++t) tile(t, std::false_type{});
   for (; t < ntiles; ++t) tile(t, std::true_type{});
   __builtin_amdgcn_s_waitcnt(0x0F70);
 

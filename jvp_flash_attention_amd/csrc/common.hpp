@@ -134,12 +134,20 @@ __device__ __forceinline__ void copy_rows_transposed(T *dst, int ld, const T *sr
   }
 }
 
-// Blocks are dealt round-robin to the 8 XCDs (each with its own L2).  Re-deal so that each XCD
-// gets a contiguous range of logical ids: blocks that share one head's K/V then share an L2.
-__device__ __forceinline__ int xcd_remap(int bid, int total) {
+// Blocks are dealt round-robin to the 8 XCDs (each with its own L2).  Re-deal them so that the blocks
+// of one head (which share its K/V) land on one XCD and are worked on there at about the same time:
+// XCD x takes heads x, x+8, x+16, ... one after another.  Dealing heads round-robin rather than in
+// contiguous ranges matters when the work per head varies with the batch entry (padded batches): every
+// XCD then gets its share of every batch entry.  Returns head * per_head + block.
+__device__ __forceinline__ int xcd_remap(int bid, int per_head, int heads) {
   constexpr int NXCD = 8;
+  const int total = per_head * heads;
+  if (heads % NXCD == 0) {
+    const int x = bid % NXCD, j = bid / NXCD;  // j: arrival order within XCD x
+    return ((j / per_head) * NXCD + x) * per_head + j % per_head;
+  }
   if (total % NXCD != 0) return bid;
-  return (bid % NXCD) * (total / NXCD) + bid / NXCD;
+  return (bid % NXCD) * (total / NXCD) + bid / NXCD;  // contiguous ranges of blocks
 }
 
 // Store 8 consecutive elements of type T converted from fp32.

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
   const int L = pr.L;
   const int nqb = (L + Cfg::BM - 1) / Cfg::BM;
   const int total = nqb * pr.Z * pr.H;
-  const int id = xcd_remap(blockIdx.x, total);
+  const int id = xcd_remap(blockIdx.x, nqb, pr.Z * pr.H);
   const int zh = id / nqb;
   // causal: the last query blocks have the longest key loops, start them first
   const int qb = pr.causal ? nqb - 1 - id % nqb : id % nqb;

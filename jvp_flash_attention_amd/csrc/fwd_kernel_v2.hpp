@@ -66,7 +66,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   const int L = pr.L;
   const int nqb = (L + Cfg::BM - 1) / Cfg::BM;
   const int total = nqb * pr.Z * pr.H;
-  const int id = xcd_remap(blockIdx.x, total);
+  const int id = xcd_remap(blockIdx.x, nqb, pr.Z * pr.H);
   const int zh = id / nqb;
   const int qb = pr.causal ? nqb - 1 - id % nqb : id % nqb;
   const int z = zh / pr.H, h = zh % pr.H;
@@ -190,7 +190,17 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     if (pr.klimit) kend = min(L, max(pr.klimit[z], 1));
   }
   if (pr.causal) kend = min(L, q0 + Cfg::BM);
-  const int ntiles = (kend + BN - 1) / BN;
+  // Tiles visited: 0 .. ceil(kend/BN)-1, or the caller's list of the tiles of this query block that
+  // hold an attended entry (ascending; fully masked tiles contribute exact zeros, so leaving them
+  // out changes nothing).  tile_at(i) is the i-th tile visited.
+  const int *tlist = nullptr;
+  if constexpr (MASK != MASK_NONE) {
+    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
+  }
+  const int ntiles = tlist ? tlist[0] : (kend + BN - 1) / BN;
+  // List elements are requested a tile ahead, unconditionally (from a harmless address when there is
+  // no list: a branch around the read would split the tile loop's straight-line body).
+  auto list_slot = [&](int i) { return tlist ? tlist + 1 + i : reinterpret_cast<const int *>(p.q); };
 
   // The loads of the next tile are not issued in one burst (the vector-memory queue would back up
   // and stall this wave for longer than a whole GEMM phase) but one instruction at a time, spread
@@ -410,27 +420,37 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       }
     }
   };
-  fetch_masks(0);
-  issue_loads(0, 0);
+  // the tile of this step and of the next
+  int tcur = tlist ? tlist[1] : 0, tnext = tlist ? tlist[1 + min(1, ntiles - 1)] : min(1, ntiles - 1);
+  fetch_masks(tcur);
+  issue_loads(0, tcur * BN);
   auto tile = [&](int t, auto EDGEc) {
-    const int j0 = t * BN;
+    const int j0 = tcur * BN;
     const int stage = t & 1;
     JVPFA_STAMP(1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
     JVPFA_STAMP(2);
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
     JVPFA_STAMP(3);
+    int tnext2 = min(t + 2, ntiles - 1), tahead = 0;
     if constexpr (MASK != MASK_NONE) {
+      tahead = list_request(list_slot(tnext2));
 #pragma unroll
       for (int i = 0; i < 4; ++i) mcur[i / 2][i % 2] = mnext[i / 2][i % 2];
-      fetch_masks(min(t + 1, ntiles - 1));
+      fetch_masks(tnext);
     }
-    prepare_loads(stage ^ 1, j0 + BN, t + 1 < ntiles);
+    prepare_loads(stage ^ 1, tnext * BN, t + 1 < ntiles);
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB;
     half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, j0);
     // always both halves: a half past the last key is fully masked and contributes exact zeros, and a
     // branch here would make the accumulators change register file around it
     half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, j0 + 32);
+    if constexpr (MASK != MASK_NONE) {
+      const int listed = list_take(tahead);
+      tnext2 = tlist ? listed : tnext2;
+    }
+    tcur = tnext;
+    tnext = tnext2;
   };
   // Tiles that need the general treatment are the last ones; they get a loop of their own so that the
   // common tile carries no limit tests.  (q0 is a multiple of the tile size.)
@@ -438,7 +458,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   if (pr.causal) t_edge = min(t_edge, q0 / BN);
   if (!(sl2 > 0.f) || (MASK != MASK_NONE && !mask_al)) t_edge = 0;
   int t = 0;
-  for (; t < min(t_edge, ntiles); ++t) tile(t, std::false_type{});
+  for (; t < ntiles && tcur < t_edge; ++t) tile(t, std::false_type{});
   for (; t < ntiles; ++t) tile(t, std::true_type{});
 
   // ---- epilogue ---------------------------------------------------------------------------------

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   const int L = pr.L;
   const int nqb = (L + Cfg::BM - 1) / Cfg::BM;
   const int total = nqb * pr.Z * pr.H;
-  const int id = xcd_remap(blockIdx.x, total);
+  const int id = xcd_remap(blockIdx.x, nqb, pr.Z * pr.H);
   const int zh = id / nqb;
   const int qb = pr.causal ? nqb - 1 - id % nqb : id % nqb;
 

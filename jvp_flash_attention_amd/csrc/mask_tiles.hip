@@ -1,0 +1,118 @@
+// C ABI: jvpfa_mask_tiles -- lists of the 64-wide tiles of a mask that hold an attended entry.
+//
+// The forward and dq kernels own 128 query rows and stream 64-key tiles; the dk/dv kernels own 128
+// keys and stream 64-query tiles.  One workgroup here walks the strip of one such owner and writes
+// the indices of the tiles worth visiting, so that the attention kernels skip the rest.  The
+// reference has nothing like it: it reads and applies the whole (Z,H,L,L) mask
+// (jvp_attention.py:2383-2388, :241-251).
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+#include "api_common.hpp"
+
+namespace jvpfa {
+
+template <typename E, bool BOOL> __device__ __forceinline__ bool attended(E x) {
+  if constexpr (BOOL) return x != 0;
+  else return (float)x != -__builtin_inff();
+}
+
+// KEYS_OWNED false: block = 128 query rows, tiles run over keys (list for forward / dq).
+// KEYS_OWNED true:  block = 128 keys, tiles run over query rows (list for dk/dv).
+// Every thread looks at 32 consecutive keys of one row of the current tile.
+template <typename E, bool BOOL, bool KEYS_OWNED>
+__global__ __launch_bounds__(256) void mask_tiles_kernel(const E *mask, int64_t s0, int64_t s1, int64_t s2,
+                                                         int64_t s3, int hm, int L, int *out) {
+  const int nblk = (L + TILE_BLOCK - 1) / TILE_BLOCK, nt = (L + TILE_W - 1) / TILE_W;
+  const int plane = blockIdx.x / nblk, blk = blockIdx.x % nblk;
+  const E *base = mask + (int64_t)(plane / hm) * s0 + (int64_t)(plane % hm) * s1;
+  int *list = out + ((size_t)plane * nblk + blk) * (size_t)(nt + 1);
+  const int tid = threadIdx.x;
+  constexpr int PARTS = KEYS_OWNED ? 4 : 2;  // 32-key pieces per row of a tile
+  const int rsub = tid / PARTS, part = tid % PARTS;
+  // 16-byte vector reads when every piece starts on a 16-byte boundary
+  constexpr int VEC = 16 / sizeof(E);
+  const bool vec_ok = s3 == 1 && (s0 % VEC) == 0 && (s1 % VEC) == 0 && (s2 % VEC) == 0 &&
+                      (reinterpret_cast<uintptr_t>(mask) % 16) == 0;
+  int count = 0;
+  for (int t = 0; t < nt; ++t) {
+    const int row = KEYS_OWNED ? t * TILE_W + rsub : blk * TILE_BLOCK + rsub;
+    const int key0 = (KEYS_OWNED ? blk * TILE_BLOCK : t * TILE_W) + 32 * part;
+    bool any = false;
+    if (row < L && key0 < L) {
+      const E *rp = base + (int64_t)row * s2;
+      if (vec_ok && key0 + 32 <= L) {
+#pragma unroll
+        for (int v = 0; v < 32 / VEC; ++v) {
+          const uint4 w = *reinterpret_cast<const uint4 *>(rp + key0 + v * VEC);
+          if constexpr (BOOL) {
+            any |= (w.x | w.y | w.z | w.w) != 0;
+          } else {
+            E e[VEC];
+            __builtin_memcpy(e, &w, 16);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) any |= attended<E, BOOL>(e[i]);
+          }
+        }
+      } else {
+        const int n = min(32, L - key0);
+        for (int i = 0; i < n; ++i) any |= attended<E, BOOL>(rp[(int64_t)(key0 + i) * s3]);
+      }
+    }
+    if (__syncthreads_or(any)) {  // uniform over the workgroup
+      if (tid == 0) list[1 + count] = t;
+      ++count;
+    }
+  }
+  if (tid == 0) {
+    // a strip without any attended entry still visits one (fully masked) tile, which keeps its
+    // output rows defined: zeros
+    if (count == 0) list[1] = 0;
+    list[0] = count == 0 ? 1 : count;
+  }
+}
+
+template <typename E, bool BOOL>
+static int launch_both(const jvpfa_problem &p, int *tq, int *tk, hipStream_t stream) {
+  const int hm = p.mask_stride[1] ? p.H : 1, zm = p.mask_stride[0] ? p.Z : 1;
+  const int nblk = (p.L + TILE_BLOCK - 1) / TILE_BLOCK;
+  const long long blocks = (long long)zm * hm * nblk;
+  if (blocks > 0x7fffffffLL) return JVPFA_E_SHAPE;
+  const E *m = static_cast<const E *>(p.mask);
+  const int64_t *s = p.mask_stride;
+  if (tq)
+    hipLaunchKernelGGL((mask_tiles_kernel<E, BOOL, false>), dim3((unsigned)blocks), dim3(256), 0, stream, m, s[0],
+                       s[1], s[2], s[3], hm, p.L, tq);
+  if (tk)
+    hipLaunchKernelGGL((mask_tiles_kernel<E, BOOL, true>), dim3((unsigned)blocks), dim3(256), 0, stream, m, s[0],
+                       s[1], s[2], s[3], hm, p.L, tk);
+  return hipGetLastError() == hipSuccess ? JVPFA_OK : JVPFA_E_LAUNCH;
+}
+
+}  // namespace jvpfa
+
+using namespace jvpfa;
+
+extern "C" size_t jvpfa_mask_tiles_bytes(const jvpfa_problem *p) {
+  if (!p || p->Z < 1 || p->H < 1 || p->L < 1) return 0;
+  const size_t planes = (size_t)(p->mask_stride[0] ? p->Z : 1) * (p->mask_stride[1] ? p->H : 1);
+  const size_t nblk = (p->L + TILE_BLOCK - 1) / TILE_BLOCK, nt = (p->L + TILE_W - 1) / TILE_W;
+  return planes * nblk * (nt + 1) * sizeof(int32_t);
+}
+
+extern "C" int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t *tiles_q, int32_t *tiles_k, void *hip_stream) {
+  if (!p || (!tiles_q && !tiles_k)) return JVPFA_E_NULL;
+  if (p->Z < 1 || p->H < 1 || p->L < 1) return JVPFA_E_SHAPE;
+  if (p->dtype < JVPFA_BF16 || p->dtype > JVPFA_FP32) return JVPFA_E_DTYPE;
+  if (p->mask_kind != JVPFA_MASK_BOOL && p->mask_kind != JVPFA_MASK_ADD) return JVPFA_E_DTYPE;
+  if (!p->mask) return JVPFA_E_NULL;
+  for (int i = 0; i < 4; ++i)
+    if (p->mask_stride[i] < 0) return JVPFA_E_SHAPE;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  if (p->mask_kind == JVPFA_MASK_BOOL) return launch_both<uint8_t, true>(*p, tiles_q, tiles_k, stream);
+  switch (p->dtype) {
+    case JVPFA_BF16: return launch_both<__bf16, false>(*p, tiles_q, tiles_k, stream);
+    case JVPFA_FP16: return launch_both<_Float16, false>(*p, tiles_q, tiles_k, stream);
+    default: return launch_both<float, false>(*p, tiles_q, tiles_k, stream);
+  }
+}

@@ -13,7 +13,20 @@ struct Problem {
   const void *mask;
   int64_t ms[4];  // element strides (z, h, query, key)
   const int *klimit;  // per batch entry: keys at or past this index are masked by the mask (hint), or null
+  // Lists of the tiles that hold an attended entry, or null: per mask plane and 128-row block,
+  // 1 + ceil(L/64) ints (count >= 1, then ascending indices of 64-wide tiles).  tiles_q: key tiles
+  // per query block; tiles_k: query tiles per key block.
+  const int *tiles_q, *tiles_k;
 };
+
+constexpr int TILE_BLOCK = 128, TILE_W = 64;  // geometry of the tile lists
+// first element of the list of (plane of (z, h), block)
+__host__ __device__ inline size_t tile_list_offset(const Problem &pr, int z, int h, int block) {
+  const int hm = pr.ms[1] ? pr.H : 1;
+  const size_t plane = (size_t)(pr.ms[0] ? z : 0) * hm + (pr.ms[1] ? h : 0);
+  const int nblk = (pr.L + TILE_BLOCK - 1) / TILE_BLOCK, nt = (pr.L + TILE_W - 1) / TILE_W;
+  return (plane * nblk + block) * (size_t)(nt + 1);
+}
 
 struct FwdParams {
   Problem pr;

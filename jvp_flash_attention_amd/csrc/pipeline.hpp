@@ -87,6 +87,20 @@ template <int N> __device__ __forceinline__ void lds_wait(u32x2 &a, u32x2 &b, u3
   asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
 }
 
+// One int of a list in global memory, read a whole tile before it is needed.  list_request is a
+// plain load, issued where it is written (memory operations are not moved across the inline-asm
+// matrix instructions and LDS reads around it); list_take, placed where the value is first needed,
+// moves it to a scalar register.  Being inline asm it stays put as well, so the wait for the load
+// (which the compiler inserts in front of it) lands there and not in the middle of the tile, where
+// it would also wait for every older load still in flight.  p must be the same address in every
+// lane.
+__device__ __forceinline__ int list_request(const int *p) { return *p; }
+__device__ __forceinline__ int list_take(int v) {
+  int s;
+  asm volatile("v_readfirstlane_b32 %0, %1\n\ts_nop 4" : "=s"(s) : "v"(v));
+  return s;
+}
+
 // chunk swizzles (row -> xor value applied to the 16-byte chunk index)
 template <int CH> __device__ __forceinline__ int swz_k(int row) { return CH == 16 ? (row & 15) : ((row >> 1) & 7); }
 template <int CH> __device__ __forceinline__ int swz_v(int row) { return CH == 16 ? ((row & 7) << 1) : (((row >> 1) & 3) << 1); }

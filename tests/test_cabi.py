@@ -89,17 +89,68 @@ def test_forward_argument_validation_codes(kw, code):
     assert lib.jvpfa_error_string(code).decode() not in ("ok", "unknown status")
 
 
-def test_version_1_struct_sizes_are_still_accepted():
-    """A caller built against version 1 passes structs that end before key_limit."""
+def test_earlier_struct_sizes_are_still_accepted():
+    """A caller built against version 1 passes structs that end before key_limit, one built against
+    version 2 structs that end before tiles_q."""
     lib = _lib.load()
     a = _fwd_args(q=None)
-    a.struct_size = _lib.FwdArgs.key_limit.offset
-    assert lib.jvpfa_fwd(C.byref(a), None) == -1  # got past the size check, to the NULL pointer check
+    for size in (_lib.FwdArgs.key_limit.offset, _lib.FwdArgs.tiles_q.offset, C.sizeof(_lib.FwdArgs)):
+        a.struct_size = size
+        assert lib.jvpfa_fwd(C.byref(a), None) == -1  # got past the size check, to the NULL pointer check
     a.struct_size = _lib.FwdArgs.key_limit.offset - 8
     assert lib.jvpfa_fwd(C.byref(a), None) == -7
     b = _lib.BwdArgs()
-    b.struct_size = _lib.BwdArgs.key_limit.offset
     b.p.Z, b.p.H, b.p.L, b.p.D = 1, 1, 32, 64
+    for size in (_lib.BwdArgs.key_limit.offset, _lib.BwdArgs.tiles_q.offset, C.sizeof(_lib.BwdArgs)):
+        b.struct_size = size
+        assert lib.jvpfa_bwd(C.byref(b), None) == -1
+
+
+def test_tile_lists_are_only_made_for_masks_with_a_row_per_query():
+    import torch
+
+    q = torch.empty(2, 2, 1024, 64, dtype=torch.bfloat16)
+    full = torch.ones(2, 1, 1024, 1024, dtype=torch.bool)
+    cases = [
+        (q, torch.ones(2, 1, 1, 1024, dtype=torch.bool)),         # key padding: the key limit covers it
+        (q[:, :, :256], full[:, :, :256, :256]),                   # too short to pay for the scan
+        (q.float(), full),                                          # fp32 kernels visit every tile
+        (torch.empty(2, 2, 1024, 32, dtype=torch.bfloat16), full),  # so do the D = 32 kernels
+        (q, None),
+    ]
+    for qq, m in cases:
+        assert _lib.tile_lists(qq, m, _lib.MASK_BOOL if m is not None else _lib.MASK_NONE, True) == (None, None)
+    _lib.set_tile_lists(False)
+    try:
+        assert _lib.tile_lists(q, full, _lib.MASK_BOOL, True) == (None, None)
+    finally:
+        _lib.set_tile_lists(True)
+
+
+def test_mask_tile_list_sizes_and_argument_checks():
+    """Host-side part of jvpfa_mask_tiles: buffer sizes and refusals (nothing is launched)."""
+    lib = _lib.load()
+    p = _lib.Problem()
+    p.Z, p.H, p.L, p.D = 3, 4, 700, 64
+    p.dtype, p.mask_kind = 0, _lib.MASK_BOOL
+    nblk, nt = 6, 11  # ceil(700/128) blocks of ceil(700/64) + 1 ints each
+    for strides, planes in (((490000 * 4, 490000, 700, 1), 12), ((490000, 0, 700, 1), 3), ((0, 0, 700, 1), 1)):
+        p.mask_stride = (C.c_int64 * 4)(*strides)
+        assert lib.jvpfa_mask_tiles_bytes(C.byref(p)) == planes * nblk * (nt + 1) * 4
+    buf = (C.c_int32 * 16)()
+    assert lib.jvpfa_mask_tiles(C.byref(p), buf, None, None) == -1  # no mask pointer
+    p.mask = C.addressof(buf)
+    assert lib.jvpfa_mask_tiles(C.byref(p), None, None, None) == -1  # no output at all
+    p.mask_kind = _lib.MASK_NONE
+    assert lib.jvpfa_mask_tiles(C.byref(p), buf, None, None) == -3
+    p.mask_kind, p.L = _lib.MASK_BOOL, 0
+    assert lib.jvpfa_mask_tiles(C.byref(p), buf, None, None) == -2
+    assert lib.jvpfa_mask_tiles_bytes(C.byref(p)) == 0
+    # the backward takes both lists or none
+    b = _lib.BwdArgs()
+    b.struct_size = C.sizeof(_lib.BwdArgs)
+    b.p.Z, b.p.H, b.p.L, b.p.D = 1, 1, 32, 64
+    b.tiles_q = C.addressof(buf)
     assert lib.jvpfa_bwd(C.byref(b), None) == -1
 
 

@@ -173,6 +173,113 @@ def test_key_padding_with_skipped_tiles(D, kind):
     assert grads[1][1, :, 256:].abs().max().item() == 0.0 and grads[2][2, :, 128:].abs().max().item() == 0.0
 
 
+def _structured_keep(kind, Z, H, L, seed=5):
+    """Boolean (Z or 1, H or 1, L, L) masks with whole tiles masked: the shapes that packed sequences,
+    local windows and padding on both axes produce."""
+    g = torch.Generator().manual_seed(seed)
+    i, j = torch.arange(L)[:, None], torch.arange(L)[None, :]
+    if kind == "blockdiag":  # packed sequences: segment boundaries at random places, one set per batch entry
+        keep = torch.zeros(Z, 1, L, L, dtype=torch.bool)
+        for z in range(Z):
+            cuts = sorted({0, L, *torch.randint(1, L, (3,), generator=g).tolist()})
+            seg = torch.zeros(L, dtype=torch.long)
+            for n, (a, b) in enumerate(zip(cuts[:-1], cuts[1:])):
+                seg[a:b] = n
+            keep[z, 0] = seg[:, None] == seg[None, :]
+        return keep
+    if kind == "band":  # local window of 100 keys either side, shared by batch and heads
+        return ((i - j).abs() <= 100).view(1, 1, L, L)
+    if kind == "pad2d":  # outer product of per-batch padding vectors; padded queries attend nothing
+        lens = torch.randint(L // 4, L + 1, (Z,), generator=g)
+        valid = torch.arange(L)[None, :] < lens[:, None]
+        return (valid[:, :, None] & valid[:, None, :]).view(Z, 1, L, L)
+    if kind == "lower":  # an explicit lower-triangular mask, per head
+        return (j <= i).view(1, 1, L, L).expand(1, H, L, L).contiguous()
+    raise ValueError(kind)
+
+
+def _numpy_tile_lists(keep, L):
+    """(tiles_q, tiles_k) as lists of index lists, from a (P, L, L) boolean array."""
+    nblk, nt = (L + 127) // 128, (L + 63) // 64
+    tq, tk = [], []
+    for pl in keep:
+        for b in range(nblk):
+            rows = pl[128 * b:128 * b + 128]
+            tq.append([t for t in range(nt) if rows[:, 64 * t:64 * t + 64].any()] or [0])
+            cols = pl[:, 128 * b:128 * b + 128]
+            tk.append([t for t in range(nt) if cols[64 * t:64 * t + 64].any()] or [0])
+    return tq, tk
+
+
+@pytest.mark.parametrize("kind", ["blockdiag", "band", "pad2d", "lower"])
+@pytest.mark.parametrize("as_bias", [False, True])
+@pytest.mark.parametrize("L", [640, 700])
+def test_mask_tile_lists_match_a_numpy_scan(kind, as_bias, L):
+    from jvp_flash_attention_amd import _lib
+
+    Z, H = 2, 2
+    keep = _structured_keep(kind, Z, H, L)
+    dtype = torch.bfloat16
+    mask = torch.where(keep, 0.5, float("-inf")).to(dtype) if as_bias else keep
+    mk = _lib.MASK_ADD if as_bias else _lib.MASK_BOOL
+    q = torch.empty(Z, H, L, 64, dtype=dtype, device="cuda")
+    tq, tk = _lib.tile_lists(q, mask.cuda(), mk, True)
+    nt = (L + 63) // 64
+    rq, rk = _numpy_tile_lists(keep.reshape(-1, L, L).numpy(), L)
+    for got, ref in ((tq, rq), (tk, rk)):
+        got = got.cpu().view(-1, nt + 1).tolist()
+        assert len(got) == len(ref)
+        for row, want in zip(got, ref):
+            assert row[0] == len(want) and row[1:1 + row[0]] == want
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("kind", ["blockdiag", "band", "pad2d", "lower"])
+@pytest.mark.parametrize("as_bias", [False, True])
+def test_structured_masks_with_skipped_tiles(D, kind, as_bias):
+    """Masks with whole tiles masked: the host scans them into tile lists and the kernels visit the
+    listed tiles only.  Checked against the oracle, and bit for bit against the same kernels made to
+    visit every tile (a fully masked tile contributes exact zeros)."""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H, L = 2, 2, 700
+    dtype = torch.bfloat16
+    q, k, v, qt, kt, vt, go, gt = _make(Z, H, L, D, dtype, 31)
+    keep = _structured_keep(kind, Z, H, L)
+    mask = torch.where(keep, 0.0, float("-inf")).to(dtype) if as_bias else keep
+    mk = _lib.MASK_ADD if as_bias else _lib.MASK_BOOL
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    be = _lib.backend()
+    scale = D**-0.5
+    print(f"case structured {kind} D{D} bias={as_bias}", flush=True)
+
+    def run(dmask):
+        o, ot, M, mu = be.fwd(*dev[:6], dmask, mk, False, scale)
+        grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, mk, False, scale, want_tangent_grads=True)
+        g1 = be.bwd(dev[0], dev[1], dev[2], None, None, None, o, None, M, None, dev[6], None, dmask, mk, False, scale)
+        return [o, ot, M, mu, *grads, *g1[:3]]
+
+    dmask = mask.cuda()
+    with_lists = run(dmask)
+    assert getattr(dmask, "_jvpfa_tiles")[1] is not None and getattr(dmask, "_jvpfa_tiles")[2] is not None
+    _lib.set_tile_lists(False)
+    try:
+        every_tile = run(mask.cuda())
+    finally:
+        _lib.set_tile_lists(True)
+    for a, b in zip(with_lists, every_tile):
+        assert torch.equal(a, b)
+
+    npm = keep.numpy()
+    ref = dense.forward(*f64[:6], mask=npm, causal=False, scale=scale)
+    rb = dense.backward(*f64, mask=npm, causal=False, scale=scale)
+    _tol_check("O", with_lists[0], ref["O"], dtype)
+    _tol_check("O'", with_lists[1], ref["Ot"], dtype)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), with_lists[4:10]):
+        _tol_check(n, t, rb[n], dtype)
+
+
 def test_mask_combined_with_causal_is_refused():
     # as in the reference, causal attention takes no explicit mask: the library reports it instead of guessing
     with pytest.raises(RuntimeError, match="causal"):
