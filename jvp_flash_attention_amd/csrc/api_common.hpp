@@ -11,8 +11,9 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 inline int check_problem(const jvpfa_problem &p) {
   if (p.Z < 1 || p.H < 1 || p.L < 1) return JVPFA_E_SHAPE;
-  if (p.D != 32 && p.D != 64 && p.D != 128) return JVPFA_E_SHAPE;
+  if (p.D != 32 && p.D != 64 && p.D != 128 && p.D != 256) return JVPFA_E_SHAPE;
   if (p.dtype < JVPFA_BF16 || p.dtype > JVPFA_FP32) return JVPFA_E_DTYPE;
+  if (p.D == 256 && p.dtype == JVPFA_FP32) return JVPFA_E_SHAPE;  // the fp32 tiles of D = 256 do not fit the LDS
   if (p.mask_kind < JVPFA_MASK_NONE || p.mask_kind > JVPFA_MASK_ADD) return JVPFA_E_DTYPE;
   if (p.mask_kind != JVPFA_MASK_NONE) {
     if (p.causal) return JVPFA_E_CONFLICT;
@@ -40,7 +41,7 @@ inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit, cons
   return r;
 }
 
-// 0..8: (dtype, head-dim) slot in the launcher tables.
-inline int slot(const jvpfa_problem &p) { return p.dtype * 3 + (p.D == 32 ? 0 : p.D == 64 ? 1 : 2); }
+// 0..11: (dtype, head-dim) slot in the launcher tables.
+inline int slot(const jvpfa_problem &p) { return p.dtype * 4 + (p.D == 32 ? 0 : p.D == 64 ? 1 : p.D == 128 ? 2 : 3); }
 
 }  // namespace jvpfa

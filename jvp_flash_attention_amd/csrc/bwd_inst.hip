@@ -1,5 +1,5 @@
 // One translation unit per (element type, head dim): compiled with
-//   -DJVPFA_T=<__bf16|_Float16|float> -DJVPFA_D=<32|64|128> -DJVPFA_NAME=<symbol>
+//   -DJVPFA_T=<__bf16|_Float16|float> -DJVPFA_D=<32|64|128|256> -DJVPFA_NAME=<symbol>
 // and exporting  int JVPFA_NAME(const BwdParams&, int mask_kind, bool dual, bool tangent_grads,
 // hipStream_t): pre-pass, then the dq and dk/dv kernels of every requested mode.
 #include "bwd_kernel.hpp"
@@ -14,7 +14,7 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
   const int nb = (p.pr.L + BWD_BLK - 1) / BWD_BLK;
   const long long blocks = (long long)nb * p.pr.Z * p.pr.H;
   if (blocks > 0x7fffffffLL) return -2;
-  if constexpr (sizeof(T) == 2 && D >= 64) {  // direct-to-LDS, double-buffered kernels
+  if constexpr (sizeof(T) == 2 && D >= 64 && D <= 128) {  // direct-to-LDS, double-buffered kernels
     using Cfg2 = Bwd2Cfg<T, D, MODE>;
     // gO may be absent only in the dual mode (loss depends on O' alone)
     const bool no_go = MODE == BWD_DUAL && p.go == nullptr;

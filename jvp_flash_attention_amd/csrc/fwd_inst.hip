@@ -1,5 +1,5 @@
 // One translation unit per (element type, head dim): compiled with
-//   -DJVPFA_T=<__bf16|_Float16|float> -DJVPFA_D=<32|64|128> -DJVPFA_NAME=<symbol>
+//   -DJVPFA_T=<__bf16|_Float16|float> -DJVPFA_D=<32|64|128|256> -DJVPFA_NAME=<symbol>
 // and exporting  int JVPFA_NAME(const FwdParams&, bool dual, int mask_kind, hipStream_t).
 #include "fwd_kernel.hpp"
 #include "fwd_kernel_v2.hpp"
@@ -21,7 +21,7 @@ static int launch_fwd_one(const FwdParams &p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }
 
-// 16-bit element types with D >= 64 take the direct-to-LDS, double-buffered kernel.
+// 16-bit element types with D = 64 or 128 take the direct-to-LDS, double-buffered kernel.
 template <typename T, int D, bool DUAL, int MASK>
 static int launch_fwd2_one(const FwdParams &p, hipStream_t stream) {
   using Cfg = Fwd2Cfg<T, D, DUAL>;
@@ -51,7 +51,7 @@ static int launch_fwd3_one(const FwdParams &p, hipStream_t stream) {
 
 template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
-  if constexpr (sizeof(T) == 2 && D >= 64) {
+  if constexpr (sizeof(T) == 2 && D >= 64 && D <= 128) {
     switch (mask) {
       case MASK_NONE:
         // the pipelined kernel pays off where a slot has enough matrix work to hide the softmax behind
@@ -72,7 +72,7 @@ static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
 }
 
 int JVPFA_NAME(const FwdParams &p, bool dual, int mask, hipStream_t stream) {
-  constexpr int BN = sizeof(JVPFA_T) == 4 ? 32 : 64;
+  constexpr int BN = (sizeof(JVPFA_T) == 4 || JVPFA_D > 128) ? 32 : 64;  // keys per tile of the LDS-copy kernel
   return dual ? launch_fwd_mask<JVPFA_T, JVPFA_D, BN, true>(p, mask, stream)
               : launch_fwd_mask<JVPFA_T, JVPFA_D, BN, false>(p, mask, stream);
 }

@@ -17,8 +17,8 @@ Differences from the reference, all deliberate:
 * ``fwd_dual`` returns an output whose tangent O' carries an autograd graph, so gradients of
   functions of O' (Hessian-vector products) reach q, k, v and the input tangents.  The
   reference's tangent is a constant (JA:2399, JA:2828) and its backward ignores it (JA:2831).
-* Any sequence length L >= 1 and head dims {32, 64, 128} (the reference: L a multiple of 32,
-  D in {32, 64, 128, 256}, JA:2371-2378, JA:2892).
+* Any sequence length L >= 1 and head dims {32, 64, 128, 256} (the reference: L a multiple of 32,
+  JA:2371-2378, JA:2892); D = 256 for bf16 / fp16 only.
 * ``attention`` notices dual inputs and then behaves like ``fwd_dual`` (the reference's ``attention``
   is ``JVPAttn.fwd`` and drops the tangent, its README.md:65-67).
 """
@@ -36,7 +36,7 @@ from . import _lib
 
 MASK_CONST = -100.0  # JA:48-50: value float masks use for "masked"; far below any real logit
 MIN_SEQUENCE_LENGTH = 32  # JA:51; kept for importers, not a limit of these kernels
-SUPPORTED_HEAD_DIMS = (32, 64, 128)
+SUPPORTED_HEAD_DIMS = (32, 64, 128, 256)  # 256: bf16 / fp16 only
 BLOCK_M = 128  # query rows per workgroup of the forward kernel (only reported through Grid)
 
 
@@ -57,6 +57,9 @@ def _validate(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dropout
     assert k.shape == q.shape and v.shape == q.shape, (
         "JVP attention requires q, k, v of one shape (no cross-attention or grouped heads),"
         f" but got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}"
+    )
+    assert not (HEAD_DIM_K == 256 and q.dtype == torch.float32), (
+        "JVP attention supports HEAD_DIM_K=256 for bfloat16 and float16 only"
     )
     assert N_CTX >= 1, f"JVP attention requires N_CTX >= 1, but got N_CTX={N_CTX}"
     assert q.dtype in _lib.DTYPES and k.dtype == q.dtype and v.dtype == q.dtype, (

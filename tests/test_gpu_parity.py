@@ -107,6 +107,18 @@ def test_dual_fwd_bwd_dense_and_causal(dt, D, mode):
     _run_case(2, 2, 256, D, DTYPES[dt], mode)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+@pytest.mark.parametrize("mode", ["none", "causal", "keypad", "bias", "bool_full"])
+def test_head_dim_256(dt, mode):
+    # the largest head dim the reference admits (its jvp_attention.py:2371-2374); 16-bit element types only here
+    _run_case(1, 2, 200, 256, DTYPES[dt], mode, seed=17)
+
+
+def test_head_dim_256_in_fp32_is_refused():
+    with pytest.raises(RuntimeError, match="unsupported shape"):
+        _run_case(1, 1, 64, 256, torch.float32, "none")
+
+
 @pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
 @pytest.mark.parametrize("mode", ["keypad", "bias", "bool_full", "bias_bcast"])
 def test_dual_fwd_bwd_masks(dt, mode):
