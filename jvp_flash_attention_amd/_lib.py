@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
+from typing import Optional, Tuple
 
 import torch
 
@@ -207,12 +208,32 @@ def _stream(t) -> int:
 
 
 class HipBackend:
-    """Device work of the forward and the backward, through the C ABI."""
+    """Device work of the forward and the backward, through the C ABI.
+
+    ``fwd`` / ``bwd`` call the library directly.  While ``torch.compile`` traces, they go through
+    the registered operators ``jvpfa::fwd`` / ``jvpfa::bwd`` instead (same code behind them), which
+    the tracer records as opaque nodes with known output shapes rather than following into ctypes."""
 
     name = "hip"
 
     def fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
         """Returns (o, ot, M, mu); ot and mu are None for a plain forward."""
+        if torch.compiler.is_compiling():
+            o, ot, M, mu = torch.ops.jvpfa.fwd(q, k, v, qt, kt, vt, mask, int(mask_kind), bool(causal), float(sm_scale))
+            return (o, ot, M, mu) if qt is not None else (o, None, M, None)
+        return self._fwd(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale)
+
+    def bwd(self, q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
+            want_tangent_grads=False):
+        """Returns (dq, dk, dv, dqt, dkt, dvt); the last three are None unless requested."""
+        if torch.compiler.is_compiling():
+            out = torch.ops.jvpfa.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, int(mask_kind), bool(causal),
+                                      float(sm_scale), bool(want_tangent_grads))
+            return tuple(out) if want_tangent_grads else (*out[:3], None, None, None)
+        return self._bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
+                         want_tangent_grads)
+
+    def _fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
         _require_gpu(q, k, v, qt, kt, vt, mask)
         lib = load()
         dual = qt is not None
@@ -235,9 +256,8 @@ class HipBackend:
             check(lib.jvpfa_fwd(C.byref(a), _stream(q)))
         return o, ot, M, mu
 
-    def bwd(self, q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
-            want_tangent_grads=False):
-        """Returns (dq, dk, dv, dqt, dkt, dvt); the last three are None unless requested."""
+    def _bwd(self, q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
+             want_tangent_grads=False):
         _require_gpu(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask)
         lib = load()
         Z, H, L, _ = q.shape
@@ -266,6 +286,41 @@ class HipBackend:
 
 
 _backend = HipBackend()
+_hip = _backend  # the operators below always mean the HIP library, whatever backend() has been pointed at
+
+_T, _OT = torch.Tensor, Optional[torch.Tensor]
+
+
+@torch.library.custom_op("jvpfa::fwd", mutates_args=(), device_types="cuda")
+def _op_fwd(q: _T, k: _T, v: _T, qt: _OT, kt: _OT, vt: _OT, mask: _OT, mask_kind: int, causal: bool,
+            sm_scale: float) -> Tuple[_T, _T, _T, _T]:
+    o, ot, M, mu = _hip._fwd(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale)
+    # an operator returns tensors only: empty ones stand for the absent tangent outputs
+    return o, (ot if ot is not None else q.new_empty(0)), M, (mu if mu is not None else M.new_empty(0))
+
+
+@_op_fwd.register_fake
+def _(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
+    Z, H, L, _ = q.shape
+    stat = q.new_empty((Z, H, L), dtype=torch.float32)
+    if qt is None:
+        return torch.empty_like(q), q.new_empty(0), stat, stat.new_empty(0)
+    return torch.empty_like(q), torch.empty_like(q), stat, torch.empty_like(stat)
+
+
+@torch.library.custom_op("jvpfa::bwd", mutates_args=(), device_types="cuda")
+def _op_bwd(q: _T, k: _T, v: _T, qt: _OT, kt: _OT, vt: _OT, o: _T, ot: _OT, M: _T, mu: _OT, go: _OT, gt: _OT,
+            mask: _OT, mask_kind: int, causal: bool, sm_scale: float,
+            want_tangent_grads: bool) -> Tuple[_T, _T, _T, _T, _T, _T]:
+    g = _hip._bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale, want_tangent_grads)
+    return tuple(t if t is not None else q.new_empty(0) for t in g)
+
+
+@_op_bwd.register_fake
+def _(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale, want_tangent_grads):
+    full = [torch.empty_like(q) for _ in range(3)]
+    rest = [torch.empty_like(q) if want_tangent_grads else q.new_empty(0) for _ in range(3)]
+    return (*full, *rest)
 
 
 def backend():

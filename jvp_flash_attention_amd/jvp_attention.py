@@ -137,6 +137,35 @@ class _DualCore(Function):
         return dq, dk, dv, dqt, dkt, dvt, None, None, None, None
 
 
+class _PlainCore(Function):
+    """(q, k, v) -> (O, M) with the first-order backward: what ``JVPAttn`` computes without tangents,
+    as a Function without a custom ``jvp`` (which ``torch.compile`` refuses to trace).  ``JVPAttn.fwd``
+    uses it while compiling."""
+
+    @staticmethod
+    def forward(q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale):
+        o, _o_t, M, _mu = _lib.backend().fwd(q, k, v, None, None, None, mask_tensor, MASK_TYPE, causal, sm_scale)
+        return o, M
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale = inputs
+        o, M = outputs
+        ctx.mark_non_differentiable(M)
+        ctx.save_for_backward(q, k, v, o, M)
+        ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale = mask_tensor, MASK_TYPE, causal, sm_scale
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, go, _gM):
+        q, k, v, o, M = ctx.saved_tensors
+        dq, dk, dv, _, _, _ = _lib.backend().bwd(
+            q, k, v, None, None, None, o, None, M, None, _dense(go), None,
+            ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale,
+        )
+        return dq, dk, dv, None, None, None, None
+
+
 class _AttachTangent(Function):
     """Identity on O whose forward-mode tangent is the precomputed O' (the reference's trick of
     JA:2688 and JA:2828, with O' an input so that it keeps its autograd graph)."""
@@ -301,6 +330,14 @@ class JVPAttn(Function):
         """Plain attention forward, differentiable in q, k, v (JA:2700-2752)."""
         if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
             q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        if torch.compiler.is_compiling():
+            # the same computation through a Function the tracer can follow (no custom jvp, no
+            # data-dependent mask checks); the kernels appear in the graph as jvpfa::fwd / jvpfa::bwd
+            _validate(q, k, v, attn_mask, dropout_p, causal)
+            scale = q.shape[-1] ** -0.5 if sm_scale is None else sm_scale
+            mask_tensor, MASK_TYPE = _classify_mask(attn_mask, q, False)
+            o, _M = _PlainCore.apply(q, k, v, mask_tensor, MASK_TYPE, causal, scale)
+            return o
         out: JVPAttn.FwdOut = JVPAttn.apply(
             q, k, v, None, None, None, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA
         )
@@ -323,6 +360,13 @@ class JVPAttn(Function):
         ``torch.func.jvp`` the result is a dual tensor whose tangent is O', computed by the same
         kernel pass as O.  Both O and O' are differentiable (reverse mode) in q, k, v and in the
         input tangents."""
+        if torch.compiler.is_compiling():
+            # The tracer cannot follow the custom jvp that hands O' to forward-mode AD.  With a
+            # forward-mode level active the call is therefore left out of the graph and runs as
+            # ordinary Python between two compiled pieces; without one no tangent can exist.
+            if fwAD._current_level >= 0:
+                return _fwd_dual_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
+            return JVPAttn.fwd(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
         if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
             q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         q_p, q_t = fwAD.unpack_dual(q)
@@ -367,6 +411,11 @@ class JVPAttn(Function):
             ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale,
         )
         return JVPAttn.BwdOut(dq, dk, dv, None, None, None, None, None, None, None, None, None, None)
+
+
+@torch.compiler.disable
+def _fwd_dual_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA):
+    return JVPAttn.fwd_dual(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
 
 
 def attention(

@@ -143,6 +143,54 @@ def test_forward_and_backward_replay_from_a_hip_graph(causal):
             assert torch.equal(a, b), f"replay {rep}"
 
 
+@pytest.mark.parametrize("masked", [False, True])
+def test_plain_attention_inside_torch_compile_without_graph_breaks(masked):
+    """``torch.compile(fullgraph=True)`` over a function that calls ``attention``: the kernels enter
+    the graph as the operators ``jvpfa::fwd`` / ``jvpfa::bwd``; output and gradients equal the eager
+    ones bit for bit (the ``aot_eager`` backend runs the traced graph with the same kernels)."""
+    from jvp_flash_attention_amd import attention
+
+    Z, H, L, D = 2, 4, 256, 64
+    q, k, v = [_randn((Z, H, L, D), torch.bfloat16, 70 + i).requires_grad_() for i in range(3)]
+    kw = dict(causal=True)
+    if masked:
+        keep = torch.rand(Z, 1, L, L, device="cuda", generator=torch.Generator(device="cuda").manual_seed(5)) > 0.3
+        keep[..., 0] = True
+        kw = dict(attn_mask=keep)
+
+    def f(q, k, v):
+        return (attention(q * 1.0, k, v, **kw) * 2.0).float().sum()
+
+    ref = f(q, k, v)
+    gref = torch.autograd.grad(ref, (q, k, v))
+    torch._dynamo.reset()
+    out = torch.compile(f, backend="aot_eager", fullgraph=True)(q, k, v)
+    g = torch.autograd.grad(out, (q, k, v))
+    assert torch.equal(out, ref)
+    for a, b in zip(g, gref):
+        assert torch.equal(a, b)
+
+
+def test_dual_tensors_inside_torch_compile_keep_their_tangent():
+    """Forward-mode AD inside a compiled function: the attention call is left out of the graph and
+    runs between two compiled pieces, so O' is what the eager call gives, not silently dropped."""
+    from jvp_flash_attention_amd import JVPAttn
+
+    Z, H, L, D = 1, 2, 128, 64
+    q, k, v, qt, kt, vt = [_randn((Z, H, L, D), torch.bfloat16, 80 + i) for i in range(6)]
+
+    def g(q, k, v, qt, kt, vt):
+        with fwAD.dual_level():
+            out = JVPAttn.fwd_dual(fwAD.make_dual(q, qt), fwAD.make_dual(k, kt), fwAD.make_dual(v, vt), causal=True)
+            o, ot = fwAD.unpack_dual(out)
+            return o.clone(), ot.clone()
+
+    o1, ot1 = g(q, k, v, qt, kt, vt)
+    torch._dynamo.reset()
+    o2, ot2 = torch.compile(g, backend="eager")(q, k, v, qt, kt, vt)
+    assert torch.equal(o1, o2) and torch.equal(ot1, ot2)
+
+
 def test_plain_attention_autograd_and_apply_tuple():
     from jvp_flash_attention_amd import JVPAttn, attention
 

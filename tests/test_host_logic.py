@@ -211,3 +211,24 @@ def test_product_has_no_cpu_path():
     q, k, v, *_ = _inputs()
     with pytest.raises(RuntimeError, match="no CPU path|There is no CPU path"):
         attention(q, k, v)
+
+
+def test_registered_operators_describe_their_outputs_without_running():
+    """``jvpfa::fwd`` / ``jvpfa::bwd`` are what ``torch.compile`` records in place of the ctypes calls;
+    their shape functions must agree with what the library returns (empty tensors stand for absent
+    tangent outputs).  Fake tensors only: nothing is launched."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from jvp_flash_attention_amd import _lib  # noqa: F401  (registers the operators)
+
+    with FakeTensorMode():
+        q = torch.empty(2, 3, 64, 64, device="cuda", dtype=torch.bfloat16)
+        o, ot, M, mu = torch.ops.jvpfa.fwd(q, q, q, None, None, None, None, 0, False, 0.125)
+        assert o.shape == q.shape and o.dtype == q.dtype and ot.numel() == 0 and mu.numel() == 0
+        assert M.shape == (2, 3, 64) and M.dtype == torch.float32
+        o, ot, M, mu = torch.ops.jvpfa.fwd(q, q, q, q, q, q, None, 0, True, 0.125)
+        assert ot.shape == q.shape and mu.shape == (2, 3, 64) and mu.dtype == torch.float32
+        g = torch.ops.jvpfa.bwd(q, q, q, q, q, q, o, ot, M, mu, q, q, None, 0, True, 0.125, True)
+        assert [t.shape for t in g] == [q.shape] * 6
+        g = torch.ops.jvpfa.bwd(q, q, q, None, None, None, o, None, M, None, q, None, None, 0, True, 0.125, False)
+        assert [t.shape for t in g[:3]] == [q.shape] * 3 and all(t.numel() == 0 for t in g[3:])
