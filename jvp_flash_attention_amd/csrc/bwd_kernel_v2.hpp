@@ -191,7 +191,8 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   if constexpr (MASK != MASK_NONE) {
     if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
   }
-  const int ntiles = tlist ? tlist[0] : (kend + BT - 1) / BT;
+  const int tmax = (L + BT - 1) / BT - 1;  // index of the last tile of the sequence: bounds whatever a list holds
+  const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1) : (kend + BT - 1) / BT;
   // List elements are requested a tile ahead, unconditionally (from a harmless address when there is
   // no list: a branch around the read would split the tile loop's straight-line body).
   auto list_slot = [&](int i) { return tlist ? tlist + 1 + i : reinterpret_cast<const int *>(p.q); };
@@ -358,7 +359,8 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
     }
   };
   // the tile of this step and of the next
-  int tcur = tlist ? tlist[1] : 0, tnext = tlist ? tlist[1 + min(1, ntiles - 1)] : min(1, ntiles - 1);
+  int tcur = tlist ? min(max(tlist[1], 0), tmax) : 0;
+  int tnext = tlist ? min(max(tlist[1 + min(1, ntiles - 1)], 0), tmax) : min(1, ntiles - 1);
   fetch_masks(tcur);
   prepare_loads(0, tcur * BT, true);
   static_for<NLOAD>([&](auto pc) { load_piece(pc); });
@@ -382,7 +384,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
     half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, j0 + 32);
     if constexpr (MASK != MASK_NONE) {
       const int listed = list_take(tahead);
-      tnext2 = tlist ? listed : tnext2;
+      tnext2 = tlist ? min(max(listed, 0), tmax) : tnext2;
     }
     tcur = tnext;
     tnext = tnext2;
@@ -510,7 +512,8 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   if constexpr (MASK != MASK_NONE) {
     if (pr.tiles_k) tlist = pr.tiles_k + tile_list_offset(pr, z, h, kb);
   }
-  const int ntiles = tlist ? tlist[0] : (L - istart + BT - 1) / BT;
+  const int tmax = (L + BT - 1) / BT - 1;  // index of the last tile of the sequence: bounds whatever a list holds
+  const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1) : (L - istart + BT - 1) / BT;
   // List elements are requested a tile ahead, unconditionally (from a harmless address when there is
   // no list: a branch around the read would split the tile loop's straight-line body).
   auto list_slot = [&](int i) { return tlist ? tlist + 1 + i : reinterpret_cast<const int *>(p.q); };
@@ -756,7 +759,8 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   };
 
   // the tile of this step and of the next
-  int tcur = tlist ? tlist[1] : 0, tnext = tlist ? tlist[1 + min(1, ntiles - 1)] : min(1, ntiles - 1);
+  int tcur = tlist ? min(max(tlist[1], 0), tmax) : 0;
+  int tnext = tlist ? min(max(tlist[1 + min(1, ntiles - 1)], 0), tmax) : min(1, ntiles - 1);
   if constexpr (MASK != MASK_NONE && MAHEAD) fetch_mask_half(istart + tcur * BT);
   prepare_loads(0, istart + tcur * BT, true);
   static_for<NLOAD>([&](auto pc) { load_piece(pc); });
@@ -777,7 +781,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
     half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32, i0n);
     if constexpr (MASK != MASK_NONE) {
       const int listed = list_take(tahead);
-      tnext2 = tlist ? listed : tnext2;
+      tnext2 = tlist ? min(max(listed, 0), tmax) : tnext2;
     }
     tcur = tnext;
     tnext = tnext2;

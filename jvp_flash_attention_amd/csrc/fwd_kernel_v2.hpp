@@ -197,7 +197,8 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   if constexpr (MASK != MASK_NONE) {
     if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
   }
-  const int ntiles = tlist ? tlist[0] : (kend + BN - 1) / BN;
+  const int tmax = (L + BN - 1) / BN - 1;  // index of the last tile of the sequence: bounds whatever a list holds
+  const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1) : (kend + BN - 1) / BN;
   // List elements are requested a tile ahead, unconditionally (from a harmless address when there is
   // no list: a branch around the read would split the tile loop's straight-line body).
   auto list_slot = [&](int i) { return tlist ? tlist + 1 + i : reinterpret_cast<const int *>(p.q); };
@@ -421,7 +422,8 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     }
   };
   // the tile of this step and of the next
-  int tcur = tlist ? tlist[1] : 0, tnext = tlist ? tlist[1 + min(1, ntiles - 1)] : min(1, ntiles - 1);
+  int tcur = tlist ? min(max(tlist[1], 0), tmax) : 0;
+  int tnext = tlist ? min(max(tlist[1 + min(1, ntiles - 1)], 0), tmax) : min(1, ntiles - 1);
   fetch_masks(tcur);
   issue_loads(0, tcur * BN);
   auto tile = [&](int t, auto EDGEc) {
@@ -447,7 +449,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, j0 + 32);
     if constexpr (MASK != MASK_NONE) {
       const int listed = list_take(tahead);
-      tnext2 = tlist ? listed : tnext2;
+      tnext2 = tlist ? min(max(listed, 0), tmax) : tnext2;
     }
     tcur = tnext;
     tnext = tnext2;
