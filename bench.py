@@ -116,6 +116,40 @@ def hvp_sweep(be, _lib):
     return rows
 
 
+def mask_rows(be, _lib, q, k, v, qt, kt, vt, go, gt, scale):
+    """The headline shape with explicit masks: dual forward / backward times for a dense random boolean
+    mask (nothing to skip), a block-diagonal mask of four segments and a band of +-256 keys (tiles
+    without an attended entry are skipped through the tile lists), and the time of the scan that makes
+    the lists (an HBM-bound pass: it reads the mask once per list)."""
+    import torch
+
+    dev = q.device
+    g = torch.Generator(device=dev).manual_seed(7)
+    idx = torch.arange(L, device=dev)
+    seg = (idx * 4) // L
+    masks = {
+        "dense_bool_ZHLL": torch.rand(Z, H, L, L, generator=g, device=dev) > 0.1,
+        "block_diagonal_x4_Z1LL": (seg[:, None] == seg[None, :]).view(1, 1, L, L).expand(Z, 1, L, L).contiguous(),
+        "band_256_11LL": ((idx[:, None] - idx[None, :]).abs() <= 256).view(1, 1, L, L),
+    }
+    rows = {}
+    for name, m in masks.items():
+        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, m, _lib.MASK_BOOL, False, scale), 10, 3)
+        o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, m, _lib.MASK_BOOL, False, scale)
+        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, m, _lib.MASK_BOOL, False, scale), 5, 2)
+
+        def scan():
+            if hasattr(m, "_jvpfa_tiles"):
+                del m._jvpfa_tiles
+            _lib.tile_lists(q, m, _lib.MASK_BOOL, True)
+
+        ms_s, _ = timed(scan, 5, 2)
+        rows[name] = {"attended_fraction": m.float().mean().item(), "fwd_ms": ms_f, "bwd_ms": ms_b, "scan_ms": ms_s,
+                      "scan_GBps": 2.0 * m.numel() / (ms_s * 1e-3) / 1e9}
+        del m
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -215,6 +249,7 @@ def main():
             "peak_hbm_allocated_mb": torch.cuda.max_memory_allocated() / 2**20,
         }
         out["extra"]["hvp_sweep_bf16_B1_H16_D128_causal"] = hvp_sweep(be, _lib)
+        out["extra"]["masks_bf16_B4_H16_L4096_D128"] = mask_rows(be, _lib, q, k, v, qt, kt, vt, go, gt, scale)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)
