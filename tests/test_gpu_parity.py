@@ -292,6 +292,42 @@ def test_structured_masks_with_skipped_tiles(D, kind, as_bias):
         _tol_check(n, t, rb[n], dtype)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_configurations(seed):
+    """Element type, head dim, batch, heads, sequence length (ragged ones included, some long enough
+    for the tile lists and the key-limit hint) and mask mode drawn from a seeded generator."""
+    from jvp_flash_attention_amd import _lib
+
+    rng = np.random.default_rng(1000 + seed)
+    dt = ["bf16", "fp16", "fp32"][rng.integers(3)]
+    D = [32, 64, 128, 256][rng.integers(4)] if dt != "fp32" else [32, 64, 128][rng.integers(3)]
+    Z, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+    long_case = seed % 3 == 0
+    L = int(rng.integers(513, 900)) if long_case else int(rng.integers(1, 300))
+    mode = ["none", "causal", "keypad", "bias", "bool_full", "blockdiag", "band", "pad2d", "lower"][rng.integers(9)]
+    dtype = DTYPES[dt]
+    if mode in ("none", "causal", "keypad", "bias", "bool_full"):
+        _run_case(Z, H, L, D, dtype, mode, seed=seed, tangent_grads=bool(rng.integers(2)))
+        return
+    keep = _structured_keep(mode, Z, H, L, seed=seed) if L > 100 or mode != "blockdiag" else _structured_keep("band", Z, H, L)
+    as_bias = bool(rng.integers(2))
+    q, k, v, qt, kt, vt, go, gt = _make(Z, H, L, D, dtype, seed)
+    mask = torch.where(keep, 0.0, float("-inf")).to(dtype) if as_bias else keep
+    mk = _lib.MASK_ADD if as_bias else _lib.MASK_BOOL
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    print(f"case random {seed}: Z{Z} H{H} L{L} D{D} {dt} {mode} bias={as_bias}", flush=True)
+    be, scale, dmask = _lib.backend(), D**-0.5, mask.cuda()
+    o, ot, M, mu = be.fwd(*dev[:6], dmask, mk, False, scale)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, mk, False, scale, want_tangent_grads=True)
+    ref = dense.forward(*f64[:6], mask=keep.numpy(), causal=False, scale=scale)
+    rb = dense.backward(*f64, mask=keep.numpy(), causal=False, scale=scale)
+    _tol_check("O", o, ref["O"], dtype)
+    _tol_check("O'", ot, ref["Ot"], dtype)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        _tol_check(n, t, rb[n], dtype)
+
+
 def test_mask_combined_with_causal_is_refused():
     # as in the reference, causal attention takes no explicit mask: the library reports it instead of guessing
     with pytest.raises(RuntimeError, match="causal"):
