@@ -151,12 +151,18 @@ def key_limit_hint(mask, mask_kind, Z, L):
 
 TILE_LISTS_MIN_L = 512  # below this a mask has too few tiles for skipping some to pay for the scan
 _tile_lists_enabled = True
+_tile_lists_additive = False
 
 
-def set_tile_lists(enabled: bool) -> None:
-    """Switch the scan of two-dimensional masks for skippable tiles on or off (default on)."""
-    global _tile_lists_enabled
+def set_tile_lists(enabled: bool, additive: bool | None = None) -> None:
+    """Switch the scan of two-dimensional masks for skippable tiles on or off (default: on for
+    boolean masks, off for additive ones).  An additive mask only has skippable tiles where it holds
+    -inf over a whole tile; a learned bias never does and the scan would read it for nothing, so
+    additive masks are scanned only after ``set_tile_lists(True, additive=True)``."""
+    global _tile_lists_enabled, _tile_lists_additive
     _tile_lists_enabled = bool(enabled)
+    if additive is not None:
+        _tile_lists_additive = bool(additive)
 
 
 def tile_lists(q, mask, mask_kind, want_k):
@@ -172,6 +178,8 @@ def tile_lists(q, mask, mask_kind, want_k):
             or q.dtype == torch.float32 or D < 64):
         return None, None
     if mask.dim() != 4 or mask.shape[2] != L or mask.shape[3] != L:
+        return None, None
+    if mask_kind == MASK_ADD and not _tile_lists_additive:
         return None, None
     cached = getattr(mask, "_jvpfa_tiles", None)
     if cached is None or cached[0] != mask._version:

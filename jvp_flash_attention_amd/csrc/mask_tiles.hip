@@ -35,33 +35,42 @@ __global__ __launch_bounds__(256) void mask_tiles_kernel(const E *mask, int64_t 
   const bool vec_ok = s3 == 1 && (s0 % VEC) == 0 && (s1 % VEC) == 0 && (s2 % VEC) == 0 &&
                       (reinterpret_cast<uintptr_t>(mask) % 16) == 0;
   int count = 0;
-  for (int t = 0; t < nt; ++t) {
-    const int row = KEYS_OWNED ? t * TILE_W + rsub : blk * TILE_BLOCK + rsub;
-    const int key0 = (KEYS_OWNED ? blk * TILE_BLOCK : t * TILE_W) + 32 * part;
-    bool any = false;
-    if (row < L && key0 < L) {
-      const E *rp = base + (int64_t)row * s2;
-      if (vec_ok && key0 + 32 <= L) {
+  constexpr int U = 4;  // tiles looked at per round: their loads are all in flight before the first vote
+  for (int t0 = 0; t0 < nt; t0 += U) {
+    bool any[U];
 #pragma unroll
-        for (int v = 0; v < 32 / VEC; ++v) {
-          const uint4 w = *reinterpret_cast<const uint4 *>(rp + key0 + v * VEC);
-          if constexpr (BOOL) {
-            any |= (w.x | w.y | w.z | w.w) != 0;
-          } else {
-            E e[VEC];
-            __builtin_memcpy(e, &w, 16);
+    for (int u = 0; u < U; ++u) {
+      const int t = t0 + u;
+      const int row = KEYS_OWNED ? t * TILE_W + rsub : blk * TILE_BLOCK + rsub;
+      const int key0 = (KEYS_OWNED ? blk * TILE_BLOCK : t * TILE_W) + 32 * part;
+      any[u] = false;
+      if (t < nt && row < L && key0 < L) {
+        const E *rp = base + (int64_t)row * s2;
+        if (vec_ok && key0 + 32 <= L) {
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) any |= attended<E, BOOL>(e[i]);
+          for (int v = 0; v < 32 / VEC; ++v) {
+            const uint4 w = *reinterpret_cast<const uint4 *>(rp + key0 + v * VEC);
+            if constexpr (BOOL) {
+              any[u] |= (w.x | w.y | w.z | w.w) != 0;
+            } else {
+              E e[VEC];
+              __builtin_memcpy(e, &w, 16);
+#pragma unroll
+              for (int i = 0; i < VEC; ++i) any[u] |= attended<E, BOOL>(e[i]);
+            }
           }
+        } else {
+          const int n = min(32, L - key0);
+          for (int i = 0; i < n; ++i) any[u] |= attended<E, BOOL>(rp[(int64_t)(key0 + i) * s3]);
         }
-      } else {
-        const int n = min(32, L - key0);
-        for (int i = 0; i < n; ++i) any |= attended<E, BOOL>(rp[(int64_t)(key0 + i) * s3]);
       }
     }
-    if (__syncthreads_or(any)) {  // uniform over the workgroup
-      if (tid == 0) list[1 + count] = t;
-      ++count;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (__syncthreads_or(any[u])) {  // uniform over the workgroup
+        if (tid == 0) list[1 + count] = t0 + u;
+        ++count;
+      }
     }
   }
   if (tid == 0) {

@@ -121,6 +121,7 @@ def test_tile_lists_are_only_made_for_masks_with_a_row_per_query():
     ]
     for qq, m in cases:
         assert _lib.tile_lists(qq, m, _lib.MASK_BOOL if m is not None else _lib.MASK_NONE, True) == (None, None)
+    assert _lib.tile_lists(q, full.to(torch.bfloat16), _lib.MASK_ADD, True) == (None, None)  # additive: on request only
     _lib.set_tile_lists(False)
     try:
         assert _lib.tile_lists(q, full, _lib.MASK_BOOL, True) == (None, None)

@@ -235,7 +235,11 @@ def test_mask_tile_lists_match_a_numpy_scan(kind, as_bias, L):
     mask = torch.where(keep, 0.5, float("-inf")).to(dtype) if as_bias else keep
     mk = _lib.MASK_ADD if as_bias else _lib.MASK_BOOL
     q = torch.empty(Z, H, L, 64, dtype=dtype, device="cuda")
-    tq, tk = _lib.tile_lists(q, mask.cuda(), mk, True)
+    _lib.set_tile_lists(True, additive=True)  # additive masks are only scanned on request
+    try:
+        tq, tk = _lib.tile_lists(q, mask.cuda(), mk, True)
+    finally:
+        _lib.set_tile_lists(True, additive=False)
     nt = (L + 63) // 64
     rq, rk = _numpy_tile_lists(keep.reshape(-1, L, L).numpy(), L)
     for got, ref in ((tq, rq), (tk, rk)):
@@ -273,13 +277,14 @@ def test_structured_masks_with_skipped_tiles(D, kind, as_bias):
         return [o, ot, M, mu, *grads, *g1[:3]]
 
     dmask = mask.cuda()
-    with_lists = run(dmask)
-    assert getattr(dmask, "_jvpfa_tiles")[1] is not None and getattr(dmask, "_jvpfa_tiles")[2] is not None
-    _lib.set_tile_lists(False)
+    _lib.set_tile_lists(True, additive=True)  # additive masks are only scanned on request
     try:
+        with_lists = run(dmask)
+        assert getattr(dmask, "_jvpfa_tiles")[1] is not None and getattr(dmask, "_jvpfa_tiles")[2] is not None
+        _lib.set_tile_lists(False)
         every_tile = run(mask.cuda())
     finally:
-        _lib.set_tile_lists(True)
+        _lib.set_tile_lists(True, additive=False)
     for a, b in zip(with_lists, every_tile):
         assert torch.equal(a, b)
 
