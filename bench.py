@@ -27,9 +27,9 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
 Z, H, L, D = 4, 16, 4096, 128
 
 # HBM bytes per forward launch measured with rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a plain
-# copy of known size gives) and WRITE_SIZE (x1.0): 406.1 MB read + 136.3 MB written; the figures
+# copy of known size gives) and WRITE_SIZE (x1.0): 403.0 MB read + 136.3 MB written; the figures
 # and commands are in profiles/fwd3_kernel_bf16_B4_H16_L4096_D128.md.
-MEASURED_FWD_TRAFFIC_BYTES = 542.4e6
+MEASURED_FWD_TRAFFIC_BYTES = 539.3e6
 
 
 def timed(fn, steps, warmup):
