@@ -72,7 +72,28 @@ def build(jobs: int | None = None, verbose: bool = True, extra_flags=(), lib: st
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
     if verbose:
         print(f"built {lib} from {len(objs)} objects", flush=True)
+    if lib == LIB:
+        build_host_check(verbose)
     return lib
+
+
+HOST_CHECK_SRC = os.path.join(os.path.dirname(HERE), "tests", "cabi_host", "host_check.cpp")
+HOST_CHECK_BIN = os.path.join(os.path.dirname(HERE), "tests", "cabi_host", "host_check")
+
+
+def build_host_check(verbose: bool = True) -> str | None:
+    """The plain C++ caller of the C ABI used by the GPU tests (no Python, no torch in the process):
+    compiled against ``include/jvpfa.h`` and linked with the library just built."""
+    if not os.path.exists(HOST_CHECK_SRC):
+        return None
+    cmd = [HIPCC, "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", "-I", os.path.join(os.path.dirname(HERE), "include"),
+           HOST_CHECK_SRC, "-o", HOST_CHECK_BIN, "-L", HERE, "-ljvpfa", "-Wl,-rpath,$ORIGIN/../../jvp_flash_attention_amd"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for the host check:\n{' '.join(cmd)}\n{r.stderr[-4000:]}")
+    if verbose:
+        print(f"built {HOST_CHECK_BIN}", flush=True)
+    return HOST_CHECK_BIN
 
 
 if __name__ == "__main__":

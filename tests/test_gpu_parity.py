@@ -508,3 +508,17 @@ def test_additive_mask_with_minus_infinity_entries(dt):
                    want_tangent_grads=True)
     for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
         _tol_check(n, t, rb[n], dtype)
+
+
+def test_c_abi_from_a_plain_cpp_program():
+    """``tests/cabi_host/host_check`` (built with the library) calls jvpfa_fwd / jvpfa_bwd from C++ with
+    memory it allocated through the HIP runtime, no Python or torch in its process, and compares with
+    its own O(L^2) double-precision evaluation: fp32, max-abs <= 1e-4, key-padding mask and causal."""
+    import os
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cabi_host", "host_check")
+    assert os.path.exists(exe), "build it with `python -m jvp_flash_attention_amd.build`"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0 and "host check ok" in r.stdout
