@@ -518,7 +518,8 @@ def test_c_abi_from_a_plain_cpp_program():
     import subprocess
 
     exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cabi_host", "host_check")
-    assert os.path.exists(exe), "build it with `python -m jvp_flash_attention_amd.build`"
+    if not os.path.exists(exe):
+        pytest.skip("tests/cabi_host/host_check is not built: run `python -m jvp_flash_attention_amd.build`")
     r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0 and "host check ok" in r.stdout
