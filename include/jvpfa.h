@@ -9,7 +9,7 @@
  * call from any thread; two calls that write the same buffers race.
  *
  * Tensors q, k, v, their tangents, outputs and gradients are dense row-major
- * (Z, H, L, D); row statistics are fp32 (Z, H, L).  The mask, when present,
+ * (Z, H, L, D) (k, v and what belongs to them: (Z, Hk, Lk, D) when a call says so); row statistics are fp32 (Z, H, L).  The mask, when present,
  * is addressed with four element strides (0 = broadcast along that axis), so
  * a key-padding mask of shape [Z,1,1,L] is read in place.
  *
@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define JVPFA_ABI_VERSION 3
+#define JVPFA_ABI_VERSION 4
 
 enum jvpfa_dtype { JVPFA_BF16 = 0, JVPFA_FP16 = 1, JVPFA_FP32 = 2 };
 
@@ -85,6 +85,14 @@ typedef struct jvpfa_fwd_args {
    * this same mask, or NULL.  Tiles not listed are skipped instead of read and masked.  When set,
    * key_limit is ignored.  Ignored without a mask. */
   const int32_t *tiles_q;
+  /* since version 4 (a caller may pass the version-3 size, which ends before this field): shape of
+   * k, v, kt, vt when it is not q's -- Lk keys (any length >= 1) and Hk key/value heads, Hk a divisor
+   * of p.H; query head h reads key/value head h / (H / Hk).  0 means "as q" (p.L, p.H).  k, v and
+   * their tangents are then (Z, Hk, Lk, D), the mask strides address (z, h, query, key) with Lk keys,
+   * and causal means key index <= query index.  The reference requires q, k, v of one shape
+   * (JA:2367-2378); such calls run on the general kernels, not the tuned ones.  key_limit and the tile
+   * lists are ignored for them. */
+  int32_t Lk, Hk;
 } jvpfa_fwd_args;
 
 int jvpfa_fwd(const jvpfa_fwd_args *args, void *hip_stream);
@@ -119,6 +127,7 @@ typedef struct jvpfa_bwd_args {
   const int32_t *tiles_q;   /* since version 3: as in jvpfa_fwd_args (used by the dq kernels) */
   const int32_t *tiles_k;   /* since version 3: the other list of jvpfa_mask_tiles() (dk/dv kernels);
                                tiles_q and tiles_k are both NULL or both set */
+  int32_t Lk, Hk;           /* since version 4: as in jvpfa_fwd_args; dk, dv, dkt, dvt have the shape of k */
 } jvpfa_bwd_args;
 
 int jvpfa_bwd(const jvpfa_bwd_args *args, void *hip_stream);

@@ -15,7 +15,7 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libjvpfa.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
 EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_bwd_workspace_bytes", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
@@ -42,6 +42,7 @@ class FwdArgs(C.Structure):
         ("M", C.c_void_p), ("mu", C.c_void_p),
         ("key_limit", C.c_void_p),
         ("tiles_q", C.c_void_p),
+        ("Lk", C.c_int32), ("Hk", C.c_int32),
     ]
 
 
@@ -59,6 +60,7 @@ class BwdArgs(C.Structure):
         ("workspace", C.c_void_p),
         ("key_limit", C.c_void_p),
         ("tiles_q", C.c_void_p), ("tiles_k", C.c_void_p),
+        ("Lk", C.c_int32), ("Hk", C.c_int32),
     ]
 
 
@@ -256,6 +258,7 @@ class HipBackend:
         a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
         a.qt, a.kt, a.vt = _ptr(qt), _ptr(kt), _ptr(vt)
         a.o, a.ot, a.M, a.mu = _ptr(o), _ptr(ot), _ptr(M), _ptr(mu)
+        a.Hk, a.Lk = k.shape[1], k.shape[2]  # key/value heads and length (may differ from q's)
         with torch.cuda.device(q.device):
             lim = key_limit_hint(mask, mask_kind, Z, L)
             a.key_limit = _ptr(lim)
@@ -284,6 +287,7 @@ class HipBackend:
         a.dq, a.dk, a.dv = _ptr(dq), _ptr(dk), _ptr(dv)
         a.dqt, a.dkt, a.dvt = _ptr(dqt), _ptr(dkt), _ptr(dvt)
         a.workspace = _ptr(ws)
+        a.Hk, a.Lk = k.shape[1], k.shape[2]
         with torch.cuda.device(q.device):
             lim = key_limit_hint(mask, mask_kind, Z, L)
             a.key_limit = _ptr(lim)
@@ -326,8 +330,8 @@ def _op_bwd(q: _T, k: _T, v: _T, qt: _OT, kt: _OT, vt: _OT, o: _T, ot: _OT, M: _
 
 @_op_bwd.register_fake
 def _(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale, want_tangent_grads):
-    full = [torch.empty_like(q) for _ in range(3)]
-    rest = [torch.empty_like(q) if want_tangent_grads else q.new_empty(0) for _ in range(3)]
+    full = [torch.empty_like(t) for t in (q, k, v)]
+    rest = [torch.empty_like(t) if want_tangent_grads else q.new_empty(0) for t in (q, k, v)]
     return (*full, *rest)
 
 

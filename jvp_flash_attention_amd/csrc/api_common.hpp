@@ -24,10 +24,20 @@ inline int check_problem(const jvpfa_problem &p) {
   return JVPFA_OK;
 }
 
+// Lk, Hk as given by the caller (0 = as q); JVPFA_E_SHAPE if they do not fit
+inline int check_kv_shape(const jvpfa_problem &p, int32_t Lk, int32_t Hk) {
+  if (Lk < 0 || Hk < 0) return JVPFA_E_SHAPE;
+  if (Hk > 0 && (Hk > p.H || p.H % Hk != 0)) return JVPFA_E_SHAPE;
+  return JVPFA_OK;
+}
+
 inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit, const int32_t *tiles_q,
-                          const int32_t *tiles_k) {
+                          const int32_t *tiles_k, int32_t Lk = 0, int32_t Hk = 0) {
   Problem r;
-  const bool masked = p.mask_kind != JVPFA_MASK_NONE;
+  r.Lk = Lk > 0 ? Lk : p.L;
+  r.Hk = Hk > 0 ? Hk : p.H;
+  // the hints are for the tuned kernels, which take k, v of q's shape only
+  const bool masked = p.mask_kind != JVPFA_MASK_NONE && r.Lk == p.L && r.Hk == p.H;
   r.tiles_q = masked ? tiles_q : nullptr;
   r.tiles_k = masked ? tiles_k : nullptr;
   r.klimit = (masked && !r.tiles_q && !r.tiles_k) ? key_limit : nullptr;

@@ -152,15 +152,17 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
-  const T *Kg = reinterpret_cast<const T *>(p.k) + head;
-  const T *Vg = reinterpret_cast<const T *>(p.v) + head;
-  const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + head : nullptr;
-  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + head : nullptr;
+  const int Lk = pr.Lk;  // keys; L counts queries
+  const size_t kvhead = ((size_t)z * pr.Hk + h / (pr.H / pr.Hk)) * Lk * D;  // grouped heads share K, V
+  const T *Kg = reinterpret_cast<const T *>(p.k) + kvhead;
+  const T *Vg = reinterpret_cast<const T *>(p.v) + kvhead;
+  const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + kvhead : nullptr;
+  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + kvhead : nullptr;
 
-  const int kend = pr.causal ? min(L, q0 + BWD_BLK) : L;
+  const int kend = pr.causal ? min(Lk, q0 + BWD_BLK) : Lk;
   for (int j0 = 0; j0 < kend; j0 += BWD_T) {
     __syncthreads();
-    const int nvalid = L - j0;
+    const int nvalid = Lk - j0;
     copy_rows<T, BWD_T, D, BWD_NT>(Kn, Cfg::LDN, Kg + (size_t)j0 * D, nvalid, tid);
     copy_rows<T, BWD_T, D, BWD_NT>(Vn, Cfg::LDN, Vg + (size_t)j0 * D, nvalid, tid);
     copy_rows_transposed<T, BWD_T, D, BWD_NT>(KT, Cfg::LDT, Kg + (size_t)j0 * D, nvalid, tid);
@@ -191,7 +193,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
     }
 
     const bool diag = pr.causal && (j0 + BWD_T - 1 > q0 + wave * 32);
-    const bool ragged = j0 + BWD_T > L;
+    const bool ragged = j0 + BWD_T > Lk;
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
       const int key0 = j0 + 16 * hf + 8 * g;
@@ -207,7 +209,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
         float pv = fast_exp2(s - Mq);
         if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
         if (diag) pv = (key0 + e <= qrow) ? pv : 0.f;
-        if (ragged) pv = (key0 + e < L) ? pv : 0.f;
+        if (ragged) pv = (key0 + e < Lk) ? pv : 0.f;
         if constexpr (MODE == BWD_PLAIN) {
           S[i] = pv * (dP[i] - d1);
         } else if constexpr (DUAL) {
@@ -271,30 +273,30 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
   float *stats = reinterpret_cast<float *>(trbase + Cfg::DKV_TR * Cfg::T_ELEMS);
   float *sM = stats, *sd1 = stats + BWD_T, *smu = stats + 2 * BWD_T, *sa = stats + 3 * BWD_T, *sd2 = stats + 4 * BWD_T;
 
+  // One workgroup per (batch entry, key/value head, block of 128 keys).  With grouped heads the query
+  // heads of the group are visited one after another and their contributions add up in dK, dV.
   const Problem &pr = p.pr;
-  const int L = pr.L;
-  const int nkb = (L + BWD_BLK - 1) / BWD_BLK;
-  const int total = nkb * pr.Z * pr.H;
-  const int id = xcd_remap(blockIdx.x, nkb, pr.Z * pr.H);
-  const int zh = id / nkb;
+  const int L = pr.L, Lk = pr.Lk;  // queries, keys
+  const int nkb = (Lk + BWD_BLK - 1) / BWD_BLK;
+  const int id = xcd_remap(blockIdx.x, nkb, pr.Z * pr.Hk);
+  const int zhk = id / nkb;
   const int kb = id % nkb;  // causal: the first key blocks have the longest query loops
-  const int z = zh / pr.H, h = zh % pr.H;
+  const int z = zhk / pr.Hk, hk = zhk % pr.Hk, group = pr.H / pr.Hk;
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int r = lane % 32, g = lane / 32, pr32 = perm32(r);
 
-  const size_t head = (size_t)zh * L * D;
-  const size_t srow = (size_t)zh * L;
+  const size_t kvhead = (size_t)zhk * Lk * D;
   const int k0 = kb * BWD_BLK;
   const int krow = k0 + wave * 32 + r;
-  const int kld = krow < L ? krow : L - 1;
+  const int kld = krow < Lk ? krow : Lk - 1;
   const bool has_go = p.go != nullptr;
 
   Frag<T> Kf[KK], Vf[KK], Ktf[DUAL ? KK : 1], Vtf[DUAL ? KK : 1];
-  load_row_frags<KK>(Kf, reinterpret_cast<const T *>(p.k) + head + (size_t)kld * D, g);
-  load_row_frags<KK>(Vf, reinterpret_cast<const T *>(p.v) + head + (size_t)kld * D, g);
+  load_row_frags<KK>(Kf, reinterpret_cast<const T *>(p.k) + kvhead + (size_t)kld * D, g);
+  load_row_frags<KK>(Vf, reinterpret_cast<const T *>(p.v) + kvhead + (size_t)kld * D, g);
   if constexpr (DUAL) {
-    load_row_frags<KK>(Ktf, reinterpret_cast<const T *>(p.kt) + head + (size_t)kld * D, g);
-    load_row_frags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + head + (size_t)kld * D, g);
+    load_row_frags<KK>(Ktf, reinterpret_cast<const T *>(p.kt) + kvhead + (size_t)kld * D, g);
+    load_row_frags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + kvhead + (size_t)kld * D, g);
   }
 
   f32x16 dK[DB], dV[DB];
@@ -305,13 +307,16 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
   }
 
   const float sl2 = pr.scale * LOG2E;
+  const int istart = pr.causal ? (k0 / BWD_T) * BWD_T : 0;
+  for (int gi = 0; gi < group; ++gi) {
+  const int h = hk * group + gi;  // query head
+  const size_t head = ((size_t)z * pr.H + h) * L * D;
+  const size_t srow = ((size_t)z * pr.H + h) * L;
   const T *Qg = reinterpret_cast<const T *>(p.q) + head;
   const T *Qtg = DUAL ? reinterpret_cast<const T *>(p.qt) + head : nullptr;
   const T *gOg = (!TAN && has_go) ? reinterpret_cast<const T *>(p.go) + head : nullptr;
   const T *gTg = (DUAL || TAN) ? reinterpret_cast<const T *>(p.gt) + head : nullptr;
   const T *Gg = TAN ? gTg : gOg;  // tensor staged in Gn / GT
-
-  const int istart = pr.causal ? (k0 / BWD_T) * BWD_T : 0;
   for (int i0 = istart; i0 < L; i0 += BWD_T) {
     __syncthreads();
     const int nvalid = L - i0;
@@ -417,10 +422,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
       }
     }
   }
+  }  // query heads of the group
 
-  if (krow < L) {
-    T *outk = reinterpret_cast<T *>(TAN ? p.dkt : p.dk) + head + (size_t)krow * D;
-    T *outv = reinterpret_cast<T *>(TAN ? p.dvt : p.dv) + head + (size_t)krow * D;
+  if (krow < Lk) {
+    T *outk = reinterpret_cast<T *>(TAN ? p.dkt : p.dk) + kvhead + (size_t)krow * D;
+    T *outv = reinterpret_cast<T *>(TAN ? p.dvt : p.dv) + kvhead + (size_t)krow * D;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
 #pragma unroll

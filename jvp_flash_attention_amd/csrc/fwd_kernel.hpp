@@ -58,13 +58,15 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
   const int r = lane % 32, g = lane / 32;
   const int pr32 = perm32(r);
 
+  const int Lk = pr.Lk;  // keys; L counts queries
   const size_t head = (size_t)zh * L * D;
+  const size_t kvhead = ((size_t)z * pr.Hk + h / (pr.H / pr.Hk)) * Lk * D;  // grouped heads share K, V
   const T *Qg = reinterpret_cast<const T *>(p.q) + head;
-  const T *Kg = reinterpret_cast<const T *>(p.k) + head;
-  const T *Vg = reinterpret_cast<const T *>(p.v) + head;
+  const T *Kg = reinterpret_cast<const T *>(p.k) + kvhead;
+  const T *Vg = reinterpret_cast<const T *>(p.v) + kvhead;
   const T *Qtg = DUAL ? reinterpret_cast<const T *>(p.qt) + head : nullptr;
-  const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + head : nullptr;
-  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + head : nullptr;
+  const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + kvhead : nullptr;
+  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + kvhead : nullptr;
 
   const int q0 = qb * Cfg::BM;         // first query row of the workgroup
   const int qrow = q0 + wave * 32 + r; // this lane's query row
@@ -91,12 +93,12 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
 
-  int kend = L;
-  if (pr.causal) kend = min(L, q0 + Cfg::BM);
+  int kend = Lk;
+  if (pr.causal) kend = min(Lk, q0 + Cfg::BM);
 
   for (int j0 = 0; j0 < kend; j0 += BN) {
     __syncthreads();
-    const int nvalid = L - j0;  // rows >= nvalid are zero-filled
+    const int nvalid = Lk - j0;  // rows >= nvalid are zero-filled
     copy_rows<T, BN, D, Cfg::NT>(Ks, Cfg::LDK, Kg + (size_t)j0 * D, nvalid, tid);
     copy_rows_transposed<T, BN, D, Cfg::NT>(Vs, Cfg::LDV, Vg + (size_t)j0 * D, nvalid, tid);
     if constexpr (DUAL) {
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
 
     // ---- online softmax in the log2 domain (per-lane query column) -------------------------
     const bool diag = pr.causal && (j0 + BN - 1 > q0 + wave * 32);  // some key may exceed a query
-    const bool ragged = j0 + BN > L;
+    const bool ragged = j0 + BN > Lk;
     float mx = NEG_INF;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
           if constexpr (MASK == MASK_ADD) s += bias[e];
           if constexpr (MASK == MASK_BOOL) s = keep[e] ? s : NEG_INF;
           if (diag) s = (key0 + e <= qrow) ? s : NEG_INF;
-          if (ragged) s = (key0 + e < L) ? s : NEG_INF;
+          if (ragged) s = (key0 + e < Lk) ? s : NEG_INF;
           S[nb][8 * hf + e] = s;
           mx = fmaxf(mx, s);
         }

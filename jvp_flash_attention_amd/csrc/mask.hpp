@@ -6,16 +6,16 @@
 namespace jvpfa {
 
 // Boolean mask bytes (nonzero = attend) for keys key0 .. key0+7 of one query row.
-// Keys >= L read as "masked".
+// Keys >= Lk read as "masked".
 __device__ __forceinline__ void mask_keep8(const Problem &pr, int64_t rowoff, int key0, bool keep[8]) {
   const uint8_t *base = reinterpret_cast<const uint8_t *>(pr.mask) + rowoff;
-  if (pr.ms[3] == 1 && key0 + 8 <= pr.L && ((reinterpret_cast<uintptr_t>(base + key0) & 7) == 0)) {
+  if (pr.ms[3] == 1 && key0 + 8 <= pr.Lk && ((reinterpret_cast<uintptr_t>(base + key0) & 7) == 0)) {
     uint64_t w = *reinterpret_cast<const uint64_t *>(base + key0);
 #pragma unroll
     for (int e = 0; e < 8; ++e) keep[e] = ((e < 4 ? (uint32_t)w : (uint32_t)(w >> 32)) & (0xffu << (8 * (e & 3)))) != 0;
   } else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) keep[e] = (key0 + e < pr.L) ? base[(int64_t)(key0 + e) * pr.ms[3]] != 0 : false;
+    for (int e = 0; e < 8; ++e) keep[e] = (key0 + e < pr.Lk) ? base[(int64_t)(key0 + e) * pr.ms[3]] != 0 : false;
   }
 }
 
@@ -23,14 +23,14 @@ __device__ __forceinline__ void mask_keep8(const Problem &pr, int64_t rowoff, in
 template <typename T>
 __device__ __forceinline__ void mask_bias8(const Problem &pr, int64_t rowoff, int key0, float bias[8]) {
   const T *base = reinterpret_cast<const T *>(pr.mask) + rowoff;
-  if (pr.ms[3] == 1 && key0 + 8 <= pr.L && ((reinterpret_cast<uintptr_t>(base + key0) & 15) == 0)) {
+  if (pr.ms[3] == 1 && key0 + 8 <= pr.Lk && ((reinterpret_cast<uintptr_t>(base + key0) & 15) == 0)) {
     Frag<T> w = ld8<T>(base + key0);
 #pragma unroll
     for (int e = 0; e < 8; ++e) bias[e] = (float)w[e] * LOG2E;
   } else {
 #pragma unroll
     for (int e = 0; e < 8; ++e)
-      bias[e] = (key0 + e < pr.L) ? (float)base[(int64_t)(key0 + e) * pr.ms[3]] * LOG2E : 0.f;
+      bias[e] = (key0 + e < pr.Lk) ? (float)base[(int64_t)(key0 + e) * pr.ms[3]] * LOG2E : 0.f;
   }
 }
 
@@ -66,7 +66,7 @@ __device__ __forceinline__ MaskAhead<T, MASK> mask_fetch8_any(const Problem &pr,
     uint32_t lo = 0, hi = 0;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const uint32_t b = base[(int64_t)min(key0 + e, pr.L - 1) * pr.ms[3]] != 0 ? 0xffu : 0u;
+      const uint32_t b = base[(int64_t)min(key0 + e, pr.Lk - 1) * pr.ms[3]] != 0 ? 0xffu : 0u;
       if (e < 4) lo |= b << (8 * e);
       else hi |= b << (8 * (e - 4));
     }
@@ -74,7 +74,7 @@ __device__ __forceinline__ MaskAhead<T, MASK> mask_fetch8_any(const Problem &pr,
   } else {
     const T *base = reinterpret_cast<const T *>(pr.mask) + rowoff;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) m.f[e] = base[(int64_t)min(key0 + e, pr.L - 1) * pr.ms[3]];
+    for (int e = 0; e < 8; ++e) m.f[e] = base[(int64_t)min(key0 + e, pr.Lk - 1) * pr.ms[3]];
   }
   return m;
 }

@@ -19,6 +19,9 @@ Differences from the reference, all deliberate:
   reference's tangent is a constant (JA:2399, JA:2828) and its backward ignores it (JA:2831).
 * Any sequence length L >= 1 and head dims {32, 64, 128, 256} (the reference: L a multiple of 32,
   JA:2371-2378, JA:2892); D = 256 for bf16 / fp16 only.
+* k and v may have fewer heads than q (grouped heads: H a multiple of H_kv) and a length of their own
+  (cross-attention); causal then means key index <= query index, as in SDPA.  The reference requires
+  q, k, v of one shape (JA:2367-2378).  Such calls run on the general kernels, not the tuned ones.
 * ``attention`` notices dual inputs and then behaves like ``fwd_dual`` (the reference's ``attention``
   is ``JVPAttn.fwd`` and drops the tangent, its README.md:65-67).
 """
@@ -54,9 +57,9 @@ def _validate(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dropout
     assert HEAD_DIM_K in SUPPORTED_HEAD_DIMS, (
         f"JVP attention only supports HEAD_DIM_K in {set(SUPPORTED_HEAD_DIMS)}, but got HEAD_DIM_K={HEAD_DIM_K}"
     )
-    assert k.shape == q.shape and v.shape == q.shape, (
-        "JVP attention requires q, k, v of one shape (no cross-attention or grouped heads),"
-        f" but got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}"
+    assert k.shape == v.shape and k.shape[0] == Z and H % k.shape[1] == 0, (
+        "JVP attention requires k and v of one shape (Z, H_kv, N_CTX_kv, HEAD_DIM) with H a multiple of H_kv,"
+        f" but got q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}"
     )
     assert not (HEAD_DIM_K == 256 and q.dtype == torch.float32), (
         "JVP attention supports HEAD_DIM_K=256 for bfloat16 and float16 only"
@@ -69,8 +72,8 @@ def _validate(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dropout
         raise ValueError("Causal attention does not support an attention mask.")
     if attn_mask is not None:
         assert attn_mask.dim() == 4 and all(
-            m in (1, full) for m, full in zip(attn_mask.shape, (Z, H, N_CTX, N_CTX))
-        ), "The provided attention mask must have 4 dimensions broadcastable to (Z, H, N_CTX, N_CTX)."
+            m in (1, full) for m, full in zip(attn_mask.shape, (Z, H, N_CTX, k.shape[2]))
+        ), "The provided attention mask must have 4 dimensions broadcastable to (Z, H, N_CTX, N_CTX_kv)."
         assert attn_mask.dtype in {torch.bool, q.dtype}, (
             "The attention mask must be of the dtype bool or that of the query tensor."
         )

@@ -33,13 +33,27 @@ import numpy as np
 LOG2E = 1.4426950408889634
 
 
+def _expand_heads(x, H):
+    """Grouped heads (not in the reference, which requires q, k, v of one shape, ``:2367-2378``): k, v
+    may have fewer heads than q; query head h reads key/value head h // (H / Hk)."""
+    Hk = x.shape[1]
+    assert H % Hk == 0, "the number of query heads must be a multiple of the number of key/value heads"
+    return x if Hk == H else np.repeat(x, H // Hk, axis=1)
+
+
+def _reduce_heads(g, Hk):
+    Z, H, L, D = g.shape
+    return g if H == Hk else g.reshape(Z, Hk, H // Hk, L, D).sum(axis=2)
+
+
 def _logits(q, k, mask, causal, scale):
-    """Scaled, masked logits S (fp64) and the boolean 'attend' pattern."""
-    L = q.shape[-2]
+    """Scaled, masked logits S (fp64) and the boolean 'attend' pattern.  q and k may differ in length;
+    causal then means key index <= query index, as in SDPA."""
+    Lq, Lk = q.shape[-2], k.shape[-2]
     s = scale * np.einsum("zhid,zhjd->zhij", q, k)
     keep = np.ones(s.shape, dtype=bool)
     if causal:
-        keep &= np.tril(np.ones((L, L), dtype=bool))
+        keep &= np.tril(np.ones((Lq, Lk), dtype=bool))
     if mask is not None:
         mask = np.asarray(mask)
         if mask.dtype == np.bool_:
@@ -65,13 +79,15 @@ def _softmax(s, keep):
 def forward(q, k, v, qt=None, kt=None, vt=None, mask=None, causal=False, scale=None):
     """Returns dict with O, M and (when tangents are given) O', mu, plus P, S' for reuse."""
     q, k, v = (np.asarray(x, dtype=np.float64) for x in (q, k, v))
-    D = q.shape[-1]
+    D, H = q.shape[-1], q.shape[1]
+    k, v = _expand_heads(k, H), _expand_heads(v, H)
     scale = D**-0.5 if scale is None else scale
     s, keep = _logits(q, k, mask, causal, scale)
     p, M = _softmax(s, keep)
     out = {"O": p @ v, "M": M, "P": p, "scale": scale}
     if qt is not None:
         qt, kt, vt = (np.asarray(x, dtype=np.float64) for x in (qt, kt, vt))
+        kt, vt = _expand_heads(kt, H), _expand_heads(vt, H)
         sp = scale * (np.einsum("zhid,zhjd->zhij", qt, k) + np.einsum("zhid,zhjd->zhij", q, kt))
         mu = (p * sp).sum(-1, keepdims=True)
         pp = p * (sp - mu)
@@ -85,6 +101,8 @@ def backward(q, k, v, qt, kt, vt, go, gt=None, mask=None, causal=False, scale=No
         qt, kt, vt = (np.zeros_like(np.asarray(x, dtype=np.float64)) for x in (q, k, v))
     f = forward(q, k, v, qt, kt, vt, mask=mask, causal=causal, scale=scale)
     q, k, v, qt, kt, vt, go = (np.asarray(x, dtype=np.float64) for x in (q, k, v, qt, kt, vt, go))
+    H, Hk = q.shape[1], k.shape[1]
+    k, v, kt, vt = (_expand_heads(x, H) for x in (k, v, kt, vt))
     p, sc = f["P"], f["scale"]
     T = lambda x: np.swapaxes(x, -1, -2)  # noqa: E731
     d1 = (go * f["O"]).sum(-1, keepdims=True)
@@ -105,9 +123,9 @@ def backward(q, k, v, qt, kt, vt, go, gt=None, mask=None, causal=False, scale=No
         dvt = T(p) @ gt
     return {
         "dq": sc * (ds @ k + dsp @ kt),
-        "dk": sc * (T(ds) @ q + T(dsp) @ qt),
-        "dv": dv,
+        "dk": _reduce_heads(sc * (T(ds) @ q + T(dsp) @ qt), Hk),
+        "dv": _reduce_heads(dv, Hk),
         "dqt": sc * (dsp @ k),
-        "dkt": sc * (T(dsp) @ q),
-        "dvt": dvt,
+        "dkt": _reduce_heads(sc * (T(dsp) @ q), Hk),
+        "dvt": _reduce_heads(dvt, Hk),
     }

@@ -22,7 +22,8 @@ class OracleBackend:
 
     def fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
         self.calls.append(("fwd", qt is not None, mask_kind, bool(causal)))
-        f = lambda t: None if t is None else t.double()  # noqa: E731
+        G = q.shape[1] // k.shape[1]  # grouped heads: the tile-loop restatement wants them repeated
+        f = lambda t: None if t is None else (t.double() if t.shape[1] == q.shape[1] else t.double().repeat_interleave(G, 1))  # noqa: E731
         m = self._mask(mask, mask_kind)
         m = m if m is None or m.dtype == torch.bool else m.double()
         o, ot, M, mu = tiled.forward(f(q), f(k), f(v), f(qt), f(kt), f(vt), mask=m, causal=causal, scale=sm_scale)
@@ -32,7 +33,8 @@ class OracleBackend:
     def bwd(self, q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
             want_tangent_grads=False):
         self.calls.append(("bwd", gt is not None, mask_kind, bool(causal), want_tangent_grads))
-        f = lambda t: None if t is None else t.double()  # noqa: E731
+        Z, H, Hk = q.shape[0], q.shape[1], k.shape[1]
+        f = lambda t: None if t is None else (t.double() if t.dim() != 4 or t.shape[1] == H else t.double().repeat_interleave(H // Hk, 1))  # noqa: E731
         m = self._mask(mask, mask_kind)
         m = m if m is None or m.dtype == torch.bool else m.double()
         if go is None:
@@ -40,8 +42,9 @@ class OracleBackend:
         g = tiled.backward(f(q), f(k), f(v), f(qt), f(kt), f(vt), f(o), f(ot), f(M), f(mu), f(go), f(gt),
                            mask=m, causal=causal, scale=sm_scale)
         c = lambda t: t.to(q.dtype)  # noqa: E731
-        tg = (c(g["dqt"]), c(g["dkt"]), c(g["dvt"])) if want_tangent_grads else (None, None, None)
-        return (c(g["dq"]), c(g["dk"]), c(g["dv"]), *tg)
+        kv = lambda t: c(t if Hk == H else t.reshape(Z, Hk, H // Hk, *t.shape[2:]).sum(2))  # noqa: E731
+        tg = (c(g["dqt"]), kv(g["dkt"]), kv(g["dvt"])) if want_tangent_grads else (None, None, None)
+        return (c(g["dq"]), kv(g["dk"]), kv(g["dv"]), *tg)
 
 
 @contextlib.contextmanager

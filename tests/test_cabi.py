@@ -90,19 +90,28 @@ def test_forward_argument_validation_codes(kw, code):
     assert lib.jvpfa_error_string(code).decode() not in ("ok", "unknown status")
 
 
+def test_key_value_shape_fields_are_checked():
+    lib = _lib.load()
+    for kw, code in ((dict(Hk=3), -2), (dict(Hk=-1), -2), (dict(Lk=-5), -2), (dict(Hk=8), -2)):
+        a = _fwd_args(p_H=4, **kw)
+        assert lib.jvpfa_fwd(C.byref(a), None) == code, kw
+    a = _fwd_args(p_H=4, Hk=2, Lk=77, q=None)
+    assert lib.jvpfa_fwd(C.byref(a), None) == -1  # shape accepted; stops at the NULL pointer
+
+
 def test_earlier_struct_sizes_are_still_accepted():
     """A caller built against version 1 passes structs that end before key_limit, one built against
-    version 2 structs that end before tiles_q."""
+    version 2 structs that end before tiles_q, one built against version 3 structs that end before Lk."""
     lib = _lib.load()
     a = _fwd_args(q=None)
-    for size in (_lib.FwdArgs.key_limit.offset, _lib.FwdArgs.tiles_q.offset, C.sizeof(_lib.FwdArgs)):
+    for size in (_lib.FwdArgs.key_limit.offset, _lib.FwdArgs.tiles_q.offset, _lib.FwdArgs.Lk.offset, C.sizeof(_lib.FwdArgs)):
         a.struct_size = size
         assert lib.jvpfa_fwd(C.byref(a), None) == -1  # got past the size check, to the NULL pointer check
     a.struct_size = _lib.FwdArgs.key_limit.offset - 8
     assert lib.jvpfa_fwd(C.byref(a), None) == -7
     b = _lib.BwdArgs()
     b.p.Z, b.p.H, b.p.L, b.p.D = 1, 1, 32, 64
-    for size in (_lib.BwdArgs.key_limit.offset, _lib.BwdArgs.tiles_q.offset, C.sizeof(_lib.BwdArgs)):
+    for size in (_lib.BwdArgs.key_limit.offset, _lib.BwdArgs.tiles_q.offset, _lib.BwdArgs.Lk.offset, C.sizeof(_lib.BwdArgs)):
         b.struct_size = size
         assert lib.jvpfa_bwd(C.byref(b), None) == -1
 

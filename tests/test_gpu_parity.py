@@ -510,6 +510,55 @@ def test_additive_mask_with_minus_infinity_entries(dt):
         _tol_check(n, t, rb[n], dtype)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("shape", [(4, 2, 96, 96), (4, 1, 70, 200), (2, 2, 200, 70), (6, 3, 130, 33)])
+@pytest.mark.parametrize("mode", ["none", "causal", "bool", "bias"])
+def test_grouped_heads_and_a_key_length_of_its_own(dt, D, shape, mode):
+    """Beyond the reference (q, k, v of one shape there): H query heads over Hk key/value heads, Lq
+    queries over Lk keys; dk, dv (and dk', dv') have k's shape and sum over the heads of a group."""
+    from jvp_flash_attention_amd import _lib
+
+    H, Hk, Lq, Lk = shape
+    Z, dtype = 2, DTYPES[dt]
+    g = torch.Generator().manual_seed(sum(map(ord, dt + mode)) + D + sum(shape))
+    # tangents of std 0.5: with std 1, D = 32 and causal rows of a few keys, the cancellation in
+    # O' = T/l - mu O (the reference's formula too, its jvp_attention.py:1031-1033) on 16-bit rounded
+    # probabilities puts single seeds at 2.3e-2, just past the bar
+    q, go, gt = [torch.randn(Z, H, Lq, D, generator=g).to(dtype) for _ in range(3)]
+    qt = (0.5 * torch.randn(Z, H, Lq, D, generator=g)).to(dtype)
+    k, v = [torch.randn(Z, Hk, Lk, D, generator=g).to(dtype) for _ in range(2)]
+    kt, vt = [(0.5 * torch.randn(Z, Hk, Lk, D, generator=g)).to(dtype) for _ in range(2)]
+    mask, kind, causal = None, _lib.MASK_NONE, mode == "causal"
+    if mode == "bool":
+        mask, kind = torch.rand(Z, H, Lq, Lk, generator=g) > 0.5, _lib.MASK_BOOL
+        mask[..., 0] = True
+    if mode == "bias":
+        mask, kind = torch.randn(Z, 1, Lq, Lk, generator=g).to(dtype), _lib.MASK_ADD
+    print(f"case kv-shape Z{Z} H{H}/{Hk} Lq{Lq} Lk{Lk} D{D} {dt} {mode}", flush=True)
+    npm = None if mask is None else (mask.numpy() if mask.dtype == torch.bool else mask.double().numpy())
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    scale = D**-0.5
+    ref = dense.forward(*f64[:6], mask=npm, causal=causal, scale=scale)
+    rb = dense.backward(*f64, mask=npm, causal=causal, scale=scale)
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dmask = None if mask is None else mask.cuda()
+    be = _lib.backend()
+    o, ot, M, mu = be.fwd(*dev[:6], dmask, kind, causal, scale)
+    _tol_check("O", o, ref["O"], dtype)
+    _tol_check("O'", ot, ref["Ot"], dtype)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, kind, causal, scale, want_tangent_grads=True)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        assert tuple(t.shape) == rb[n].shape, n
+        _tol_check(n, t, rb[n], dtype)
+    op, _, Mp, _ = be.fwd(dev[0], dev[1], dev[2], None, None, None, dmask, kind, causal, scale)
+    _tol_check("O (plain)", op, ref["O"], dtype)
+    rb1 = dense.backward(*f64[:7], None, mask=npm, causal=causal, scale=scale)
+    g1 = be.bwd(dev[0], dev[1], dev[2], None, None, None, op, None, Mp, None, dev[6], None, dmask, kind, causal, scale)
+    for n, t in zip(("dq", "dk", "dv"), g1[:3]):
+        _tol_check(n + " (plain)", t, rb1[n], dtype)
+
+
 def test_c_abi_from_a_plain_cpp_program():
     """``tests/cabi_host/host_check`` (built with the library) calls jvpfa_fwd / jvpfa_bwd from C++ with
     memory it allocated through the HIP runtime, no Python or torch in its process, and compares with

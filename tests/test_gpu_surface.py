@@ -191,6 +191,39 @@ def test_dual_tensors_inside_torch_compile_keep_their_tangent():
     assert torch.equal(o1, o2) and torch.equal(ot1, ot2)
 
 
+def test_surface_grouped_heads_and_cross_attention():
+    """k, v with fewer heads and another length than q through the public functions: forward-mode
+    tangent, and gradients of a loss on O and O' with k's shape for dk, dv (summed over each group)."""
+    from jvp_flash_attention_amd import JVPAttn, attention
+
+    Z, H, Hk, Lq, Lk, D = 2, 4, 2, 100, 150, 64
+    dt = torch.bfloat16
+    q, qt, go, gt = [_randn((Z, H, Lq, D), dt, 90 + i) for i in range(4)]
+    k, v, kt, vt = [_randn((Z, Hk, Lk, D), dt, 95 + i) for i in range(4)]
+    mask = torch.rand(Z, 1, Lq, Lk, device="cuda", generator=torch.Generator(device="cuda").manual_seed(3)) > 0.4
+    mask[..., 0] = True
+    f64 = [x.double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    ref = dense.forward(*f64[:6], mask=mask.cpu().numpy())
+    rb = dense.backward(*f64, mask=mask.cpu().numpy())
+    leaves = [x.clone().requires_grad_() for x in (q, k, v, qt, kt, vt)]
+    with fwAD.dual_level():
+        out = JVPAttn.fwd_dual(*(fwAD.make_dual(p, t) for p, t in zip(leaves[:3], leaves[3:])), attn_mask=mask)
+        o, ot = fwAD.unpack_dual(out)
+        loss = (o.float() * go.float()).sum() + (ot.float() * gt.float()).sum()
+        grads = torch.autograd.grad(loss, leaves)
+    assert _rel(o, ref["O"]) <= 2e-2 and _rel(ot, ref["Ot"]) <= 2e-2
+    for n, g in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        assert tuple(g.shape) == rb[n].shape and _rel(g, rb[n]) <= 2e-2, n
+    ql, kl, vl = [x.clone().requires_grad_() for x in (q, k, v)]
+    o_plain = attention(ql, kl, vl, causal=True)
+    g1 = torch.autograd.grad((o_plain.float() * go.float()).sum(), (ql, kl, vl))
+    refc = dense.forward(*f64[:3], causal=True)
+    rbc = dense.backward(*f64[:3], None, None, None, f64[6], None, causal=True)
+    assert _rel(o_plain, refc["O"]) <= 2e-2
+    for n, g in zip(("dq", "dk", "dv"), g1):
+        assert _rel(g, rbc[n]) <= 2e-2, n
+
+
 def test_plain_attention_autograd_and_apply_tuple():
     from jvp_flash_attention_amd import JVPAttn, attention
 

@@ -58,6 +58,37 @@ def test_dense_matches_sdpa_library_route(mode):
         assert np.abs(b1[name]).max() == 0.0
 
 
+@pytest.mark.parametrize("mode", ["none", "causal", "bool", "bias"])
+@pytest.mark.parametrize("Hk,Lk", [(1, 24), (2, 40), (4, 24)])
+def test_dense_with_grouped_heads_and_unequal_lengths_matches_the_library_route(mode, Hk, Lk):
+    """Beyond the reference (which requires q, k, v of one shape): fewer key/value heads than query
+    heads and a key length that differs from the query length.  The library route repeats the
+    key/value heads explicitly, so autograd sums their gradients over each group."""
+    Z, H, Lq, D = 2, 4, 24, 16
+    g = torch.Generator().manual_seed(7)
+    q, qt, go, gt = [torch.randn(Z, H, Lq, D, generator=g, dtype=torch.float64) for _ in range(4)]
+    k, v, kt, vt = [torch.randn(Z, Hk, Lk, D, generator=g, dtype=torch.float64) for _ in range(4)]
+    mask, causal = None, mode == "causal"
+    if mode == "bool":
+        mask = torch.rand(Z, H, Lq, Lk, generator=g) > 0.5
+        mask[..., 0] = True
+    if mode == "bias":
+        mask = torch.randn(Z, 1, Lq, Lk, generator=g, dtype=torch.float64)
+    leaves = [x.clone().requires_grad_() for x in (q, k, v, qt, kt, vt)]
+    rep = lambda x: x.repeat_interleave(H // Hk, dim=1)  # noqa: E731
+    o, ot = sdpa_jvp.forward(leaves[0], rep(leaves[1]), rep(leaves[2]), leaves[3], rep(leaves[4]), rep(leaves[5]),
+                             attn_mask=mask, causal=causal)
+    grads = torch.autograd.grad((o * go).sum() + (ot * gt).sum(), leaves)
+    npm = None if mask is None else mask.numpy()
+    f = dense.forward(*(x.numpy() for x in (q, k, v, qt, kt, vt)), mask=npm, causal=causal)
+    b = dense.backward(*(x.numpy() for x in (q, k, v, qt, kt, vt, go, gt)), mask=npm, causal=causal)
+    assert np.abs(f["O"] - o.detach().numpy()).max() < 1e-12
+    assert np.abs(f["Ot"] - ot.detach().numpy()).max() < 1e-12
+    for name, ref in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        assert b[name].shape == tuple(ref.shape), name
+        assert np.abs(b[name] - ref.numpy()).max() < 1e-11, name
+
+
 def test_dense_M_and_mu_definitions():
     q, k, v, qt, kt, vt, _, _ = _inputs()
     f = dense.forward(*(x.numpy() for x in (q, k, v, qt, kt, vt)))
