@@ -4,4 +4,9 @@ from jvp_flash_attention_amd.jvp_attention import (  # noqa: F401
     MIN_SEQUENCE_LENGTH,
     JVPAttn,
     attention,
+    is_blackwell,
+    is_cuda,
+    is_hip,
+    supports_host_descriptor,
+    supports_tma,
 )

@@ -43,6 +43,27 @@ SUPPORTED_HEAD_DIMS = (32, 64, 128, 256)  # 256: bf16 / fp16 only
 BLOCK_M = 128  # query rows per workgroup of the forward kernel (only reported through Grid)
 
 
+def is_hip() -> bool:
+    """Platform probes of the reference (JA:54-92), kept for importers: this build is HIP-only."""
+    return True
+
+
+def is_cuda() -> bool:
+    return False
+
+
+def supports_host_descriptor() -> bool:
+    return False
+
+
+def supports_tma() -> bool:
+    return False
+
+
+def is_blackwell() -> bool:
+    return False
+
+
 def _validate(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dropout_p: float, causal: bool):
     """Argument checks of JA:2356-2392, with this build's shape limits."""
     if dropout_p != 0.0:
