@@ -211,6 +211,51 @@ class _AttachTangent(Function):
         return g, None, None, None, None
 
 
+# Twins of the three Functions above in the older style (``forward(ctx, ...)``, no ``setup_context``).
+# ``Function.apply`` binds the arguments of a ``setup_context`` Function through ``inspect.signature``
+# on every call, about 25 us each; that style is only needed under ``torch.func`` transforms and
+# while ``torch.compile`` traces, so ordinary eager calls take these.
+
+
+class _DualCoreEager(Function):
+    @staticmethod
+    def forward(ctx, q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale):
+        o, o_t, M, mu = _lib.backend().fwd(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale)
+        ctx.mark_non_differentiable(M, mu)
+        ctx.save_for_backward(q, k, v, q_t, k_t, v_t, o, o_t, M, mu)
+        ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale = mask_tensor, MASK_TYPE, causal, sm_scale
+        return o, o_t, M, mu
+
+    backward = _DualCore.backward
+
+
+class _PlainCoreEager(Function):
+    @staticmethod
+    def forward(ctx, q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale):
+        o, _o_t, M, _mu = _lib.backend().fwd(q, k, v, None, None, None, mask_tensor, MASK_TYPE, causal, sm_scale)
+        ctx.mark_non_differentiable(M)
+        ctx.save_for_backward(q, k, v, o, M)
+        ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale = mask_tensor, MASK_TYPE, causal, sm_scale
+        return o, M
+
+    backward = _PlainCore.backward
+
+
+class _AttachTangentEager(Function):
+    @staticmethod
+    def forward(ctx, o, o_t, q, k, v):
+        ctx.save_for_forward(o_t)
+        return o.view_as(o)
+
+    jvp = _AttachTangent.jvp
+    backward = _AttachTangent.backward
+
+
+def _transforms_active() -> bool:
+    """A ``torch.func`` transform (jvp, vmap, grad ...) is running."""
+    return torch._C._functorch.peek_interpreter_stack() is not None
+
+
 class JVPAttn(Function):
     """JVP (Jacobian-Vector Product) for Attention Mechanism."""
 
@@ -362,6 +407,14 @@ class JVPAttn(Function):
             mask_tensor, MASK_TYPE = _classify_mask(attn_mask, q, False)
             o, _M = _PlainCore.apply(q, k, v, mask_tensor, MASK_TYPE, causal, scale)
             return o
+        if fwAD._current_level < 0 and not _transforms_active():
+            # no forward-mode level anywhere: nothing can ask for a tangent, so the plain Function
+            # (same kernels, same backward) stands in for JVPAttn.apply and its per-call set-up
+            _validate(q, k, v, attn_mask, dropout_p, causal)
+            scale = q.shape[-1] ** -0.5 if sm_scale is None else sm_scale
+            mask_tensor, MASK_TYPE = _classify_mask(attn_mask, q, True)
+            o, _M = _PlainCoreEager.apply(q, k, v, mask_tensor, MASK_TYPE, causal, scale)
+            return o
         out: JVPAttn.FwdOut = JVPAttn.apply(
             q, k, v, None, None, None, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA
         )
@@ -406,11 +459,12 @@ class JVPAttn(Function):
         q_t = torch.zeros_like(q_p) if q_t is None else _dense(q_t)
         k_t = torch.zeros_like(k_p) if k_t is None else _dense(k_t)
         v_t = torch.zeros_like(v_p) if v_t is None else _dense(v_t)
-        o, o_t, _M, _mu = _DualCore.apply(
+        core, attach = (_DualCore, _AttachTangent) if _transforms_active() else (_DualCoreEager, _AttachTangentEager)
+        o, o_t, _M, _mu = core.apply(
             _dense(q_p), _dense(k_p), _dense(v_p), q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale
         )
         # NOTE: q, k, v are passed as dual tensors so that autograd calls jvp(), which hands back O'.
-        return _AttachTangent.apply(o, o_t, q, k, v)
+        return attach.apply(o, o_t, q, k, v)
 
     @staticmethod
     def jvp(ctx: "JVPAttn.FnCtx", gq: Tensor, gk: Tensor, gv: Tensor, *_) -> "JVPAttn.JVPOut":
