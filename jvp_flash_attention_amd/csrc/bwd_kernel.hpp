@@ -79,6 +79,10 @@ template <typename T, int D, int MODE> struct BwdCfg {
   static constexpr size_t DKV_LDS = (size_t)(DKV_NAT * N_ELEMS + DKV_TR * T_ELEMS) * sizeof(T) + 5 * BWD_T * sizeof(float);
 };
 
+// whether the dq / dk,dv kernels fetch the next tile into registers during the current one's
+// computation (needs up to 64 registers; see the forward kernel)
+template <typename T, int D> constexpr bool BWD_FETCH_AHEAD = D == 64 || (D == 32 && sizeof(T) == 4);
+
 template <int KK, typename T>
 __device__ __forceinline__ void load_row_frags(Frag<T> *f, const T *row, int g) {
 #pragma unroll
@@ -160,18 +164,50 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
   const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + kvhead : nullptr;
 
   const int kend = pr.causal ? min(Lk, q0 + BWD_BLK) : Lk;
+  // The next tile is fetched into registers while this one is computed and written to LDS behind the
+  // barrier that follows; K (, K') is fetched once and written both ways.  (See the forward kernel for
+  // where this is left out.)
+  constexpr bool AHEAD = BWD_FETCH_AHEAD<T, D>;
+  QuadChunks<T, BWD_T, D, BWD_NT> rk, rkt;
+  RowChunks<T, BWD_T, D, BWD_NT> rv, rvt;
+  auto fetch_tile = [&](int j0) {
+    const int nvalid = Lk - j0;
+    fetch_quads(rk, Kg + (size_t)j0 * D, nvalid, tid);
+    fetch_rows(rv, Vg + (size_t)j0 * D, nvalid, tid);
+    if constexpr (DUAL) {
+      fetch_quads(rkt, Ktg + (size_t)j0 * D, nvalid, tid);
+      fetch_rows(rvt, Vtg + (size_t)j0 * D, nvalid, tid);
+    }
+  };
+  if constexpr (AHEAD) {
+    if (kend > 0) fetch_tile(0);
+  }
   for (int j0 = 0; j0 < kend; j0 += BWD_T) {
     __syncthreads();
-    const int nvalid = Lk - j0;
-    copy_rows<T, BWD_T, D, BWD_NT>(Kn, Cfg::LDN, Kg + (size_t)j0 * D, nvalid, tid);
-    copy_rows<T, BWD_T, D, BWD_NT>(Vn, Cfg::LDN, Vg + (size_t)j0 * D, nvalid, tid);
-    copy_rows_transposed<T, BWD_T, D, BWD_NT>(KT, Cfg::LDT, Kg + (size_t)j0 * D, nvalid, tid);
-    if constexpr (DUAL) {
-      copy_rows<T, BWD_T, D, BWD_NT>(Ktn, Cfg::LDN, Ktg + (size_t)j0 * D, nvalid, tid);
-      copy_rows<T, BWD_T, D, BWD_NT>(Vtn, Cfg::LDN, Vtg + (size_t)j0 * D, nvalid, tid);
-      copy_rows_transposed<T, BWD_T, D, BWD_NT>(KtT, Cfg::LDT, Ktg + (size_t)j0 * D, nvalid, tid);
+    if constexpr (AHEAD) {
+      put_quads_rows(Kn, Cfg::LDN, rk, tid);
+      put_quads_transposed(KT, Cfg::LDT, rk, tid);
+      put_rows(Vn, Cfg::LDN, rv, tid);
+      if constexpr (DUAL) {
+        put_quads_rows(Ktn, Cfg::LDN, rkt, tid);
+        put_quads_transposed(KtT, Cfg::LDT, rkt, tid);
+        put_rows(Vtn, Cfg::LDN, rvt, tid);
+      }
+    } else {
+      const int nvalid = Lk - j0;
+      copy_rows<T, BWD_T, D, BWD_NT>(Kn, Cfg::LDN, Kg + (size_t)j0 * D, nvalid, tid);
+      copy_rows<T, BWD_T, D, BWD_NT>(Vn, Cfg::LDN, Vg + (size_t)j0 * D, nvalid, tid);
+      copy_rows_transposed<T, BWD_T, D, BWD_NT>(KT, Cfg::LDT, Kg + (size_t)j0 * D, nvalid, tid);
+      if constexpr (DUAL) {
+        copy_rows<T, BWD_T, D, BWD_NT>(Ktn, Cfg::LDN, Ktg + (size_t)j0 * D, nvalid, tid);
+        copy_rows<T, BWD_T, D, BWD_NT>(Vtn, Cfg::LDN, Vtg + (size_t)j0 * D, nvalid, tid);
+        copy_rows_transposed<T, BWD_T, D, BWD_NT>(KtT, Cfg::LDT, Ktg + (size_t)j0 * D, nvalid, tid);
+      }
     }
     __syncthreads();
+    if constexpr (AHEAD) {
+      if (j0 + BWD_T < kend) fetch_tile(j0 + BWD_T);
+    }
 
     f32x16 S, dP, Sp, At, Bt;
     zero16(S);
@@ -317,31 +353,76 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
   const T *gOg = (!TAN && has_go) ? reinterpret_cast<const T *>(p.go) + head : nullptr;
   const T *gTg = (DUAL || TAN) ? reinterpret_cast<const T *>(p.gt) + head : nullptr;
   const T *Gg = TAN ? gTg : gOg;  // tensor staged in Gn / GT
-  for (int i0 = istart; i0 < L; i0 += BWD_T) {
-    __syncthreads();
-    const int nvalid = L - i0;
-    copy_rows<T, BWD_T, D, BWD_NT>(Qn, Cfg::LDN, Qg + (size_t)i0 * D, nvalid, tid);
-    copy_rows_transposed<T, BWD_T, D, BWD_NT>(QT, Cfg::LDT, Qg + (size_t)i0 * D, nvalid, tid);
-    if (Gg) {
-      copy_rows<T, BWD_T, D, BWD_NT>(Gn, Cfg::LDN, Gg + (size_t)i0 * D, nvalid, tid);
-      copy_rows_transposed<T, BWD_T, D, BWD_NT>(GT, Cfg::LDT, Gg + (size_t)i0 * D, nvalid, tid);
-    }
-    if constexpr (DUAL) {
-      copy_rows<T, BWD_T, D, BWD_NT>(Qtn, Cfg::LDN, Qtg + (size_t)i0 * D, nvalid, tid);
-      copy_rows_transposed<T, BWD_T, D, BWD_NT>(QtT, Cfg::LDT, Qtg + (size_t)i0 * D, nvalid, tid);
-      copy_rows<T, BWD_T, D, BWD_NT>(GTn, Cfg::LDN, gTg + (size_t)i0 * D, nvalid, tid);
-      copy_rows_transposed<T, BWD_T, D, BWD_NT>(GTT, Cfg::LDT, gTg + (size_t)i0 * D, nvalid, tid);
-    }
+  // The next tile (each tensor once, written to LDS both ways) and its row statistics are fetched
+  // into registers while this tile is computed, as in the dq kernel.
+  constexpr bool AHEAD = BWD_FETCH_AHEAD<T, D>;
+  QuadChunks<T, BWD_T, D, BWD_NT> rq, rg, rqt, rgt;
+  float rs[5] = {0.f, 0.f, 0.f, 0.f, 0.f};  // M, d1, mu, a, d2 of query row i0 + tid
+  auto fetch_stats = [&](int i0) {
     if (tid < BWD_T) {
       const bool ok = i0 + tid < L;
       const size_t si = srow + (ok ? i0 + tid : 0);
-      sM[tid] = ok ? p.M[si] : __builtin_inff();
-      sd1[tid] = (ok && MODE == BWD_PLAIN) ? p.d1[si] : 0.f;  // BWD_DUAL: d2 already holds d1 + d2
-      smu[tid] = (ok && DUAL) ? p.mu[si] : 0.f;
-      sa[tid] = (ok && (DUAL || TAN)) ? p.a[si] : 0.f;
-      sd2[tid] = (ok && DUAL) ? p.d2[si] : 0.f;
+      rs[0] = ok ? p.M[si] : __builtin_inff();
+      rs[1] = (ok && MODE == BWD_PLAIN) ? p.d1[si] : 0.f;  // BWD_DUAL: d2 already holds d1 + d2
+      rs[2] = (ok && DUAL) ? p.mu[si] : 0.f;
+      rs[3] = (ok && (DUAL || TAN)) ? p.a[si] : 0.f;
+      rs[4] = (ok && DUAL) ? p.d2[si] : 0.f;
     }
+  };
+  auto put_stats = [&]() {
+    if (tid < BWD_T) {
+      sM[tid] = rs[0], sd1[tid] = rs[1], smu[tid] = rs[2], sa[tid] = rs[3], sd2[tid] = rs[4];
+    }
+  };
+  auto fetch_tile = [&](int i0) {
+    const int nvalid = L - i0;
+    fetch_quads(rq, Qg + (size_t)i0 * D, nvalid, tid);
+    if (Gg) fetch_quads(rg, Gg + (size_t)i0 * D, nvalid, tid);
+    if constexpr (DUAL) {
+      fetch_quads(rqt, Qtg + (size_t)i0 * D, nvalid, tid);
+      fetch_quads(rgt, gTg + (size_t)i0 * D, nvalid, tid);
+    }
+    fetch_stats(i0);
+  };
+  if constexpr (AHEAD) {
+    if (istart < L) fetch_tile(istart);
+  }
+  for (int i0 = istart; i0 < L; i0 += BWD_T) {
     __syncthreads();
+    if constexpr (AHEAD) {
+      put_quads_rows(Qn, Cfg::LDN, rq, tid);
+      put_quads_transposed(QT, Cfg::LDT, rq, tid);
+      if (Gg) {
+        put_quads_rows(Gn, Cfg::LDN, rg, tid);
+        put_quads_transposed(GT, Cfg::LDT, rg, tid);
+      }
+      if constexpr (DUAL) {
+        put_quads_rows(Qtn, Cfg::LDN, rqt, tid);
+        put_quads_transposed(QtT, Cfg::LDT, rqt, tid);
+        put_quads_rows(GTn, Cfg::LDN, rgt, tid);
+        put_quads_transposed(GTT, Cfg::LDT, rgt, tid);
+      }
+    } else {
+      const int nvalid = L - i0;
+      copy_rows<T, BWD_T, D, BWD_NT>(Qn, Cfg::LDN, Qg + (size_t)i0 * D, nvalid, tid);
+      copy_rows_transposed<T, BWD_T, D, BWD_NT>(QT, Cfg::LDT, Qg + (size_t)i0 * D, nvalid, tid);
+      if (Gg) {
+        copy_rows<T, BWD_T, D, BWD_NT>(Gn, Cfg::LDN, Gg + (size_t)i0 * D, nvalid, tid);
+        copy_rows_transposed<T, BWD_T, D, BWD_NT>(GT, Cfg::LDT, Gg + (size_t)i0 * D, nvalid, tid);
+      }
+      if constexpr (DUAL) {
+        copy_rows<T, BWD_T, D, BWD_NT>(Qtn, Cfg::LDN, Qtg + (size_t)i0 * D, nvalid, tid);
+        copy_rows_transposed<T, BWD_T, D, BWD_NT>(QtT, Cfg::LDT, Qtg + (size_t)i0 * D, nvalid, tid);
+        copy_rows<T, BWD_T, D, BWD_NT>(GTn, Cfg::LDN, gTg + (size_t)i0 * D, nvalid, tid);
+        copy_rows_transposed<T, BWD_T, D, BWD_NT>(GTT, Cfg::LDT, gTg + (size_t)i0 * D, nvalid, tid);
+      }
+      fetch_stats(i0);
+    }
+    put_stats();
+    __syncthreads();
+    if constexpr (AHEAD) {
+      if (i0 + BWD_T < L) fetch_tile(i0 + BWD_T);
+    }
 
     f32x16 S, dP, Sp, At, Bt;
     zero16(S);

@@ -134,6 +134,92 @@ __device__ __forceinline__ void copy_rows_transposed(T *dst, int ld, const T *sr
   }
 }
 
+// The two movers above cut in two, so that the global loads of the next tile travel while the
+// current tile is computed: fetch_* issues the loads into registers, put_* (after the compute, behind
+// a barrier) writes them to LDS.
+template <typename T, int ROWS, int D, int NT> struct RowChunks {
+  static constexpr int EPC = 16 / sizeof(T), CPR = D / EPC, TOTAL = ROWS * CPR, N = (TOTAL + NT - 1) / NT;
+  u32x4 x[N];
+};
+template <typename T, int ROWS, int D, int NT>
+__device__ __forceinline__ void fetch_rows(RowChunks<T, ROWS, D, NT> &r, const T *src, int nvalid, int tid) {
+  using R = RowChunks<T, ROWS, D, NT>;
+#pragma unroll
+  for (int it = 0; it < R::N; ++it) {
+    const int c = tid + it * NT;
+    if (R::TOTAL % NT == 0 || c < R::TOTAL) {
+      const int row = c / R::CPR, col = (c % R::CPR) * R::EPC;
+      r.x[it] = ld_chunk(src + (size_t)row * D + col, row < nvalid);
+    }
+  }
+}
+template <typename T, int ROWS, int D, int NT>
+__device__ __forceinline__ void put_rows(T *dst, int ld, const RowChunks<T, ROWS, D, NT> &r, int tid) {
+  using R = RowChunks<T, ROWS, D, NT>;
+#pragma unroll
+  for (int it = 0; it < R::N; ++it) {
+    const int c = tid + it * NT;
+    if (R::TOTAL % NT == 0 || c < R::TOTAL) {
+      const int row = c / R::CPR, col = (c % R::CPR) * R::EPC;
+      *reinterpret_cast<u32x4 *>(dst + row * ld + col) = r.x[it];
+    }
+  }
+}
+// tasks of 4 rows x one 16-byte chunk of columns; one fetch serves a transposed put and, where a
+// tile is needed both ways, a row-major put as well
+template <typename T, int ROWS, int D, int NT> struct QuadChunks {
+  static constexpr int EPC = 16 / sizeof(T), CPR = D / EPC, RG = ROWS / 4, TOTAL = RG * CPR, N = (TOTAL + NT - 1) / NT;
+  u32x4 x[N][4];
+};
+template <typename T, int ROWS, int D, int NT>
+__device__ __forceinline__ void fetch_quads(QuadChunks<T, ROWS, D, NT> &r, const T *src, int nvalid, int tid) {
+  using R = QuadChunks<T, ROWS, D, NT>;
+#pragma unroll
+  for (int it = 0; it < R::N; ++it) {
+    const int c = tid + it * NT;
+    if (R::TOTAL % NT == 0 || c < R::TOTAL) {
+      const int rg = c % R::RG, cc = c / R::RG;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        r.x[it][i] = ld_chunk(src + (size_t)(4 * rg + i) * D + cc * R::EPC, 4 * rg + i < nvalid);
+    }
+  }
+}
+template <typename T, int ROWS, int D, int NT>
+__device__ __forceinline__ void put_quads_transposed(T *dst, int ld, const QuadChunks<T, ROWS, D, NT> &r, int tid) {
+  using R = QuadChunks<T, ROWS, D, NT>;
+#pragma unroll
+  for (int it = 0; it < R::N; ++it) {
+    const int c = tid + it * NT;
+    if (R::TOTAL % NT == 0 || c < R::TOTAL) {
+      const int rg = c % R::RG, cc = c / R::RG;
+      union { u32x4 v; T e[R::EPC]; } in[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) in[i].v = r.x[it][i];
+#pragma unroll
+      for (int e = 0; e < R::EPC; ++e) {
+        Quad<T> o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = in[i].e[e];
+        *reinterpret_cast<Quad<T> *>(dst + (cc * R::EPC + e) * ld + 4 * rg) = o;
+      }
+    }
+  }
+}
+template <typename T, int ROWS, int D, int NT>
+__device__ __forceinline__ void put_quads_rows(T *dst, int ld, const QuadChunks<T, ROWS, D, NT> &r, int tid) {
+  using R = QuadChunks<T, ROWS, D, NT>;
+#pragma unroll
+  for (int it = 0; it < R::N; ++it) {
+    const int c = tid + it * NT;
+    if (R::TOTAL % NT == 0 || c < R::TOTAL) {
+      const int rg = c % R::RG, cc = c / R::RG;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4 *>(dst + (4 * rg + i) * ld + cc * R::EPC) = r.x[it][i];
+    }
+  }
+}
+
 // Blocks are dealt round-robin to the 8 XCDs (each with its own L2).  Re-deal them so that the blocks
 // of one head (which share its K/V) land on one XCD and are worked on there at about the same time:
 // XCD x takes heads x, x+8, x+16, ... one after another.  Dealing heads round-robin rather than in
