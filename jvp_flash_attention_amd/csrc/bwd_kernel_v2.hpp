@@ -60,7 +60,7 @@ template <int N> __device__ __forceinline__ void lds_wait4(u32x4 &a, u32x4 &b, u
 #ifndef JVPFA_BWD_SPREAD
 #define JVPFA_BWD_SPREAD(n) (3 * (n) / 4)
 #endif
-#define JVPFA_BWD2_COMMON(Cfg)                                                                                      \
+#define JVPFA_BWD2_COMMON(Cfg, STREAMED_ROWS)                                                                                      \
   constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT;                   \
   constexpr int KK = D / 16, DB = D / 32;                                                                           \
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];                                        \
@@ -93,7 +93,7 @@ template <int N> __device__ __forceinline__ void lds_wait4(u32x4 &a, u32x4 &b, u
   uint32_t ld_dst = 0;                                                                                              \
   __amdgpu_buffer_rsrc_t ld_rs[4];                                                                                  \
   auto tile_rsrc = [&](const char *base, int j, bool exists) {                                                      \
-    const int rows = exists ? max(L - j, 0) : 0;                                                                    \
+    const int rows = exists ? max((STREAMED_ROWS) - j, 0) : 0;                                                                    \
     return __builtin_amdgcn_make_buffer_rsrc((void *)(base + (size_t)j * ROWB), 0, rows * ROWB, 0x00020000);       \
   };                                                                                                                \
   auto load_piece = [&](auto pc) {                                                                                  \
@@ -139,7 +139,7 @@ template <typename T, int D, int MODE, int MASK, bool GO>
 __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
-  JVPFA_BWD2_COMMON(Cfg)
+  JVPFA_BWD2_COMMON(Cfg, pr.Lk)  // streams key tiles
   const int qb = pr.causal ? nblk - 1 - id % nblk : id % nblk;
   const int q0 = qb * Cfg::BLK;
   const int qrow = q0 + wave * 32 + r;
@@ -176,12 +176,16 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
   bool mask_al = false;  // mask rows can be fetched with aligned vector loads
   if constexpr (MASK != MASK_NONE) mask_al = mask_rows_aligned<T, MASK>(pr);
-  const char *Kb = reinterpret_cast<const char *>(p.k) + head * sizeof(T);
-  const char *Vb = reinterpret_cast<const char *>(p.v) + head * sizeof(T);
-  const char *Ktb = DUAL ? reinterpret_cast<const char *>(p.kt) + head * sizeof(T) : nullptr;
-  const char *Vtb = DUAL ? reinterpret_cast<const char *>(p.vt) + head * sizeof(T) : nullptr;
+  // keys: Lk of them, in head h / (H / Hk) of the key/value tensors (L and h themselves for the
+  // shapes the reference admits)
+  const int Lk = pr.Lk;
+  const size_t kvhead = ((size_t)z * pr.Hk + h / (pr.H / pr.Hk)) * Lk * D;
+  const char *Kb = reinterpret_cast<const char *>(p.k) + kvhead * sizeof(T);
+  const char *Vb = reinterpret_cast<const char *>(p.v) + kvhead * sizeof(T);
+  const char *Ktb = DUAL ? reinterpret_cast<const char *>(p.kt) + kvhead * sizeof(T) : nullptr;
+  const char *Vtb = DUAL ? reinterpret_cast<const char *>(p.vt) + kvhead * sizeof(T) : nullptr;
 
-  int kend = pr.causal ? min(L, q0 + Cfg::BLK) : L;
+  int kend = pr.causal ? min(Lk, q0 + Cfg::BLK) : Lk;
   if constexpr (MASK != MASK_NONE) {  // key tiles that the caller's hint declares fully masked are not visited
     if (pr.klimit) kend = min(kend, max(pr.klimit[z], 1));
   }
@@ -191,7 +195,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   if constexpr (MASK != MASK_NONE) {
     if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
   }
-  const int tmax = (L + BT - 1) / BT - 1;  // index of the last tile of the sequence: bounds whatever a list holds
+  const int tmax = (Lk + BT - 1) / BT - 1;  // index of the last tile of the sequence: bounds whatever a list holds
   const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1) : (kend + BT - 1) / BT;
   // List elements are requested a tile ahead, unconditionally (from a harmless address when there is
   // no list: a branch around the read would split the tile loop's straight-line body).
@@ -272,7 +276,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
     else tiles_ready(S, dP);
 
     // ---- P and the score gradients -------------------------------------------------------------
-    const int klim = min(pr.causal ? qrow : 0x7fffffff, L - 1);  // keys above this index are masked
+    const int klim = min(pr.causal ? qrow : 0x7fffffff, Lk - 1);  // keys above this index are masked
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
       const int key0 = jh + 16 * hf + 8 * g;
@@ -349,7 +353,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   auto fetch_masks = [&](int tn) {
     if constexpr (MASK != MASK_NONE) {
       const int jn = tn * BT;
-      if (mask_al && jn + BT <= L) {  // aligned rows, all 64 keys exist: one vector load per 8 keys
+      if (mask_al && jn + BT <= Lk) {  // aligned rows, all 64 keys exist: one vector load per 8 keys
 #pragma unroll
         for (int i = 0; i < 4; ++i) mnext[i / 2][i % 2] = mask_fetch8<T, MASK>(pr, mrow, jn + 16 * i + 8 * g);
       } else {
@@ -391,7 +395,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   };
   // Tiles that cross the diagonal or the end of the sequence are the last ones; they get a loop of their
   // own so that the common tile carries no limit tests.  (q0 is a multiple of the tile size.)
-  int t_edge = L / BT;
+  int t_edge = Lk / BT;
   if (pr.causal) t_edge = min(t_edge, q0 / BT);
   if (MASK != MASK_NONE && !mask_al) t_edge = 0;  // interior tiles fetch mask rows with aligned vector loads
   int t = 0;
@@ -438,7 +442,7 @@ template <typename T, int D, int MODE, int MASK, bool GO>
 __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
-  JVPFA_BWD2_COMMON(Cfg)
+  JVPFA_BWD2_COMMON(Cfg, pr.L)  // streams query tiles
   const int kb = id % nblk;  // causal: the first key blocks have the longest query loops
   const int k0 = kb * Cfg::BLK;
   const int krow = k0 + wave * 32 + r;

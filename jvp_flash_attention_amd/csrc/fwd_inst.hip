@@ -51,28 +51,24 @@ static int launch_fwd3_one(const FwdParams &p, hipStream_t stream) {
 
 template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
-  // key/value tensors of the query tensors' shape (the reference's case) take the tuned kernels;
-  // grouped heads and a key length of its own go through the LDS-copy kernel
-  const bool one_shape = p.pr.Lk == p.pr.L && p.pr.Hk == p.pr.H;
   if constexpr (sizeof(T) == 2 && D >= 64 && D <= 128) {
-    if (one_shape) {
-      switch (mask) {
-        case MASK_NONE:
-          // the pipelined kernel pays off where a slot has enough matrix work to hide the softmax behind
-          if constexpr (D >= 128) return launch_fwd3_one<T, D, DUAL>(p, stream);
-          else return launch_fwd2_one<T, D, DUAL, MASK_NONE>(p, stream);
-        case MASK_BOOL: return launch_fwd2_one<T, D, DUAL, MASK_BOOL>(p, stream);
-        case MASK_ADD: return launch_fwd2_one<T, D, DUAL, MASK_ADD>(p, stream);
-      }
-      return -3;
+    switch (mask) {
+      case MASK_NONE:
+        // the pipelined kernel pays off where a slot has enough matrix work to hide the softmax behind
+        if constexpr (D >= 128) return launch_fwd3_one<T, D, DUAL>(p, stream);
+        else return launch_fwd2_one<T, D, DUAL, MASK_NONE>(p, stream);
+      case MASK_BOOL: return launch_fwd2_one<T, D, DUAL, MASK_BOOL>(p, stream);
+      case MASK_ADD: return launch_fwd2_one<T, D, DUAL, MASK_ADD>(p, stream);
     }
+    return -3;
+  } else {
+    switch (mask) {
+      case MASK_NONE: return launch_fwd_one<T, D, BN, DUAL, MASK_NONE>(p, stream);
+      case MASK_BOOL: return launch_fwd_one<T, D, BN, DUAL, MASK_BOOL>(p, stream);
+      case MASK_ADD: return launch_fwd_one<T, D, BN, DUAL, MASK_ADD>(p, stream);
+    }
+    return -3;
   }
-  switch (mask) {
-    case MASK_NONE: return launch_fwd_one<T, D, BN, DUAL, MASK_NONE>(p, stream);
-    case MASK_BOOL: return launch_fwd_one<T, D, BN, DUAL, MASK_BOOL>(p, stream);
-    case MASK_ADD: return launch_fwd_one<T, D, BN, DUAL, MASK_ADD>(p, stream);
-  }
-  return -3;
 }
 
 int JVPFA_NAME(const FwdParams &p, bool dual, int mask, hipStream_t stream) {

@@ -77,12 +77,16 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   const int pr32 = perm32(r);
 
   const size_t head = (size_t)zh * L * D;
+  // keys: Lk of them, in head h / (H / Hk) of the key/value tensors (L and h themselves for the
+  // shapes the reference admits)
+  const int Lk = pr.Lk;
+  const size_t kvhead = ((size_t)z * pr.Hk + h / (pr.H / pr.Hk)) * Lk * D;
   const T *Qg = reinterpret_cast<const T *>(p.q) + head;
-  const T *Kg = reinterpret_cast<const T *>(p.k) + head;
-  const T *Vg = reinterpret_cast<const T *>(p.v) + head;
+  const T *Kg = reinterpret_cast<const T *>(p.k) + kvhead;
+  const T *Vg = reinterpret_cast<const T *>(p.v) + kvhead;
   const T *Qtg = DUAL ? reinterpret_cast<const T *>(p.qt) + head : nullptr;
-  const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + head : nullptr;
-  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + head : nullptr;
+  const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + kvhead : nullptr;
+  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + kvhead : nullptr;
 
   const int q0 = qb * Cfg::BM;
   const int qrow = q0 + wave * 32 + r;
@@ -110,12 +114,12 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     const char *kp = reinterpret_cast<const char *>(Kg) + tb, *vp = reinterpret_cast<const char *>(Vg) + tb;
     const char *ktp = DUAL ? reinterpret_cast<const char *>(Ktg) + tb : nullptr;
     const char *vtp = DUAL ? reinterpret_cast<const char *>(Vtg) + tb : nullptr;
-    const bool ragged_tile = j0 + BN > L;
+    const bool ragged_tile = j0 + BN > Lk;
 #pragma unroll
     for (int i = 0; i < IPW; ++i) {
       uint32_t ok = ld_bk[i], ov = ld_bv[i];
       if (ragged_tile) {  // rows past the end re-read the last row; their scores are masked
-        const int row = min(ld_row[i], L - 1 - j0);
+        const int row = min(ld_row[i], Lk - 1 - j0);
         ok = row * ROWB + ld_ck[i];
         ov = row * ROWB + ld_cv[i];
       }
@@ -183,13 +187,13 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   bool mask_al = false;  // mask rows can be fetched with aligned vector loads
   if constexpr (MASK != MASK_NONE) mask_al = mask_rows_aligned<T, MASK>(pr);
 
-  int kend = L;
+  int kend = Lk;
   // padded batches: the caller's hint says the mask hides every key from klimit[z] on, so those tiles
   // need not be visited (at least one tile is, which keeps rows without any key well defined)
   if constexpr (MASK != MASK_NONE) {
-    if (pr.klimit) kend = min(L, max(pr.klimit[z], 1));
+    if (pr.klimit) kend = min(Lk, max(pr.klimit[z], 1));
   }
-  if (pr.causal) kend = min(L, q0 + Cfg::BM);
+  if (pr.causal) kend = min(Lk, q0 + Cfg::BM);
   // Tiles visited: 0 .. ceil(kend/BN)-1, or the caller's list of the tiles of this query block that
   // hold an attended entry (ascending; fully masked tiles contribute exact zeros, so leaving them
   // out changes nothing).  tile_at(i) is the i-th tile visited.
@@ -197,7 +201,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   if constexpr (MASK != MASK_NONE) {
     if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
   }
-  const int tmax = (L + BN - 1) / BN - 1;  // index of the last tile of the sequence: bounds whatever a list holds
+  const int tmax = (Lk + BN - 1) / BN - 1;  // index of the last tile of the sequence: bounds whatever a list holds
   const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1) : (kend + BN - 1) / BN;
   // List elements are requested a tile ahead, unconditionally (from a harmless address when there is
   // no list: a branch around the read would split the tile loop's straight-line body).
@@ -215,7 +219,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   // predicated off, which keeps every step of the tile loop one straight-line block.
   auto prepare_loads = [&](int stage, int j0, bool on) {
     j0 = on ? j0 : 0;
-    ld_rows = L - 1 - j0;  // rows past the end re-read the last row; their scores are masked
+    ld_rows = Lk - 1 - j0;  // rows past the end re-read the last row; their scores are masked
     ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
     const size_t tb = (size_t)j0 * ROWB;
     ld_p[0] = reinterpret_cast<const char *>(Kg) + tb;
@@ -251,7 +255,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   // tiles where the running maximum really grows.  O = acc / l is unchanged by the choice of m_i.
   constexpr float RESCALE_TAU = 8.f;
   MaskAhead<T, MASK> mcur[2][2], mnext[2][2];  // mask values of this tile and the next: [half tile][16-key group]
-  const int klim = min(pr.causal ? qrow : 0x7fffffff, L - 1);  // keys above this index are masked
+  const int klim = min(pr.causal ? qrow : 0x7fffffff, Lk - 1);  // keys above this index are masked
   // EDGE: the half tile may cross the causal diagonal or the end of the sequence, the scale may be
   // negative, or the mask rows are not aligned for vector fetches
   auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, int jh) {
@@ -412,7 +416,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   auto fetch_masks = [&](int tn) {
     if constexpr (MASK != MASK_NONE) {
       const int jn = tn * BN;
-      if (mask_al && jn + BN <= L) {  // aligned rows, all 64 keys exist: one vector load per 8 keys
+      if (mask_al && jn + BN <= Lk) {  // aligned rows, all 64 keys exist: one vector load per 8 keys
 #pragma unroll
         for (int i = 0; i < 4; ++i) mnext[i / 2][i % 2] = mask_fetch8<T, MASK>(pr, mrow, jn + 16 * i + 8 * g);
       } else {
@@ -456,7 +460,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   };
   // Tiles that need the general treatment are the last ones; they get a loop of their own so that the
   // common tile carries no limit tests.  (q0 is a multiple of the tile size.)
-  int t_edge = L / BN;
+  int t_edge = Lk / BN;
   if (pr.causal) t_edge = min(t_edge, q0 / BN);
   if (!(sl2 > 0.f) || (MASK != MASK_NONE && !mask_al)) t_edge = 0;
   int t = 0;

@@ -78,12 +78,16 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   const int pr32 = perm32(r);
 
   const size_t head = (size_t)zh * L * D;
+  // keys: Lk of them, in head h / (H / Hk) of the key/value tensors (L and h themselves for the
+  // shapes the reference admits)
+  const int Lk = pr.Lk;
+  const size_t kvhead = ((size_t)(zh / pr.H) * pr.Hk + (zh % pr.H) / (pr.H / pr.Hk)) * Lk * D;
   const T *Qg = reinterpret_cast<const T *>(p.q) + head;
-  const char *Kg = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.k) + head);
-  const char *Vg = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.v) + head);
+  const char *Kg = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.k) + kvhead);
+  const char *Vg = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.v) + kvhead);
   const T *Qtg = DUAL ? reinterpret_cast<const T *>(p.qt) + head : nullptr;
-  const char *Ktg = DUAL ? reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.kt) + head) : nullptr;
-  const char *Vtg = DUAL ? reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.vt) + head) : nullptr;
+  const char *Ktg = DUAL ? reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.kt) + kvhead) : nullptr;
+  const char *Vtg = DUAL ? reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.vt) + kvhead) : nullptr;
 
   const int q0 = qb * Cfg::BM;
   const int qrow = q0 + wave * 32 + r;
@@ -147,7 +151,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
 
   const float sl2 = pr.scale * LOG2E;
   const bool neg_scale = !(sl2 > 0.f);
-  const int kend = pr.causal ? min(L, q0 + Cfg::BM) : L;
+  const int kend = pr.causal ? min(Lk, q0 + Cfg::BM) : Lk;
   const int ntiles = (kend + BN - 1) / BN;
   const int qlim = pr.causal ? qrow : 0x7fffffff;  // keys above this index are masked
 
@@ -168,7 +172,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     ldo_v[i] = ld_row[i] * ROWB + ld_cv[i];
   }
   auto tile_rsrc = [&](const char *base, int j, bool exists) {
-    const int rows = exists ? max(L - j, 0) : 0;
+    const int rows = exists ? max(Lk - j, 0) : 0;
     return __builtin_amdgcn_make_buffer_rsrc((void *)(base + (size_t)j * ROWB), 0, rows * ROWB, 0x00020000);
   };
   // iteration t loads K(t+1) into the K half of stage (t+1)&1 and V(t) into the V half of stage t&1
@@ -247,7 +251,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
             const int key = jh + 16 * (e / 8) + 8 * g + (e % 8);
             float s = Sc[e] * sl2;
             s = (key <= qlim) ? s : NEG_INF;
-            s = (key < L) ? s : NEG_INF;
+            s = (key < Lk) ? s : NEG_INF;
             Sc[e] = s;
             m8 = fmaxf(m8, s);
           } else {
@@ -459,7 +463,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   slot(B1{}, B0{}, B1{}, B1{}, std::integral_constant<int, NSS>{}, B0{}, B0{}, kad(0, 1), 0u, SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0);
   // Iterations whose softmax needs the causal / sequence-end limits form the tail of the loop; they
   // get a loop of their own so that the common iteration is one straight-line block.
-  int t_gen = (L >= 32) ? (L - 32) / BN + 1 : 0;
+  int t_gen = (Lk >= 32) ? (Lk - 32) / BN + 1 : 0;
   if (pr.causal) t_gen = min(t_gen, (q0 + 32) / BN);
   t_gen = neg_scale ? 1 : max(1, t_gen);
   int t = 1;
