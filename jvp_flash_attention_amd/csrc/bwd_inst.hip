@@ -14,10 +14,8 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
   const int nb = (p.pr.L + BWD_BLK - 1) / BWD_BLK;
   const long long blocks = (long long)nb * p.pr.Z * p.pr.H;
   if (blocks > 0x7fffffffLL) return -2;
-  // key/value tensors of the query tensors' shape (the reference's case) take the tuned kernels below;
-  // with grouped heads or a key length of its own the dq kernel still does (it owns query rows), and
-  // dk, dv, which add up over the heads of a group, come from the LDS-copy kernel
-  const bool one_shape = p.pr.Lk == p.pr.L && p.pr.Hk == p.pr.H;
+  // the dk/dv kernels run one workgroup per 128 keys of a key/value head (the same count as for dq
+  // when k, v have q's shape)
   const long long kv_blocks = (long long)((p.pr.Lk + BWD_BLK - 1) / BWD_BLK) * p.pr.Z * p.pr.Hk;
   if (kv_blocks > 0x7fffffffLL) return -2;
   if constexpr (sizeof(T) == 2 && D >= 64 && D <= 128) {  // direct-to-LDS, double-buffered kernels
@@ -40,14 +38,7 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
     int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
     if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);
     if (rc != 0) return rc;
-    if (one_shape) {
-      hipLaunchKernelGGL(kkv, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
-    } else {
-      auto kkv1 = bwd_dkdv_kernel<T, D, MODE, MASK>;
-      rc = allow_lds(reinterpret_cast<const void *>(kkv1), Cfg::DKV_LDS);
-      if (rc != 0) return rc;
-      hipLaunchKernelGGL(kkv1, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
-    }
+    hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
     hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
    }

@@ -60,23 +60,23 @@ template <int N> __device__ __forceinline__ void lds_wait4(u32x4 &a, u32x4 &b, u
 #ifndef JVPFA_BWD_SPREAD
 #define JVPFA_BWD_SPREAD(n) (3 * (n) / 4)
 #endif
-#define JVPFA_BWD2_COMMON(Cfg, STREAMED_ROWS)                                                                                      \
+#define JVPFA_BWD2_COMMON(Cfg, STREAMED_ROWS, OWN_ROWS, OWN_HEADS)                                                                                      \
   constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT;                   \
   constexpr int KK = D / 16, DB = D / 32;                                                                           \
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];                                        \
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem_raw;                                                              \
   const Problem &pr = p.pr;                                                                                         \
   const int L = pr.L;                                                                                               \
-  const int nblk = (L + Cfg::BLK - 1) / Cfg::BLK;                                                                   \
-  const int total = nblk * pr.Z * pr.H;                                                                             \
-  const int id = xcd_remap(blockIdx.x, nblk, pr.Z * pr.H);                                                                      \
+  /* a workgroup owns 128 of the OWN_ROWS rows of one (z, head out of OWN_HEADS) */                               \
+  const int nblk = ((OWN_ROWS) + Cfg::BLK - 1) / Cfg::BLK;                                                          \
+  const int id = xcd_remap(blockIdx.x, nblk, pr.Z * (OWN_HEADS));                                                   \
   const int zh = id / nblk;                                                                                         \
-  const int z = zh / pr.H, h = zh % pr.H;                                                                           \
+  const int z = zh / (OWN_HEADS), h = zh % (OWN_HEADS);                                                             \
   const int tid = threadIdx.x;                                                                                      \
   const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;                                   \
   const int r = lane % 32, g = lane / 32, pr32 = perm32(r);                                                         \
-  const size_t head = (size_t)zh * L * D;                                                                           \
-  const size_t srow = (size_t)zh * L;                                                                               \
+  const size_t head = (size_t)zh * (OWN_ROWS) * D;                                                                  \
+  const size_t srow = (size_t)zh * (OWN_ROWS);                                                                      \
   (void)z; (void)h; (void)srow;                                                                                     \
   /* direct loads: instruction i of this wave fills LDS chunks 64*(wave*IPW+i) .. +63 of a tile */                   \
   int ld_row[IPW];                                                                                                  \
@@ -139,7 +139,7 @@ template <typename T, int D, int MODE, int MASK, bool GO>
 __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
-  JVPFA_BWD2_COMMON(Cfg, pr.Lk)  // streams key tiles
+  JVPFA_BWD2_COMMON(Cfg, pr.Lk, pr.L, pr.H)  // owns query rows, streams key tiles
   const int qb = pr.causal ? nblk - 1 - id % nblk : id % nblk;
   const int q0 = qb * Cfg::BLK;
   const int qrow = q0 + wave * 32 + r;
@@ -442,15 +442,16 @@ template <typename T, int D, int MODE, int MASK, bool GO>
 __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
-  JVPFA_BWD2_COMMON(Cfg, pr.L)  // streams query tiles
+  JVPFA_BWD2_COMMON(Cfg, pr.L, pr.Lk, pr.Hk)  // owns key rows (h: key/value head), streams query tiles
   const int kb = id % nblk;  // causal: the first key blocks have the longest query loops
   const int k0 = kb * Cfg::BLK;
   const int krow = k0 + wave * 32 + r;
-  const int kld = krow < L ? krow : L - 1;
+  const int Lk = pr.Lk;  // keys; L counts queries
+  const int kld = krow < Lk ? krow : Lk - 1;
   if constexpr (MASK != MASK_NONE) {
     // a key block that the caller's hint declares fully masked has zero gradients
     if (pr.klimit && k0 >= pr.klimit[z]) {
-      if (krow < L) {
+      if (krow < Lk) {
         T *outk = reinterpret_cast<T *>(MODE == BWD_TANGENT ? p.dkt : p.dk) + head + (size_t)krow * D;
         T *outv = reinterpret_cast<T *>(MODE == BWD_TANGENT ? p.dvt : p.dv) + head + (size_t)krow * D;
         float zero8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -496,17 +497,30 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   uint32_t mlane = 0;
   if constexpr (MASK != MASK_NONE) {
     const int64_t lim = (int64_t)1 << 31;
-    mask_small = pr.ms[2] >= 0 && pr.ms[3] >= 0 && 8 * pr.ms[2] + (int64_t)L * pr.ms[3] < lim;
+    mask_small = pr.ms[2] >= 0 && pr.ms[3] >= 0 && 8 * pr.ms[2] + (int64_t)Lk * pr.ms[3] < lim;
     mlane = (uint32_t)(8 * g * pr.ms[2] + (int64_t)kld * pr.ms[3]);
   }
-  // tile slots: 0 Q, 1 G (gO; gT in TANGENT; gT again in DUAL without gO), 2 Q', 3 gT
-  const char *Qb = reinterpret_cast<const char *>(p.q) + head * sizeof(T);
-  const char *gTb = (DUAL || TAN) ? reinterpret_cast<const char *>(p.gt) + head * sizeof(T) : nullptr;
-  const char *Gb = TAN ? gTb : (has_go ? reinterpret_cast<const char *>(p.go) + head * sizeof(T) : gTb);
-  const char *Qtb = DUAL ? reinterpret_cast<const char *>(p.qt) + head * sizeof(T) : nullptr;
-  // statistics slots: PLAIN M, d1 | DUAL M, mu, a, d2 (= d1 + d2) | TANGENT M, a
-  const float *st_p[4] = {p.M + srow, MODE == BWD_PLAIN ? p.d1 + srow : (DUAL ? p.mu + srow : p.a + srow),
-                          DUAL ? p.a + srow : nullptr, DUAL ? p.d2 + srow : nullptr};
+  // The query heads that read this key/value head are visited one after another (one, h itself, for
+  // the shapes the reference admits); hq is the current one, and what depends on it is set per head:
+  // tile slots 0 Q, 1 G (gO; gT in TANGENT; gT again in DUAL without gO), 2 Q', 3 gT, and the
+  // statistics slots PLAIN M, d1 | DUAL M, mu, a, d2 (= d1 + d2) | TANGENT M, a
+  const int group = pr.H / pr.Hk;
+  int hq = h * group;
+  const char *Qb = nullptr, *gTb = nullptr, *Gb = nullptr, *Qtb = nullptr;
+  const float *st_p[4] = {nullptr, nullptr, nullptr, nullptr};
+  auto set_query_head = [&](int hq_) {
+    hq = hq_;
+    const size_t qhead = ((size_t)z * pr.H + hq) * L * D * sizeof(T), qrow0 = ((size_t)z * pr.H + hq) * L;
+    Qb = reinterpret_cast<const char *>(p.q) + qhead;
+    gTb = (DUAL || TAN) ? reinterpret_cast<const char *>(p.gt) + qhead : nullptr;
+    Gb = TAN ? gTb : (has_go ? reinterpret_cast<const char *>(p.go) + qhead : gTb);
+    Qtb = DUAL ? reinterpret_cast<const char *>(p.qt) + qhead : nullptr;
+    st_p[0] = p.M + qrow0;
+    st_p[1] = MODE == BWD_PLAIN ? p.d1 + qrow0 : (DUAL ? p.mu + qrow0 : p.a + qrow0);
+    st_p[2] = DUAL ? p.a + qrow0 : nullptr;
+    st_p[3] = DUAL ? p.d2 + qrow0 : nullptr;
+  };
+  set_query_head(h * group);
 
   const int istart = pr.causal ? (k0 / BT) * BT : 0;
   // Query tiles visited, counted from istart: 0 .. ntiles-1, or the caller's list of the tiles of this
@@ -514,7 +528,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   // tile_at(i) is the i-th one.
   const int *tlist = nullptr;
   if constexpr (MASK != MASK_NONE) {
-    if (pr.tiles_k) tlist = pr.tiles_k + tile_list_offset(pr, z, h, kb);
+    if (pr.tiles_k) tlist = pr.tiles_k + tile_list_offset(pr, z, h, kb);  // only given when Hk == H
   }
   const int tmax = (L + BT - 1) / BT - 1;  // index of the last tile of the sequence: bounds whatever a list holds
   const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1) : (L - istart + BT - 1) / BT;
@@ -567,7 +581,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
     if constexpr (MASK != MASK_NONE) {
       if (mask_small && ihn + 32 <= L) {
         // uniform 64-bit row pointer + 32-bit lane offset: no per-lane address arithmetic per element
-        const int64_t mrow0 = z * pr.ms[0] + h * pr.ms[1];
+        const int64_t mrow0 = z * pr.ms[0] + hq * pr.ms[1];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int64_t urow = mrow0 + (int64_t)(ihn + 16 * (e / 8) + (e % 8)) * pr.ms[2];
@@ -575,7 +589,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
           if constexpr (MASK == MASK_BOOL) mnext_b[e] = (reinterpret_cast<const uint8_t *>(pr.mask) + urow)[mlane];
         }
       } else {  // rows past the end are read from the last row (their scores are masked by index)
-        const int64_t mcol = z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3];
+        const int64_t mcol = z * pr.ms[0] + hq * pr.ms[1] + (int64_t)kld * pr.ms[3];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int qi = ihn + 16 * (e / 8) + 8 * g + (e % 8);
@@ -611,7 +625,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
     // 16(e/8) + 8g + e%8): requested one half tile earlier (see fetch_mask_half), taken over here
     T mraw_a[MASK == MASK_ADD ? 16 : 1];
     uint8_t mraw_b[MASK == MASK_BOOL ? 16 : 1];
-    const int64_t mcol_use = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3] : 0;
+    const int64_t mcol_use = MASK != MASK_NONE ? z * pr.ms[0] + hq * pr.ms[1] + (int64_t)kld * pr.ms[3] : 0;
     if constexpr (MASK != MASK_NONE && MAHEAD) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
@@ -701,7 +715,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
           bool keep = true;
           if constexpr (MASK != MASK_NONE && !MAHEAD) {
             if constexpr (!EDGE) {  // uniform row pointer + 32-bit lane offset, as above
-              const int64_t urow = z * pr.ms[0] + h * pr.ms[1] + (int64_t)(ih + 16 * (e / 8) + (e % 8)) * pr.ms[2];
+              const int64_t urow = z * pr.ms[0] + hq * pr.ms[1] + (int64_t)(ih + 16 * (e / 8) + (e % 8)) * pr.ms[2];
               if constexpr (MASK == MASK_ADD) mraw_a[0] = (reinterpret_cast<const T *>(pr.mask) + urow)[mlane];
               if constexpr (MASK == MASK_BOOL) mraw_b[0] = (reinterpret_cast<const uint8_t *>(pr.mask) + urow)[mlane];
             } else {
@@ -762,13 +776,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
     });
   };
 
-  // the tile of this step and of the next
-  int tcur = tlist ? min(max(tlist[1], 0), tmax) : 0;
-  int tnext = tlist ? min(max(tlist[1 + min(1, ntiles - 1)], 0), tmax) : min(1, ntiles - 1);
-  if constexpr (MASK != MASK_NONE && MAHEAD) fetch_mask_half(istart + tcur * BT);
-  prepare_loads(0, istart + tcur * BT, true);
-  static_for<NLOAD>([&](auto pc) { load_piece(pc); });
-  load_stats();
+  int tcur = 0, tnext = 0;  // the tile of this step and of the next
   auto tile = [&](int t, auto EDGEc) {
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -794,13 +802,25 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   // last; the tiles in between run without limit tests.
   const int t_diag = pr.causal ? min(ntiles, (k0 + Cfg::BLK - istart + BT - 1) / BT) : 0;
   const int t_end = mask_small ? max(t_diag, (L - istart) / BT) : t_diag;  // first tile that crosses the end
-  int t = 0;
-  for (; t < t_diag; ++t) tile(t, std::true_type{});
-  for (; t < ntiles && tcur < t_end; ++t) tile(t, std::false_type{});
-  for (; t < ntiles; ++t) tile(t, std::true_type{});
-  __builtin_amdgcn_s_waitcnt(0x0F70);
+  for (int gi = 0; gi < group; ++gi) {
+    if (gi > 0) {
+      __syncthreads();  // every wave is done with the previous head's last tile: its stage may be refilled
+      set_query_head(h * group + gi);
+    }
+    tcur = tlist ? min(max(tlist[1], 0), tmax) : 0;
+    tnext = tlist ? min(max(tlist[1 + min(1, ntiles - 1)], 0), tmax) : min(1, ntiles - 1);
+    if constexpr (MASK != MASK_NONE && MAHEAD) fetch_mask_half(istart + tcur * BT);
+    prepare_loads(0, istart + tcur * BT, true);
+    static_for<NLOAD>([&](auto pc) { load_piece(pc); });
+    load_stats();
+    int t = 0;
+    for (; t < t_diag; ++t) tile(t, std::true_type{});
+    for (; t < ntiles && tcur < t_end; ++t) tile(t, std::false_type{});
+    for (; t < ntiles; ++t) tile(t, std::true_type{});
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+  }
 
-  if (krow < L) {
+  if (krow < Lk) {
     T *outk = reinterpret_cast<T *>(TAN ? p.dkt : p.dk) + head + (size_t)krow * D;
     T *outv = reinterpret_cast<T *>(TAN ? p.dvt : p.dv) + head + (size_t)krow * D;
 #pragma unroll

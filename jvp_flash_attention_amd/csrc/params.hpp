@@ -9,8 +9,7 @@ enum MaskKind { MASK_NONE = 0, MASK_BOOL = 1, MASK_ADD = 2 };
 struct Problem {
   int Z, H, L;  // batch, query heads, query length
   // Key/value length and heads; equal to L and H for the shapes the reference admits
-  // (jvp_attention.py:2367-2378).  Query head h reads key/value head h / (H / Hk).  The tuned
-  // dk/dv kernel (bwd_kernel_v2.hpp) is the one kernel that needs Lk == L and Hk == H.
+  // (jvp_attention.py:2367-2378).  Query head h reads key/value head h / (H / Hk).
   int Lk, Hk;
   int causal;
   float scale;

@@ -21,7 +21,7 @@ Differences from the reference, all deliberate:
   JA:2371-2378, JA:2892); D = 256 for bf16 / fp16 only.
 * k and v may have fewer heads than q (grouped heads: H a multiple of H_kv) and a length of their own
   (cross-attention); causal then means key index <= query index, as in SDPA.  The reference requires
-  q, k, v of one shape (JA:2367-2378).  dk, dv of such calls come from the general kernel.
+  q, k, v of one shape (JA:2367-2378).
 * ``attention`` notices dual inputs and then behaves like ``fwd_dual`` (the reference's ``attention``
   is ``JVPAttn.fwd`` and drops the tangent, its README.md:65-67).
 """
