@@ -90,7 +90,7 @@ typedef struct jvpfa_fwd_args {
    * of p.H; query head h reads key/value head h / (H / Hk).  0 means "as q" (p.L, p.H).  k, v and
    * their tangents are then (Z, Hk, Lk, D), the mask strides address (z, h, query, key) with Lk keys,
    * and causal means key index <= query index.  The reference requires q, k, v of one shape
-   * (JA:2367-2378).  key_limit and the tile lists are ignored for such calls. */
+   * (JA:2367-2378).  key_limit then counts the Lk keys; the tile lists are ignored for such calls. */
   int32_t Lk, Hk;
 } jvpfa_fwd_args;
 

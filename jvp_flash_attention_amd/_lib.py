@@ -260,9 +260,9 @@ class HipBackend:
         a.o, a.ot, a.M, a.mu = _ptr(o), _ptr(ot), _ptr(M), _ptr(mu)
         a.Hk, a.Lk = k.shape[1], k.shape[2]  # key/value heads and length (may differ from q's)
         with torch.cuda.device(q.device):
-            lim = key_limit_hint(mask, mask_kind, Z, L)
+            lim = key_limit_hint(mask, mask_kind, Z, k.shape[2])
             a.key_limit = _ptr(lim)
-            tq, _ = tile_lists(q, mask, mask_kind, False)
+            tq, _ = tile_lists(q, mask, mask_kind, False) if k.shape == q.shape else (None, None)
             a.tiles_q = _ptr(tq)
             check(lib.jvpfa_fwd(C.byref(a), _stream(q)))
         return o, ot, M, mu
@@ -289,9 +289,9 @@ class HipBackend:
         a.workspace = _ptr(ws)
         a.Hk, a.Lk = k.shape[1], k.shape[2]
         with torch.cuda.device(q.device):
-            lim = key_limit_hint(mask, mask_kind, Z, L)
+            lim = key_limit_hint(mask, mask_kind, Z, k.shape[2])
             a.key_limit = _ptr(lim)
-            tq, tk = tile_lists(q, mask, mask_kind, True)
+            tq, tk = tile_lists(q, mask, mask_kind, True) if k.shape == q.shape else (None, None)
             a.tiles_q, a.tiles_k = _ptr(tq), _ptr(tk)
             check(lib.jvpfa_bwd(C.byref(a), _stream(q)))
         return dq, dk, dv, dqt, dkt, dvt

@@ -36,10 +36,11 @@ inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit, cons
   Problem r;
   r.Lk = Lk > 0 ? Lk : p.L;
   r.Hk = Hk > 0 ? Hk : p.H;
-  // the hints are for the tuned kernels, which take k, v of q's shape only
-  const bool masked = p.mask_kind != JVPFA_MASK_NONE && r.Lk == p.L && r.Hk == p.H;
-  r.tiles_q = masked ? tiles_q : nullptr;
-  r.tiles_k = masked ? tiles_k : nullptr;
+  const bool masked = p.mask_kind != JVPFA_MASK_NONE;
+  // the tile lists are laid out for k, v of q's shape; the key limit counts keys whatever the shape
+  const bool lists = masked && r.Lk == p.L && r.Hk == p.H;
+  r.tiles_q = lists ? tiles_q : nullptr;
+  r.tiles_k = lists ? tiles_k : nullptr;
   r.klimit = (masked && !r.tiles_q && !r.tiles_k) ? key_limit : nullptr;
   r.Z = p.Z;
   r.H = p.H;

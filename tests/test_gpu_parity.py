@@ -559,6 +559,34 @@ def test_grouped_heads_and_a_key_length_of_its_own(dt, D, shape, mode):
         _tol_check(n + " (plain)", t, rb1[n], dtype)
 
 
+def test_grouped_heads_with_key_padding_and_skipped_tiles():
+    """The key-limit hint with 8 query heads over 2 key/value heads and 700 keys for 300 queries."""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H, Hk, Lq, Lk, D = 2, 8, 2, 300, 700, 64
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(77)
+    q, go, gt = [torch.randn(Z, H, Lq, D, generator=g).to(dtype) for _ in range(3)]
+    qt = (0.5 * torch.randn(Z, H, Lq, D, generator=g)).to(dtype)
+    k, v = [torch.randn(Z, Hk, Lk, D, generator=g).to(dtype) for _ in range(2)]
+    kt, vt = [(0.5 * torch.randn(Z, Hk, Lk, D, generator=g)).to(dtype) for _ in range(2)]
+    lens = [700, 130]
+    mask = (torch.arange(Lk)[None, :] < torch.tensor(lens)[:, None]).view(Z, 1, 1, Lk)
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dmask, scale, be = mask.cuda(), D**-0.5, _lib.backend()
+    assert _lib.key_limit_hint(dmask, _lib.MASK_BOOL, Z, Lk).tolist() == lens
+    ref = dense.forward(*f64[:6], mask=mask.numpy(), scale=scale)
+    rb = dense.backward(*f64, mask=mask.numpy(), scale=scale)
+    o, ot, M, mu = be.fwd(*dev[:6], dmask, _lib.MASK_BOOL, False, scale)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, _lib.MASK_BOOL, False, scale, want_tangent_grads=True)
+    _tol_check("O", o, ref["O"], dtype)
+    _tol_check("O'", ot, ref["Ot"], dtype)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        _tol_check(n, t, rb[n], dtype)
+    assert grads[1][1, :, 256:].abs().max().item() == 0.0  # key blocks past the limit of batch entry 1
+
+
 def test_c_abi_from_a_plain_cpp_program():
     """``tests/cabi_host/host_check`` (built with the library) calls jvpfa_fwd / jvpfa_bwd from C++ with
     memory it allocated through the HIP runtime, no Python or torch in its process, and compares with
