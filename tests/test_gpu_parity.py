@@ -512,7 +512,7 @@ def test_additive_mask_with_minus_infinity_entries(dt):
 
 @pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
 @pytest.mark.parametrize("D", [32, 64, 128])
-@pytest.mark.parametrize("shape", [(4, 2, 96, 96), (4, 1, 70, 200), (2, 2, 200, 70), (6, 3, 130, 33)])
+@pytest.mark.parametrize("shape", [(4, 2, 96, 96), (4, 1, 70, 200), (2, 2, 200, 70), (6, 3, 130, 33), (2, 1, 3, 5), (2, 2, 5, 2)])
 @pytest.mark.parametrize("mode", ["none", "causal", "bool", "bias"])
 def test_grouped_heads_and_a_key_length_of_its_own(dt, D, shape, mode):
     """Beyond the reference (q, k, v of one shape there): H query heads over Hk key/value heads, Lq
