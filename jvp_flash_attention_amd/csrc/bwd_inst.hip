@@ -25,15 +25,20 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
     const bool no_go = MODE == BWD_DUAL && p.go == nullptr;
     constexpr bool NG = MODE != BWD_DUAL;  // the GO template argument of the kernels without gO
     void (*kq)(const BwdParams), (*kkv)(const BwdParams);
+    const bool grouped = p.pr.Hk != p.pr.H;  // a key/value head serves several query heads
     if constexpr (D <= 64) {  // the register-capped twins: two workgroups per compute unit
       kq = no_go ? bwd2_dq_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dq_kernel_2wg<T, D, MODE, MASK, true>;
-      if constexpr (MASK == MASK_NONE || MODE != BWD_DUAL)
-        kkv = no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, true>;
-      else  // the masked dual dk/dv kernel needs a few registers more than the cap leaves
-        kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
+      if constexpr (MASK == MASK_NONE || MODE != BWD_DUAL) {
+        if (grouped) kkv = no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, true, true>;
+        else kkv = no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, true>;
+      } else {  // the masked dual dk/dv kernel needs a few registers more than the cap leaves
+        if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true>;
+        else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
+      }
     } else {
       kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG> : bwd2_dq_kernel<T, D, MODE, MASK, true>;
-      kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
+      if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true>;
+      else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
     }
     int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
     if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);

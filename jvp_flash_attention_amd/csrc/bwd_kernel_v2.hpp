@@ -438,7 +438,9 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(160))) void 
 // of Q, G (, Q', gT), G = gO (gT in TANGENT).  Scores are S = Q K^T (lane = key, registers =
 // queries) so P, dS are the B operands of dV^T += G^T P and dK^T += Q^T dS.
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stubs (and has no buffer descriptor type)
-template <typename T, int D, int MODE, int MASK, bool GO>
+// GROUPED: the key/value head serves several query heads (compiled apart, so that the common case of
+// one keeps its pointers loop-invariant).
+template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED>
 __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
@@ -504,7 +506,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   // the shapes the reference admits); hq is the current one, and what depends on it is set per head:
   // tile slots 0 Q, 1 G (gO; gT in TANGENT; gT again in DUAL without gO), 2 Q', 3 gT, and the
   // statistics slots PLAIN M, d1 | DUAL M, mu, a, d2 (= d1 + d2) | TANGENT M, a
-  const int group = pr.H / pr.Hk;
+  const int group = GROUPED ? pr.H / pr.Hk : 1;
   int hq = h * group;
   const char *Qb = nullptr, *gTb = nullptr, *Gb = nullptr, *Qtb = nullptr;
   const float *st_p[4] = {nullptr, nullptr, nullptr, nullptr};
@@ -840,18 +842,18 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   }
 }
 #endif
-template <typename T, int D, int MODE, int MASK, bool GO>
+template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED = false>
 __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dkdv_body<T, D, MODE, MASK, GO>(p);
+  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED>(p);
 #endif
 }
 // The same code with the vector registers capped, for D = 64: together with the accumulation registers
 // the kernel then needs at most 256 registers and two workgroups share a compute unit.
-template <typename T, int D, int MODE, int MASK, bool GO>
+template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED = false>
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(144))) void bwd2_dkdv_kernel_2wg(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dkdv_body<T, D, MODE, MASK, GO>(p);
+  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED>(p);
 #endif
 }
 
