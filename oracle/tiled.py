@@ -19,6 +19,10 @@ reference does not have (its ``backward`` ignores the second incoming
 gradient, ``:2831``).
 
 Mask semantics follow SDPA (bool True = attend; float added after scaling).
+
+Beyond the reference's one shape for q, k and v: k and v may be ``(Z, H_kv, L_kv, D)`` with
+``H % H_kv == 0`` (query head ``h`` reads key/value head ``h // (H / H_kv)``; their gradients
+are summed over the group) and any ``L_kv`` (causal = key index <= query index).
 """
 from __future__ import annotations
 
@@ -39,8 +43,8 @@ def _tile_logits(qi, kj, scale, mask, causal, i0, j0):
         cols = torch.arange(j0, j0 + bj).unsqueeze(0)
         keep = keep & (rows >= cols)
     if mask is not None:
-        Lk = mask.shape[-1]
-        mt = mask.expand(s.shape[0], s.shape[1], Lk, Lk)[..., i0 : i0 + bi, j0 : j0 + bj]
+        Lq = max(mask.shape[-2], i0 + bi)  # a mask row of extent 1 is shared by every query
+        mt = mask.expand(s.shape[0], s.shape[1], Lq, mask.shape[-1])[..., i0 : i0 + bi, j0 : j0 + bj]
         if mask.dtype == torch.bool:
             keep = keep & mt
         else:
@@ -49,9 +53,22 @@ def _tile_logits(qi, kj, scale, mask, causal, i0, j0):
     return s * LOG2E, keep
 
 
+def _group(x, H):
+    """Key/value heads repeated so that each query head finds its own at the same index."""
+    return x if x is None or x.shape[1] == H else x.repeat_interleave(H // x.shape[1], dim=1)
+
+
+def _ungroup(x, Hk):
+    """Per-query-head key/value gradients summed over each group of heads."""
+    Z, H, Lk, D = x.shape
+    return x if H == Hk else x.view(Z, Hk, H // Hk, Lk, D).sum(2)
+
+
 def forward(q, k, v, qt=None, kt=None, vt=None, mask=None, causal=False, scale=None, bm=32, bn=32):
     """Online-softmax dual forward.  Returns (O, O' or None, M, mu or None)."""
     Z, H, L, D = q.shape
+    Lk = k.shape[2]
+    k, v, kt, vt = (_group(x, H) for x in (k, v, kt, vt))
     scale = D**-0.5 if scale is None else scale
     dual = qt is not None
     o = torch.zeros_like(q)
@@ -67,9 +84,9 @@ def forward(q, k, v, qt=None, kt=None, vt=None, mask=None, causal=False, scale=N
         acc = torch.zeros(Z, H, rows, D, dtype=q.dtype)
         t_acc = torch.zeros_like(acc)
         mu = torch.zeros_like(l)
-        hi = min(i1, L) if causal else L  # causal: tiles right of the diagonal are skipped
+        hi = min(i1, Lk) if causal else Lk  # causal: tiles right of the diagonal are skipped
         for j0 in range(0, hi, bn):
-            j1 = min(j0 + bn, L)
+            j1 = min(j0 + bn, Lk)
             s2, keep = _tile_logits(qi, k[:, :, j0:j1], scale, mask, causal, i0, j0)
             s2 = torch.where(keep, s2, torch.full_like(s2, -math.inf))
             m_new = torch.maximum(m, s2.amax(-1, keepdim=True))
@@ -107,9 +124,12 @@ def backward(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt=None, mask=None, causal=F
     plain forward).
     """
     Z, H, L, D = q.shape
+    Hk, Lk = k.shape[1], k.shape[2]
+    k, v, kt, vt = (_group(x, H) for x in (k, v, kt, vt))
     scale = D**-0.5 if scale is None else scale
     dual = gt is not None
-    g = {n: torch.zeros_like(q) for n in ("dq", "dk", "dv", "dqt", "dkt", "dvt")}
+    g = {n: torch.zeros_like(q) for n in ("dq", "dqt")}
+    g.update({n: torch.zeros_like(k) for n in ("dk", "dv", "dkt", "dvt")})
     # pre-pass row statistics (reference delta at jvp_attention.py:1384-1411, plus the tangent ones)
     d1 = (go * o).sum(-1, keepdim=True)
     if dual:
@@ -117,10 +137,10 @@ def backward(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt=None, mask=None, causal=F
         d2 = (gt * ot).sum(-1, keepdim=True) - a * mu.unsqueeze(-1)
     for i0 in range(0, L, bm):
         i1 = min(i0 + bm, L)
-        hi = i1 if causal else L
+        hi = min(i1, Lk) if causal else Lk
         Mi = M[:, :, i0:i1].unsqueeze(-1)
         for j0 in range(0, hi, bn):
-            j1 = min(j0 + bn, L)
+            j1 = min(j0 + bn, Lk)
             kj, vj = k[:, :, j0:j1], v[:, :, j0:j1]
             s2, keep = _tile_logits(q[:, :, i0:i1], kj, scale, mask, causal, i0, j0)
             p = torch.where(keep, torch.exp2(s2 - Mi), torch.zeros_like(s2))
@@ -147,4 +167,6 @@ def backward(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt=None, mask=None, causal=F
                 g["dkt"][:, :, j0:j1] += scale * torch.matmul(dsp.transpose(-1, -2), q[:, :, i0:i1])
             g["dq"][:, :, i0:i1] += scale * torch.matmul(ds, kj)
             g["dk"][:, :, j0:j1] += scale * torch.matmul(ds.transpose(-1, -2), q[:, :, i0:i1])
+    for n in ("dk", "dv", "dkt", "dvt"):
+        g[n] = _ungroup(g[n], Hk)
     return g

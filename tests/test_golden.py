@@ -23,7 +23,7 @@ def _load(path):
 
 
 def test_the_fixtures_are_there():
-    assert len(FILES) == 5
+    assert len(FILES) == 6
 
 
 @pytest.mark.parametrize("path", FILES, ids=NAMES)
