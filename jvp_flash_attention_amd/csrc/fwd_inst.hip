@@ -4,6 +4,7 @@
 #include "fwd_kernel.hpp"
 #include "fwd_kernel_v2.hpp"
 #include "fwd_kernel_v3.hpp"
+#include "fwd_kernel_wide.hpp"
 #include "launch.hpp"
 
 namespace jvpfa {
@@ -49,9 +50,30 @@ static int launch_fwd3_one(const FwdParams &p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }
 
+// D = 256: two workgroups per query block, each with 128 of the output columns.
+template <typename T, int D, bool DUAL, int MASK>
+static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
+  using Cfg = FwdWideCfg<T, D, 128, DUAL>;
+  auto kern = fwd_wide_kernel<T, D, 128, DUAL, MASK>;
+  int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
+  if (rc != 0) return rc;
+  const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
+  const long long blocks = (long long)nqb * Cfg::NS * p.pr.Z * p.pr.H;
+  if (blocks > 0x7fffffffLL) return -2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : -6;
+}
+
 template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
-  if constexpr (sizeof(T) == 2 && D >= 64 && D <= 128) {
+  if constexpr (sizeof(T) == 2 && D == 256) {
+    switch (mask) {
+      case MASK_NONE: return launch_fwd_wide_one<T, D, DUAL, MASK_NONE>(p, stream);
+      case MASK_BOOL: return launch_fwd_wide_one<T, D, DUAL, MASK_BOOL>(p, stream);
+      case MASK_ADD: return launch_fwd_wide_one<T, D, DUAL, MASK_ADD>(p, stream);
+    }
+    return -3;
+  } else if constexpr (sizeof(T) == 2 && D >= 64 && D <= 128) {
     switch (mask) {
       case MASK_NONE:
         // the pipelined kernel pays off where a slot has enough matrix work to hide the softmax behind
