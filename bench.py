@@ -116,6 +116,34 @@ def hvp_sweep(be, _lib):
     return rows
 
 
+def shape_rows(be, _lib):
+    """Shapes next to the headline one, bf16, no mask: D = 256 (the largest head dim the reference
+    admits), 16 query heads over 4 key/value heads, and 4096 queries over 512 keys (the last two are
+    shapes the reference refuses).  Dual forward and dual backward, counted as 12 and 24 flops per
+    (query, key, d) triple."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    rows = {}
+    for name, (Zs, Hs, Hk, Lq, Lk, Ds) in {
+        "B4_H16_L2048_D256": (4, 16, 16, 2048, 2048, 256),
+        "B4_H16_over_4_kv_heads_L4096_D128": (4, 16, 4, 4096, 4096, 128),
+        "B4_H16_Lq4096_Lk512_D128": (4, 16, 16, 4096, 512, 128),
+    }.items():
+        g = torch.Generator(device=dev).manual_seed(11)
+        mk = lambda h, l: torch.randn(Zs, h, l, Ds, generator=g, device=dev).to(torch.bfloat16)  # noqa: E731
+        q, qt, go, gt = [mk(Hs, Lq) for _ in range(4)]
+        k, v, kt, vt = [mk(Hk, Lk) for _ in range(4)]
+        scale = Ds**-0.5
+        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale), 10, 3)
+        o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale)
+        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, False, scale), 5, 2)
+        n = float(Zs) * Hs * Lq * Lk * Ds
+        rows[name] = {"fwd_ms": ms_f, "fwd_tflops": 12 * n / (ms_f * 1e-3) / 1e12,
+                      "bwd_ms": ms_b, "bwd_tflops": 24 * n / (ms_b * 1e-3) / 1e12}
+    return rows
+
+
 def mask_rows(be, _lib, q, k, v, qt, kt, vt, go, gt, scale):
     """The headline shape with explicit masks: dual forward / backward times for a dense random boolean
     mask (nothing to skip), a block-diagonal mask of four segments and a band of +-256 keys (tiles
@@ -250,6 +278,7 @@ def main():
         }
         out["extra"]["hvp_sweep_bf16_B1_H16_D128_causal"] = hvp_sweep(be, _lib)
         out["extra"]["masks_bf16_B4_H16_L4096_D128"] = mask_rows(be, _lib, q, k, v, qt, kt, vt, go, gt, scale)
+        out["extra"]["other_shapes_bf16"] = shape_rows(be, _lib)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)
