@@ -83,14 +83,16 @@ typedef struct jvpfa_fwd_args {
   /* since version 3 (a caller may pass the version-2 size, which ends before this field):
    * optional lists of the key tiles that hold an attended entry, written by jvpfa_mask_tiles() for
    * this same mask, or NULL.  Tiles not listed are skipped instead of read and masked.  When set,
-   * key_limit is ignored.  Ignored without a mask. */
+   * key_limit is ignored.  Ignored (and key_limit used) without a mask, for fp32 and for D other
+   * than 64 and 128, whose kernels visit every tile up to the key limit. */
   const int32_t *tiles_q;
   /* since version 4 (a caller may pass the version-3 size, which ends before this field): shape of
    * k, v, kt, vt when it is not q's -- Lk keys (any length >= 1) and Hk key/value heads, Hk a divisor
    * of p.H; query head h reads key/value head h / (H / Hk).  0 means "as q" (p.L, p.H).  k, v and
    * their tangents are then (Z, Hk, Lk, D), the mask strides address (z, h, query, key) with Lk keys,
    * and causal means key index <= query index.  The reference requires q, k, v of one shape
-   * (JA:2367-2378).  key_limit then counts the Lk keys; the tile lists are ignored for such calls. */
+   * (JA:2367-2378).  key_limit then counts the Lk keys; the tile lists are used when Lk equals p.L
+   * (any Hk: they belong to the mask planes, which follow the query heads) and ignored otherwise. */
   int32_t Lk, Hk;
 } jvpfa_fwd_args;
 

@@ -177,7 +177,7 @@ def tile_lists(q, mask, mask_kind, want_k):
     counter, so that layers and the backward reuse one scan."""
     Z, H, L, D = q.shape
     if (not _tile_lists_enabled or mask is None or mask_kind == MASK_NONE or L < TILE_LISTS_MIN_L
-            or q.dtype == torch.float32 or D < 64):
+            or q.dtype == torch.float32 or D not in (64, 128)):
         return None, None
     if mask.dim() != 4 or mask.shape[2] != L or mask.shape[3] != L:
         return None, None
@@ -262,7 +262,7 @@ class HipBackend:
         with torch.cuda.device(q.device):
             lim = key_limit_hint(mask, mask_kind, Z, k.shape[2])
             a.key_limit = _ptr(lim)
-            tq, _ = tile_lists(q, mask, mask_kind, False) if k.shape == q.shape else (None, None)
+            tq, _ = tile_lists(q, mask, mask_kind, False) if k.shape[2] == q.shape[2] else (None, None)
             a.tiles_q = _ptr(tq)
             check(lib.jvpfa_fwd(C.byref(a), _stream(q)))
         return o, ot, M, mu
@@ -291,7 +291,7 @@ class HipBackend:
         with torch.cuda.device(q.device):
             lim = key_limit_hint(mask, mask_kind, Z, k.shape[2])
             a.key_limit = _ptr(lim)
-            tq, tk = tile_lists(q, mask, mask_kind, True) if k.shape == q.shape else (None, None)
+            tq, tk = tile_lists(q, mask, mask_kind, True) if k.shape[2] == q.shape[2] else (None, None)
             a.tiles_q, a.tiles_k = _ptr(tq), _ptr(tk)
             check(lib.jvpfa_bwd(C.byref(a), _stream(q)))
         return dq, dk, dv, dqt, dkt, dvt

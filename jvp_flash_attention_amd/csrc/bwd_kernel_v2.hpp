@@ -528,12 +528,20 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   // Query tiles visited, counted from istart: 0 .. ntiles-1, or the caller's list of the tiles of this
   // key block that hold an attended entry (ascending; only with a mask, where istart is 0);
   // tile_at(i) is the i-th one.
+  // The lists belong to the mask planes, one per query head: with grouped heads the list changes with
+  // the head visited.
   const int *tlist = nullptr;
-  if constexpr (MASK != MASK_NONE) {
-    if (pr.tiles_k) tlist = pr.tiles_k + tile_list_offset(pr, z, h, kb);  // only given when Hk == H
-  }
   const int tmax = (L + BT - 1) / BT - 1;  // index of the last tile of the sequence: bounds whatever a list holds
-  const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1) : (L - istart + BT - 1) / BT;
+  int ntiles = (L - istart + BT - 1) / BT;
+  auto set_list = [&](int hq_) {
+    if constexpr (MASK != MASK_NONE) {
+      if (pr.tiles_k) {
+        tlist = pr.tiles_k + tile_list_offset(pr, z, hq_, kb);
+        ntiles = min(max(tlist[0], 1), tmax + 1);
+      }
+    }
+  };
+  set_list(h * group);
   // List elements are requested a tile ahead, unconditionally (from a harmless address when there is
   // no list: a branch around the read would split the tile loop's straight-line body).
   auto list_slot = [&](int i) { return tlist ? tlist + 1 + i : reinterpret_cast<const int *>(p.q); };
@@ -808,6 +816,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
     if (gi > 0) {
       __syncthreads();  // every wave is done with the previous head's last tile: its stage may be refilled
       set_query_head(h * group + gi);
+      if constexpr (GROUPED) set_list(h * group + gi);
     }
     tcur = tlist ? min(max(tlist[1], 0), tmax) : 0;
     tnext = tlist ? min(max(tlist[1 + min(1, ntiles - 1)], 0), tmax) : min(1, ntiles - 1);

@@ -126,6 +126,7 @@ def test_tile_lists_are_only_made_for_masks_with_a_row_per_query():
         (q[:, :, :256], full[:, :, :256, :256]),                   # too short to pay for the scan
         (q.float(), full),                                          # fp32 kernels visit every tile
         (torch.empty(2, 2, 1024, 32, dtype=torch.bfloat16), full),  # so do the D = 32 kernels
+        (torch.empty(2, 2, 1024, 256, dtype=torch.bfloat16), full),  # and the D = 256 ones (key limit only)
         (q, None),
     ]
     for qq, m in cases:

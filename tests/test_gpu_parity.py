@@ -587,6 +587,54 @@ def test_grouped_heads_with_key_padding_and_skipped_tiles():
     assert grads[1][1, :, 256:].abs().max().item() == 0.0  # key blocks past the limit of batch entry 1
 
 
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("kind", ["blockdiag", "band", "per_head"])
+def test_grouped_heads_with_structured_masks_and_skipped_tiles(D, kind):
+    """Tile lists with 4 query heads over 2 key/value heads: the lists belong to the mask planes (one
+    per query head when the mask has a head axis), so the dk/dv kernel changes list with every query
+    head of a group.  Against the oracle, and bit for bit against visiting every tile."""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H, Hk, L = 2, 4, 2, 700
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(91)
+    q, go, gt = [torch.randn(Z, H, L, D, generator=g).to(dtype) for _ in range(3)]
+    qt = (0.5 * torch.randn(Z, H, L, D, generator=g)).to(dtype)
+    k, v = [torch.randn(Z, Hk, L, D, generator=g).to(dtype) for _ in range(2)]
+    kt, vt = [(0.5 * torch.randn(Z, Hk, L, D, generator=g)).to(dtype) for _ in range(2)]
+    if kind == "per_head":  # a band whose width and offset differ from head to head
+        i, j = torch.arange(L)[:, None], torch.arange(L)[None, :]
+        keep = torch.stack([((i - j) <= 40 + 90 * h) & ((j - i) <= 200 - 60 * h) for h in range(H)]).view(1, H, L, L)
+    else:
+        keep = _structured_keep(kind, Z, H, L)
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    be, scale = _lib.backend(), D**-0.5
+    print(f"case grouped structured {kind} D{D}", flush=True)
+
+    def run(dmask):
+        o, ot, M, mu = be.fwd(*dev[:6], dmask, _lib.MASK_BOOL, False, scale)
+        grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, _lib.MASK_BOOL, False, scale, want_tangent_grads=True)
+        return [o, ot, M, mu, *grads]
+
+    dmask = keep.cuda()
+    try:
+        with_lists = run(dmask)
+        assert getattr(dmask, "_jvpfa_tiles")[1] is not None and getattr(dmask, "_jvpfa_tiles")[2] is not None
+        _lib.set_tile_lists(False)
+        every_tile = run(keep.cuda())
+    finally:
+        _lib.set_tile_lists(True, additive=False)
+    for a, b in zip(with_lists, every_tile):
+        assert torch.equal(a, b)
+    ref = dense.forward(*f64[:6], mask=keep.numpy(), scale=scale)
+    rb = dense.backward(*f64, mask=keep.numpy(), scale=scale)
+    _tol_check("O", with_lists[0], ref["O"], dtype)
+    _tol_check("O'", with_lists[1], ref["Ot"], dtype)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), with_lists[4:10]):
+        _tol_check(n, t, rb[n], dtype)
+
+
 def test_c_abi_from_a_plain_cpp_program():
     """``tests/cabi_host/host_check`` (built with the library) calls jvpfa_fwd / jvpfa_bwd from C++ with
     memory it allocated through the HIP runtime, no Python or torch in its process, and compares with
