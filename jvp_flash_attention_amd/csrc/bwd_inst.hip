@@ -47,6 +47,19 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
     hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
    }
+  } else if constexpr (D == 256 && MODE == BWD_DUAL) {
+    // dk/dv in two launches, each with a register set that fits: dV from K, K' alone, then dK
+    auto kq = bwd_dq_kernel<T, D, MODE, MASK>;
+    auto kv = bwd_dkdv_kernel<T, D, MODE, MASK, DKDV_ONLY_DV>;
+    auto kk = bwd_dkdv_kernel<T, D, MODE, MASK, DKDV_ONLY_DK>;
+    int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);
+    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kv), Cfg::DKV_LDS);
+    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kk), Cfg::DKV_LDS);
+    if (rc != 0) return rc;
+    hipLaunchKernelGGL(kv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+    hipLaunchKernelGGL(kk, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+    hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DQ_LDS, stream, p);
+    return hipGetLastError() == hipSuccess ? 0 : -6;
   } else {
     auto kq = bwd_dq_kernel<T, D, MODE, MASK>;
     auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK>;
