@@ -517,6 +517,21 @@ def test_additive_mask_with_minus_infinity_entries(dt):
 def test_grouped_heads_and_a_key_length_of_its_own(dt, D, shape, mode):
     """Beyond the reference (q, k, v of one shape there): H query heads over Hk key/value heads, Lq
     queries over Lk keys; dk, dv (and dk', dv') have k's shape and sum over the heads of a group."""
+    _run_kv_shape_case(dt, D, shape, mode)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(4, 2, 96, 96), (2, 1, 70, 200), (2, 2, 200, 70), (1, 1, 1, 3), (1, 1, 33, 31), (2, 2, 5, 2)])
+@pytest.mark.parametrize("mode", ["none", "causal", "bool", "bias"])
+def test_head_dim_256_with_grouped_heads_key_lengths_and_tiny_shapes(dt, shape, mode):
+    """The D = 256 forward (two workgroups per query block, 32-key tiles) and the split dk/dv launches
+    on the shapes of the test above, down to a single query."""
+    if mode == "causal" and shape == (1, 1, 1, 3):
+        pytest.skip("one query sees one key under the causal rule: every gradient of q is exactly zero")
+    _run_kv_shape_case(dt, 256, shape, mode)
+
+
+def _run_kv_shape_case(dt, D, shape, mode):
     from jvp_flash_attention_amd import _lib
 
     H, Hk, Lq, Lk = shape
