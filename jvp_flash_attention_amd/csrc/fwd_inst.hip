@@ -73,7 +73,7 @@ static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
       case MASK_ADD: return launch_fwd_wide_one<T, D, DUAL, MASK_ADD>(p, stream);
     }
     return -3;
-  } else if constexpr (sizeof(T) == 2 && D >= 64 && D <= 128) {
+  } else if constexpr (sizeof(T) == 2 && D <= 128) {
     switch (mask) {
       case MASK_NONE:
         // the pipelined kernel pays off where a slot has enough matrix work to hide the softmax behind

@@ -102,14 +102,21 @@ __device__ __forceinline__ int list_take(int v) {
 }
 
 // chunk swizzles (row -> xor value applied to the 16-byte chunk index)
-template <int CH> __device__ __forceinline__ int swz_k(int row) { return CH == 16 ? (row & 15) : ((row >> 1) & 7); }
-template <int CH> __device__ __forceinline__ int swz_v(int row) { return CH == 16 ? ((row & 7) << 1) : (((row >> 1) & 3) << 1); }
+// (CH = 4, rows of 64 bytes: four rows share a line of 256 bytes, which the transposing read of four
+// consecutive rows covers exactly, so only the row-wise read needs its chunks moved)
+template <int CH> __device__ __forceinline__ int swz_k(int row) {
+  return CH == 16 ? (row & 15) : CH == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3);
+}
+template <int CH> __device__ __forceinline__ int swz_v(int row) {
+  return CH == 16 ? ((row & 7) << 1) : CH == 8 ? (((row >> 1) & 3) << 1) : 0;
+}
 
 // Swizzle for tiles that are read both ways (ds_read_b128 along rows and the transposing
 // ds_read_b64_tr_b16 across rows): 16 consecutive rows get 16 different values for the former,
 // and 4 consecutive rows move an aligned chunk pair to 4 different pairs for the latter.
 template <int CH> __device__ __forceinline__ int swz_u(int row) {
   if (CH == 16) return ((row & 7) << 1) | ((row >> 3) & 1);
+  if (CH == 4) return (row >> 2) & 3;
   const int x = (row >> 1) & 7;
   return ((x & 3) << 1) | ((x >> 2) & 1);
 }
