@@ -1,0 +1,114 @@
+"""Lint of the compiled kernels around their inline-asm matrix instructions.
+
+The tuned kernels issue some ``v_mfma`` instructions through inline asm (result tile in ordinary
+vector registers, B operand resident in the accumulation file).  The compiler schedules and
+allocates registers around inline asm but does not look inside it, so it cannot add the idle issue
+slots that the hardware needs
+
+1. between a vector-ALU write to a register (for instance ``v_accvgpr_read_b32`` bringing back a
+   value the allocator parked in the accumulation file) and a matrix instruction that reads it, and
+2. between a matrix instruction and anything else that reads its result.
+
+The sources provide those slots themselves (``s_nop 1`` in front of the matrix instructions whose
+operands live long enough to be parked, ``tiles_ready()`` = ``s_nop 15; s_nop 3`` after each group).
+This module compiles translation units to ISA text and checks that every inline-asm matrix
+instruction in it is covered: ``python -m jvp_flash_attention_amd.asm_lint [unit names]``.
+"""
+from __future__ import annotations
+
+import os
+import re
+import subprocess
+import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+
+from . import build as _build
+
+
+def _regs(tok: str) -> set[int]:
+    tok = tok.strip()
+    m = re.fullmatch(r"v(\d+)", tok)
+    if m:
+        return {int(m.group(1))}
+    m = re.fullmatch(r"v\[(\d+):(\d+)\]", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    return set()
+
+
+def scan(isa_text: str, where: str = "") -> list[str]:
+    """Findings (one line each) in the ISA text of one translation unit."""
+    out = []
+    kern, inasm, hist, pending = "?", False, [], set()
+    for ln in isa_text.splitlines():
+        t = ln.strip()
+        if t.startswith("_Z") and ":" in t and "$" not in t.split(":")[0]:
+            kern, hist, pending = t.split(":")[0], [], set()
+            continue
+        if "ASMSTART" in t:
+            inasm = True
+            continue
+        if "ASMEND" in t:
+            inasm = False
+            continue
+        if not t or t[0] in ";.":
+            continue
+        t = t.split(";")[0].strip()
+        if not t:
+            continue
+        op = t.split()[0]
+        ops = [x.strip() for x in t.split(None, 1)[1].split(",")] if " " in t else []
+        if op == "s_nop" and ops and int(ops[0]) >= 15:
+            pending = set()  # tiles_ready(): results of the group are readable from here on
+        if op.startswith("v_mfma"):
+            dst, srcs = _regs(ops[0]), set()
+            for o in ops[1:4]:
+                srcs |= _regs(o)
+            if inasm:
+                guarded = bool(hist) and hist[-1][0] == "s_nop"
+                if not guarded:
+                    for pop, pops in hist[-2:]:
+                        if pop.startswith("v_") and not pop.startswith("v_mfma") and pops and (_regs(pops[0]) & srcs):
+                            out.append(f"{where} {kern}: '{pop} {pops[0]}' feeds '{t[:60]}' without idle slots")
+                pending |= dst
+            else:
+                pending -= dst
+        elif pending and op.startswith(("v_", "ds_write", "global_store", "buffer_store", "scratch_store")):
+            srcs = set()
+            for o in (ops[1:] if op.startswith("v_") else ops):
+                srcs |= _regs(o)
+            if srcs & pending:
+                out.append(f"{where} {kern}: '{t[:60]}' reads a matrix result before the wait that follows its group")
+        hist.append((op, ops))
+    return out
+
+
+def isa_of(unit) -> str:
+    """Device ISA text of one translation unit of ``build.units()``."""
+    name, src, defs = unit
+    with tempfile.TemporaryDirectory() as td:
+        path = os.path.join(td, name + ".s")
+        cmd = [_build.HIPCC, *_build.FLAGS, *defs, "-S", "--cuda-device-only", src, "-o", path]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc -S failed for {name}:\n{r.stderr[-4000:]}")
+        with open(path) as f:
+            return f.read()
+
+
+def lint(names=None, jobs: int | None = None) -> list[str]:
+    """Compile the named units (default: every kernel unit) to ISA and scan them."""
+    units = [u for u in _build.units() if u[0].startswith(("fwd_", "bwd_")) and (not names or u[0] in names)]
+    with ThreadPoolExecutor(max_workers=jobs or min(8, os.cpu_count() or 1)) as ex:
+        texts = list(ex.map(isa_of, units))
+    findings = []
+    for u, text in zip(units, texts):
+        findings += scan(text, u[0])
+    return findings
+
+
+if __name__ == "__main__":
+    found = lint(sys.argv[1:] or None)
+    print("\n".join(found) if found else "asm lint: clean")
+    sys.exit(1 if found else 0)

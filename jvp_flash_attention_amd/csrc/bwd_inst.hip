@@ -18,7 +18,7 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
   // when k, v have q's shape)
   const long long kv_blocks = (long long)((p.pr.Lk + BWD_BLK - 1) / BWD_BLK) * p.pr.Z * p.pr.Hk;
   if (kv_blocks > 0x7fffffffLL) return -2;
-  if constexpr (sizeof(T) == 2 && D >= 64 && D <= 128) {  // direct-to-LDS, double-buffered kernels
+  if constexpr (sizeof(T) == 2 && D <= 128) {  // direct-to-LDS, double-buffered kernels
    {
     using Cfg2 = Bwd2Cfg<T, D, MODE>;
     // gO may be absent only in the dual mode (loss depends on O' alone)
@@ -26,7 +26,7 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
     constexpr bool NG = MODE != BWD_DUAL;  // the GO template argument of the kernels without gO
     void (*kq)(const BwdParams), (*kkv)(const BwdParams);
     const bool grouped = p.pr.Hk != p.pr.H;  // a key/value head serves several query heads
-    if constexpr (D <= 64) {  // the register-capped twins: two workgroups per compute unit
+    if constexpr (D == 64) {  // the register-capped twins: two workgroups per compute unit (D = 32 needs no cap for that)
       kq = no_go ? bwd2_dq_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dq_kernel_2wg<T, D, MODE, MASK, true>;
       if constexpr (MASK == MASK_NONE || MODE != BWD_DUAL) {
         if (grouped) kkv = no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, true, true>;

@@ -203,7 +203,9 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   // tile slots in a stage: 0 K, 1 V, 2 K', 3 V'
   constexpr int NLOAD = IPW * Cfg::NTILE;
   constexpr int NACC = DUAL ? 2 : 1;            // operand tensors of the accumulation (K, K')
-  constexpr int NPV = 2 * DB / 2;               // accumulation steps of a half: (chunk c, pair of d-blocks)
+  constexpr int PW = DB >= 2 ? 2 : 1;           // d-blocks per accumulation step (one for D = 32)
+  constexpr int NDP = DB / PW;
+  constexpr int NPV = 2 * NDP;                  // accumulation steps of a half: (chunk c, group of PW d-blocks)
   constexpr int NSTEP = 2 * (KK + NPV);
   auto prepare_loads = [&](int stage, int j0, bool on) {
     ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
@@ -316,13 +318,13 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
     }
 
     // ---- dQ^T += K^T dS^T (+ K'^T dS'^T): steps over (key chunk c, pair of d-blocks) -------------
-    FragT tk[2][2], tkt[2][2];  // [ring slot][d-block of the pair]
+    FragT tk[2][PW], tkt[2][PW];  // [ring slot][d-block of the group]
     auto issue_t = [&](auto ic) {
-      constexpr int i = decltype(ic)::value, c = i / (DB / 2), dp = i % (DB / 2), sl = i % 2;
+      constexpr int i = decltype(ic)::value, c = i / NDP, dp = i % NDP, sl = i % 2;
       constexpr int TO = (HB * 32 + c * 16) * ROWB;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const uint32_t a0 = sbase + toff[2 * dp + u][0], a1 = sbase + toff[2 * dp + u][1];
+      for (int u = 0; u < PW; ++u) {
+        const uint32_t a0 = sbase + toff[PW * dp + u][0], a1 = sbase + toff[PW * dp + u][1];
         tk[sl][u].lo = lds_tr64<TO>(a0);
         tk[sl][u].hi = lds_tr64<TO>(a1);
         if constexpr (DUAL) {
@@ -331,19 +333,25 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
         }
       }
     };
-    constexpr int NRT = 4 * NACC;
+    constexpr int NRT = 2 * PW * NACC;
     issue_t(std::integral_constant<int, 0>{});
     static_for<NPV>([&](auto ic) {
-      constexpr int i = decltype(ic)::value, c = i / (DB / 2), dp = i % (DB / 2), sl = i % 2;
+      constexpr int i = decltype(ic)::value, c = i / NDP, dp = i % NDP, sl = i % 2;
       if constexpr (i + 1 < NPV) issue_t(std::integral_constant<int, i + 1>{});
-      if constexpr (DUAL) lds_wait<(i + 1 < NPV) ? NRT : 0>(tk[sl][0], tk[sl][1], tkt[sl][0], tkt[sl][1]);
-      else lds_wait<(i + 1 < NPV) ? NRT : 0>(tk[sl][0], tk[sl][1]);
+      constexpr int younger = (i + 1 < NPV) ? NRT : 0;
+      if constexpr (PW == 2) {
+        if constexpr (DUAL) lds_wait<younger>(tk[sl][0], tk[sl][1], tkt[sl][0], tkt[sl][1]);
+        else lds_wait<younger>(tk[sl][0], tk[sl][1]);
+      } else {
+        if constexpr (DUAL) lds_wait<younger>(tk[sl][0], tkt[sl][0]);
+        else lds_wait<younger>(tk[sl][0].lo, tk[sl][0].hi);
+      }
       load_step(std::integral_constant<int, 2 * KK + HB * NPV + i>{});
-      mma(acc[2 * dp], as_frag<T>(tk[sl][0]), dsf[c]);
-      mma(acc[2 * dp + 1], as_frag<T>(tk[sl][1]), dsf[c]);
+#pragma unroll
+      for (int u = 0; u < PW; ++u) mma(acc[PW * dp + u], as_frag<T>(tk[sl][u]), dsf[c]);
       if constexpr (DUAL) {
-        mma(acc[2 * dp], as_frag<T>(tkt[sl][0]), dspf[c]);
-        mma(acc[2 * dp + 1], as_frag<T>(tkt[sl][1]), dspf[c]);
+#pragma unroll
+        for (int u = 0; u < PW; ++u) mma(acc[PW * dp + u], as_frag<T>(tkt[sl][u]), dspf[c]);
       }
     });
   };

@@ -57,14 +57,17 @@ template <bool FIRST> __device__ __forceinline__ void mma_vra(f32x16 &c, const f
   if constexpr (FIRST) asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
   else asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
 }
-// the same with the B operand in ordinary vector registers
+// The same with the B operand in ordinary vector registers.  Under register pressure the compiler may
+// park such a long-lived operand in the accumulation file and copy it back just before its use; a
+// matrix instruction must not read a register within two issue slots of a vector-ALU write to it, and
+// the compiler does not look inside inline asm, so the two slots are written here.
 template <bool FIRST> __device__ __forceinline__ void mma_vrv(f32x16 &c, const bf16x8 &a, const bf16x8 &b) {
-  if constexpr (FIRST) asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
-  else asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  if constexpr (FIRST) asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  else asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
 template <bool FIRST> __device__ __forceinline__ void mma_vrv(f32x16 &c, const f16x8 &a, const f16x8 &b) {
-  if constexpr (FIRST) asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
-  else asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  if constexpr (FIRST) asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  else asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
 // 16 + 4 idle issue slots: the last matrix-core pass has written its registers when this returns
 __device__ __forceinline__ void tiles_ready(f32x16 &a) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a)); }

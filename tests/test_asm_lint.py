@@ -1,0 +1,44 @@
+"""The lint that checks the idle issue slots around inline-asm matrix instructions
+(``jvp_flash_attention_amd/asm_lint.py``): it must flag the two patterns on hand-written ISA text and
+find none in freshly compiled kernels."""
+from jvp_flash_attention_amd import asm_lint
+
+PARKED_OPERAND = """
+_ZN5jvpfa4kernEv:
+	v_accvgpr_read_b32 v19, a61
+	;;#ASMSTART
+	v_mfma_f32_32x32x16_bf16 v[32:47], v[64:67], v[16:19], v[32:47]
+	;;#ASMEND
+	s_nop 15
+	s_nop 3
+	v_mul_f32_e32 v1, v32, v2
+"""
+
+EARLY_READ = """
+_ZN5jvpfa4kernEv:
+	;;#ASMSTART
+	v_mfma_f32_32x32x16_bf16 v[32:47], v[64:67], a[16:19], 0
+	;;#ASMEND
+	v_accvgpr_write_b32 a70, v33
+	s_nop 15
+	s_nop 3
+"""
+
+
+def test_a_parked_operand_restored_right_before_its_matrix_instruction_is_flagged():
+    found = asm_lint.scan(PARKED_OPERAND, "unit")
+    assert len(found) == 1 and "without idle slots" in found[0]
+    guarded = PARKED_OPERAND.replace("\tv_mfma", "\ts_nop 1\n\tv_mfma")
+    assert asm_lint.scan(guarded, "unit") == []
+
+
+def test_a_result_read_before_the_wait_is_flagged():
+    found = asm_lint.scan(EARLY_READ, "unit")
+    assert len(found) == 1 and "before the wait" in found[0]
+    assert asm_lint.scan(EARLY_READ.replace("\tv_accvgpr_write_b32 a70, v33\n", ""), "unit") == []
+
+
+def test_compiled_kernels_are_clean():
+    # the D = 32 backward is where the allocator once parked a resident operand in the accumulation
+    # file and restored it in front of its matrix instruction
+    assert asm_lint.lint(["bwd_bf16_32", "fwd_bf16_64"]) == []
