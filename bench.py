@@ -117,8 +117,8 @@ def hvp_sweep(be, _lib):
 
 
 def shape_rows(be, _lib):
-    """Shapes next to the headline one, bf16, no mask: D = 256 (the largest head dim the reference
-    admits), 16 query heads over 4 key/value heads, and 4096 queries over 512 keys (the last two are
+    """Shapes next to the headline one, bf16, no mask: D = 32 and D = 256 (the smallest and the largest
+    head dim the reference admits), 16 query heads over 4 key/value heads, and 4096 queries over 512 keys (the last two are
     shapes the reference refuses).  Dual forward and dual backward, counted as 12 and 24 flops per
     (query, key, d) triple."""
     import torch
@@ -126,6 +126,7 @@ def shape_rows(be, _lib):
     dev = torch.device("cuda:0")
     rows = {}
     for name, (Zs, Hs, Hk, Lq, Lk, Ds) in {
+        "B4_H16_L2048_D32": (4, 16, 16, 2048, 2048, 32),
         "B4_H16_L2048_D256": (4, 16, 16, 2048, 2048, 256),
         "B4_H16_over_4_kv_heads_L4096_D128": (4, 16, 4, 4096, 4096, 128),
         "B4_H16_Lq4096_Lk512_D128": (4, 16, 16, 4096, 512, 128),
