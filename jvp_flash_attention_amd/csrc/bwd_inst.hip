@@ -47,7 +47,7 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
     hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
    }
-  } else if constexpr (D == 256 && MODE == BWD_DUAL) {
+  } else if constexpr (BWD_WIDE_ROWS<T, D> && sizeof(T) == 2 && MODE == BWD_DUAL) {  // (fp32 D = 128 is bound by its matrix rate either way)
     // dk/dv in two launches, each with a register set that fits: dV from K, K' alone, then dK
     auto kq = bwd_dq_kernel<T, D, MODE, MASK>;
     auto kv = bwd_dkdv_kernel<T, D, MODE, MASK, DKDV_ONLY_DV>;

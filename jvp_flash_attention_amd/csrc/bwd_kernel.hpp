@@ -82,6 +82,8 @@ template <typename T, int D, int MODE> struct BwdCfg {
 // whether the dq / dk,dv kernels fetch the next tile into registers during the current one's
 // computation (needs up to 64 registers; see the forward kernel)
 template <typename T, int D> constexpr bool BWD_FETCH_AHEAD = D == 64 || (D == 32 && sizeof(T) == 4);
+// rows of 512 bytes: the resident operands of the dual backward fill the register file by themselves
+template <typename T, int D> constexpr bool BWD_WIDE_ROWS = D * sizeof(T) >= 512;
 
 template <int KK, typename T>
 __device__ __forceinline__ void load_row_frags(Frag<T> *f, const T *row, int g) {
@@ -94,9 +96,9 @@ __device__ __forceinline__ void gemm_tile(f32x16 &acc, const T *tile, int ld, in
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) {
     mma(acc, lds_frag(tile + arow * ld + 16 * kk + 8 * g), b[kk]);
-    // D = 256: the register file is full of resident operands; keep the scheduler from hoisting
-    // more than four fragment reads above the products that consume them
-    if constexpr (KK >= 16) {
+    // rows of 512 bytes (D = 256; fp32 D = 128): the register file is full of resident operands; keep
+    // the scheduler from hoisting more than four fragment reads above the products that consume them
+    if constexpr (KK * sizeof(Frag<T>) >= 256) {
       if (kk % 4 == 3) __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -273,7 +275,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
       for (int db = 0; db < DB; ++db) {
         mma(acc[db], lds_frag(KT + (32 * db + pr32) * Cfg::LDT + 16 * c + 8 * g), dsf);
         if constexpr (DUAL) mma(acc[db], lds_frag(KtT + (32 * db + pr32) * Cfg::LDT + 16 * c + 8 * g), dspf);
-        if constexpr (DB >= 8) {  // D = 256: as in gemm_tile, bound the fragment reads in flight
+        if constexpr (BWD_WIDE_ROWS<T, D>) {  // as in gemm_tile, bound the fragment reads in flight
           if (db % 2 == 1) __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
 // dk, dv (MODE PLAIN / DUAL) or dk', dv' (MODE TANGENT).  Scores are S = Q K^T (lane = key,
 // registers = queries), so P and dS are the B operands of dV^T += gO^T P and dK^T += Q^T dS.
 //
-// PART (BWD_DUAL only) splits the work over two launches for D = 256, where the resident operands
+// PART (BWD_DUAL only) splits the work over two launches for rows of 512 bytes, where the resident operands
 // (K, K', V, V': 4 x 64 registers) and both accumulators (2 x 128) do not fit one wave:
 // DKDV_ONLY_DV keeps K, K' and dV (it needs S, S' only), DKDV_ONLY_DK keeps all four and dK.
 enum DkdvPart { DKDV_BOTH = 0, DKDV_ONLY_DV = 1, DKDV_ONLY_DK = 2 };
@@ -527,7 +529,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
           mma(dK[db], lds_frag(QT + off), dspf);
           mma(dV[db], lds_frag(GT + off), pf);
         }
-        if constexpr (DB >= 8) {  // D = 256: as in gemm_tile, bound the fragment reads in flight
+        if constexpr (BWD_WIDE_ROWS<T, D>) {  // as in gemm_tile, bound the fragment reads in flight
           if (db % 2 == 1) __builtin_amdgcn_sched_barrier(0);
         }
       }
