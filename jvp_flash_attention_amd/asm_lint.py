@@ -26,14 +26,15 @@ from concurrent.futures import ThreadPoolExecutor
 from . import build as _build
 
 
-def _regs(tok: str) -> set[int]:
+def _regs(tok: str) -> set[tuple[str, int]]:
+    """Registers named by an operand: ('v', n) ordinary, ('a', n) accumulation file."""
     tok = tok.strip()
-    m = re.fullmatch(r"v(\d+)", tok)
+    m = re.fullmatch(r"([va])(\d+)", tok)
     if m:
-        return {int(m.group(1))}
-    m = re.fullmatch(r"v\[(\d+):(\d+)\]", tok)
+        return {(m.group(1), int(m.group(2)))}
+    m = re.fullmatch(r"([va])\[(\d+):(\d+)\]", tok)
     if m:
-        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+        return {(m.group(1), n) for n in range(int(m.group(2)), int(m.group(3)) + 1)}
     return set()
 
 
@@ -71,7 +72,7 @@ def scan(isa_text: str, where: str = "") -> list[str]:
                     for pop, pops in hist[-2:]:
                         if pop.startswith("v_") and not pop.startswith("v_mfma") and pops and (_regs(pops[0]) & srcs):
                             out.append(f"{where} {kern}: '{pop} {pops[0]}' feeds '{t[:60]}' without idle slots")
-                pending |= dst
+                pending |= {r for r in dst if r[0] == "v"}  # results in the accumulation file are only read by matrix instructions
             else:
                 pending -= dst
         elif pending and op.startswith(("v_", "ds_write", "global_store", "buffer_store", "scratch_store")):

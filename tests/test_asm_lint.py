@@ -32,6 +32,12 @@ def test_a_parked_operand_restored_right_before_its_matrix_instruction_is_flagge
     assert asm_lint.scan(guarded, "unit") == []
 
 
+def test_a_resident_operand_rewritten_right_before_its_matrix_instruction_is_flagged():
+    text = PARKED_OPERAND.replace("v_accvgpr_read_b32 v19, a61", "v_accvgpr_write_b32 a18, v7").replace("v[16:19]", "a[16:19]")
+    found = asm_lint.scan(text, "unit")
+    assert len(found) == 1 and "without idle slots" in found[0]
+
+
 def test_a_result_read_before_the_wait_is_flagged():
     found = asm_lint.scan(EARLY_READ, "unit")
     assert len(found) == 1 and "before the wait" in found[0]
