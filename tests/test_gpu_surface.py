@@ -283,6 +283,37 @@ def test_config2_dense_bf16_full_size_properties():
     assert _rel(dvt, g1[2]) <= 1e-2
 
 
+@pytest.mark.parametrize("D,causal", [(32, False), (32, True), (256, False), (256, True)])
+def test_other_head_dims_at_benchmark_size(D, causal):
+    """bf16 B4 H16 L2048 with D = 32 and D = 256: a head computed inside the whole batch (more workgroups
+    than compute units, heads spread over the dies, for D = 256 two workgroups per query block) equals the
+    same head computed alone, bit for bit, forward and backward; one slab is checked against the oracle."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    Z, H, L = 4, 16, 2048
+    dt, scale = torch.bfloat16, D**-0.5
+    q, k, v, go, gt = [_randn((Z, H, L, D), dt, 80 + i) for i in range(5)]
+    qt, kt, vt = [_randn((Z, H, L, D), dt, 90 + i, std=0.5) for i in range(3)]
+    o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, 0, causal, scale)
+    grads = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, 0, causal, scale, want_tangent_grads=True)
+    for z, h in ((0, 0), (3, 15), (2, 9)):
+        one = [x[z:z + 1, h:h + 1].contiguous() for x in (q, k, v, qt, kt, vt, go, gt)]
+        o1, ot1, M1, mu1 = be.fwd(*one[:6], None, 0, causal, scale)
+        assert torch.equal(o[z, h], o1[0, 0]) and torch.equal(ot[z, h], ot1[0, 0])
+        assert torch.equal(M[z, h], M1[0, 0]) and torch.equal(mu[z, h], mu1[0, 0])
+        g1 = be.bwd(*one[:6], o1, ot1, M1, mu1, one[6], one[7], None, 0, causal, scale, want_tangent_grads=True)
+        for n, a_, b_ in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads, g1):
+            assert torch.equal(a_[z, h], b_[0, 0]), n
+    z, h = 1, 5
+    f64 = [x[z, h:h + 1][None].double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    ref = dense.forward(*f64[:6], causal=causal)
+    rb = dense.backward(*f64, causal=causal)
+    assert _rel(o[z, h], ref["O"][0, 0]) <= 2e-2 and _rel(ot[z, h], ref["Ot"][0, 0]) <= 2e-2
+    for n, g in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        assert _rel(g[z, h], rb[n][0, 0]) <= 2e-2, n
+
+
 def test_config3_causal_long_full_size_properties():
     """benchmark configuration 3: fp16 B2 H32 L4096 D128 causal, and the headline bf16 B4 H16 L4096 D128."""
     from jvp_flash_attention_amd import _lib
