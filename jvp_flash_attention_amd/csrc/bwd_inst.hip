@@ -4,6 +4,7 @@
 // hipStream_t): pre-pass, then the dq and dk/dv kernels of every requested mode.
 #include "bwd_kernel.hpp"
 #include "bwd_kernel_v2.hpp"
+#include "bwd_kernel_wide.hpp"
 #include "launch.hpp"
 
 namespace jvpfa {
@@ -47,18 +48,31 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
     hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
    }
-  } else if constexpr (BWD_WIDE_ROWS<T, D> && sizeof(T) == 2 && MODE == BWD_DUAL) {  // (fp32 D = 128 is bound by its matrix rate either way)
-    // dk/dv in two launches, each with a register set that fits: dV from K, K' alone, then dK
-    auto kq = bwd_dq_kernel<T, D, MODE, MASK>;
-    auto kv = bwd_dkdv_kernel<T, D, MODE, MASK, DKDV_ONLY_DV>;
-    auto kk = bwd_dkdv_kernel<T, D, MODE, MASK, DKDV_ONLY_DK>;
-    int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);
-    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kv), Cfg::DKV_LDS);
-    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kk), Cfg::DKV_LDS);
+  } else if constexpr (sizeof(T) == 2 && D == 256) {
+    // dq: two workgroups per query block, each with 128 of its columns, on the direct-to-LDS pipeline
+    using CfgW = BwdWideCfg<T, D, 128, MODE>;
+    const bool no_go = MODE == BWD_DUAL && p.go == nullptr;
+    constexpr bool NG = MODE != BWD_DUAL;
+    void (*kq)(const BwdParams) = no_go ? bwdw_dq_kernel<T, D, 128, MODE, MASK, NG> : bwdw_dq_kernel<T, D, 128, MODE, MASK, true>;
+    if (blocks * CfgW::NS > 0x7fffffffLL) return -2;
+    int rc = allow_lds(reinterpret_cast<const void *>(kq), CfgW::DQ_LDS);
     if (rc != 0) return rc;
-    hipLaunchKernelGGL(kv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
-    hipLaunchKernelGGL(kk, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
-    hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DQ_LDS, stream, p);
+    if constexpr (MODE == BWD_DUAL) {
+      // dk/dv in two launches, each with a register set that fits: dV from K, K' alone, then dK
+      auto kv = bwd_dkdv_kernel<T, D, MODE, MASK, DKDV_ONLY_DV>;
+      auto kk = bwd_dkdv_kernel<T, D, MODE, MASK, DKDV_ONLY_DK>;
+      rc = allow_lds(reinterpret_cast<const void *>(kv), Cfg::DKV_LDS);
+      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kk), Cfg::DKV_LDS);
+      if (rc != 0) return rc;
+      hipLaunchKernelGGL(kv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+      hipLaunchKernelGGL(kk, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+    } else {
+      auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK>;
+      rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg::DKV_LDS);
+      if (rc != 0) return rc;
+      hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+    }
+    hipLaunchKernelGGL(kq, dim3((unsigned)(blocks * CfgW::NS)), dim3(CfgW::NT), CfgW::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
   } else {
     auto kq = bwd_dq_kernel<T, D, MODE, MASK>;

@@ -49,13 +49,27 @@ __device__ __forceinline__ float acc_scale(float x, float alpha) {
 // result may only be read by other instruction kinds after tiles_ready().
 __device__ __forceinline__ void pin_acc(bf16x8 &f) { asm volatile("" : "+a"(f)); }
 __device__ __forceinline__ void pin_acc(f16x8 &f) { asm volatile("" : "+a"(f)); }
-template <bool FIRST> __device__ __forceinline__ void mma_vra(f32x16 &c, const bf16x8 &a, const bf16x8 &b) {
-  if constexpr (FIRST) asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-  else asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+// GUARD: two idle issue slots in front, for kernels whose resident operands fill the accumulation file
+// to the last register, where the allocator moves them through a spare register right before their
+// use (a matrix instruction must not read a register that soon after a vector-ALU write to it, and
+// the compiler does not look inside inline asm).
+template <bool FIRST, bool GUARD = false> __device__ __forceinline__ void mma_vra(f32x16 &c, const bf16x8 &a, const bf16x8 &b) {
+  if constexpr (GUARD) {
+    if constexpr (FIRST) asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+    else asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  } else {
+    if constexpr (FIRST) asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+    else asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  }
 }
-template <bool FIRST> __device__ __forceinline__ void mma_vra(f32x16 &c, const f16x8 &a, const f16x8 &b) {
-  if constexpr (FIRST) asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-  else asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+template <bool FIRST, bool GUARD = false> __device__ __forceinline__ void mma_vra(f32x16 &c, const f16x8 &a, const f16x8 &b) {
+  if constexpr (GUARD) {
+    if constexpr (FIRST) asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+    else asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  } else {
+    if constexpr (FIRST) asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+    else asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  }
 }
 // The same with the B operand in ordinary vector registers.  Under register pressure the compiler may
 // park such a long-lived operand in the accumulation file and copy it back just before its use; a
