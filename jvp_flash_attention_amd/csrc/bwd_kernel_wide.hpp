@@ -343,4 +343,441 @@ template <typename T, int D, int DV, int MODE, int MASK, bool GO>
 __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {}
 #endif
 
+// ------------------------------------------------------------------------------------------------
+// dk, dv (PLAIN / DUAL) or dk', dv' (TANGENT) for D = 256: workgroup = 128 keys of a head, loop over
+// 32-query tiles of Q, G (, Q', gT) with their row statistics.  What a launch produces:
+//   WIDE_DV    (DUAL) dV, all 256 columns: it needs S and S' only, so K, K' are resident (2 x 64
+//              registers) next to the accumulators (128)
+//   WIDE_DK    (DUAL) 128 columns of dK, two workgroups per key block: K, V, K', V' resident (the
+//              whole accumulation file), the accumulators in ordinary registers
+//   WIDE_BOTH  (PLAIN, TANGENT) 128 columns of dK and of dV, two workgroups per key block
+// k, v must have q's heads (grouped heads take the LDS-copy kernels).
+enum WidePart { WIDE_BOTH = 0, WIDE_DV = 1, WIDE_DK = 2 };
+
+template <typename T, int D, int DV, int MODE> struct BwdWideKvCfg : BwdWideCfg<T, D, DV, MODE> {
+  static constexpr int NSTAT = MODE == BWD_DUAL ? 4 : 2;
+  static constexpr int STATB = NSTAT * 64 * 4;  // 64 floats per statistic and stage (32 used)
+  static constexpr size_t DKV_LDS = 2 * (size_t)BwdWideCfg<T, D, DV, MODE>::STAGEB + 2 * (size_t)STATB;
+};
+
+#if defined(__HIP_DEVICE_COMPILE__)
+template <typename T, int D, int DV, int MODE, int MASK, bool GO, int PART>
+__global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
+  using Cfg = BwdWideKvCfg<T, D, DV, MODE>;
+  constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
+  static_assert(DUAL ? (PART == WIDE_DV || PART == WIDE_DK) : PART == WIDE_BOTH);
+  constexpr bool WANT_DK = PART != WIDE_DV, WANT_DV = PART != WIDE_DK;
+  constexpr bool NEED_V = !DUAL || WANT_DK;  // V (, V') enter only through dP, A, B
+  constexpr int NSL = PART == WIDE_DV ? 1 : Cfg::NS;  // workgroups per key block
+  constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT;
+  constexpr int KK = D / 16;
+  constexpr int DBK = WANT_DK ? DV / 32 : 1;                             // d-blocks of the dK accumulator
+  constexpr int DBV = WANT_DV ? (PART == WIDE_DV ? D / 32 : DV / 32) : 1;  // ... of the dV accumulator
+  constexpr int DBS = PART == WIDE_DV ? D / 32 : DV / 32;                // d-blocks visited by a step
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem_raw;
+  const Problem &pr = p.pr;
+  const int L = pr.L, Lk = pr.Lk;  // queries, keys
+  const int nblk = (Lk + Cfg::BLK - 1) / Cfg::BLK;
+  const int id = xcd_remap(blockIdx.x, nblk * NSL, pr.Z * pr.H);
+  const int zh = id / (nblk * NSL);
+  const int rem = id % (nblk * NSL);
+  const int slice = rem % NSL;
+  const int kb = rem / NSL;  // causal: the first key blocks have the longest query loops
+  const int z = zh / pr.H, h = zh % pr.H;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
+  const int r = lane % 32, g = lane / 32, pr32 = perm32(r);
+  const size_t head = (size_t)zh * Lk * D;   // of k, v and their gradients (as many heads as q)
+  const size_t qhead = (size_t)zh * L * D;   // of q, gO, q', gT
+  const size_t srow = (size_t)zh * L;
+  const int k0 = kb * Cfg::BLK;
+  const int krow = k0 + wave * 32 + r;
+  const int kld = krow < Lk ? krow : Lk - 1;
+  constexpr bool has_go = GO;
+  T *outk = reinterpret_cast<T *>(TAN ? p.dkt : p.dk) + head + (size_t)krow * D + slice * DV;
+  T *outv = reinterpret_cast<T *>(TAN ? p.dvt : p.dv) + head + (size_t)krow * D + (PART == WIDE_DV ? 0 : slice * DV);
+  if constexpr (MASK != MASK_NONE) {
+    // a key block that the caller's hint declares fully masked has zero gradients
+    if (pr.klimit && k0 >= pr.klimit[z]) {
+      if (krow < Lk) {
+        float zero8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int d0 = 8 * g; d0 < 32 * DBS; d0 += 16) {
+          if constexpr (WANT_DK) store8<T>(outk + d0, zero8);
+          if constexpr (WANT_DV) store8<T>(outv + d0, zero8);
+        }
+      }
+      return;
+    }
+  }
+
+  // direct loads of the streamed tiles, as in the dq kernel above
+  uint32_t ld_o[IPW];
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) {
+    const int lc = 64 * (wave * IPW + i) + lane;
+    const int row = lc / CH;
+    ld_o[i] = row * ROWB + (((lc % CH) ^ swz_w(row)) * 16);
+  }
+  uint32_t ld_dst = 0;
+  __amdgpu_buffer_rsrc_t ld_rs[4];
+  auto tile_rsrc = [&](const char *base, int j, bool exists) {
+    const int rows = exists ? max(L - j, 0) : 0;
+    return __builtin_amdgcn_make_buffer_rsrc((void *)(base + (size_t)j * ROWB), 0, rows * ROWB, 0x00020000);
+  };
+  auto load_piece = [&](auto pc) {
+    constexpr int pi = decltype(pc)::value, i = pi / Cfg::NTILE, ts = pi % Cfg::NTILE;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ld_rs[ts], (JVPFA_LDS(void))(uintptr_t)(ld_dst + i * 1024 + ts * TILEB),
+                                             16, ld_o[i], 0, 0, 0);
+  };
+  uint32_t noff[8];  // row-major fragment, steps kk and kk+8 differ by 256 bytes
+  {
+    const int x = swz_w(pr32);
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) noff[kk] = pr32 * ROWB + (((2 * kk + g) ^ x) * 16);
+  }
+  // transposed fragment: d-block db of this launch's columns is at toff[db % 4] + 256 * (db / 4)
+  uint32_t toff[4][2];
+  {
+    const int a_ = (lane >> 4) & 1, j_ = lane & 15;
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int row = 8 * g + 4 * hh + (j_ >> 2);
+        const int ch = (4 * db + 2 * a_ + (j_ & 1)) ^ swz_w(row);
+        toff[db][hh] = row * ROWB + (16 * (PART == WIDE_DV ? 0 : slice) + ch) * 16 + 8 * ((j_ >> 1) & 1);
+      }
+    }
+  }
+  const uint32_t stat0 = lds0 + 2 * Cfg::STAGEB;  // row statistics, two stages of NSTAT x 64 floats
+
+  Frag<T> Kf[KK], Vf[NEED_V ? KK : 1], Ktf[DUAL ? KK : 1], Vtf[DUAL && NEED_V ? KK : 1];
+  load_bfrags<KK>(Kf, reinterpret_cast<const T *>(p.k) + head + (size_t)kld * D, g);
+  if constexpr (NEED_V) load_bfrags<KK>(Vf, reinterpret_cast<const T *>(p.v) + head + (size_t)kld * D, g);
+  if constexpr (DUAL) {
+    load_bfrags<KK>(Ktf, reinterpret_cast<const T *>(p.kt) + head + (size_t)kld * D, g);
+    if constexpr (NEED_V) load_bfrags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + head + (size_t)kld * D, g);
+  }
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    pin_acc(Kf[kk]);
+    if constexpr (NEED_V) pin_acc(Vf[kk]);
+    if constexpr (DUAL) {
+      pin_acc(Ktf[kk]);
+      if constexpr (NEED_V) pin_acc(Vtf[kk]);
+    }
+  }
+  // the accumulation file is full (or nearly) in every variant: see mma_vra
+  constexpr bool GD = true;
+
+  f32x16 dK[DBK], dV[DBV];
+#pragma unroll
+  for (int db = 0; db < DBK; ++db) zero_acc(dK[db]);
+#pragma unroll
+  for (int db = 0; db < DBV; ++db) zero_acc(dV[db]);
+
+  const float sl2 = pr.scale * LOG2E;
+  bool mask_small = true;
+  uint32_t mlane = 0;
+  if constexpr (MASK != MASK_NONE) {
+    const int64_t lim = (int64_t)1 << 31;
+    mask_small = pr.ms[2] >= 0 && pr.ms[3] >= 0 && 8 * pr.ms[2] + (int64_t)Lk * pr.ms[3] < lim;
+    mlane = (uint32_t)(8 * g * pr.ms[2] + (int64_t)kld * pr.ms[3]);
+  }
+  // tile slots 0 Q, 1 G (gO; gT in TANGENT; gT again in DUAL without gO), 2 Q', 3 gT, and the
+  // statistics slots PLAIN M, d1 | DUAL M, mu, a, d2 (= d1 + d2) | TANGENT M, a
+  const char *Qb = reinterpret_cast<const char *>(p.q) + qhead * sizeof(T);
+  const char *gTb = (DUAL || TAN) ? reinterpret_cast<const char *>(p.gt) + qhead * sizeof(T) : nullptr;
+  const char *Gb = TAN ? gTb : (has_go ? reinterpret_cast<const char *>(p.go) + qhead * sizeof(T) : gTb);
+  const char *Qtb = DUAL ? reinterpret_cast<const char *>(p.qt) + qhead * sizeof(T) : nullptr;
+  const float *st_p[4] = {p.M + srow, MODE == BWD_PLAIN ? p.d1 + srow : (DUAL ? p.mu + srow : p.a + srow),
+                          DUAL ? p.a + srow : nullptr, DUAL ? p.d2 + srow : nullptr};
+
+  const int istart = pr.causal ? (k0 / BT) * BT : 0;
+  const int ntiles = (L - istart + BT - 1) / BT;
+  constexpr int NLOAD = IPW * Cfg::NTILE;
+  constexpr int NPV = 2 * DBS;  // accumulation steps: (16-query chunk c, d-block db)
+  constexpr int NSTEP = KK + NPV;
+  int st_row = 0;
+  uint32_t st_dst = 0;
+  auto prepare_loads = [&](int stage, int i0, bool on) {
+    ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
+    ld_rs[0] = tile_rsrc(Qb, i0, on);
+    ld_rs[1] = tile_rsrc(Gb, i0, on);
+    if constexpr (DUAL) {
+      ld_rs[2] = tile_rsrc(Qtb, i0, on);
+      ld_rs[3] = tile_rsrc(gTb, i0, on);
+    }
+    i0 = on ? i0 : istart;
+    st_row = min(i0 + lane, L - 1);
+    st_dst = stat0 + stage * Cfg::STATB;
+  };
+  // one 4-byte-per-lane direct load per statistic (64 rows, the first 32 are the tile's); wave s loads statistic s
+  auto load_stats = [&]() {
+    if (wave < Cfg::NSTAT) {
+      __builtin_amdgcn_global_load_lds((JVPFA_GLB(const void))(st_p[wave] + st_row),
+                                       (JVPFA_LDS(void))(uintptr_t)(st_dst + wave * 64 * 4), 4, 0, 0);
+    }
+  };
+  auto load_step = [&](auto gc) {
+    constexpr int gi = decltype(gc)::value;
+    constexpr int NSPREAD = JVPFA_BWD_SPREAD(NSTEP);
+    if constexpr (gi < NSPREAD) {
+      constexpr int lo = (gi * NLOAD + NSPREAD - 1) / NSPREAD, hi = ((gi + 1) * NLOAD + NSPREAD - 1) / NSPREAD;
+      static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+    }
+  };
+
+  // mask values of the tile that starts at query ihn, for this lane's key, requested a tile ahead
+  T mnext_a[MASK == MASK_ADD ? 16 : 1];
+  uint8_t mnext_b[MASK == MASK_BOOL ? 16 : 1];
+  auto fetch_mask_tile = [&](int ihn) {
+    if constexpr (MASK != MASK_NONE) {
+      if (mask_small && ihn + 32 <= L) {
+        const int64_t mrow0 = z * pr.ms[0] + h * pr.ms[1];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int64_t urow = mrow0 + (int64_t)(ihn + 16 * (e / 8) + (e % 8)) * pr.ms[2];
+          if constexpr (MASK == MASK_ADD) mnext_a[e] = (reinterpret_cast<const T *>(pr.mask) + urow)[mlane];
+          if constexpr (MASK == MASK_BOOL) mnext_b[e] = (reinterpret_cast<const uint8_t *>(pr.mask) + urow)[mlane];
+        }
+      } else {  // rows past the end are read from the last row (their scores are masked by index)
+        const int64_t mcol = z * pr.ms[0] + h * pr.ms[1] + (int64_t)kld * pr.ms[3];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int qi = ihn + 16 * (e / 8) + 8 * g + (e % 8);
+          const int64_t off = mcol + (int64_t)min(qi, L - 1) * pr.ms[2];
+          if constexpr (MASK == MASK_ADD) mnext_a[e] = reinterpret_cast<const T *>(pr.mask)[off];
+          if constexpr (MASK == MASK_BOOL) mnext_b[e] = reinterpret_cast<const uint8_t *>(pr.mask)[off];
+        }
+      }
+    }
+  };
+  // ih: first query of this tile; ihn: of the tile that follows it
+  auto tile_body = [&](auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn) {
+    constexpr bool EDGE = decltype(EDGEc)::value;
+    // ---- recompute ------------------------------------------------------------------------------
+    FragN fq[2], fg[2], fqt[2], fgt[2];
+    auto issue_n = [&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value, sl = kk % 2, HI = (kk / 8) * 256;
+      const uint32_t ad = sbase + noff[kk % 8];
+      fq[sl].v = lds_b128<HI>(ad);
+      if constexpr (NEED_V) fg[sl].v = lds_b128<HI + TILEB>(ad);
+      if constexpr (DUAL) {
+        fqt[sl].v = lds_b128<HI + 2 * TILEB>(ad);
+        if constexpr (NEED_V) fgt[sl].v = lds_b128<HI + 3 * TILEB>(ad);
+      }
+    };
+    constexpr int NRN = (DUAL ? 2 : 1) * (NEED_V ? 2 : 1);
+    T mraw_a[MASK == MASK_ADD ? 16 : 1];
+    uint8_t mraw_b[MASK == MASK_BOOL ? 16 : 1];
+    if constexpr (MASK != MASK_NONE) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        if constexpr (MASK == MASK_ADD) mraw_a[e] = mnext_a[e];
+        if constexpr (MASK == MASK_BOOL) mraw_b[e] = mnext_b[e];
+      }
+      fetch_mask_tile(ihn);
+    }
+    f32x16 S, dP, Sp, At;  // DUAL: dP also collects gT V'^T (the B term)
+    issue_n(std::integral_constant<int, 0>{});
+    static_for<KK>([&](auto kkc) {
+      constexpr int kk = decltype(kkc)::value, sl = kk % 2;
+      constexpr bool F = kk == 0;
+      if constexpr (kk + 1 < KK) issue_n(std::integral_constant<int, kk + 1>{});
+      constexpr int younger_n = (kk + 1 < KK) ? NRN : 0;
+      if constexpr (DUAL && NEED_V) lds_wait<younger_n>(fq[sl], fg[sl], fqt[sl], fgt[sl]);
+      else if constexpr (DUAL) lds_wait<younger_n>(fq[sl], fqt[sl]);
+      else lds_wait<younger_n>(fq[sl], fg[sl]);
+      load_step(std::integral_constant<int, kk>{});
+      const Frag<T> q_ = as_frag<T>(fq[sl]);
+      mma_vra<F, GD>(S, q_, Kf[kk]);
+      if constexpr (MODE == BWD_PLAIN) mma_vra<F, GD>(dP, as_frag<T>(fg[sl]), Vf[kk]);
+      if constexpr (TAN) mma_vra<F, GD>(At, as_frag<T>(fg[sl]), Vf[kk]);
+      if constexpr (DUAL) {
+        mma_vra<F, GD>(Sp, as_frag<T>(fqt[sl]), Kf[kk]);
+        mma_vra<false, GD>(Sp, q_, Ktf[kk]);
+        if constexpr (NEED_V) {
+          const Frag<T> gt_ = as_frag<T>(fgt[sl]);
+          if constexpr (has_go) mma_vra<F, GD>(dP, as_frag<T>(fg[sl]), Vf[kk]);
+          mma_vra<F, GD>(At, gt_, Vf[kk]);
+          mma_vra<F && !has_go, GD>(dP, gt_, Vtf[kk]);
+        }
+      }
+    });
+    if constexpr (DUAL && NEED_V) tiles_ready(S, dP, Sp, At);
+    else if constexpr (DUAL) tiles_ready(S, Sp);
+    else if constexpr (TAN) tiles_ready(S, At);
+    else tiles_ready(S, dP);
+
+    // ---- row statistics of the 32 queries: register e belongs to query 16(e/8) + 8g + e%8, read one
+    // quad of registers at a time, one quad ahead
+    u32x4 stq[2][Cfg::NSTAT];
+    const uint32_t sad = sstat + 8 * g * 4;
+    auto issue_s = [&](auto c4c) {
+      constexpr int c4 = decltype(c4c)::value;
+      static_for<Cfg::NSTAT>([&](auto sc) {
+        constexpr int s_ = decltype(sc)::value;
+        stq[c4 % 2][s_] = lds_b128<s_ * 64 * 4 + (c4 / 2) * 64 + (c4 % 2) * 16>(sad);
+      });
+    };
+    const int qmin = pr.causal ? krow : 0;  // queries below this index do not see this key
+    FragT tq[2], tg[2], tqt[2], tgt[2];
+    // one step: transposed fragments of d-block db of chunk c; Q, Q' feed dK, G, gT feed dV
+    auto issue_t = [&](auto ic) {
+      constexpr int i = decltype(ic)::value, c = i / DBS, db = i % DBS, sl = i % 2;
+      constexpr int TO = c * 16 * ROWB + (db / 4) * 256;
+      const uint32_t a0 = sbase + toff[db % 4][0], a1 = sbase + toff[db % 4][1];
+      if constexpr (WANT_DK) {
+        tq[sl].lo = lds_tr64<TO>(a0);
+        tq[sl].hi = lds_tr64<TO>(a1);
+      }
+      if constexpr (WANT_DV && (!DUAL || has_go)) {
+        tg[sl].lo = lds_tr64<TO + TILEB>(a0);
+        tg[sl].hi = lds_tr64<TO + TILEB>(a1);
+      }
+      if constexpr (DUAL && WANT_DK) {
+        tqt[sl].lo = lds_tr64<TO + 2 * TILEB>(a0);
+        tqt[sl].hi = lds_tr64<TO + 2 * TILEB>(a1);
+      }
+      if constexpr (DUAL && WANT_DV) {
+        tgt[sl].lo = lds_tr64<TO + 3 * TILEB>(a0);
+        tgt[sl].hi = lds_tr64<TO + 3 * TILEB>(a1);
+      }
+    };
+    // LDS reads of a step (each FragT is two)
+    constexpr int NRT = 2 * ((WANT_DK ? 1 : 0) + ((WANT_DV && (!DUAL || has_go)) ? 1 : 0) + ((DUAL && WANT_DK) ? 1 : 0) +
+                             ((DUAL && WANT_DV) ? 1 : 0));
+    issue_s(std::integral_constant<int, 0>{});
+    static_for<2>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      f32x8 Pp;  // P * (S' - mu) of this chunk
+      static_for<2>([&](auto hc) {
+        constexpr int c4 = 2 * c + decltype(hc)::value, sl = c4 % 2;
+        if constexpr (c4 + 1 < 4) issue_s(std::integral_constant<int, c4 + 1>{});
+        // waits also cover the transposed fragments issued before (LDS reads complete in order)
+        constexpr int younger = (c4 + 1 < 4) ? Cfg::NSTAT : 0;
+        if constexpr (Cfg::NSTAT == 4) lds_wait4<younger>(stq[sl][0], stq[sl][1], stq[sl][2], stq[sl][3]);
+        else lds_wait<younger>(stq[sl][0], stq[sl][1]);
+        auto stat = [&](int s_, int e) { return __uint_as_float(stq[sl][s_][e % 4]); };
+#pragma unroll
+        for (int e = 4 * c4; e < 4 * c4 + 4; ++e) {
+          const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
+          float s = S[e] * sl2;
+          bool keep = true;
+          if constexpr (MASK == MASK_ADD) s += (float)mraw_a[e] * LOG2E;
+          if constexpr (MASK == MASK_BOOL) keep = mraw_b[e] != 0;
+          float pv = fast_exp2(s - stat(0, e));
+          if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
+          if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
+          S[e] = pv;
+          if constexpr (MODE == BWD_PLAIN) {
+            dP[e] = pv * (dP[e] - stat(1, e));
+          } else if constexpr (DUAL) {
+            const float sp = Sp[e] * pr.scale, m_ = stat(1, e);
+            if constexpr (WANT_DV) Pp[e - 8 * c] = pv * (sp - m_);
+            if constexpr (WANT_DK) {
+              const float am = At[e] - stat(2, e);
+              Sp[e] = pv * am;
+              dP[e] = pv * (dP[e] + am * sp - At[e] * m_ - stat(3, e));
+            }
+          } else {
+            Sp[e] = pv * (At[e] - stat(1, e));
+          }
+        }
+      });
+      Frag<T> pf, dsf, dspf, ppf;
+      if constexpr (WANT_DV) pf = to_frag<T>(S, c);
+      if constexpr (!TAN && WANT_DK) dsf = to_frag<T>(dP, c);
+      if constexpr ((DUAL && WANT_DK) || TAN) dspf = to_frag<T>(Sp, c);
+      if constexpr (DUAL && WANT_DV) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ppf[e] = (T)Pp[e];
+      }
+      issue_t(std::integral_constant<int, c * DBS>{});
+      static_for<DBS>([&](auto dbc) {
+        constexpr int db = decltype(dbc)::value, i = c * DBS + db, sl = i % 2;
+        if constexpr (db + 1 < DBS) issue_t(std::integral_constant<int, i + 1>{});
+        constexpr int younger = (db + 1 < DBS) ? NRT : 0;
+        if constexpr (MODE != BWD_DUAL) lds_wait<younger>(tq[sl], tg[sl]);
+        else if constexpr (WANT_DK) lds_wait<younger>(tq[sl], tqt[sl]);
+        else if constexpr (has_go) lds_wait<younger>(tg[sl], tgt[sl]);
+        else lds_wait<younger>(tgt[sl].lo, tgt[sl].hi);
+        load_step(std::integral_constant<int, KK + i>{});
+        if constexpr (MODE == BWD_PLAIN) {
+          mma(dK[db], as_frag<T>(tq[sl]), dsf);
+          mma(dV[db], as_frag<T>(tg[sl]), pf);
+        } else if constexpr (DUAL) {
+          if constexpr (WANT_DK) {
+            mma(dK[db], as_frag<T>(tq[sl]), dsf);
+            mma(dK[db], as_frag<T>(tqt[sl]), dspf);
+          } else {
+            if constexpr (has_go) mma(dV[db], as_frag<T>(tg[sl]), pf);
+            mma(dV[db], as_frag<T>(tgt[sl]), ppf);
+          }
+        } else {
+          mma(dK[db], as_frag<T>(tq[sl]), dspf);
+          mma(dV[db], as_frag<T>(tg[sl]), pf);
+        }
+      });
+    });
+  };
+
+  auto tile = [&](int t, auto EDGEc) {
+    const int stage = t & 1;
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    const int i0 = istart + t * BT, i0n = istart + min(t + 1, ntiles - 1) * BT;
+    prepare_loads(stage ^ 1, i0n, t + 1 < ntiles);
+    load_stats();
+    tile_body(EDGEc, lds0 + stage * Cfg::STAGEB, stat0 + stage * Cfg::STATB, i0, i0n);
+  };
+  // Query tiles that cross the diagonal come first (causal), those that cross the end of the sequence
+  // last; the tiles in between run without limit tests.
+  const int t_diag = pr.causal ? min(ntiles, (k0 + Cfg::BLK - istart + BT - 1) / BT) : 0;
+  const int t_end = mask_small ? max(t_diag, (L - istart) / BT) : t_diag;
+  if constexpr (MASK != MASK_NONE) fetch_mask_tile(istart);
+  prepare_loads(0, istart, true);
+  static_for<NLOAD>([&](auto pc) { load_piece(pc); });
+  load_stats();
+  int t = 0;
+  for (; t < t_diag; ++t) tile(t, std::true_type{});
+  for (; t < ntiles && t < t_end; ++t) tile(t, std::false_type{});
+  for (; t < ntiles; ++t) tile(t, std::true_type{});
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+
+  if (krow < Lk) {
+    if constexpr (WANT_DK) {
+#pragma unroll
+      for (int db = 0; db < DBK; ++db) {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          float x[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[e] = dK[db][8 * hf + e] * pr.scale;
+          store8<T>(outk + 32 * db + 16 * hf + 8 * g, x);
+        }
+      }
+    }
+    if constexpr (WANT_DV) {
+#pragma unroll
+      for (int db = 0; db < DBV; ++db) {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          float x[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[e] = dV[db][8 * hf + e];
+          store8<T>(outv + 32 * db + 16 * hf + 8 * g, x);
+        }
+      }
+    }
+  }
+}
+#else
+template <typename T, int D, int DV, int MODE, int MASK, bool GO, int PART>
+__global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {}
+#endif
+
 }  // namespace jvpfa
