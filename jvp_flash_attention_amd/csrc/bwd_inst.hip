@@ -57,41 +57,25 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
     if (blocks * CfgW::NS > 0x7fffffffLL) return -2;
     int rc = allow_lds(reinterpret_cast<const void *>(kq), CfgW::DQ_LDS);
     if (rc != 0) return rc;
-    if (p.pr.Hk == p.pr.H) {
-      // dk/dv on the same pipeline: dV from K, K' alone, then dK in two column halves (dual); both in
-      // two column halves (otherwise)
-      using CfgK = BwdWideKvCfg<T, D, 128, MODE>;
-      if (kv_blocks * CfgK::NS > 0x7fffffffLL) return -2;
-      if constexpr (MODE == BWD_DUAL) {
-        void (*kv)(const BwdParams) = no_go ? bwdw_dkdv_kernel<T, D, 128, MODE, MASK, NG, WIDE_DV>
-                                            : bwdw_dkdv_kernel<T, D, 128, MODE, MASK, true, WIDE_DV>;
-        void (*kk)(const BwdParams) = no_go ? bwdw_dkdv_kernel<T, D, 128, MODE, MASK, NG, WIDE_DK>
-                                            : bwdw_dkdv_kernel<T, D, 128, MODE, MASK, true, WIDE_DK>;
-        rc = allow_lds(reinterpret_cast<const void *>(kv), CfgK::DKV_LDS);
-        if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kk), CfgK::DKV_LDS);
-        if (rc != 0) return rc;
-        hipLaunchKernelGGL(kv, dim3((unsigned)kv_blocks), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
-        hipLaunchKernelGGL(kk, dim3((unsigned)(kv_blocks * CfgK::NS)), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
-      } else {
-        auto kkv = bwdw_dkdv_kernel<T, D, 128, MODE, MASK, true, WIDE_BOTH>;
-        rc = allow_lds(reinterpret_cast<const void *>(kkv), CfgK::DKV_LDS);
-        if (rc != 0) return rc;
-        hipLaunchKernelGGL(kkv, dim3((unsigned)(kv_blocks * CfgK::NS)), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
-      }
-    } else if constexpr (MODE == BWD_DUAL) {
-      // grouped heads: the LDS-copy kernels, dk/dv in two launches with register sets that fit
-      auto kv = bwd_dkdv_kernel<T, D, MODE, MASK, DKDV_ONLY_DV>;
-      auto kk = bwd_dkdv_kernel<T, D, MODE, MASK, DKDV_ONLY_DK>;
-      rc = allow_lds(reinterpret_cast<const void *>(kv), Cfg::DKV_LDS);
-      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kk), Cfg::DKV_LDS);
+    // dk/dv on the same pipeline: dV from K, K' alone, then dK in two column halves (dual); both in two
+    // column halves (otherwise)
+    using CfgK = BwdWideKvCfg<T, D, 128, MODE>;
+    if (kv_blocks * CfgK::NS > 0x7fffffffLL) return -2;
+    if constexpr (MODE == BWD_DUAL) {
+      void (*kv)(const BwdParams) = no_go ? bwdw_dkdv_kernel<T, D, 128, MODE, MASK, NG, WIDE_DV>
+                                          : bwdw_dkdv_kernel<T, D, 128, MODE, MASK, true, WIDE_DV>;
+      void (*kk)(const BwdParams) = no_go ? bwdw_dkdv_kernel<T, D, 128, MODE, MASK, NG, WIDE_DK>
+                                          : bwdw_dkdv_kernel<T, D, 128, MODE, MASK, true, WIDE_DK>;
+      rc = allow_lds(reinterpret_cast<const void *>(kv), CfgK::DKV_LDS);
+      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kk), CfgK::DKV_LDS);
       if (rc != 0) return rc;
-      hipLaunchKernelGGL(kv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
-      hipLaunchKernelGGL(kk, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+      hipLaunchKernelGGL(kv, dim3((unsigned)kv_blocks), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
+      hipLaunchKernelGGL(kk, dim3((unsigned)(kv_blocks * CfgK::NS)), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
     } else {
-      auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK>;
-      rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg::DKV_LDS);
+      auto kkv = bwdw_dkdv_kernel<T, D, 128, MODE, MASK, true, WIDE_BOTH>;
+      rc = allow_lds(reinterpret_cast<const void *>(kkv), CfgK::DKV_LDS);
       if (rc != 0) return rc;
-      hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+      hipLaunchKernelGGL(kkv, dim3((unsigned)(kv_blocks * CfgK::NS)), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
     }
     hipLaunchKernelGGL(kq, dim3((unsigned)(blocks * CfgW::NS)), dim3(CfgW::NT), CfgW::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;

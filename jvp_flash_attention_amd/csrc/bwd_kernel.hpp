@@ -96,8 +96,8 @@ __device__ __forceinline__ void gemm_tile(f32x16 &acc, const T *tile, int ld, in
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) {
     mma(acc, lds_frag(tile + arow * ld + 16 * kk + 8 * g), b[kk]);
-    // rows of 512 bytes (D = 256; fp32 D = 128): the register file is full of resident operands; keep
-    // the scheduler from hoisting more than four fragment reads above the products that consume them
+    // rows of 512 bytes (fp32 D = 128): the register file is full of resident operands; keep the
+    // scheduler from hoisting more than four fragment reads above the products that consume them
     if constexpr (KK * sizeof(Frag<T>) >= 256) {
       if (kk % 4 == 3) __builtin_amdgcn_sched_barrier(0);
     }
@@ -300,19 +300,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // dk, dv (MODE PLAIN / DUAL) or dk', dv' (MODE TANGENT).  Scores are S = Q K^T (lane = key,
 // registers = queries), so P and dS are the B operands of dV^T += gO^T P and dK^T += Q^T dS.
-//
-// PART (BWD_DUAL only) splits the work over two launches for rows of 512 bytes, where the resident operands
-// (K, K', V, V': 4 x 64 registers) and both accumulators (2 x 128) do not fit one wave:
-// DKDV_ONLY_DV keeps K, K' and dV (it needs S, S' only), DKDV_ONLY_DK keeps all four and dK.
-enum DkdvPart { DKDV_BOTH = 0, DKDV_ONLY_DV = 1, DKDV_ONLY_DK = 2 };
-
-template <typename T, int D, int MODE, int MASK, int PART = DKDV_BOTH>
+template <typename T, int D, int MODE, int MASK>
 __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
   using Cfg = BwdCfg<T, D, MODE>;
   constexpr int KK = D / 16, DB = D / 32;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
-  static_assert(PART == DKDV_BOTH || (DUAL && !BWD_FETCH_AHEAD<T, D>));
-  constexpr bool WANT_DK = PART != DKDV_ONLY_DV, WANT_DV = PART != DKDV_ONLY_DK;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   // row-major tiles first, then transposed ones, then the row statistics
@@ -346,19 +338,19 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
   const int kld = krow < Lk ? krow : Lk - 1;
   const bool has_go = p.go != nullptr;
 
-  Frag<T> Kf[KK], Vf[WANT_DK ? KK : 1], Ktf[DUAL ? KK : 1], Vtf[DUAL && WANT_DK ? KK : 1];
+  Frag<T> Kf[KK], Vf[KK], Ktf[DUAL ? KK : 1], Vtf[DUAL ? KK : 1];
   load_row_frags<KK>(Kf, reinterpret_cast<const T *>(p.k) + kvhead + (size_t)kld * D, g);
-  if constexpr (WANT_DK) load_row_frags<KK>(Vf, reinterpret_cast<const T *>(p.v) + kvhead + (size_t)kld * D, g);
+  load_row_frags<KK>(Vf, reinterpret_cast<const T *>(p.v) + kvhead + (size_t)kld * D, g);
   if constexpr (DUAL) {
     load_row_frags<KK>(Ktf, reinterpret_cast<const T *>(p.kt) + kvhead + (size_t)kld * D, g);
-    if constexpr (WANT_DK) load_row_frags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + kvhead + (size_t)kld * D, g);
+    load_row_frags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + kvhead + (size_t)kld * D, g);
   }
 
-  f32x16 dK[WANT_DK ? DB : 1], dV[WANT_DV ? DB : 1];
+  f32x16 dK[DB], dV[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db) {
-    if constexpr (WANT_DK) zero16(dK[db]);
-    if constexpr (WANT_DV) zero16(dV[db]);
+    zero16(dK[db]);
+    zero16(dV[db]);
   }
 
   const float sl2 = pr.scale * LOG2E;
@@ -423,21 +415,17 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
       }
     } else {
       const int nvalid = L - i0;
-      // row-major copies feed the recomputed products, transposed ones the accumulations: a part
-      // of the work copies only what it reads
       copy_rows<T, BWD_T, D, BWD_NT>(Qn, Cfg::LDN, Qg + (size_t)i0 * D, nvalid, tid);
-      if constexpr (WANT_DK) copy_rows_transposed<T, BWD_T, D, BWD_NT>(QT, Cfg::LDT, Qg + (size_t)i0 * D, nvalid, tid);
+      copy_rows_transposed<T, BWD_T, D, BWD_NT>(QT, Cfg::LDT, Qg + (size_t)i0 * D, nvalid, tid);
       if (Gg) {
-        if constexpr (WANT_DK) copy_rows<T, BWD_T, D, BWD_NT>(Gn, Cfg::LDN, Gg + (size_t)i0 * D, nvalid, tid);
-        if constexpr (WANT_DV) copy_rows_transposed<T, BWD_T, D, BWD_NT>(GT, Cfg::LDT, Gg + (size_t)i0 * D, nvalid, tid);
+        copy_rows<T, BWD_T, D, BWD_NT>(Gn, Cfg::LDN, Gg + (size_t)i0 * D, nvalid, tid);
+        copy_rows_transposed<T, BWD_T, D, BWD_NT>(GT, Cfg::LDT, Gg + (size_t)i0 * D, nvalid, tid);
       }
       if constexpr (DUAL) {
         copy_rows<T, BWD_T, D, BWD_NT>(Qtn, Cfg::LDN, Qtg + (size_t)i0 * D, nvalid, tid);
-        if constexpr (WANT_DK) {
-          copy_rows_transposed<T, BWD_T, D, BWD_NT>(QtT, Cfg::LDT, Qtg + (size_t)i0 * D, nvalid, tid);
-          copy_rows<T, BWD_T, D, BWD_NT>(GTn, Cfg::LDN, gTg + (size_t)i0 * D, nvalid, tid);
-        }
-        if constexpr (WANT_DV) copy_rows_transposed<T, BWD_T, D, BWD_NT>(GTT, Cfg::LDT, gTg + (size_t)i0 * D, nvalid, tid);
+        copy_rows_transposed<T, BWD_T, D, BWD_NT>(QtT, Cfg::LDT, Qtg + (size_t)i0 * D, nvalid, tid);
+        copy_rows<T, BWD_T, D, BWD_NT>(GTn, Cfg::LDN, gTg + (size_t)i0 * D, nvalid, tid);
+        copy_rows_transposed<T, BWD_T, D, BWD_NT>(GTT, Cfg::LDT, gTg + (size_t)i0 * D, nvalid, tid);
       }
       fetch_stats(i0);
     }
@@ -450,7 +438,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
     f32x16 S, dP, Sp, At;  // DUAL: dP also collects V' gT^T (the B term)
     zero16(S);
     gemm_tile<KK>(S, Qn, Cfg::LDN, pr32, g, Kf);
-    if constexpr (!TAN && WANT_DK) {
+    if constexpr (!TAN) {
       zero16(dP);
       if (has_go) gemm_tile<KK>(dP, Gn, Cfg::LDN, pr32, g, Vf);
     }
@@ -458,11 +446,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
       zero16(Sp);
       gemm_tile<KK>(Sp, Qtn, Cfg::LDN, pr32, g, Kf);
       gemm_tile<KK>(Sp, Qn, Cfg::LDN, pr32, g, Ktf);
-      if constexpr (WANT_DK) {
-        zero16(At);
-        gemm_tile<KK>(At, GTn, Cfg::LDN, pr32, g, Vf);
-        gemm_tile<KK>(dP, GTn, Cfg::LDN, pr32, g, Vtf);
-      }
+      zero16(At);
+      gemm_tile<KK>(At, GTn, Cfg::LDN, pr32, g, Vf);
+      gemm_tile<KK>(dP, GTn, Cfg::LDN, pr32, g, Vtf);
     }
     if constexpr (TAN) {
       zero16(At);
@@ -492,11 +478,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
       } else if constexpr (DUAL) {
         const float sp = Sp[e] * pr.scale, m_ = smu[ql], a_ = sa[ql];
         S[e] = pv;
-        if constexpr (WANT_DV) Pp[e] = pv * (sp - m_);
-        if constexpr (WANT_DK) {
-          Sp[e] = pv * (At[e] - a_);
-          dP[e] = pv * (dP[e] - sd1[ql] + At[e] * (sp - m_) - a_ * sp - sd2[ql]);
-        }
+        Pp[e] = pv * (sp - m_);
+        Sp[e] = pv * (At[e] - a_);
+        dP[e] = pv * (dP[e] - sd1[ql] + At[e] * (sp - m_) - a_ * sp - sd2[ql]);
       } else {
         S[e] = pv;
         Sp[e] = pv * (At[e] - sa[ql]);
@@ -507,9 +491,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
     for (int c = 0; c < BWD_T / 16; ++c) {
       Frag<T> pf = to_frag<T>(S, c);
       Frag<T> dsf, dspf, ppf;
-      if constexpr (!TAN && WANT_DK) dsf = to_frag<T>(dP, c);
-      if constexpr ((DUAL && WANT_DK) || TAN) dspf = to_frag<T>(Sp, c);
-      if constexpr (DUAL && WANT_DV) ppf = to_frag<T>(Pp, c);
+      if constexpr (!TAN) dsf = to_frag<T>(dP, c);
+      if constexpr (DUAL || TAN) dspf = to_frag<T>(Sp, c);
+      if constexpr (DUAL) ppf = to_frag<T>(Pp, c);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const int off = (32 * db + pr32) * Cfg::LDT + 16 * c + 8 * g;
@@ -517,14 +501,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
           mma(dK[db], lds_frag(QT + off), dsf);
           mma(dV[db], lds_frag(GT + off), pf);
         } else if constexpr (DUAL) {
-          if constexpr (WANT_DK) {
-            mma(dK[db], lds_frag(QT + off), dsf);
-            mma(dK[db], lds_frag(QtT + off), dspf);
-          }
-          if constexpr (WANT_DV) {
-            if (has_go) mma(dV[db], lds_frag(GT + off), pf);
-            mma(dV[db], lds_frag(GTT + off), ppf);
-          }
+          mma(dK[db], lds_frag(QT + off), dsf);
+          mma(dK[db], lds_frag(QtT + off), dspf);
+          if (has_go) mma(dV[db], lds_frag(GT + off), pf);
+          mma(dV[db], lds_frag(GTT + off), ppf);
         } else {
           mma(dK[db], lds_frag(QT + off), dspf);
           mma(dV[db], lds_frag(GT + off), pf);
@@ -547,11 +527,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
         float xk[8], xv[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          if constexpr (WANT_DK) xk[e] = dK[db][8 * hf + e] * pr.scale;
-          if constexpr (WANT_DV) xv[e] = dV[db][8 * hf + e];
+          xk[e] = dK[db][8 * hf + e] * pr.scale;
+          xv[e] = dV[db][8 * hf + e];
         }
-        if constexpr (WANT_DK) store8<T>(outk + 32 * db + 16 * hf + 8 * g, xk);
-        if constexpr (WANT_DV) store8<T>(outv + 32 * db + 16 * hf + 8 * g, xv);
+        store8<T>(outk + 32 * db + 16 * hf + 8 * g, xk);
+        store8<T>(outv + 32 * db + 16 * hf + 8 * g, xv);
       }
     }
   }

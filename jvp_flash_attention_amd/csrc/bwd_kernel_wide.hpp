@@ -351,7 +351,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {}
 //   WIDE_DK    (DUAL) 128 columns of dK, two workgroups per key block: K, V, K', V' resident (the
 //              whole accumulation file), the accumulators in ordinary registers
 //   WIDE_BOTH  (PLAIN, TANGENT) 128 columns of dK and of dV, two workgroups per key block
-// k, v must have q's heads (grouped heads take the LDS-copy kernels).
+// With grouped heads the query heads that read this key/value head are visited one after another.
 enum WidePart { WIDE_BOTH = 0, WIDE_DV = 1, WIDE_DK = 2 };
 
 template <typename T, int D, int DV, int MODE> struct BwdWideKvCfg : BwdWideCfg<T, D, DV, MODE> {
@@ -379,18 +379,16 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   const Problem &pr = p.pr;
   const int L = pr.L, Lk = pr.Lk;  // queries, keys
   const int nblk = (Lk + Cfg::BLK - 1) / Cfg::BLK;
-  const int id = xcd_remap(blockIdx.x, nblk * NSL, pr.Z * pr.H);
+  const int id = xcd_remap(blockIdx.x, nblk * NSL, pr.Z * pr.Hk);
   const int zh = id / (nblk * NSL);
   const int rem = id % (nblk * NSL);
   const int slice = rem % NSL;
   const int kb = rem / NSL;  // causal: the first key blocks have the longest query loops
-  const int z = zh / pr.H, h = zh % pr.H;
+  const int z = zh / pr.Hk, hk = zh % pr.Hk, group = pr.H / pr.Hk;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
   const int r = lane % 32, g = lane / 32, pr32 = perm32(r);
-  const size_t head = (size_t)zh * Lk * D;   // of k, v and their gradients (as many heads as q)
-  const size_t qhead = (size_t)zh * L * D;   // of q, gO, q', gT
-  const size_t srow = (size_t)zh * L;
+  const size_t head = (size_t)zh * Lk * D;   // of k, v and their gradients
   const int k0 = kb * Cfg::BLK;
   const int krow = k0 + wave * 32 + r;
   const int kld = krow < Lk ? krow : Lk - 1;
@@ -488,12 +486,22 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   }
   // tile slots 0 Q, 1 G (gO; gT in TANGENT; gT again in DUAL without gO), 2 Q', 3 gT, and the
   // statistics slots PLAIN M, d1 | DUAL M, mu, a, d2 (= d1 + d2) | TANGENT M, a
-  const char *Qb = reinterpret_cast<const char *>(p.q) + qhead * sizeof(T);
-  const char *gTb = (DUAL || TAN) ? reinterpret_cast<const char *>(p.gt) + qhead * sizeof(T) : nullptr;
-  const char *Gb = TAN ? gTb : (has_go ? reinterpret_cast<const char *>(p.go) + qhead * sizeof(T) : gTb);
-  const char *Qtb = DUAL ? reinterpret_cast<const char *>(p.qt) + qhead * sizeof(T) : nullptr;
-  const float *st_p[4] = {p.M + srow, MODE == BWD_PLAIN ? p.d1 + srow : (DUAL ? p.mu + srow : p.a + srow),
-                          DUAL ? p.a + srow : nullptr, DUAL ? p.d2 + srow : nullptr};
+  // h is the query head being visited; what depends on it is set per head
+  int h = hk * group;
+  const char *Qb = nullptr, *gTb = nullptr, *Gb = nullptr, *Qtb = nullptr;
+  const float *st_p[4] = {nullptr, nullptr, nullptr, nullptr};
+  auto set_query_head = [&](int hq) {
+    h = hq;
+    const size_t qhead = ((size_t)z * pr.H + hq) * L * D * sizeof(T), srow = ((size_t)z * pr.H + hq) * L;
+    Qb = reinterpret_cast<const char *>(p.q) + qhead;
+    gTb = (DUAL || TAN) ? reinterpret_cast<const char *>(p.gt) + qhead : nullptr;
+    Gb = TAN ? gTb : (has_go ? reinterpret_cast<const char *>(p.go) + qhead : gTb);
+    Qtb = DUAL ? reinterpret_cast<const char *>(p.qt) + qhead : nullptr;
+    st_p[0] = p.M + srow;
+    st_p[1] = MODE == BWD_PLAIN ? p.d1 + srow : (DUAL ? p.mu + srow : p.a + srow);
+    st_p[2] = DUAL ? p.a + srow : nullptr;
+    st_p[3] = DUAL ? p.d2 + srow : nullptr;
+  };
 
   const int istart = pr.causal ? (k0 / BT) * BT : 0;
   const int ntiles = (L - istart + BT - 1) / BT;
@@ -738,15 +746,19 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   // last; the tiles in between run without limit tests.
   const int t_diag = pr.causal ? min(ntiles, (k0 + Cfg::BLK - istart + BT - 1) / BT) : 0;
   const int t_end = mask_small ? max(t_diag, (L - istart) / BT) : t_diag;
-  if constexpr (MASK != MASK_NONE) fetch_mask_tile(istart);
-  prepare_loads(0, istart, true);
-  static_for<NLOAD>([&](auto pc) { load_piece(pc); });
-  load_stats();
-  int t = 0;
-  for (; t < t_diag; ++t) tile(t, std::true_type{});
-  for (; t < ntiles && t < t_end; ++t) tile(t, std::false_type{});
-  for (; t < ntiles; ++t) tile(t, std::true_type{});
-  __builtin_amdgcn_s_waitcnt(0x0F70);
+  for (int gi = 0; gi < group; ++gi) {
+    if (gi > 0) __syncthreads();  // every wave is done with the previous head's last tile: its stage may be refilled
+    set_query_head(hk * group + gi);
+    if constexpr (MASK != MASK_NONE) fetch_mask_tile(istart);
+    prepare_loads(0, istart, true);
+    static_for<NLOAD>([&](auto pc) { load_piece(pc); });
+    load_stats();
+    int t = 0;
+    for (; t < t_diag; ++t) tile(t, std::true_type{});
+    for (; t < ntiles && t < t_end; ++t) tile(t, std::false_type{});
+    for (; t < ntiles; ++t) tile(t, std::true_type{});
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+  }
 
   if (krow < Lk) {
     if constexpr (WANT_DK) {
