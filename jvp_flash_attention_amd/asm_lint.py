@@ -11,8 +11,9 @@ slots that the hardware needs
 
 The sources provide those slots themselves (``s_nop 1`` in front of the matrix instructions whose
 operands live long enough to be parked, ``tiles_ready()`` = ``s_nop 15; s_nop 3`` after each group).
-This module compiles translation units to ISA text and checks that every inline-asm matrix
-instruction in it is covered: ``python -m jvp_flash_attention_amd.asm_lint [unit names]``.
+``scan()`` checks the ISA text of a translation unit for both; ``build()`` runs it on every kernel unit it
+compiles and fails on a finding.  ``python -m jvp_flash_attention_amd.asm_lint [unit names]`` compiles
+units to ISA text on its own and scans them.
 """
 from __future__ import annotations
 
@@ -23,7 +24,6 @@ import sys
 import tempfile
 from concurrent.futures import ThreadPoolExecutor
 
-from . import build as _build
 
 
 def _regs(tok: str) -> set[tuple[str, int]]:
@@ -87,6 +87,8 @@ def scan(isa_text: str, where: str = "") -> list[str]:
 
 def isa_of(unit) -> str:
     """Device ISA text of one translation unit of ``build.units()``."""
+    from . import build as _build
+
     name, src, defs = unit
     with tempfile.TemporaryDirectory() as td:
         path = os.path.join(td, name + ".s")
@@ -100,6 +102,8 @@ def isa_of(unit) -> str:
 
 def lint(names=None, jobs: int | None = None) -> list[str]:
     """Compile the named units (default: every kernel unit) to ISA and scan them."""
+    from . import build as _build
+
     units = [u for u in _build.units() if u[0].startswith(("fwd_", "bwd_")) and (not names or u[0] in names)]
     with ThreadPoolExecutor(max_workers=jobs or min(8, os.cpu_count() or 1)) as ex:
         texts = list(ex.map(isa_of, units))

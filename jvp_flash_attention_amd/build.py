@@ -48,13 +48,29 @@ def units():
     return out
 
 
+def isa_path(name: str, objdir: str = OBJ) -> str:
+    """Where ``build()`` leaves the device ISA text of a translation unit."""
+    return os.path.join(objdir, name, name + ".s")
+
+
 def _compile(unit):
     name, src, defs, objdir, extra = unit
-    obj = os.path.join(objdir, name + ".o")
-    cmd = [HIPCC, *FLAGS, *extra, *defs, "-c", src, "-o", obj]
+    # a directory per unit: the compiler names its intermediate files after the source, and several
+    # units share one source
+    udir = os.path.join(objdir, name)
+    os.makedirs(udir, exist_ok=True)
+    obj = os.path.join(udir, name + ".o")
+    cmd = [HIPCC, *FLAGS, *extra, *defs, "-save-temps=obj", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {name}:\n{' '.join(cmd)}\n{r.stderr[-4000:]}")
+    # of the intermediate files keep the device ISA text (the asm lint reads it)
+    for f in os.listdir(udir):
+        path = os.path.join(udir, f)
+        if f.endswith(".s") and "-hip-amdgcn-" in f:
+            os.replace(path, isa_path(name, objdir))
+        elif path != obj:
+            os.remove(path)
     return obj
 
 
@@ -72,6 +88,19 @@ def build(jobs: int | None = None, verbose: bool = True, extra_flags=(), lib: st
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
     if verbose:
         print(f"built {lib} from {len(objs)} objects", flush=True)
+    # the inline-asm matrix instructions of every kernel unit must carry the idle issue slots the
+    # compiler cannot add for them (see asm_lint.py); a finding fails the build
+    from . import asm_lint
+
+    findings = []
+    for name, _src, _defs, *_ in us:
+        if name.startswith(("fwd_", "bwd_")):
+            with open(isa_path(name, objdir)) as f:
+                findings += asm_lint.scan(f.read(), name)
+    if findings:
+        raise RuntimeError("asm lint:\n" + "\n".join(findings))
+    if verbose:
+        print("asm lint: clean", flush=True)
     if lib == LIB:
         build_host_check(verbose)
     return lib
