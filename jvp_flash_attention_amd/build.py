@@ -65,11 +65,13 @@ def _compile(unit):
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {name}:\n{' '.join(cmd)}\n{r.stderr[-4000:]}")
     # of the intermediate files keep the device ISA text (the asm lint reads it)
+    isa = isa_path(name, objdir)
+    for f in os.listdir(udir):
+        if f.endswith(".s") and "-hip-amdgcn-" in f:
+            os.replace(os.path.join(udir, f), isa)
     for f in os.listdir(udir):
         path = os.path.join(udir, f)
-        if f.endswith(".s") and "-hip-amdgcn-" in f:
-            os.replace(path, isa_path(name, objdir))
-        elif path != obj:
+        if path not in (obj, isa):
             os.remove(path)
     return obj
 

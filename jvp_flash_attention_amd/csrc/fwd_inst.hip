@@ -50,11 +50,12 @@ static int launch_fwd3_one(const FwdParams &p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }
 
-// D = 256: two workgroups per query block, each with 128 of the output columns.
+// D = 256: two workgroups per query block, each with 128 of the output columns (dual forward).
 template <typename T, int D, bool DUAL, int MASK>
 static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
-  using Cfg = FwdWideCfg<T, D, 128, DUAL>;
-  auto kern = fwd_wide_kernel<T, D, 128, DUAL, MASK>;
+  constexpr int DV = DUAL ? 128 : D;  // without tangents one workgroup holds all columns
+  using Cfg = FwdWideCfg<T, D, DV, DUAL>;
+  auto kern = fwd_wide_kernel<T, D, DV, DUAL, MASK>;
   int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
   if (rc != 0) return rc;
   const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;

@@ -4,7 +4,8 @@
 // 2 x 128) of 32 query rows do not fit one wave next to the score tiles.  Here a workgroup
 // produces DV = 128 of the D output columns: it forms the scores over the whole of D (both
 // workgroups of a query block do, which is the price) and multiplies them with a 128-column slice
-// of V, V', so a wave holds 2 x 64 + 2 x 64 registers in the accumulation file, all of it.
+// of V, V', so a wave holds 2 x 64 + 2 x 64 registers in the accumulation file, all of it.  (Without
+// tangents Q and O alone fit, 64 + 128, and one workgroup produces all columns: DV = D.)
 //
 // Memory side as in fwd_kernel_v2.hpp: direct-to-LDS loads, double buffered, one barrier per tile,
 // XOR-swizzled 16-byte chunks, ds_read_b128 for K / K' fragments and the transposing
@@ -37,7 +38,7 @@ template <typename T, int D, int DV, bool DUAL> struct FwdWideCfg {
   static constexpr size_t LDS_BYTES = 2 * (size_t)STAGEB;
   static constexpr int IPWK = TILEBK / 1024 / NW;      // direct-load instructions per wave per tile
   static constexpr int IPWV = TILEBV / 1024 / NW;
-  static_assert(IPWK >= 1 && IPWV >= 1 && CHK == 32 && CHV == 16);
+  static_assert(IPWK >= 1 && IPWV >= 1 && CHK == 32 && (CHV == 16 || (CHV == 32 && !DUAL)));
 };
 
 template <typename T, int D, int DV, bool DUAL, int MASK>

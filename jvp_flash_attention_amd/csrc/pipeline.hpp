@@ -124,8 +124,10 @@ __device__ __forceinline__ int list_take(int v) {
 template <int CH> __device__ __forceinline__ int swz_k(int row) {
   return CH == 16 ? (row & 15) : CH == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
+// (CH = 32, rows of 512 bytes: every row starts a 256-byte line, so the four consecutive rows of a
+// transposing read need their groups of four chunks moved apart)
 template <int CH> __device__ __forceinline__ int swz_v(int row) {
-  return CH == 16 ? ((row & 7) << 1) : CH == 8 ? (((row >> 1) & 3) << 1) : 0;
+  return CH == 32 ? ((row & 3) << 2) : CH == 16 ? ((row & 7) << 1) : CH == 8 ? (((row >> 1) & 3) << 1) : 0;
 }
 
 // Swizzle for tiles that are read both ways (ds_read_b128 along rows and the transposing
