@@ -83,8 +83,8 @@ typedef struct jvpfa_fwd_args {
   /* since version 3 (a caller may pass the version-2 size, which ends before this field):
    * optional lists of the key tiles that hold an attended entry, written by jvpfa_mask_tiles() for
    * this same mask, or NULL.  Tiles not listed are skipped instead of read and masked.  When set,
-   * key_limit is ignored.  Ignored (and key_limit used) for fp32 and for D = 256, whose kernels
-   * visit every tile up to the key limit.  Ignored without a mask. */
+   * key_limit is ignored.  Ignored (and key_limit used) for fp32, whose kernels visit every tile
+   * up to the key limit.  Ignored without a mask. */
   const int32_t *tiles_q;
   /* since version 4 (a caller may pass the version-3 size, which ends before this field): shape of
    * k, v, kt, vt when it is not q's -- Lk keys (any length >= 1) and Hk key/value heads, Hk a divisor

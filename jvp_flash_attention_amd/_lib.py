@@ -177,7 +177,7 @@ def tile_lists(q, mask, mask_kind, want_k):
     counter, so that layers and the backward reuse one scan."""
     Z, H, L, D = q.shape
     if (not _tile_lists_enabled or mask is None or mask_kind == MASK_NONE or L < TILE_LISTS_MIN_L
-            or q.dtype == torch.float32 or D > 128):
+            or q.dtype == torch.float32):
         return None, None
     if mask.dim() != 4 or mask.shape[2] != L or mask.shape[3] != L:
         return None, None

@@ -147,7 +147,22 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   if constexpr (MASK != MASK_NONE) {
     if (pr.klimit) kend = min(kend, max(pr.klimit[z], 1));
   }
-  const int ntiles = (kend + BT - 1) / BT;
+  // Key tiles visited: the 32-key tiles 0 .. ceil(kend/32)-1, or both halves of every 64-key tile of the
+  // caller's list for this query block (the second half of the last one is dropped when it lies past
+  // the last key).
+  const int *tlist = nullptr;
+  if constexpr (MASK != MASK_NONE) {
+    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
+  }
+  const int tmax = (Lk + TILE_W - 1) / TILE_W - 1;  // bounds whatever a list holds
+  int ntiles = (kend + BT - 1) / BT;
+  if (tlist) {
+    const int cnt = min(max(tlist[0], 1), tmax + 1);
+    const int last = min(max(tlist[cnt], 0), tmax);
+    ntiles = 2 * cnt - (last * TILE_W + BT >= Lk ? 1 : 0);
+  }
+  auto list_slot = [&](int t) { return tlist ? tlist + 1 + (t >> 1) : reinterpret_cast<const int *>(p.q); };
+  auto key_of = [&](int entry, int t) { return tlist ? min(max(entry, 0), tmax) * TILE_W + (t & 1) * BT : t * BT; };
   // tile slots in a stage: 0 K, 1 V, 2 K', 3 V'
   constexpr int NLOAD = IPW * Cfg::NTILE;
   constexpr int NACC = DUAL ? 2 : 1;
@@ -288,9 +303,8 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   };
 
   // mask values of tile t+1 are requested at the top of tile t
-  auto fetch_masks = [&](int tn) {
+  auto fetch_masks = [&](int jn) {
     if constexpr (MASK != MASK_NONE) {
-      const int jn = tn * BT;
       if (mask_al && jn + BT <= Lk) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) mnext[i] = mask_fetch8<T, MASK>(pr, mrow, jn + 16 * i + 8 * g);
@@ -300,27 +314,37 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
       }
     }
   };
-  fetch_masks(0);
-  prepare_loads(0, 0, true);
+  // first keys of the tile of this step and of the next
+  int jcur = key_of(tlist ? tlist[1] : 0, 0);
+  int jnext = key_of(tlist ? tlist[1 + (min(1, ntiles - 1) >> 1)] : 0, min(1, ntiles - 1));
+  fetch_masks(jcur);
+  prepare_loads(0, jcur, true);
   static_for<NLOAD>([&](auto pc) { load_piece(pc); });
   auto tile = [&](int t, auto EDGEc) {
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
+    const int tnext2 = min(t + 2, ntiles - 1);
+    int tahead = 0;
     if constexpr (MASK != MASK_NONE) {
+      tahead = list_request(list_slot(tnext2));  // read a tile ahead, taken at the end of this one
       mcur[0] = mnext[0];
       mcur[1] = mnext[1];
-      fetch_masks(min(t + 1, ntiles - 1));
+      fetch_masks(jnext);
     }
-    prepare_loads(stage ^ 1, (t + 1) * BT, t + 1 < ntiles);
-    tile_body(EDGEc, lds0 + stage * Cfg::STAGEB, t * BT);
+    prepare_loads(stage ^ 1, jnext, t + 1 < ntiles);
+    tile_body(EDGEc, lds0 + stage * Cfg::STAGEB, jcur);
+    int jnext2 = tnext2 * BT;
+    if constexpr (MASK != MASK_NONE) jnext2 = key_of(list_take(tahead), tnext2);
+    jcur = jnext;
+    jnext = jnext2;
   };
   // tiles that cross the diagonal or the end of the sequence are the last ones
   int t_edge = Lk / BT;
   if (pr.causal) t_edge = min(t_edge, q0 / BT);
   if (MASK != MASK_NONE && !mask_al) t_edge = 0;
   int t = 0;
-  for (; t < ntiles && t < t_edge; ++t) tile(t, std::false_type{});
+  for (; t < ntiles && jcur < t_edge * BT; ++t) tile(t, std::false_type{});
   for (; t < ntiles; ++t) tile(t, std::true_type{});
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the redirected loads of the last iteration must not outlive the kernel
 
@@ -504,7 +528,26 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   };
 
   const int istart = pr.causal ? (k0 / BT) * BT : 0;
-  const int ntiles = (L - istart + BT - 1) / BT;
+  // Query tiles visited, counted from istart: the 32-query tiles 0 .. ntiles-1, or both halves of every
+  // 64-query tile of the caller's list for this key block and the query head visited (only with a
+  // mask, where istart is 0); the second half of the last one is dropped when it lies past the end.
+  const int *tlist = nullptr;
+  const int tmax = (L + TILE_W - 1) / TILE_W - 1;  // bounds whatever a list holds
+  int ntiles = (L - istart + BT - 1) / BT;
+  auto set_list = [&](int hq) {
+    if constexpr (MASK != MASK_NONE) {
+      if (pr.tiles_k) {
+        tlist = pr.tiles_k + tile_list_offset(pr, z, hq, kb);
+        const int cnt = min(max(tlist[0], 1), tmax + 1);
+        const int last = min(max(tlist[cnt], 0), tmax);
+        ntiles = 2 * cnt - (last * TILE_W + BT >= L ? 1 : 0);
+      }
+    }
+  };
+  auto list_slot = [&](int t) { return tlist ? tlist + 1 + (t >> 1) : reinterpret_cast<const int *>(p.q); };
+  auto query_of = [&](int entry, int t) {
+    return tlist ? min(max(entry, 0), tmax) * TILE_W + (t & 1) * BT : istart + t * BT;
+  };
   constexpr int NLOAD = IPW * Cfg::NTILE;
   constexpr int NPV = 2 * DBS;  // accumulation steps: (16-query chunk c, d-block db)
   constexpr int NSTEP = KK + NPV;
@@ -733,14 +776,21 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
     });
   };
 
+  int icur = 0, inext = 0;  // first queries of the tile of this step and of the next
   auto tile = [&](int t, auto EDGEc) {
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    const int i0 = istart + t * BT, i0n = istart + min(t + 1, ntiles - 1) * BT;
-    prepare_loads(stage ^ 1, i0n, t + 1 < ntiles);
+    const int tnext2 = min(t + 2, ntiles - 1);
+    int tahead = 0;
+    if constexpr (MASK != MASK_NONE) tahead = list_request(list_slot(tnext2));  // read a tile ahead
+    prepare_loads(stage ^ 1, inext, t + 1 < ntiles);
     load_stats();
-    tile_body(EDGEc, lds0 + stage * Cfg::STAGEB, stat0 + stage * Cfg::STATB, i0, i0n);
+    tile_body(EDGEc, lds0 + stage * Cfg::STAGEB, stat0 + stage * Cfg::STATB, icur, inext);
+    int inext2 = istart + tnext2 * BT;
+    if constexpr (MASK != MASK_NONE) inext2 = query_of(list_take(tahead), tnext2);
+    icur = inext;
+    inext = inext2;
   };
   // Query tiles that cross the diagonal come first (causal), those that cross the end of the sequence
   // last; the tiles in between run without limit tests.
@@ -749,13 +799,16 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   for (int gi = 0; gi < group; ++gi) {
     if (gi > 0) __syncthreads();  // every wave is done with the previous head's last tile: its stage may be refilled
     set_query_head(hk * group + gi);
-    if constexpr (MASK != MASK_NONE) fetch_mask_tile(istart);
-    prepare_loads(0, istart, true);
+    set_list(hk * group + gi);
+    icur = query_of(tlist ? tlist[1] : 0, 0);
+    inext = query_of(tlist ? tlist[1 + (min(1, ntiles - 1) >> 1)] : 0, min(1, ntiles - 1));
+    if constexpr (MASK != MASK_NONE) fetch_mask_tile(icur);
+    prepare_loads(0, icur, true);
     static_for<NLOAD>([&](auto pc) { load_piece(pc); });
     load_stats();
     int t = 0;
     for (; t < t_diag; ++t) tile(t, std::true_type{});
-    for (; t < ntiles && t < t_end; ++t) tile(t, std::false_type{});
+    for (; t < ntiles && icur < istart + t_end * BT; ++t) tile(t, std::false_type{});
     for (; t < ntiles; ++t) tile(t, std::true_type{});
     __builtin_amdgcn_s_waitcnt(0x0F70);
   }

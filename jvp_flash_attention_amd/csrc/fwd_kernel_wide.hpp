@@ -10,7 +10,7 @@
 // Memory side as in fwd_kernel_v2.hpp: direct-to-LDS loads, double buffered, one barrier per tile,
 // XOR-swizzled 16-byte chunks, ds_read_b128 for K / K' fragments and the transposing
 // ds_read_b64_tr_b16 for V / V'.  A tile is 32 keys (K, K' rows are 512 bytes; two stages of
-// 64-key tiles would not fit the LDS).  No tile lists; the key-limit hint is honoured.
+// 64-key tiles would not fit the LDS); a listed 64-key tile is visited as its two halves.
 #pragma once
 #include <utility>
 
@@ -156,7 +156,24 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
     if (pr.klimit) kend = min(Lk, max(pr.klimit[z], 1));
   }
   if (pr.causal) kend = min(Lk, q0 + Cfg::BM);
-  const int ntiles = (kend + BN - 1) / BN;
+  // Tiles visited: the 32-key tiles 0 .. ceil(kend/32)-1, or both halves of every 64-key tile of the
+  // caller's list for this query block (ascending; a tile without an attended entry contributes exact
+  // zeros, so leaving it out changes nothing).  The second half of the last listed tile is dropped
+  // when it lies past the last key.
+  const int *tlist = nullptr;
+  if constexpr (MASK != MASK_NONE) {
+    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
+  }
+  const int tmax = (Lk + TILE_W - 1) / TILE_W - 1;  // bounds whatever a list holds
+  int ntiles = (kend + BN - 1) / BN;
+  if (tlist) {
+    const int cnt = min(max(tlist[0], 1), tmax + 1);
+    const int last = min(max(tlist[cnt], 0), tmax);
+    ntiles = 2 * cnt - (last * TILE_W + BN >= Lk ? 1 : 0);
+  }
+  // first key of the t-th tile visited, given the list entry that covers it
+  auto list_slot = [&](int t) { return tlist ? tlist + 1 + (t >> 1) : reinterpret_cast<const int *>(p.q); };
+  auto key_of = [&](int entry, int t) { return tlist ? min(max(entry, 0), tmax) * TILE_W + (t & 1) * BN : t * BN; };
 
   // The loads of the next tile are issued one instruction at a time, spread over the steps of the
   // current tile's matrix products.  Past the last tile they are pointed at tile 0 again (never
@@ -344,9 +361,8 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
   };
 
   // mask values of tile t+1 are requested at the top of tile t
-  auto fetch_masks = [&](int tn) {
+  auto fetch_masks = [&](int jn) {
     if constexpr (MASK != MASK_NONE) {
-      const int jn = tn * BN;
       if (mask_al && jn + BN <= Lk) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) mnext[i] = mask_fetch8<T, MASK>(pr, mrow, jn + 16 * i + 8 * g);
@@ -356,22 +372,32 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
       }
     }
   };
-  fetch_masks(0);
+  // first keys of the tile of this step and of the next
+  int jcur = key_of(tlist ? tlist[1] : 0, 0);
+  int jnext = key_of(tlist ? tlist[1 + (min(1, ntiles - 1) >> 1)] : 0, min(1, ntiles - 1));
+  fetch_masks(jcur);
   {
-    prepare_loads(0, 0, true);
+    prepare_loads(0, jcur, true);
     static_for<NLOAD>([&](auto pc) { load_piece(pc); });
   }
   auto tile = [&](int t, auto EDGEc) {
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
+    const int tnext2 = min(t + 2, ntiles - 1);
+    int tahead = 0;
     if constexpr (MASK != MASK_NONE) {
+      tahead = list_request(list_slot(tnext2));  // read a tile ahead, taken at the end of this one
       mcur[0] = mnext[0];
       mcur[1] = mnext[1];
-      fetch_masks(min(t + 1, ntiles - 1));
+      fetch_masks(jnext);
     }
-    prepare_loads(stage ^ 1, (t + 1) * BN, t + 1 < ntiles);
-    tile_body(EDGEc, lds0 + stage * Cfg::STAGEB, t * BN);
+    prepare_loads(stage ^ 1, jnext, t + 1 < ntiles);
+    tile_body(EDGEc, lds0 + stage * Cfg::STAGEB, jcur);
+    int jnext2 = tnext2 * BN;
+    if constexpr (MASK != MASK_NONE) jnext2 = key_of(list_take(tahead), tnext2);
+    jcur = jnext;
+    jnext = jnext2;
   };
   // Tiles that need the general treatment are the last ones; they get a loop of their own so that the
   // common tile carries no limit tests.
@@ -379,7 +405,7 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
   if (pr.causal) t_edge = min(t_edge, q0 / BN);
   if (!(sl2 > 0.f) || (MASK != MASK_NONE && !mask_al)) t_edge = 0;
   int t = 0;
-  for (; t < ntiles && t < t_edge; ++t) tile(t, std::false_type{});
+  for (; t < ntiles && jcur < t_edge * BN; ++t) tile(t, std::false_type{});
   for (; t < ntiles; ++t) tile(t, std::true_type{});
 
   // ---- epilogue ---------------------------------------------------------------------------------

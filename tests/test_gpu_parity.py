@@ -249,7 +249,7 @@ def test_mask_tile_lists_match_a_numpy_scan(kind, as_bias, L):
             assert row[0] == len(want) and row[1:1 + row[0]] == want
 
 
-@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128, 256])
 @pytest.mark.parametrize("kind", ["blockdiag", "band", "pad2d", "lower"])
 @pytest.mark.parametrize("as_bias", [False, True])
 def test_structured_masks_with_skipped_tiles(D, kind, as_bias):
@@ -602,7 +602,7 @@ def test_grouped_heads_with_key_padding_and_skipped_tiles():
     assert grads[1][1, :, 256:].abs().max().item() == 0.0  # key blocks past the limit of batch entry 1
 
 
-@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128, 256])
 @pytest.mark.parametrize("kind", ["blockdiag", "band", "per_head"])
 def test_grouped_heads_with_structured_masks_and_skipped_tiles(D, kind):
     """Tile lists with 4 query heads over 2 key/value heads: the lists belong to the mask planes (one
