@@ -1,16 +1,21 @@
-// Fused dual forward for 16-bit element types with D = 256.
+// Forward for 16-bit element types with D = 256.
 //
 // With D = 256 the operands that stay in registers (Q, Q': 2 x 64) and the accumulators (O, T:
-// 2 x 128) of 32 query rows do not fit one wave next to the score tiles.  Here a workgroup
-// produces DV = 128 of the D output columns: it forms the scores over the whole of D (both
-// workgroups of a query block do, which is the price) and multiplies them with a 128-column slice
-// of V, V', so a wave holds 2 x 64 + 2 x 64 registers in the accumulation file, all of it.  (Without
-// tangents Q and O alone fit, 64 + 128, and one workgroup produces all columns: DV = D.)
+// 2 x 128) of 32 query rows do not fit one wave next to the score tiles.  Without tangents Q and O
+// alone do (64 + 128 in the accumulation file), and that is the first of two passes of the dual
+// forward: O and M.  The second pass (TPASS) holds Q, Q' and T (all of the accumulation file), takes
+// the final M of the first, so that p = exp2(s - M) needs no running maximum, and writes
+// O' = T - mu O and mu.  S is formed twice (seven matrix products instead of six).
+//
+// (The template can also split the output columns over workgroups, DV < D: each then forms the
+// scores over all of D and multiplies with a DV-column slice of V, V'.  Two halves compute nine
+// products for the dual forward and measured 11 % slower than the two passes; the launcher does not
+// use it.)
 //
 // Memory side as in fwd_kernel_v2.hpp: direct-to-LDS loads, double buffered, one barrier per tile,
 // XOR-swizzled 16-byte chunks, ds_read_b128 for K / K' fragments and the transposing
-// ds_read_b64_tr_b16 for V / V'.  A tile is 32 keys (K, K' rows are 512 bytes; two stages of
-// 64-key tiles would not fit the LDS); a listed 64-key tile is visited as its two halves.
+// ds_read_b64_tr_b16 for V / V'.  A tile is 32 keys (rows are 512 bytes; two stages of 64-key tiles
+// would not fit the LDS); a listed 64-key tile is visited as its two halves.
 #pragma once
 #include <utility>
 
@@ -38,12 +43,15 @@ template <typename T, int D, int DV, bool DUAL> struct FwdWideCfg {
   static constexpr size_t LDS_BYTES = 2 * (size_t)STAGEB;
   static constexpr int IPWK = TILEBK / 1024 / NW;      // direct-load instructions per wave per tile
   static constexpr int IPWV = TILEBV / 1024 / NW;
-  static_assert(IPWK >= 1 && IPWV >= 1 && CHK == 32 && (CHV == 16 || (CHV == 32 && !DUAL)));
+  static_assert(IPWK >= 1 && IPWV >= 1 && CHK == 32 && (CHV == 16 || CHV == 32));
 };
 
-template <typename T, int D, int DV, bool DUAL, int MASK>
+// TPASS (with DUAL and DV = D): the second pass of the dual forward, see above.
+template <typename T, int D, int DV, bool DUAL, int MASK, bool TPASS = false>
 __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
+  static_assert(!TPASS || (DUAL && DV == D));
   using Cfg = FwdWideCfg<T, D, DV, DUAL>;
+  constexpr bool GD = TPASS;  // the accumulation file is full: see mma_vra
   constexpr int BN = Cfg::BN, NS = Cfg::NS, NK = Cfg::NK;
   constexpr int ROWBK = Cfg::ROWBK, ROWBV = Cfg::ROWBV, TILEBK = Cfg::TILEBK, TILEBV = Cfg::TILEBV;
   constexpr int IPWK = Cfg::IPWK, IPWV = Cfg::IPWV, VBASE = Cfg::VBASE;
@@ -135,16 +143,17 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
     if constexpr (DUAL) pin_acc(Qtf[kk]);
   }
 
-  f32x16 Oacc[DB], Tacc[DUAL ? DB : 1];
+  f32x16 Oacc[TPASS ? 1 : DB], Tacc[DUAL ? DB : 1];
 #pragma unroll
   for (int db = 0; db < DB; ++db) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      Oacc[db][e] = 0.f;
+      if constexpr (!TPASS) Oacc[db][e] = 0.f;
       if constexpr (DUAL) Tacc[db][e] = 0.f;
     }
   }
   float m_i = NEG_INF, l_i = 0.f, mu_i = 0.f;
+  if constexpr (TPASS) m_i = qrow < L ? p.M[(size_t)zh * L + qld] : __builtin_inff();  // +inf: a row without keys
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
@@ -258,13 +267,13 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
       if constexpr (kk + PD < KK) issue_k(std::integral_constant<int, kk + PD>{});
       load_step(std::integral_constant<int, kk>{});
       const Frag<T> a = __builtin_bit_cast(Frag<T>, ka[kk % RD]);
-      if constexpr (DUAL) mma_vra<kk == 0>(Sp, a, Qtf[kk]);
-      mma_vra<kk == 0>(S, a, Qf[kk]);
-      if constexpr (DUAL) mma_vra<false>(Sp, __builtin_bit_cast(Frag<T>, kb[kk % RD]), Qf[kk]);
+      if constexpr (DUAL) mma_vra<kk == 0, GD>(Sp, a, Qtf[kk]);
+      mma_vra<kk == 0, GD>(S, a, Qf[kk]);
+      if constexpr (DUAL) mma_vra<false, GD>(Sp, __builtin_bit_cast(Frag<T>, kb[kk % RD]), Qf[kk]);
     });
     if constexpr (DUAL) tiles_ready(S, Sp);
     else tiles_ready(S);
-    float mx;
+    float mx = 0.f;
     constexpr bool general = MASK != MASK_NONE || EDGE;
     if constexpr (general) {
       mx = NEG_INF;
@@ -291,24 +300,26 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
         }
       }
       mx = pair_max(mx);
-    } else {
+    } else if constexpr (!TPASS) {
       mx = S[0];
 #pragma unroll
       for (int e = 1; e < 16; ++e) mx = fmaxf(mx, S[e]);
       mx = pair_max(mx) * sl2;
     }
-    if (__any(mx > m_i + RESCALE_TAU)) {
-      const float m_new = fmaxf(m_i, mx);
-      const float alpha = fast_exp2(m_i - ((m_new == NEG_INF) ? 0.f : m_new));
-      m_i = m_new;
-      l_i *= alpha;
-      if constexpr (DUAL) mu_i *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          Oacc[db][e] = acc_scale(Oacc[db][e], alpha);
-          if constexpr (DUAL) Tacc[db][e] = acc_scale(Tacc[db][e], alpha);
+    if constexpr (!TPASS) {
+      if (__any(mx > m_i + RESCALE_TAU)) {
+        const float m_new = fmaxf(m_i, mx);
+        const float alpha = fast_exp2(m_i - ((m_new == NEG_INF) ? 0.f : m_new));
+        m_i = m_new;
+        l_i *= alpha;
+        if constexpr (DUAL) mu_i *= alpha;
+  #pragma unroll
+        for (int db = 0; db < DB; ++db) {
+  #pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            Oacc[db][e] = acc_scale(Oacc[db][e], alpha);
+            if constexpr (DUAL) Tacc[db][e] = acc_scale(Tacc[db][e], alpha);
+          }
         }
       }
     }
@@ -351,7 +362,7 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
       load_step(std::integral_constant<int, KK + i>{});
       const u32x4 av = {va[sl][0][0], va[sl][0][1], va[sl][1][0], va[sl][1][1]};
       const Frag<T> a = __builtin_bit_cast(Frag<T>, av);
-      mma(Oacc[db], a, pf[c]);
+      if constexpr (!TPASS) mma(Oacc[db], a, pf[c]);
       if constexpr (DUAL) {
         mma(Tacc[db], a, psf[c]);
         const u32x4 bv = {vb[sl][0][0], vb[sl][0][1], vb[sl][1][0], vb[sl][1][1]};
@@ -411,30 +422,51 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
   // ---- epilogue ---------------------------------------------------------------------------------
   l_i += xor32(l_i);
   if constexpr (DUAL) mu_i += xor32(mu_i);
-  const bool dead = !(l_i > 0.f);
-  const float inv = dead ? 0.f : 1.f / l_i;
-  const float mu_n = mu_i * inv;
-  if (qrow < L) {
-    T *Og = reinterpret_cast<T *>(p.o) + head + (size_t)qrow * D + slice * DV;
-    T *Otg = DUAL ? reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D + slice * DV : nullptr;
+  if constexpr (TPASS) {
+    // p was normalised by the final M, so T and mu are final as they stand; O comes from the first pass
+    if (qrow < L) {
+      const T *Og = reinterpret_cast<const T *>(p.o) + head + (size_t)qrow * D;
+      T *Otg = reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+      for (int db = 0; db < DB; ++db) {
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        float o8[8], t8[8];
+        for (int hf = 0; hf < 2; ++hf) {
+          const int d0 = 32 * db + 16 * hf + 8 * g;
+          const Frag<T> o8 = ld8<T>(Og + d0);
+          float t8[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          o8[e] = Oacc[db][8 * hf + e] * inv;
-          if constexpr (DUAL) t8[e] = Tacc[db][8 * hf + e] * inv - mu_n * o8[e];
+          for (int e = 0; e < 8; ++e) t8[e] = Tacc[db][8 * hf + e] - mu_i * (float)o8[e];
+          store8<T>(Otg + d0, t8);
         }
-        const int d0 = 32 * db + 16 * hf + 8 * g;
-        store8<T>(Og + d0, o8);
-        if constexpr (DUAL) store8<T>(Otg + d0, t8);
       }
+      if (g == 0) p.mu[(size_t)zh * L + qrow] = mu_i;
     }
-    if (g == 0 && slice == 0) {  // every slice holds the same row statistics
-      p.M[(size_t)zh * L + qrow] = dead ? __builtin_inff() : m_i + __builtin_amdgcn_logf(l_i);
-      if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = mu_n;
+  } else {
+    const bool dead = !(l_i > 0.f);
+    const float inv = dead ? 0.f : 1.f / l_i;
+    const float mu_n = mu_i * inv;
+    if (qrow < L) {
+      T *Og = reinterpret_cast<T *>(p.o) + head + (size_t)qrow * D + slice * DV;
+      T *Otg = DUAL ? reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D + slice * DV : nullptr;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          float o8[8], t8[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            o8[e] = Oacc[db][8 * hf + e] * inv;
+            if constexpr (DUAL) t8[e] = Tacc[db][8 * hf + e] * inv - mu_n * o8[e];
+          }
+          const int d0 = 32 * db + 16 * hf + 8 * g;
+          store8<T>(Og + d0, o8);
+          if constexpr (DUAL) store8<T>(Otg + d0, t8);
+        }
+      }
+      if (g == 0 && slice == 0) {  // every slice holds the same row statistics
+        p.M[(size_t)zh * L + qrow] = dead ? __builtin_inff() : m_i + __builtin_amdgcn_logf(l_i);
+        if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = mu_n;
+      }
     }
   }
 }
