@@ -117,22 +117,25 @@ def hvp_sweep(be, _lib):
 
 
 def shape_rows(be, _lib):
-    """Shapes next to the headline one, bf16, no mask: D = 32 and D = 256 (the smallest and the largest
-    head dim the reference admits), 16 query heads over 4 key/value heads, and 4096 queries over 512 keys (the last two are
+    """Shapes next to the headline one, no mask: the other benchmark configurations' shapes, D = 32 and
+    D = 256 (the smallest and the largest head dim the reference admits), 16 query heads over 4 key/value heads, and 4096 queries over 512 keys (the last two are
     shapes the reference refuses).  Dual forward and dual backward, counted as 12 and 24 flops per
     (query, key, d) triple."""
     import torch
 
     dev = torch.device("cuda:0")
     rows = {}
-    for name, (Zs, Hs, Hk, Lq, Lk, Ds) in {
-        "B4_H16_L2048_D32": (4, 16, 16, 2048, 2048, 32),
-        "B4_H16_L2048_D256": (4, 16, 16, 2048, 2048, 256),
-        "B4_H16_over_4_kv_heads_L4096_D128": (4, 16, 4, 4096, 4096, 128),
-        "B4_H16_Lq4096_Lk512_D128": (4, 16, 16, 4096, 512, 128),
+    for name, (Zs, Hs, Hk, Lq, Lk, Ds, dtype) in {
+        "bf16_B4_H16_L2048_D32": (4, 16, 16, 2048, 2048, 32, torch.bfloat16),
+        "bf16_B4_H16_L2048_D64_config2": (4, 16, 16, 2048, 2048, 64, torch.bfloat16),
+        "bf16_B4_H16_L2048_D256": (4, 16, 16, 2048, 2048, 256, torch.bfloat16),
+        "fp16_B2_H32_L4096_D128_config3_noncausal": (2, 32, 32, 4096, 4096, 128, torch.float16),
+        "fp32_B4_H8_L1024_D64_config4_nomask": (4, 8, 8, 1024, 1024, 64, torch.float32),
+        "bf16_B4_H16_over_4_kv_heads_L4096_D128": (4, 16, 4, 4096, 4096, 128, torch.bfloat16),
+        "bf16_B4_H16_Lq4096_Lk512_D128": (4, 16, 16, 4096, 512, 128, torch.bfloat16),
     }.items():
         g = torch.Generator(device=dev).manual_seed(11)
-        mk = lambda h, l: torch.randn(Zs, h, l, Ds, generator=g, device=dev).to(torch.bfloat16)  # noqa: E731
+        mk = lambda h, l: torch.randn(Zs, h, l, Ds, generator=g, device=dev).to(dtype)  # noqa: E731
         q, qt, go, gt = [mk(Hs, Lq) for _ in range(4)]
         k, v, kt, vt = [mk(Hk, Lk) for _ in range(4)]
         scale = Ds**-0.5
@@ -279,7 +282,7 @@ def main():
         }
         out["extra"]["hvp_sweep_bf16_B1_H16_D128_causal"] = hvp_sweep(be, _lib)
         out["extra"]["masks_bf16_B4_H16_L4096_D128"] = mask_rows(be, _lib, q, k, v, qt, kt, vt, go, gt, scale)
-        out["extra"]["other_shapes_bf16"] = shape_rows(be, _lib)
+        out["extra"]["other_shapes"] = shape_rows(be, _lib)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)
