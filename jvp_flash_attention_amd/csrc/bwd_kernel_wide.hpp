@@ -1,11 +1,15 @@
-// dq (PLAIN / DUAL) or dq' (TANGENT) for 16-bit element types with D = 256, on the memory pipeline of
-// bwd_kernel_v2.hpp.
+// Backward kernels for 16-bit element types with D = 256, on the memory pipeline of bwd_kernel_v2.hpp.
 //
-// The resident operands of 32 query rows (Q, gO, Q', gT: 4 x 64 registers) are the whole
-// accumulation file, so, as in fwd_kernel_wide.hpp, two workgroups share a query block: each
-// recomputes the score tiles over all of D and accumulates DV = 128 of the dq columns, in ordinary
-// vector registers.  Key tiles are 32 rows (K, V, K', V' rows are 512 bytes: two stages of four
-// 16 KB tiles fill 128 KB of LDS); a tile is read both ways from its one row-major copy, as there.
+// With D = 256 the operands that stay in registers are the whole accumulation file (dq: Q, gO, Q',
+// gT; dk: K, V, K', V': 4 x 64 registers), so the accumulators live in ordinary vector registers and
+// cover DV = 128 columns: two workgroups per block of 128 rows recompute the score tiles over all of
+// D and each accumulates half of the output.  (dV needs S and S' only: in the dual mode it is a launch
+// of its own with K, K' resident and all 256 columns.)  Streamed tiles are 32 rows of 512 bytes: two
+// stages of four 16 KB tiles fill 128 KB of LDS; a tile is read both ways from its one row-major copy.
+// The inline-asm matrix instructions are the guarded form (see mma_vra): with the accumulation file
+// full the allocator moves resident operands through a spare register right before their use.
+//
+// First kernel: dq (PLAIN / DUAL) or dq' (TANGENT).
 #pragma once
 #include "bwd_kernel_v2.hpp"
 
