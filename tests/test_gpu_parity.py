@@ -351,12 +351,16 @@ def test_small_tangents_config2_shape_slice():
     _run_case(1, 4, 512, 64, torch.bfloat16, "none", tangent_std=0.1)
 
 
-def test_fully_masked_rows_are_zero():
+@pytest.mark.parametrize("dt,D", [("fp32", 64), ("bf16", 32), ("bf16", 64), ("bf16", 128), ("fp16", 256), ("bf16", 256)])
+def test_fully_masked_rows_are_zero(dt, D):
+    """Rows without any attended key: O = O' = 0, M = +inf, mu = 0 and zero gradients, in every kernel
+    family (the reference gives O = 0 there too, its jvp_attention.py:1011-1015)."""
     from jvp_flash_attention_amd import _lib
 
     be = _lib.backend()
-    Z, H, L, D = 1, 2, 64, 64
-    q, k, v, qt, kt, vt, go, gt = [x.cuda() for x in _make(Z, H, L, D, torch.float32, 3)]
+    Z, H, L = 1, 2, 64
+    dtype = DTYPES[dt]
+    q, k, v, qt, kt, vt, go, gt = [x.cuda() for x in _make(Z, H, L, D, dtype, 3)]
     mask = torch.ones(Z, H, L, L, dtype=torch.bool)
     mask[0, 1, 5, :] = False
     mask[0, 0, 40, :] = False
@@ -373,7 +377,7 @@ def test_fully_masked_rows_are_zero():
     f64 = [x.double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
     rb = dense.backward(*f64, mask=mask.cpu().numpy(), scale=D**-0.5)
     for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
-        _tol_check(n, t, rb[n], torch.float32)
+        _tol_check(n, t, rb[n], dtype)
 
 
 def test_only_tangent_gradient_hvp_style():
