@@ -100,21 +100,40 @@ def _validate(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dropout
         )
 
 
+def _already_verified(mask: Tensor) -> bool:
+    """The checks of ``verify_attn_mask`` read the whole mask and wait for the answer; a mask that
+    passed them is remembered on the tensor, keyed by its version counter, so that the layers of a
+    model and the steps of a loop that share one mask pay once."""
+    return getattr(mask, "_jvpfa_verified", None) == mask._version
+
+
+def _remember_verified(mask: Tensor) -> None:
+    try:
+        mask._jvpfa_verified = mask._version
+    except (AttributeError, RuntimeError):
+        pass
+
+
 def _classify_mask(attn_mask: Tensor | None, q: Tensor, verify_attn_mask: bool):
     """Mask kind and the tensor the kernels read (JA:2429-2462)."""
     if attn_mask is None:
         return torch.empty(0, device=q.device, dtype=q.dtype), _lib.MASK_NONE
     if attn_mask.dtype == torch.bool:
         mask_tensor = attn_mask
-        if verify_attn_mask:
+        if verify_attn_mask and not _already_verified(attn_mask):
             assert mask_tensor.any(dim=-1).any(dim=-1).all(), (
                 "The attention mask cannot be all False for any head."
             )
+            _remember_verified(attn_mask)
         return mask_tensor, _lib.MASK_BOOL
     mask_tensor = attn_mask.to(q.dtype)
-    if verify_attn_mask:
-        assert not torch.isnan(mask_tensor).any(), "The attention mask cannot contain NaNs."
-        assert not torch.isposinf(mask_tensor).any(), "The attention mask cannot contain +inf."
+    if verify_attn_mask and not _already_verified(attn_mask):
+        # one pass: neither NaN nor +inf compares <= the largest finite value; the reference's two
+        # messages (JA:2447-2456) are told apart only when the pass fails
+        if not bool((mask_tensor <= torch.finfo(mask_tensor.dtype).max).all()):
+            assert not torch.isnan(mask_tensor).any(), "The attention mask cannot contain NaNs."
+            assert not torch.isposinf(mask_tensor).any(), "The attention mask cannot contain +inf."
+        _remember_verified(attn_mask)
     return mask_tensor, _lib.MASK_ADD
 
 

@@ -232,3 +232,30 @@ def test_registered_operators_describe_their_outputs_without_running():
         assert [t.shape for t in g] == [q.shape] * 6
         g = torch.ops.jvpfa.bwd(q, q, q, None, None, None, o, None, M, None, q, None, None, 0, True, 0.125, False)
         assert [t.shape for t in g[:3]] == [q.shape] * 3 and all(t.numel() == 0 for t in g[3:])
+
+
+def test_mask_verification_is_remembered_per_mask_version():
+    """``verify_attn_mask`` reads the whole mask; a mask that passed is not read again until it changes."""
+    import torch
+
+    from jvp_flash_attention_amd import jvp_attention as ja
+
+    q = torch.zeros(1, 1, 4, 32)
+    mask = torch.ones(1, 1, 4, 4, dtype=torch.bool)
+    ja._classify_mask(mask, q, True)
+    assert ja._already_verified(mask)
+    mask[0, 0] = False  # an in-place change bumps the version: the check runs again and fails
+    assert not ja._already_verified(mask)
+    with pytest.raises(AssertionError, match="all False"):
+        ja._classify_mask(mask, q, True)
+    bias = torch.zeros(1, 1, 4, 4)
+    ja._classify_mask(bias, q, True)
+    assert ja._already_verified(bias)
+    bias[0, 0, 1, 2] = float("nan")
+    with pytest.raises(AssertionError, match="NaN"):
+        ja._classify_mask(bias, q, True)
+    bias[0, 0, 1, 2] = float("inf")
+    with pytest.raises(AssertionError, match=r"\+inf"):
+        ja._classify_mask(bias, q, True)
+    bias[0, 0, 1, 2] = float("-inf")  # -inf is a legal "masked" value
+    ja._classify_mask(bias, q, True)
