@@ -314,6 +314,33 @@ def test_other_head_dims_at_benchmark_size(D, causal):
         assert _rel(g[z, h], rb[n][0, 0]) <= 2e-2, n
 
 
+@pytest.mark.parametrize("D", [32, 64, 256])
+def test_long_causal_sequences_prefix_properties(D):
+    """bf16 B1 H4 L16384 causal: causal rows never see later keys, so the first half of the outputs equals a
+    run on the truncated sequence bit for bit, and with the incoming gradients of the second half set
+    to zero the gradients of the first half equal those of the truncated run while dk, dv of the second
+    half are exactly zero."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    Z, H, L = 1, 4, 16384
+    dt, scale = torch.bfloat16, D**-0.5
+    q, k, v, qt, kt, vt, go, gt = [_randn((Z, H, L, D), dt, 70 + i) for i in range(8)]
+    o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, 0, True, scale)
+    assert all(torch.isfinite(t).all() for t in (o, ot, M, mu))
+    h = L // 2
+    cut = [x[:, :, :h].contiguous() for x in (q, k, v, qt, kt, vt)]
+    o2, ot2, M2, mu2 = be.fwd(*cut, None, 0, True, scale)
+    assert torch.equal(o[:, :, :h], o2) and torch.equal(ot[:, :, :h], ot2) and torch.equal(M[:, :, :h], M2)
+    go[:, :, h:] = 0
+    gt[:, :, h:] = 0
+    full = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, 0, True, scale)
+    part = be.bwd(*cut, o2, ot2, M2, mu2, go[:, :, :h].contiguous(), gt[:, :, :h].contiguous(), None, 0, True, scale)
+    for n, a_, b_ in zip(("dq", "dk", "dv"), full[:3], part[:3]):
+        assert torch.equal(a_[:, :, :h], b_), n
+    assert full[1][:, :, h:].abs().max().item() == 0.0 and full[2][:, :, h:].abs().max().item() == 0.0
+
+
 def test_config3_causal_long_full_size_properties():
     """benchmark configuration 3: fp16 B2 H32 L4096 D128 causal, and the headline bf16 B4 H16 L4096 D128."""
     from jvp_flash_attention_amd import _lib
