@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define JVPFA_ABI_VERSION 4
+#define JVPFA_ABI_VERSION 5
 
 enum jvpfa_dtype { JVPFA_BF16 = 0, JVPFA_FP16 = 1, JVPFA_FP32 = 2 };
 
@@ -41,7 +41,7 @@ enum jvpfa_status {
   JVPFA_E_ALIGN = -4,     /* a tensor pointer is not 16-byte aligned */
   JVPFA_E_CONFLICT = -5,  /* causal together with a mask (JA:2380-2381 raises ValueError) */
   JVPFA_E_LAUNCH = -6,    /* hipGetLastError() reported a launch failure */
-  JVPFA_E_ABI = -7        /* struct_size is neither this version's nor an earlier version's */
+  JVPFA_E_ABI = -7        /* struct_size is not this library's: caller built from another header */
 };
 
 /* Shape, numeric type and masking shared by forward and backward. */
@@ -74,20 +74,17 @@ typedef struct jvpfa_fwd_args {
   const void *qt, *kt, *vt; /* all three NULL, or all three set */
   void *o, *ot;
   float *M, *mu;
-  /* since version 2 (a caller may pass the version-1 size, which ends before this field):
-   * optional hint for padded batches, Z int32 values on the device or NULL.  The caller promises
+  /* optional hint for padded batches, Z int32 values on the device or NULL.  The caller promises
    * that the mask itself masks every key index >= key_limit[z] for all heads and queries of batch
    * z; key tiles past the limit are then skipped instead of read and masked.  No counterpart in the
    * reference, which reads the full (Z,H,L,L) mask (JA:2383-2388).  Ignored without a mask. */
   const int32_t *key_limit;
-  /* since version 3 (a caller may pass the version-2 size, which ends before this field):
-   * optional lists of the key tiles that hold an attended entry, written by jvpfa_mask_tiles() for
+  /* optional lists of the key tiles that hold an attended entry, written by jvpfa_mask_tiles() for
    * this same mask, or NULL.  Tiles not listed are skipped instead of read and masked.  When set,
    * key_limit is ignored.  Ignored (and key_limit used) for fp32, whose kernels visit every tile
    * up to the key limit.  Ignored without a mask. */
   const int32_t *tiles_q;
-  /* since version 4 (a caller may pass the version-3 size, which ends before this field): shape of
-   * k, v, kt, vt when it is not q's -- Lk keys (any length >= 1) and Hk key/value heads, Hk a divisor
+  /* shape of k, v, kt, vt when it is not q's -- Lk keys (any length >= 1) and Hk key/value heads, Hk a divisor
    * of p.H; query head h reads key/value head h / (H / Hk).  0 means "as q" (p.L, p.H).  k, v and
    * their tangents are then (Z, Hk, Lk, D), the mask strides address (z, h, query, key) with Lk keys,
    * and causal means key index <= query index.  The reference requires q, k, v of one shape
@@ -124,11 +121,11 @@ typedef struct jvpfa_bwd_args {
   void *dq, *dk, *dv;
   void *dqt, *dkt, *dvt;
   void *workspace;
-  const int32_t *key_limit; /* since version 2: as in jvpfa_fwd_args */
-  const int32_t *tiles_q;   /* since version 3: as in jvpfa_fwd_args (used by the dq kernels) */
-  const int32_t *tiles_k;   /* since version 3: the other list of jvpfa_mask_tiles() (dk/dv kernels);
+  const int32_t *key_limit; /* as in jvpfa_fwd_args */
+  const int32_t *tiles_q;   /* as in jvpfa_fwd_args (used by the dq kernels) */
+  const int32_t *tiles_k;   /* the other list of jvpfa_mask_tiles() (dk/dv kernels);
                                tiles_q and tiles_k are both NULL or both set */
-  int32_t Lk, Hk;           /* since version 4: as in jvpfa_fwd_args; dk, dv, dkt, dvt have the shape of k */
+  int32_t Lk, Hk;           /* as in jvpfa_fwd_args; dk, dv, dkt, dvt have the shape of k */
 } jvpfa_bwd_args;
 
 int jvpfa_bwd(const jvpfa_bwd_args *args, void *hip_stream);

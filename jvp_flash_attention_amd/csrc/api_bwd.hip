@@ -27,14 +27,10 @@ extern "C" size_t jvpfa_bwd_workspace_bytes(int32_t Z, int32_t H, int32_t L) {
 
 extern "C" int jvpfa_bwd(const jvpfa_bwd_args *a, void *hip_stream) {
   if (!a) return JVPFA_E_NULL;
-  // versions 1, 2 and 3 of the struct end before key_limit / tiles_q / Lk
-  const bool v4 = a->struct_size == sizeof(jvpfa_bwd_args);
-  const bool v3 = v4 || a->struct_size == offsetof(jvpfa_bwd_args, Lk);
-  const bool v2 = v3 || a->struct_size == offsetof(jvpfa_bwd_args, tiles_q);
-  if (!v2 && a->struct_size != offsetof(jvpfa_bwd_args, key_limit)) return JVPFA_E_ABI;
-  if (v3 && (a->tiles_q != nullptr) != (a->tiles_k != nullptr)) return JVPFA_E_NULL;
+  if (a->struct_size != sizeof(jvpfa_bwd_args)) return JVPFA_E_ABI;
+  if ((a->tiles_q != nullptr) != (a->tiles_k != nullptr)) return JVPFA_E_NULL;
   int rc = check_problem(a->p);
-  if (rc == JVPFA_OK && v4) rc = check_kv_shape(a->p, a->Lk, a->Hk);
+  if (rc == JVPFA_OK) rc = check_kv_shape(a->p, a->Lk, a->Hk);
   if (rc != JVPFA_OK) return rc;
   if (!a->q || !a->k || !a->v || !a->o || !a->M || !a->dq || !a->dk || !a->dv || !a->workspace)
     return JVPFA_E_NULL;
@@ -52,8 +48,7 @@ extern "C" int jvpfa_bwd(const jvpfa_bwd_args *a, void *hip_stream) {
     if (ptr && !aligned16(ptr)) return JVPFA_E_ALIGN;
 
   BwdParams p;
-  p.pr = to_problem(a->p, v2 ? a->key_limit : nullptr, v3 ? a->tiles_q : nullptr, v3 ? a->tiles_k : nullptr, v4 ? a->Lk : 0,
-                    v4 ? a->Hk : 0);
+  p.pr = to_problem(a->p, a->key_limit, a->tiles_q, a->tiles_k, a->Lk, a->Hk);
   p.q = a->q; p.k = a->k; p.v = a->v;
   p.qt = a->qt; p.kt = a->kt; p.vt = a->vt;
   p.o = a->o; p.ot = a->ot; p.M = a->M; p.mu = a->mu;

@@ -19,13 +19,9 @@ using namespace jvpfa;
 
 extern "C" int jvpfa_fwd(const jvpfa_fwd_args *a, void *hip_stream) {
   if (!a) return JVPFA_E_NULL;
-  // versions 1, 2 and 3 of the struct end before key_limit / tiles_q / Lk
-  const bool v4 = a->struct_size == sizeof(jvpfa_fwd_args);
-  const bool v3 = v4 || a->struct_size == offsetof(jvpfa_fwd_args, Lk);
-  const bool v2 = v3 || a->struct_size == offsetof(jvpfa_fwd_args, tiles_q);
-  if (!v2 && a->struct_size != offsetof(jvpfa_fwd_args, key_limit)) return JVPFA_E_ABI;
+  if (a->struct_size != sizeof(jvpfa_fwd_args)) return JVPFA_E_ABI;
   int rc = check_problem(a->p);
-  if (rc == JVPFA_OK && v4) rc = check_kv_shape(a->p, a->Lk, a->Hk);
+  if (rc == JVPFA_OK) rc = check_kv_shape(a->p, a->Lk, a->Hk);
   if (rc != JVPFA_OK) return rc;
   if (!a->q || !a->k || !a->v || !a->o || !a->M) return JVPFA_E_NULL;
   const int ntan = (a->qt != nullptr) + (a->kt != nullptr) + (a->vt != nullptr);
@@ -37,7 +33,7 @@ extern "C" int jvpfa_fwd(const jvpfa_fwd_args *a, void *hip_stream) {
     if (ptr && !aligned16(ptr)) return JVPFA_E_ALIGN;
 
   FwdParams p;
-  p.pr = to_problem(a->p, v2 ? a->key_limit : nullptr, v3 ? a->tiles_q : nullptr, nullptr, v4 ? a->Lk : 0, v4 ? a->Hk : 0);
+  p.pr = to_problem(a->p, a->key_limit, a->tiles_q, nullptr, a->Lk, a->Hk);
   p.q = a->q; p.k = a->k; p.v = a->v;
   p.qt = a->qt; p.kt = a->kt; p.vt = a->vt;
   p.o = a->o; p.ot = a->ot; p.M = a->M; p.mu = a->mu;
@@ -55,7 +51,7 @@ extern "C" const char *jvpfa_error_string(int status) {
     case JVPFA_E_ALIGN: return "tensor pointer not 16-byte aligned";
     case JVPFA_E_CONFLICT: return "causal attention does not take a mask";
     case JVPFA_E_LAUNCH: return "HIP kernel launch failed";
-    case JVPFA_E_ABI: return "struct_size does not match this library (nor an earlier version)";
+    case JVPFA_E_ABI: return "struct_size does not match this library: caller and library were built from different headers";
   }
   return "unknown status";
 }

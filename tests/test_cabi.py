@@ -99,21 +99,20 @@ def test_key_value_shape_fields_are_checked():
     assert lib.jvpfa_fwd(C.byref(a), None) == -1  # shape accepted; stops at the NULL pointer
 
 
-def test_earlier_struct_sizes_are_still_accepted():
-    """A caller built against version 1 passes structs that end before key_limit, one built against
-    version 2 structs that end before tiles_q, one built against version 3 structs that end before Lk."""
+def test_struct_size_must_be_this_library_s():
+    """One size per struct: a caller built from another header is told so instead of being guessed at."""
     lib = _lib.load()
     a = _fwd_args(q=None)
-    for size in (_lib.FwdArgs.key_limit.offset, _lib.FwdArgs.tiles_q.offset, _lib.FwdArgs.Lk.offset, C.sizeof(_lib.FwdArgs)):
+    assert lib.jvpfa_fwd(C.byref(a), None) == -1  # got past the size check, to the NULL pointer check
+    for size in (_lib.FwdArgs.key_limit.offset, _lib.FwdArgs.Lk.offset, C.sizeof(_lib.FwdArgs) + 8):
         a.struct_size = size
-        assert lib.jvpfa_fwd(C.byref(a), None) == -1  # got past the size check, to the NULL pointer check
-    a.struct_size = _lib.FwdArgs.key_limit.offset - 8
-    assert lib.jvpfa_fwd(C.byref(a), None) == -7
+        assert lib.jvpfa_fwd(C.byref(a), None) == -7
     b = _lib.BwdArgs()
     b.p.Z, b.p.H, b.p.L, b.p.D = 1, 1, 32, 64
-    for size in (_lib.BwdArgs.key_limit.offset, _lib.BwdArgs.tiles_q.offset, _lib.BwdArgs.Lk.offset, C.sizeof(_lib.BwdArgs)):
-        b.struct_size = size
-        assert lib.jvpfa_bwd(C.byref(b), None) == -1
+    b.struct_size = C.sizeof(_lib.BwdArgs)
+    assert lib.jvpfa_bwd(C.byref(b), None) == -1
+    b.struct_size = _lib.BwdArgs.Lk.offset
+    assert lib.jvpfa_bwd(C.byref(b), None) == -7
 
 
 def test_tile_lists_are_only_made_for_masks_with_a_row_per_query():
