@@ -41,7 +41,8 @@ enum jvpfa_status {
   JVPFA_E_ALIGN = -4,     /* a tensor pointer is not 16-byte aligned */
   JVPFA_E_CONFLICT = -5,  /* causal together with a mask (JA:2380-2381 raises ValueError) */
   JVPFA_E_LAUNCH = -6,    /* hipGetLastError() reported a launch failure */
-  JVPFA_E_ABI = -7        /* struct_size is not this library's: caller built from another header */
+  JVPFA_E_ABI = -7,       /* struct_size is not this library's: caller built from another header */
+  JVPFA_E_SCRATCH = -8    /* jvpfa_bwd_static: Z*H*L is more than jvpfa_bwd_static_max_rows() */
 };
 
 /* Shape, numeric type and masking shared by forward and backward. */
@@ -131,6 +132,22 @@ typedef struct jvpfa_bwd_args {
 int jvpfa_bwd(const jvpfa_bwd_args *args, void *hip_stream);
 
 size_t jvpfa_bwd_workspace_bytes(int32_t Z, int32_t H, int32_t L);
+
+/*
+ * jvpfa_bwd for callers that cannot hand over a workspace because they cannot allocate one: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
+ * the reference (whose backward allocates its `delta` with torch, JA:2883).  Same arguments and
+ * results as jvpfa_bwd; args->workspace is ignored, the row statistics of the pre-pass live in an
+ * array inside the library instead: 3 * JVPFA_STATIC_ROWS floats (12 MiB) of device memory per GPU
+ * the library runs on, held until the process ends.  The call allocates nothing and frees nothing.
+ * Limit: Z*H*L (rounded up to a multiple of 4) <= JVPFA_STATIC_ROWS, otherwise JVPFA_E_SCRATCH and
+ * nothing is launched.  The GPU the stream belongs to must be the current device.  Every call on a
+ * GPU uses that GPU's one array: two calls that overlap in time on one GPU (different streams, or
+ * different threads) race; calls on one stream, one after another, are fine.
+ */
+#define JVPFA_STATIC_ROWS (1 << 20)
+int jvpfa_bwd_static(const jvpfa_bwd_args *args, void *hip_stream);
+size_t jvpfa_bwd_static_max_rows(void);
 
 /*
  * Tile lists of a mask: which 64-wide tiles hold at least one attended entry (boolean: nonzero;

@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(HERE, "libjvpfa.so")
 ABI_VERSION = 5
 DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
-EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_bwd_workspace_bytes", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
+EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_bwd_workspace_bytes", "jvpfa_bwd_static", "jvpfa_bwd_static_max_rows", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
            "jvpfa_abi_version", "jvpfa_error_string")
 
 
@@ -83,6 +83,10 @@ def load() -> C.CDLL:
         lib.jvpfa_bwd.restype = C.c_int
         lib.jvpfa_bwd_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         lib.jvpfa_bwd_workspace_bytes.restype = C.c_size_t
+        lib.jvpfa_bwd_static.argtypes = [C.POINTER(BwdArgs), C.c_void_p]
+        lib.jvpfa_bwd_static.restype = C.c_int
+        lib.jvpfa_bwd_static_max_rows.argtypes = []
+        lib.jvpfa_bwd_static_max_rows.restype = C.c_size_t
         lib.jvpfa_mask_tiles_bytes.argtypes = [C.POINTER(Problem)]
         lib.jvpfa_mask_tiles_bytes.restype = C.c_size_t
         lib.jvpfa_mask_tiles.argtypes = [C.POINTER(Problem), C.c_void_p, C.c_void_p, C.c_void_p]

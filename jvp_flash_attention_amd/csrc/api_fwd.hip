@@ -51,6 +51,7 @@ extern "C" const char *jvpfa_error_string(int status) {
     case JVPFA_E_ALIGN: return "tensor pointer not 16-byte aligned";
     case JVPFA_E_CONFLICT: return "causal attention does not take a mask";
     case JVPFA_E_LAUNCH: return "HIP kernel launch failed";
+    case JVPFA_E_SCRATCH: return "Z*H*L exceeds the rows of the library's static scratch (jvpfa_bwd_static_max_rows())";
     case JVPFA_E_ABI: return "struct_size does not match this library: caller and library were built from different headers";
   }
   return "unknown status";
