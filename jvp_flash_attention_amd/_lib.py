@@ -130,6 +130,27 @@ def make_problem(q, mask, mask_kind, causal, sm_scale) -> Problem:
     return p
 
 
+def mask_version(mask):
+    """The version counter of a mask tensor, or None when it has none (tensors created under
+    ``torch.inference_mode()`` do not track versions): None means "do not cache, look again"."""
+    try:
+        return mask._version
+    except RuntimeError:
+        return None
+
+
+def forget_mask(mask) -> None:
+    """Drop what has been remembered about a mask tensor (verification, key limit, tile lists).  The caches
+    are keyed by the tensor's version counter, which ordinary in-place operations bump; writes that bypass it
+    (``mask.data``, a custom kernel writing through ``data_ptr()``, a dlpack / numpy alias) do not, and after
+    such a write this must be called before the mask is used again."""
+    for name in ("_jvpfa_verified", "_jvpfa_key_limit", "_jvpfa_tiles"):
+        try:
+            delattr(mask, name)
+        except AttributeError:
+            pass
+
+
 KEY_LIMIT_MIN_L = 512  # below this the two small reductions cost more than the skipped tiles save
 
 
@@ -142,17 +163,21 @@ def key_limit_hint(mask, mask_kind, Z, L):
         return None
     if mask.dim() != 4 or mask.shape[1] != 1 or mask.shape[2] != 1 or mask.shape[3] != L:
         return None
+    version = mask_version(mask)
     cached = getattr(mask, "_jvpfa_key_limit", None)
-    if cached is not None and cached[0] == mask._version:
-        return cached[1]
-    alive = mask if mask.dtype == torch.bool else mask > float("-inf")
-    idx = torch.arange(1, L + 1, device=mask.device, dtype=torch.int32)
-    lim = (alive.view(mask.shape[0], L) * idx).amax(dim=1).to(torch.int32).expand(Z).contiguous()
-    try:
-        mask._jvpfa_key_limit = (mask._version, lim)
-    except (AttributeError, RuntimeError):
-        pass
-    return lim
+    if cached is not None and version is not None and cached[0] == version:
+        lim = cached[1]
+    else:
+        alive = mask if mask.dtype == torch.bool else mask > float("-inf")
+        idx = torch.arange(1, L + 1, device=mask.device, dtype=torch.int32)
+        lim = (alive.view(mask.shape[0], L) * idx).amax(dim=1).to(torch.int32)  # one value per row of the mask
+        if version is not None:
+            try:
+                mask._jvpfa_key_limit = (version, lim)
+            except (AttributeError, RuntimeError):
+                pass
+    # the kernels index the limits by batch entry: a mask shared by the batch ([1,1,1,L]) is spread over Z
+    return lim if lim.shape[0] == Z else lim.expand(Z).contiguous()
 
 
 TILE_LISTS_MIN_L = 512  # below this a mask has too few tiles for skipping some to pay for the scan
@@ -187,9 +212,10 @@ def tile_lists(q, mask, mask_kind, want_k):
         return None, None
     if mask_kind == MASK_ADD and not _tile_lists_additive:
         return None, None
+    version = mask_version(mask)
     cached = getattr(mask, "_jvpfa_tiles", None)
-    if cached is None or cached[0] != mask._version:
-        cached = [mask._version, None, None]
+    if cached is None or version is None or cached[0] != version:
+        cached = [version, None, None]
     tq, tk = cached[1], cached[2]
     if tq is None or (want_k and tk is None):
         lib = load()
@@ -201,10 +227,11 @@ def tile_lists(q, mask, mask_kind, want_k):
         tq = new_q if tq is None else tq
         tk = new_k if new_k is not None else tk
         cached[1], cached[2] = tq, tk
-        try:
-            mask._jvpfa_tiles = cached
-        except (AttributeError, RuntimeError):
-            pass
+        if version is not None:
+            try:
+                mask._jvpfa_tiles = cached
+            except (AttributeError, RuntimeError):
+                pass
     return tq, (tk if want_k else None)
 
 

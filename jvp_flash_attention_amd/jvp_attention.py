@@ -12,6 +12,11 @@ Differences from the reference, all deliberate:
   are part of the backward recomputation (the reference scales the mask too, JA:247-251, and
   leaves it out of the backward, JA:1519-1522).  A float mask without any ``MASK_CONST`` entry is
   accepted (the reference raises ``UserWarning``, JA:2459-2462).
+* Boolean masks mask exactly: a masked key gets probability 0, and a query row with every key masked gives
+  O = O' = 0, M = +inf and zero gradients.  The reference adds ``MASK_CONST`` = -100 to the unscaled logits
+  (JA:241-245), so a masked key keeps a weight of about exp(-100 * sm_scale) next to the attended ones (1e-4 at
+  D = 128) and a fully masked row comes out as plain unmasked softmax; neither is reproduced, and no fixture of
+  the reference pins either, so for those rows the comparison with the reference is unpinned.
 * Masks may broadcast: any shape whose axes are 1 or (Z, H, L, L); a key-padding mask
   ``[Z,1,1,L]`` is read in place.  The reference requires the full shape (JA:2383-2388).
 * ``fwd_dual`` returns an output whose tangent O' carries an autograd graph, so gradients of
@@ -104,12 +109,16 @@ def _already_verified(mask: Tensor) -> bool:
     """The checks of ``verify_attn_mask`` read the whole mask and wait for the answer; a mask that
     passed them is remembered on the tensor, keyed by its version counter, so that the layers of a
     model and the steps of a loop that share one mask pay once."""
-    return getattr(mask, "_jvpfa_verified", None) == mask._version
+    version = _lib.mask_version(mask)
+    return version is not None and getattr(mask, "_jvpfa_verified", None) == version
 
 
 def _remember_verified(mask: Tensor) -> None:
+    version = _lib.mask_version(mask)
+    if version is None:
+        return
     try:
-        mask._jvpfa_verified = mask._version
+        mask._jvpfa_verified = version
     except (AttributeError, RuntimeError):
         pass
 

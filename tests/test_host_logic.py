@@ -259,3 +259,49 @@ def test_mask_verification_is_remembered_per_mask_version():
         ja._classify_mask(bias, q, True)
     bias[0, 0, 1, 2] = float("-inf")  # -inf is a legal "masked" value
     ja._classify_mask(bias, q, True)
+
+
+def test_key_limit_of_a_mask_shared_by_the_batch_follows_the_batch_size_of_each_call():
+    """One [1,1,1,L] key-padding mask used with two batch sizes: the kernels index the limits by batch entry,
+    so each call must get as many as it has batch entries (the cache keeps one value per row of the mask)."""
+    L = _lib.KEY_LIMIT_MIN_L
+    mask = torch.ones(1, 1, 1, L, dtype=torch.bool)
+    mask[..., 300:] = False
+    assert _lib.key_limit_hint(mask, _lib.MASK_BOOL, 2, L).tolist() == [300, 300]
+    assert _lib.key_limit_hint(mask, _lib.MASK_BOOL, 8, L).tolist() == [300] * 8
+    assert _lib.key_limit_hint(mask, _lib.MASK_BOOL, 1, L).tolist() == [300]
+    assert mask._jvpfa_key_limit[1].shape == (1,)
+
+
+def test_masks_made_in_inference_mode_have_no_version_counter_and_are_not_cached():
+    from jvp_flash_attention_amd import jvp_attention as ja
+
+    L = _lib.KEY_LIMIT_MIN_L
+    with torch.inference_mode():
+        mask = torch.ones(2, 1, 1, L, dtype=torch.bool)
+        mask[1, ..., 100:] = False
+        bias = torch.zeros(1, 1, 4, 4)
+    assert _lib.mask_version(mask) is None
+    q = torch.zeros(2, 1, 4, 32)
+    assert ja._classify_mask(mask, q, True)[1] == _lib.MASK_BOOL     # verified, every time
+    assert not ja._already_verified(mask)
+    assert ja._classify_mask(bias, q[:1], True)[1] == _lib.MASK_ADD
+    assert _lib.key_limit_hint(mask, _lib.MASK_BOOL, 2, L).tolist() == [L, 100]
+    assert not hasattr(mask, "_jvpfa_key_limit")
+    with torch.inference_mode(), oracle_backend():
+        o = attention(torch.randn(2, 1, L, 32), torch.randn(2, 1, L, 32), torch.randn(2, 1, L, 32), attn_mask=mask)
+    assert torch.isfinite(o).all()
+
+
+def test_forget_mask_drops_what_was_remembered():
+    from jvp_flash_attention_amd import jvp_attention as ja
+
+    L = _lib.KEY_LIMIT_MIN_L
+    mask = torch.ones(2, 1, 1, L, dtype=torch.bool)
+    ja._classify_mask(mask, torch.zeros(2, 1, 4, 32), True)
+    _lib.key_limit_hint(mask, _lib.MASK_BOOL, 2, L)
+    mask.data[1, ..., 7:] = False  # a write that does not bump the version counter
+    assert _lib.key_limit_hint(mask, _lib.MASK_BOOL, 2, L).tolist() == [L, L]  # stale, as documented
+    _lib.forget_mask(mask)
+    assert not ja._already_verified(mask)
+    assert _lib.key_limit_hint(mask, _lib.MASK_BOOL, 2, L).tolist() == [L, 7]
