@@ -179,8 +179,22 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       Oacc[db][e] = 0.f;
       if constexpr (DUAL) Tacc[db][e] = 0.f;
     }
+    if constexpr (DUAL) {
+      pin_acc(Oacc[db]);
+      pin_acc(Tacc[db]);
+    }
   }
   float m_i = NEG_INF, l_i = 0.f, mu_i = 0.f;
+  // The tangent accumulators work with S' - c_i, c_i a per-row reference close to the row's mu:
+  // O' = (P (S' - mu)) V + P V' does not change when a row constant is taken off S', but the 16-bit
+  // operand P (S' - c) of the matrix product is rounded in proportion to |S' - c|, and where one key
+  // holds most of a row's weight that rounding error is the same multiple of V's row in every column
+  // of O', which the backward's row statistic rowsum(gT O') then adds up instead of averaging out.
+  // c_i follows the running mu: it is moved to it whenever a half tile brings over four times the weight of
+  // everything before it (so always on the first one, and whenever a key arrives that dominates its row),
+  // which for ordinary inputs happens on the first tile only; the accumulators are moved along
+  // (T -= shift O, mu_acc -= shift l).
+  float c_i = 0.f;
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
@@ -346,21 +360,10 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       for (int e = 1; e < 16; ++e) mx = fmaxf(mx, S[e]);
       mx = pair_max(mx) * sl2;
     }
-    if (__any(mx > m_i + RESCALE_TAU)) {
-      const float m_new = fmaxf(m_i, mx);
-      const float alpha = fast_exp2(m_i - ((m_new == NEG_INF) ? 0.f : m_new));
-      m_i = m_new;
-      l_i *= alpha;
-      if constexpr (DUAL) mu_i *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          Oacc[db][e] = acc_scale(Oacc[db][e], alpha);
-          if constexpr (DUAL) Tacc[db][e] = acc_scale(Tacc[db][e], alpha);
-        }
-      }
-    }
+    // lazy rescaling, decided per query row; the accumulators follow further down, in the one rare block
+    const bool up = mx > m_i + RESCALE_TAU;
+    const float alpha = up ? fast_exp2(m_i - mx) : 1.f;
+    m_i = up ? mx : m_i;
     // V fragments of the first PV steps travel while the softmax runs
     static_for<(PD < NPV ? PD : NPV)>([&](auto ic) { issue_v(ic); });
 
@@ -374,10 +377,37 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       for (int e = 0; e < 16; ++e) S[e] = fast_exp2(__builtin_fmaf(S[e], sl2, -m_use));
     }
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      rs += S[e];
+    for (int e = 0; e < 16; ++e) rs += S[e];
+    // rare: some row's reference point moved, or (dual) this half tile outweighs what came before it four times
+    const bool outweighs = DUAL && rs > 4.f * l_i * alpha;
+    if (__builtin_expect(__any(up || outweighs), 0)) {
+      float neg_shift = 0.f;
       if constexpr (DUAL) {
-        const float ps = S[e] * (Sp[e] * pr.scale);
+        // both lanes of a query column must decide alike
+        const bool move = rare_pair_max(outweighs ? 1.f : 0.f) > 0.f;
+        float rc = 0.f;  // rowsum of P (S' - c) over this half tile, old reference
+#pragma unroll
+        for (int e = 0; e < 16; ++e) rc += S[e] * __builtin_fmaf(Sp[e], pr.scale, -c_i);
+        const float tot_l = rare_pair_sum(__builtin_fmaf(l_i, alpha, rs)), tot_mu = rare_pair_sum(__builtin_fmaf(mu_i, alpha, rc));
+        const float shift = (move && tot_l > 0.f) ? tot_mu / tot_l : 0.f;
+        neg_shift = -shift;
+        c_i += shift;
+        mu_i = alpha * __builtin_fmaf(neg_shift, l_i, mu_i);
+      }
+      l_i *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          if constexpr (DUAL) acc_move_in_place(Tacc[db][e], Oacc[db][e], alpha, neg_shift);
+          else Oacc[db][e] = acc_scale(Oacc[db][e], alpha);
+        }
+      }
+    }
+    if constexpr (DUAL) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float ps = S[e] * __builtin_fmaf(Sp[e], pr.scale, -c_i);
         Sp[e] = ps;
         rmu += ps;
       }
@@ -392,6 +422,8 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       pf[c] = to_frag<T>(S, c);
       if constexpr (DUAL) psf[c] = to_frag<T>(Sp, c);
     }
+    // the conversions are done (and two issue slots have passed) before the first in-place product reads them
+    if constexpr (DUAL) asm volatile("s_nop 1" : "+v"(pf[0]), "+v"(pf[1]), "+v"(psf[0]), "+v"(psf[1]));
     static_for<NPV>([&](auto ic) {
       constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % RD;
       constexpr int younger = (NPV - 1 - i < PD - 1) ? NPV - 1 - i : PD - 1;
@@ -401,11 +433,14 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       load_step(std::integral_constant<int, HB * (KK + NPV) + KK + i>{});
       const u32x4 av = {va[sl][0][0], va[sl][0][1], va[sl][1][0], va[sl][1][1]};
       const Frag<T> a = __builtin_bit_cast(Frag<T>, av);
-      mma(Oacc[db], a, pf[c]);
       if constexpr (DUAL) {
-        mma(Tacc[db], a, psf[c]);
+        // in place (see mfma_acc), and no two consecutive products on the same tile
         const u32x4 bv = {vb[sl][0][0], vb[sl][0][1], vb[sl][1][0], vb[sl][1][1]};
-        mma(Tacc[db], __builtin_bit_cast(Frag<T>, bv), pf[c]);
+        mfma_acc(Tacc[db], a, psf[c]);
+        mfma_acc(Oacc[db], a, pf[c]);
+        mfma_acc(Tacc[db], __builtin_bit_cast(Frag<T>, bv), pf[c]);
+      } else {
+        mma(Oacc[db], a, pf[c]);
       }
     });
     JVPFA_STAMP(7);
@@ -468,11 +503,12 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   for (; t < ntiles; ++t) tile(t, std::true_type{});
 
   // ---- epilogue ---------------------------------------------------------------------------------
+  if constexpr (DUAL) asm volatile("s_nop 15\n\ts_nop 15");  // the last in-place accumulation has written its registers
   l_i += xor32(l_i);
   if constexpr (DUAL) mu_i += xor32(mu_i);
   const bool dead = !(l_i > 0.f);
   const float inv = dead ? 0.f : 1.f / l_i;
-  const float mu_n = mu_i * inv;
+  const float mu_n = mu_i * inv;  // rowsum(P (S' - c)) = mu - c
   if (qrow < L) {
     T *Og = reinterpret_cast<T *>(p.o) + head + (size_t)qrow * D;
     T *Otg = DUAL ? reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D : nullptr;
@@ -493,7 +529,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     }
     if (g == 0) {
       p.M[(size_t)zh * L + qrow] = dead ? __builtin_inff() : m_i + __builtin_amdgcn_logf(l_i);
-      if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = mu_n;
+      if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = dead ? 0.f : mu_n + c_i;
     }
   }
 }

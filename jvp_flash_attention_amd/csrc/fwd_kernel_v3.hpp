@@ -28,14 +28,6 @@ template <bool FIRST> __device__ __forceinline__ void mfma_s(f32x16 &c, const f1
   if constexpr (FIRST) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
   else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
 }
-__device__ __forceinline__ void mfma_acc(f32x16 &c, const bf16x8 &a, const bf16x8 &b) {
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void mfma_acc(f32x16 &c, const f16x8 &a, const f16x8 &b) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void pin_acc(f32x16 &c) { asm volatile("" : "+a"(c)); }
-
 __device__ __forceinline__ void anchor(float &x) { asm volatile("" : "+v"(x)); }
 __device__ __forceinline__ void anchor(bf16x8 &x) { asm volatile("" : "+v"(x)); }
 __device__ __forceinline__ void anchor(f16x8 &x) { asm volatile("" : "+v"(x)); }
@@ -148,6 +140,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     if constexpr (DUAL) pin_acc(Tacc[db]);
   }
   float m_i = NEG_INF, l_i = 0.f, mu_i = 0.f;
+  float c_i = 0.f;  // per-row reference taken off S' (see fwd_kernel_v2.hpp): follows the running mu
 
   const float sl2 = pr.scale * LOG2E;
   const bool neg_scale = !(sl2 > 0.f);
@@ -240,7 +233,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     // ---- softmax state and units ----------------------------------------------------------------
     float mxa = NEG_INF, mxb = NEG_INF, mx = NEG_INF, alpha = 1.f, m_use = 0.f, rs = 0.f, rmu = 0.f;
     float pv[16], sv[16];
-    bool any_up = false;
+    bool any_up = false, outweighs = false;
     auto unit = [&](auto uc) {
       constexpr int u = decltype(uc)::value;
       if constexpr (u == 0 || u == 1) {  // row maximum over registers 8u .. 8u+7
@@ -280,7 +273,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
         if constexpr ((u - 5) % 2 == 0) {
           if constexpr (GEN) pv[e] = fast_exp2(Sc[e] - m_use);
           else pv[e] = fast_exp2(__builtin_fmaf(Sc[e], sl2, -m_use));
-          if constexpr (DUAL) sv[e] = Spc[e] * pr.scale;
+          if constexpr (DUAL) sv[e] = __builtin_fmaf(Spc[e], pr.scale, -c_i);
           anchor(pv[e]);
         } else {
           rs += pv[e];
@@ -305,7 +298,12 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
         }
       } else {
         l_i = __builtin_fmaf(l_i, alpha, rs);
-        if constexpr (DUAL) mu_i = __builtin_fmaf(mu_i, alpha, rmu);
+        if constexpr (DUAL) {
+          mu_i = __builtin_fmaf(mu_i, alpha, rmu);
+          // this half tile holds over 4/5 of the row's weight so far: the reference of S' follows (rare)
+          outweighs = 1.25f * rs > l_i;
+          any_up = any_up || __any(outweighs);
+        }
       }
     };
     // (anchor(): an empty asm statement that consumes a value; it keeps the unit that produced the value
@@ -428,14 +426,36 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     });
     JVPFA_STAMP(6);
     if constexpr (SM) {
-      if (any_up) {  // rare: some row's reference point moved; the accumulators follow it
+      if (any_up) {  // rare: some row's reference point (of S or of S') moved; the accumulators follow it
         asm volatile("s_nop 15\n\ts_nop 15");  // the last accumulation above has written its registers
+        float neg_shift = 0.f;
+        if constexpr (DUAL) {
+          // l_i, mu_i already hold this half tile (with the old reference); both lanes of a query column
+          // must decide alike
+          const bool move = rare_pair_max(outweighs ? 1.f : 0.f) > 0.f;
+          const float tot_l = rare_pair_sum(l_i), tot_mu = rare_pair_sum(mu_i);
+          const float shift = (move && tot_l > 0.f) ? tot_mu / tot_l : 0.f;
+          neg_shift = -shift;
+          c_i += shift;
+          mu_i = __builtin_fmaf(neg_shift, l_i, mu_i);
+          // the operand P (S' - c) of this half tile again, with the new reference (the exponentials come
+          // out exactly as before: same instructions on the same registers)
+          float m_again = m_use;
+          anchor(m_again);  // a value of its own: otherwise every exponential above is kept alive for this path
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            float pe;
+            if constexpr (GEN) pe = fast_exp2(Sc[e] - m_again);
+            else pe = fast_exp2(__builtin_fmaf(Sc[e], sl2, -m_again));
+            psfn[e / 8][e % 8] = (T)(pe * __builtin_fmaf(Spc[e], pr.scale, -c_i));
+          }
+        }
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
-            Oacc[db][e] = acc_scale(Oacc[db][e], alpha);
-            if constexpr (DUAL) Tacc[db][e] = acc_scale(Tacc[db][e], alpha);
+            if constexpr (DUAL) acc_move_in_place(Tacc[db][e], Oacc[db][e], alpha, neg_shift);
+            else Oacc[db][e] = acc_scale(Oacc[db][e], alpha);
           }
         }
       }
@@ -520,7 +540,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     }
     if (g == 0) {
       p.M[(size_t)zh * L + qrow] = dead ? __builtin_inff() : m_i + __builtin_amdgcn_logf(l_i);
-      if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = mu_n;
+      if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = dead ? 0.f : mu_n + c_i;  // mu_n = rowsum(P (S' - c))
     }
   }
 #endif

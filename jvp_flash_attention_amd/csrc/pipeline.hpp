@@ -44,6 +44,43 @@ __device__ __forceinline__ float acc_scale(float x, float alpha) {
                : "v"(alpha));
   return x;
 }
+// pair_sum / pair_max (common.hpp) for use inside a rarely taken block of a hot loop.  The compiler treats
+// the cross-lane builtin as a convergent operation, restructures the branch around it and then copies every
+// accumulator on the path that skips the block; written as asm the exchange is an ordinary statement.
+__device__ __forceinline__ void rare_pair(float x, float &lo, float &hi) {
+  lo = x;
+  hi = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lo), "+v"(hi));
+}
+__device__ __forceinline__ float rare_pair_sum(float x) {
+  float lo, hi;
+  rare_pair(x, lo, hi);
+  return lo + hi;
+}
+__device__ __forceinline__ float rare_pair_max(float x) {
+  float lo, hi;
+  rare_pair(x, lo, hi);
+  return fmaxf(lo, hi);
+}
+
+// (t, o) <- (alpha * (t + neg_shift * o), alpha * o) for two values that live in accumulation registers, done
+// where they stand: the tangent accumulator is re-centred on a new reference for S' (see fwd_kernel_v2.hpp) and
+// both follow a new reference point of the exponentials.
+// The registers are named as inputs and written all the same.  That is sound only where nothing but in-place
+// statements (mfma_acc, this one) touches the tiles from their first product to the end of the tile loop, so
+// that the compiler never holds a value of theirs anywhere else.  (With the elements as in/out operands the
+// compiler gives the tiles a second home after the rarely taken block this is used in, and copies all of
+// them there on the path that skips the block, on every half tile.)
+__device__ __forceinline__ void acc_move_in_place(float t, float o, float alpha, float neg_shift) {
+  float a, b;
+  asm volatile(
+      "v_accvgpr_read_b32 %0, %2\n\tv_accvgpr_read_b32 %1, %3\n\tv_fma_f32 %0, %1, %5, %0\n\t"
+      "v_mul_f32 %1, %1, %4\n\tv_mul_f32 %0, %0, %4\n\ts_nop 1\n\t"
+      "v_accvgpr_write_b32 %3, %1\n\tv_accvgpr_write_b32 %2, %0\n\ts_nop 1"
+      : "=&v"(a), "=&v"(b)
+      : "a"(t), "a"(o), "v"(alpha), "v"(neg_shift)
+      : "memory");
+}
 // Products whose B operand stays resident in the accumulation register file for the whole kernel
 // while the result tile lives in ordinary vector registers: c = a*b (FIRST) or c += a*b.  The
 // result may only be read by other instruction kinds after tiles_ready().
@@ -83,6 +120,16 @@ template <bool FIRST> __device__ __forceinline__ void mma_vrv(f32x16 &c, const f
   if constexpr (FIRST) asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
   else asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
+// Accumulation in place: the tile is read and written in the same accumulation registers, so the
+// register allocator can never give it a second home (and copy it there on the common path).
+__device__ __forceinline__ void mfma_acc(f32x16 &c, const bf16x8 &a, const bf16x8 &b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_acc(f32x16 &c, const f16x8 &a, const f16x8 &b) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void pin_acc(f32x16 &c) { asm volatile("" : "+a"(c)); }
+
 // 16 + 4 idle issue slots: the last matrix-core pass has written its registers when this returns
 __device__ __forceinline__ void tiles_ready(f32x16 &a) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a)); }
 __device__ __forceinline__ void tiles_ready(f32x16 &a, f32x16 &b) {

@@ -448,7 +448,7 @@ def test_growing_row_maximum_exercises_the_rescale_path(dt, D, causal):
     for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
         got = t.double().cpu().numpy()
         rel = np.abs(got - rb[n]).max() / np.abs(rb[n]).max()
-        assert np.isfinite(got).all() and rel <= (5e-5 if dtype == torch.float32 else 3e-2), (n, rel)
+        assert np.isfinite(got).all() and rel <= (5e-5 if dtype == torch.float32 else 2e-2), (n, rel)
 
 
 @pytest.mark.parametrize("dt,D", [("bf16", 64), ("fp32", 64), ("bf16", 32), ("bf16", 128), ("bf16", 256)])
@@ -541,13 +541,9 @@ def _run_kv_shape_case(dt, D, shape, mode):
     H, Hk, Lq, Lk = shape
     Z, dtype = 2, DTYPES[dt]
     g = torch.Generator().manual_seed(sum(map(ord, dt + mode)) + D + sum(shape))
-    # tangents of std 0.5: with std 1, D = 32 and causal rows of a few keys, the cancellation in
-    # O' = T/l - mu O (the reference's formula too, its jvp_attention.py:1031-1033) on 16-bit rounded
-    # probabilities puts single seeds at 2.3e-2, just past the bar
-    q, go, gt = [torch.randn(Z, H, Lq, D, generator=g).to(dtype) for _ in range(3)]
-    qt = (0.5 * torch.randn(Z, H, Lq, D, generator=g)).to(dtype)
-    k, v = [torch.randn(Z, Hk, Lk, D, generator=g).to(dtype) for _ in range(2)]
-    kt, vt = [(0.5 * torch.randn(Z, Hk, Lk, D, generator=g)).to(dtype) for _ in range(2)]
+    # tangents ~ N(0,1), as large as the primals (what the benchmark configurations with causal masks use)
+    q, go, gt, qt = [torch.randn(Z, H, Lq, D, generator=g).to(dtype) for _ in range(4)]
+    k, v, kt, vt = [torch.randn(Z, Hk, Lk, D, generator=g).to(dtype) for _ in range(4)]
     mask, kind, causal = None, _lib.MASK_NONE, mode == "causal"
     if mode == "bool":
         mask, kind = torch.rand(Z, H, Lq, Lk, generator=g) > 0.5, _lib.MASK_BOOL

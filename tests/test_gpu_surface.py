@@ -371,6 +371,91 @@ def test_config3_causal_long_full_size_properties():
         torch.cuda.empty_cache()
 
 
+def test_headline_shape_non_causal_full_size_against_the_oracle():
+    """The benchmarked launch itself: bf16 B4 H16 L4096 D128, no mask, not causal (64 interior tiles per
+    query block).  Two (z, h) slabs of O, O' and of all six gradients against the oracle, tangents ~ N(0,1)."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    Z, H, L, D = 4, 16, 4096, 128
+    dt, scale = torch.bfloat16, D**-0.5
+    q, k, v, qt, kt, vt, go, gt = [_randn((Z, H, L, D), dt, 160 + i) for i in range(8)]
+    o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, 0, False, scale)
+    grads = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, 0, False, scale, want_tangent_grads=True)
+    for z, h in ((0, 0), (3, 13)):
+        print(f"case headline slab z{z} h{h}", flush=True)
+        f64 = [x[z, h:h + 1][None].double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+        ref = dense.forward(*f64[:6], scale=scale)
+        assert _rel(o[z, h], ref["O"][0, 0]) <= 2e-2 and _rel(ot[z, h], ref["Ot"][0, 0]) <= 2e-2
+        assert np.abs(M[z, h].double().cpu().numpy() - ref["M"][0, 0]).max() <= 2e-2
+        assert np.abs(mu[z, h].double().cpu().numpy() - ref["mu"][0, 0]).max() <= 2e-2
+        rb = dense.backward(*f64, scale=scale)
+        for n, g in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+            assert _rel(g[z, h], rb[n][0, 0]) <= 2e-2, n
+        del ref, rb
+
+
+@pytest.mark.parametrize("L", [1024, 4096, 16384, 32768])
+def test_config5_hvp_sweep_at_every_length(L):
+    """benchmark configuration 5: bf16 B1 H16 D128 causal, tangents ~ N(0,1), the gradient of sum(O' * gO')
+    with respect to q, k, v (no gO), at each length of the sweep.
+
+    * L <= 4096: one whole head of O, O', dq, dk, dv against the oracle.
+    * every L: the tail, where 32-bit offsets would wrap first.  Row i of O, O', dq depends on q[i], q'[i],
+      gO'[i] and the keys up to i only, so the last 64 queries of a head over all L keys are an exact
+      oracle problem of their own (a boolean mask states the causal limit of each row); dk, dv of the last
+      64 keys receive contributions from those 64 queries only, so the same problem gives them too.
+    * every L: causal rows never see later keys, so the first half equals a run on the truncated sequence,
+      bit for bit, forward and (with the incoming gradient of the second half set to zero) backward."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    Z, H, D = 1, 16, 128
+    dt, scale = torch.bfloat16, D**-0.5
+    q, k, v, qt, kt, vt, gt = [_randn((Z, H, L, D), dt, 170 + i) for i in range(7)]
+    print(f"case config5 L{L}", flush=True)
+    o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, 0, True, scale)
+    dq, dk, dv, *_ = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, None, gt, None, 0, True, scale)
+    assert all(torch.isfinite(t).all() for t in (o, ot, M, mu, dq, dk, dv))
+    np64 = lambda x: x.double().cpu().numpy()  # noqa: E731
+    if L <= 4096:
+        h = 11
+        f64 = [np64(x[:, h:h + 1]) for x in (q, k, v, qt, kt, vt)]
+        g64 = np64(gt[:, h:h + 1])
+        ref = dense.forward(*f64, causal=True, scale=scale)
+        assert _rel(o[0, h], ref["O"][0, 0]) <= 2e-2 and _rel(ot[0, h], ref["Ot"][0, 0]) <= 2e-2
+        rb = dense.backward(*f64, np.zeros_like(g64), g64, causal=True, scale=scale)
+        for n, g in zip(("dq", "dk", "dv"), (dq, dk, dv)):
+            assert _rel(g[0, h], rb[n][0, 0]) <= 2e-2, n
+        del ref, rb
+    # the tail: last T queries of two heads over all keys
+    T = 64
+    for h in (0, H - 1):
+        rows = slice(L - T, L)
+        f64 = [np64(q[:, h:h + 1, rows]), np64(k[:, h:h + 1]), np64(v[:, h:h + 1]),
+               np64(qt[:, h:h + 1, rows]), np64(kt[:, h:h + 1]), np64(vt[:, h:h + 1])]
+        g64 = np64(gt[:, h:h + 1, rows])
+        keep = (np.arange(L)[None, :] <= (L - T + np.arange(T))[:, None])[None, None]
+        ref = dense.forward(*f64, mask=keep, scale=scale)
+        assert _rel(o[0, h, rows], ref["O"][0, 0]) <= 2e-2 and _rel(ot[0, h, rows], ref["Ot"][0, 0]) <= 2e-2
+        assert np.abs(np64(M[0, h, rows]) - ref["M"][0, 0]).max() <= 2e-2
+        rb = dense.backward(*f64, np.zeros_like(g64), g64, mask=keep, scale=scale)
+        assert _rel(dq[0, h, rows], rb["dq"][0, 0]) <= 2e-2
+        assert _rel(dk[0, h, rows], rb["dk"][0, 0, rows]) <= 2e-2 and _rel(dv[0, h, rows], rb["dv"][0, 0, rows]) <= 2e-2
+    # the prefix
+    half = L // 2
+    cut = [x[:, :, :half].contiguous() for x in (q, k, v, qt, kt, vt)]
+    o2, ot2, M2, mu2 = be.fwd(*cut, None, 0, True, scale)
+    assert torch.equal(o[:, :, :half], o2) and torch.equal(ot[:, :, :half], ot2)
+    assert torch.equal(M[:, :, :half], M2) and torch.equal(mu[:, :, :half], mu2)
+    gt[:, :, half:] = 0
+    full = be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, None, gt, None, 0, True, scale)
+    part = be.bwd(*cut, o2, ot2, M2, mu2, None, gt[:, :, :half].contiguous(), None, 0, True, scale)
+    for n, a_, b_ in zip(("dq", "dk", "dv"), full[:3], part[:3]):
+        assert torch.equal(a_[:, :, :half], b_), n
+    assert full[1][:, :, half:].abs().max().item() == 0.0 and full[2][:, :, half:].abs().max().item() == 0.0
+
+
 def test_config4_mask_modes_fp32_full_size():
     """benchmark configuration 4: fp32 B4 H8 L1024 D64; (a) key padding [B,1,1,L], (b) additive bias [B,H,L,L]."""
     from jvp_flash_attention_amd import _lib
