@@ -166,25 +166,32 @@ __device__ __forceinline__ int list_take(int v) {
 }
 
 // chunk swizzles (row -> xor value applied to the 16-byte chunk index)
+//
+// The LDS has 64 banks of 4 bytes.  A ds_read_b128 is served 16 lanes at a time (16 x 16 bytes = all banks
+// once if the 16 lanes, which read 16 consecutive rows at one logical chunk, land in 16 different chunks of
+// a 256-byte line); a ds_read_b64_tr_b16 is served 32 lanes at a time: the lanes 16a + j of a half wave
+// read row 4hh + j/4, the 8-byte half (j/2)%2 of logical chunk 4db + 2a + j%2, so the four rows j/4 must
+// move the chunk index in bits that neither a nor j%2 occupies (bits 2 and up), or two lanes of the half
+// wave meet in a bank and the read takes twice as long (measured before: 2 conflict cycles per
+// transposing read, 33 % of the LDS cycles of the headline forward).
 // (CH = 4, rows of 64 bytes: four rows share a line of 256 bytes, which the transposing read of four
 // consecutive rows covers exactly, so only the row-wise read needs its chunks moved)
 template <int CH> __device__ __forceinline__ int swz_k(int row) {
   return CH == 16 ? (row & 15) : CH == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
-// (CH = 32, rows of 512 bytes: every row starts a 256-byte line, so the four consecutive rows of a
-// transposing read need their groups of four chunks moved apart)
+// Tiles read by the transposing read only.  (CH = 32, 16: every row starts a 256-byte line, rows 0..3 move
+// bits 2-3; CH = 8: two rows share a line and differ in the bank already, rows 2-3 move bit 2.)
 template <int CH> __device__ __forceinline__ int swz_v(int row) {
-  return CH == 32 ? ((row & 3) << 2) : CH == 16 ? ((row & 7) << 1) : CH == 8 ? (((row >> 1) & 3) << 1) : 0;
+  return (CH == 32 || CH == 16) ? ((row & 3) << 2) : CH == 8 ? (((row >> 1) & 1) << 2) : 0;
 }
 
-// Swizzle for tiles that are read both ways (ds_read_b128 along rows and the transposing
-// ds_read_b64_tr_b16 across rows): 16 consecutive rows get 16 different values for the former,
-// and 4 consecutive rows move an aligned chunk pair to 4 different pairs for the latter.
+// Swizzle for tiles that are read both ways: 16 consecutive rows (8 pairs for CH = 8) get different values
+// for the row-wise read, and the rows j/4 of a transposing read move bits 2 and up.
 template <int CH> __device__ __forceinline__ int swz_u(int row) {
-  if (CH == 16) return ((row & 7) << 1) | ((row >> 3) & 1);
+  if (CH == 16) return ((row & 3) << 2) | ((row >> 2) & 3);
   if (CH == 4) return (row >> 2) & 3;
   const int x = (row >> 1) & 7;
-  return ((x & 3) << 1) | ((x >> 2) & 1);
+  return ((x & 1) << 2) | (x >> 1);
 }
 
 }  // namespace jvpfa
