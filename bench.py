@@ -26,10 +26,11 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
 Z, H, L, D = 4, 16, 4096, 128
 
-# HBM bytes per forward launch measured with rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a plain
-# copy of known size gives) and WRITE_SIZE (x1.0): 403.0 MB read + 136.3 MB written; the figures
-# and commands are in profiles/fwd3_kernel_bf16_B4_H16_L4096_D128.md.
+# HBM bytes per forward launch.  A recorded constant, not measured in this run: rocprofv3 --pmc
+# FETCH_SIZE (x2.0, the factor a plain copy of known size gives) and WRITE_SIZE (x1.0) read 403.0 MB +
+# 136.3 MB; the counter runs and their commands are in profiles/fwd3_kernel_bf16_B4_H16_L4096_D128.md.
 MEASURED_FWD_TRAFFIC_BYTES = 539.3e6
+TRAFFIC_SOURCE = "recorded from the rocprofv3 --pmc runs in profiles/fwd3_kernel_bf16_B4_H16_L4096_D128.md, not measured in this run"
 
 
 def timed(fn, steps, warmup):
@@ -248,7 +249,7 @@ def main():
         "ms_per_step": ms_fwd,
         "higher_is_better": True,
         "scaling": "weak",
-        "vs_baseline": None,
+        "vs_baseline": None,  # the reference publishes no number for this shape or for any AMD GPU
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "bf16 B4 H16 L4096 D128 dual forward (O, O'), no mask, sm_scale=D^-0.5",
@@ -262,11 +263,18 @@ def main():
             "unit": "TFLOP/s",
             "frac": fwd_flops / (ms_fwd * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
             "traffic": MEASURED_FWD_TRAFFIC_BYTES,
+            "traffic_source": TRAFFIC_SOURCE,
             "kernel": "fwd3_kernel<bf16, D=128, dual>",
         },
     }
     if not args.fwd_only:
         ms_fc, _ = timed(lambda: fwd(True), args.steps, args.warmup)
+        o, ot, M, mu = fwd()
+        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, False, scale),
+                        max(1, args.steps // 2), 2)
+        ms_b6, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, False, scale,
+                                        want_tangent_grads=True), max(1, args.steps // 2), 2)
+        del o, ot, M, mu
         ms_fb, _ = timed(fwd_bwd, max(1, args.steps // 2), 2)
         ms_fbc, _ = timed(lambda: fwd_bwd(True), max(1, args.steps // 2), 2)
         tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12  # noqa: E731
@@ -277,6 +285,14 @@ def main():
                         "pct_mfma_peak": 100 * tf(fwd_flops + bwd_flops, ms_fb) / PEAK_BF16_TFLOPS},
             "fwd_bwd_causal": {"ms": ms_fbc, "tflops": tf((fwd_flops + bwd_flops) / 2, ms_fbc),
                                "pct_mfma_peak": 100 * tf((fwd_flops + bwd_flops) / 2, ms_fbc) / PEAK_BF16_TFLOPS},
+            # the backward alone: pre-pass + bwd2_dkdv (10 products executed) + bwd2_dq (8 executed), 12 counted
+            "roofline_backward": {"bound": "mfma", "achieved": tf(bwd_flops, ms_b), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                  "frac": tf(bwd_flops, ms_b) / PEAK_BF16_TFLOPS, "ms": ms_b,
+                                  "executed_tflops": tf(bwd_flops * 18 / 12, ms_b),
+                                  "kernels": "bwd_prepass + bwd2_dkdv + bwd2_dq <bf16, D=128, dual>"},
+            # all six gradients (dq, dk, dv and dq', dk', dv'): 15 products counted
+            "bwd_six_gradients": {"ms": ms_b6, "tflops": tf(bwd_flops * 15 / 12, ms_b6),
+                                  "pct_mfma_peak": 100 * tf(bwd_flops * 15 / 12, ms_b6) / PEAK_BF16_TFLOPS},
             "fwd_tflops_reference_flop_convention": tf(ref_conv_flops, ms_fwd),
             "peak_hbm_allocated_mb": torch.cuda.max_memory_allocated() / 2**20,
         }

@@ -57,9 +57,8 @@ template <int N> __device__ __forceinline__ void lds_wait4(u32x4 &a, u32x4 &b, u
 
 // Everything the two kernels share: tile geometry, direct loads spread over steps, fragment reads.
 // SLOTn are LDS tile slots inside a stage; a tile is BT rows, row-major, chunks swizzled by swz_u.
-#ifndef JVPFA_BWD_SPREAD
-#define JVPFA_BWD_SPREAD(n) (3 * (n) / 4)
-#endif
+// the loads of the next tile are spread over the first three quarters of a tile's steps
+constexpr int bwd_spread(int nstep) { return 3 * nstep / 4; }
 #define JVPFA_BWD2_COMMON(Cfg, STREAMED_ROWS, OWN_ROWS, OWN_HEADS)                                                                                      \
   constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT;                   \
   constexpr int KK = D / 16, DB = D / 32;                                                                           \
@@ -219,7 +218,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
     // spread over the first NSPREAD steps only: the last load then has time to land before the barrier
-    constexpr int NSPREAD = JVPFA_BWD_SPREAD(NSTEP);
+    constexpr int NSPREAD = bwd_spread(NSTEP);
     if constexpr (gi < NSPREAD) {
       constexpr int lo = (gi * NLOAD + NSPREAD - 1) / NSPREAD, hi = ((gi + 1) * NLOAD + NSPREAD - 1) / NSPREAD;
       static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
@@ -580,7 +579,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
     // spread over the first NSPREAD steps only: the last load then has time to land before the barrier
-    constexpr int NSPREAD = JVPFA_BWD_SPREAD(NSTEP);
+    constexpr int NSPREAD = bwd_spread(NSTEP);
     if constexpr (gi < NSPREAD) {
       constexpr int lo = (gi * NLOAD + NSPREAD - 1) / NSPREAD, hi = ((gi + 1) * NLOAD + NSPREAD - 1) / NSPREAD;
       static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });

@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   };
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
-    constexpr int NSPREAD = JVPFA_BWD_SPREAD(NSTEP);
+    constexpr int NSPREAD = bwd_spread(NSTEP);
     if constexpr (gi < NSPREAD) {
       constexpr int lo = (gi * NLOAD + NSPREAD - 1) / NSPREAD, hi = ((gi + 1) * NLOAD + NSPREAD - 1) / NSPREAD;
       static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
@@ -578,7 +578,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   };
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
-    constexpr int NSPREAD = JVPFA_BWD_SPREAD(NSTEP);
+    constexpr int NSPREAD = bwd_spread(NSTEP);
     if constexpr (gi < NSPREAD) {
       constexpr int lo = (gi * NLOAD + NSPREAD - 1) / NSPREAD, hi = ((gi + 1) * NLOAD + NSPREAD - 1) / NSPREAD;
       static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });

@@ -56,8 +56,8 @@ static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
   // Without tangents one workgroup holds all columns.  The dual forward runs that kernel first (O, M)
   // and then the tangent pass (O', mu) with the final M: seven products, where two workgroups with a
   // column half each would compute nine.
-  using Cfg = FwdWideCfg<T, D, D, false>;
-  auto kern = fwd_wide_kernel<T, D, D, false, MASK>;
+  using Cfg = FwdWideCfg<T, D, false>;
+  auto kern = fwd_wide_kernel<T, D, false, MASK>;
   int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
   if (rc != 0) return rc;
   const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
@@ -65,8 +65,8 @@ static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
   if (blocks > 0x7fffffffLL) return -2;
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
   if constexpr (DUAL) {
-    using CfgT = FwdWideCfg<T, D, D, true>;
-    auto kt = fwd_wide_kernel<T, D, D, true, MASK, true>;
+    using CfgT = FwdWideCfg<T, D, true>;
+    auto kt = fwd_wide_kernel<T, D, true, MASK, true>;
     rc = allow_lds(reinterpret_cast<const void *>(kt), CfgT::LDS_BYTES);
     if (rc != 0) return rc;
     hipLaunchKernelGGL(kt, dim3((unsigned)blocks), dim3(CfgT::NT), CfgT::LDS_BYTES, stream, p);

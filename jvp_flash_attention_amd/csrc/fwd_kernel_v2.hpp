@@ -19,21 +19,7 @@
 #include "params.hpp"
 #include "pipeline.hpp"
 
-#ifndef JVPFA_RING
-#define JVPFA_RING 5
-#endif
-
 namespace jvpfa {
-
-#ifdef JVPFA_TRACE
-__device__ long long *g_trace = nullptr;  // debugging aid: time stamps of one wave
-#define JVPFA_STAMP(slot)                                                        \
-  do {                                                                           \
-    if (g_trace && blockIdx.x == 0 && threadIdx.x == 0 && trace_n < 4096) g_trace[trace_n++] = ((long long)(slot) << 48) | (clock64() & 0xffffffffffffLL); \
-  } while (0)
-#else
-#define JVPFA_STAMP(slot) do {} while (0)
-#endif
 
 template <typename T, int D, bool DUAL> struct Fwd2Cfg {
   static constexpr int NW = 4;
@@ -56,8 +42,6 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   constexpr int NB = BN / 32, KK = D / 16, DB = D / 32;
   constexpr float NEG_INF = -__builtin_inff();
 
-  int trace_n = 0;
-  (void)trace_n;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   // stage s: [K | V | K' | V'] each TILEB bytes
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem_raw;
@@ -280,7 +264,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     constexpr int NRV = DUAL ? 4 : 2;   // LDS reads per PV step
     constexpr int NPV = 2 * DB;         // PV steps: (16-key chunk c, d-block db)
 
-    constexpr int RD = MASK != MASK_NONE ? 4 : JVPFA_RING;  // fragment ring slots (reads run RD-1 steps ahead); the masked kernels need the registers
+    constexpr int RD = MASK != MASK_NONE ? 4 : 5;  // fragment ring slots (reads run RD-1 steps ahead); the masked kernels need the registers
     constexpr int PD = RD - 1;
     u32x4 ka[RD], kb[RD];
     auto issue_k = [&](auto kkc) {
@@ -326,7 +310,6 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     });
     if constexpr (DUAL) tiles_ready(S, Sp);
     else tiles_ready(S);
-    JVPFA_STAMP(5);
     float mx;
     constexpr bool general = MASK != MASK_NONE || EDGE;
     if constexpr (general) {
@@ -414,8 +397,6 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     }
     l_i += rs;
     if constexpr (DUAL) mu_i += rmu;
-
-    JVPFA_STAMP(6);
     Frag<T> pf[2], psf[2];
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
@@ -443,7 +424,6 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
         mma(Oacc[db], a, pf[c]);
       }
     });
-    JVPFA_STAMP(7);
   };
 
   // Mask values travel from HBM or the far caches, further than one phase of matrix products hides:
@@ -468,11 +448,8 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   auto tile = [&](int t, auto EDGEc) {
     const int j0 = tcur * BN;
     const int stage = t & 1;
-    JVPFA_STAMP(1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile t has landed
-    JVPFA_STAMP(2);
     __syncthreads();                      // ... everyone's has, and stage^1 is no longer being read
-    JVPFA_STAMP(3);
     int tnext2 = min(t + 2, ntiles - 1), tahead = 0;
     if constexpr (MASK != MASK_NONE) {
       tahead = list_request(list_slot(tnext2));

@@ -49,8 +49,6 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   constexpr int NSS = KK;  // super-steps of a slot: one contraction step of the scores + one (chunk, d-block) of PV
   static_assert(2 * DB == KK, "a slot pairs score step kk with accumulation step kk");
   constexpr float NEG_INF = -__builtin_inff();
-  int trace_n = 0;
-  (void)trace_n;
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   // stage s: [K | V | K' | V'] each TILEB bytes; the K-type and V-type halves hold different tiles
@@ -203,10 +201,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   constexpr int NRS = DUAL ? 2 : 1, NRV = DUAL ? 4 : 2;  // LDS reads per super-step
   constexpr int NU = 38;                                 // vector units of one softmax
   constexpr int NU0 = 5;                                 // ... of which this many form its front
-#ifndef JVPFA_F3_RD
-#define JVPFA_F3_RD 4
-#endif
-  constexpr int RD = JVPFA_F3_RD, PD = RD - 1;           // fragment ring slots; reads run PD super-steps ahead
+  constexpr int RD = 4, PD = RD - 1;           // fragment ring slots; reads run PD super-steps ahead
 
   // One slot.  QK: scores of a half tile (K rows at LDS address kaddr) into Sn, Spn.  PV: accumulate
   // the half tile whose V rows are at vaddr, with fragments pfp, psfp.  SM: softmax of Sc, Spc (first
@@ -347,7 +342,6 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
       if constexpr (DUAL) tiles_ready(Sc, Spc);
       else tiles_ready(Sc);
     }
-    JVPFA_STAMP(4);
     if constexpr (!PRE) static_for<(PD < NSS ? PD : NSS)>([&](auto ic) { issue(ic); });
     // the front of the softmax (row maximum, reference point) runs while the first fragments travel
     if constexpr (SM) static_for<NU0>([&](auto uc) { unit(uc); });
@@ -364,7 +358,6 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
         if constexpr (DUAL) lds_wait<younger>(va[sl][0], va[sl][1], vb[sl][0], vb[sl][1]);
         else lds_wait<younger>(va[sl][0], va[sl][1]);
       }
-      if constexpr (i == 0) JVPFA_STAMP(5);
       if constexpr (i + PD < NSS || NEXT) issue(std::integral_constant<int, i + PD>{});
       if constexpr (LB >= 0) load_step(std::integral_constant<int, (LB >= 0 ? LB : 0) + i>{});
       constexpr int c = i / DB, db = i % DB;
@@ -424,7 +417,6 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
         }
       }
     });
-    JVPFA_STAMP(6);
     if constexpr (SM) {
       if (any_up) {  // rare: some row's reference point (of S or of S') moved; the accumulators follow it
         asm volatile("s_nop 15\n\ts_nop 15");  // the last accumulation above has written its registers
@@ -488,11 +480,8 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   t_gen = neg_scale ? 1 : max(1, t_gen);
   int t = 1;
   for (; t < min(t_gen, ntiles); ++t) {
-    JVPFA_STAMP(1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of K(t), V(t-1) has landed
-    JVPFA_STAMP(2);
     __syncthreads();                      // ... everyone's has, and K(t-1), V(t-2) are no longer read
-    JVPFA_STAMP(3);
     prepare_loads(t);
     slot(B1{}, B1{}, B1{}, B0{}, std::integral_constant<int, 0>{}, B0{}, XP{}, kad(t, 0), kad(t - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB, 0);
     slot(B1{}, B1{}, B1{}, B0{}, std::integral_constant<int, NSS>{}, XP{}, B0{}, kad(t, 1), kad(t - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0);

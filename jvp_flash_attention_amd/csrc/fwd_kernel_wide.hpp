@@ -7,11 +7,6 @@
 // the final M of the first, so that p = exp2(s - M) needs no running maximum, and writes
 // O' = T - mu O and mu.  S is formed twice (seven matrix products instead of six).
 //
-// (The template can also split the output columns over workgroups, DV < D: each then forms the
-// scores over all of D and multiplies with a DV-column slice of V, V'.  Two halves compute nine
-// products for the dual forward and measured 11 % slower than the two passes; the launcher does not
-// use it.)
-//
 // Memory side as in fwd_kernel_v2.hpp: direct-to-LDS loads, double buffered, one barrier per tile,
 // XOR-swizzled 16-byte chunks, ds_read_b128 for K / K' fragments and the transposing
 // ds_read_b64_tr_b16 for V / V'.  A tile is 32 keys (rows are 512 bytes; two stages of 64-key tiles
@@ -26,13 +21,13 @@
 
 namespace jvpfa {
 
-template <typename T, int D, int DV, bool DUAL> struct FwdWideCfg {
-  static_assert(sizeof(T) == 2 && D % DV == 0 && DV % 32 == 0);
+template <typename T, int D, bool DUAL> struct FwdWideCfg {
+  static_assert(sizeof(T) == 2 && D % 32 == 0);
+  static constexpr int DV = D;                         // columns of V, V' (all of them)
   static constexpr int NW = 4;
   static constexpr int NT = NW * WAVE;
   static constexpr int BM = NW * 32;
   static constexpr int BN = 32;
-  static constexpr int NS = D / DV;                    // workgroups per query block
   static constexpr int NK = DUAL ? 2 : 1;              // K (, K') and V (, V')
   static constexpr int ROWBK = D * sizeof(T);          // bytes per K-type row (LDS and global)
   static constexpr int ROWBV = DV * sizeof(T);         // bytes per V-type row in LDS (global rows: ROWBK)
@@ -43,16 +38,17 @@ template <typename T, int D, int DV, bool DUAL> struct FwdWideCfg {
   static constexpr size_t LDS_BYTES = 2 * (size_t)STAGEB;
   static constexpr int IPWK = TILEBK / 1024 / NW;      // direct-load instructions per wave per tile
   static constexpr int IPWV = TILEBV / 1024 / NW;
-  static_assert(IPWK >= 1 && IPWV >= 1 && CHK == 32 && (CHV == 16 || CHV == 32));
+  static_assert(IPWK >= 1 && IPWV >= 1 && CHK == 32 && CHV == 32);
 };
 
-// TPASS (with DUAL and DV = D): the second pass of the dual forward, see above.
-template <typename T, int D, int DV, bool DUAL, int MASK, bool TPASS = false>
+// TPASS (with DUAL): the second pass of the dual forward, see above.
+template <typename T, int D, bool DUAL, int MASK, bool TPASS = false>
 __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
-  static_assert(!TPASS || (DUAL && DV == D));
-  using Cfg = FwdWideCfg<T, D, DV, DUAL>;
+  static_assert(!TPASS || DUAL);
+  using Cfg = FwdWideCfg<T, D, DUAL>;
+  constexpr int DV = Cfg::DV;
   constexpr bool GD = TPASS;  // the accumulation file is full: see mma_vra
-  constexpr int BN = Cfg::BN, NS = Cfg::NS, NK = Cfg::NK;
+  constexpr int BN = Cfg::BN, NK = Cfg::NK;
   constexpr int ROWBK = Cfg::ROWBK, ROWBV = Cfg::ROWBV, TILEBK = Cfg::TILEBK, TILEBV = Cfg::TILEBV;
   constexpr int IPWK = Cfg::IPWK, IPWV = Cfg::IPWV, VBASE = Cfg::VBASE;
   constexpr int KK = D / 16, DB = DV / 32;
@@ -64,12 +60,10 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
   const Problem &pr = p.pr;
   const int L = pr.L;
   const int nqb = (L + Cfg::BM - 1) / Cfg::BM;
-  // the workgroups of one query block follow each other, so they share K, K' in the same L2
-  const int id = xcd_remap(blockIdx.x, nqb * NS, pr.Z * pr.H);
-  const int zh = id / (nqb * NS);
-  const int rem = id % (nqb * NS);
-  const int slice = rem % NS;
-  const int qb = pr.causal ? nqb - 1 - rem / NS : rem / NS;
+  const int id = xcd_remap(blockIdx.x, nqb, pr.Z * pr.H);
+  const int zh = id / nqb;
+  const int rem = id % nqb;
+  const int qb = pr.causal ? nqb - 1 - rem : rem;
   const int z = zh / pr.H, h = zh % pr.H;
 
   const int tid = threadIdx.x;
@@ -82,10 +76,10 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
   const size_t kvhead = ((size_t)z * pr.Hk + h / (pr.H / pr.Hk)) * Lk * D;
   const T *Qg = reinterpret_cast<const T *>(p.q) + head;
   const T *Kg = reinterpret_cast<const T *>(p.k) + kvhead;
-  const T *Vg = reinterpret_cast<const T *>(p.v) + kvhead + slice * DV;
+  const T *Vg = reinterpret_cast<const T *>(p.v) + kvhead;
   const T *Qtg = DUAL ? reinterpret_cast<const T *>(p.qt) + head : nullptr;
   const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + kvhead : nullptr;
-  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + kvhead + slice * DV : nullptr;
+  const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + kvhead : nullptr;
 
   const int q0 = qb * Cfg::BM;
   const int qrow = q0 + wave * 32 + r;
@@ -116,7 +110,7 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
   for (int kk = 0; kk < KK; ++kk) koff[kk] = pr32 * ROWBK + (((2 * kk + g) ^ (pr32 & 15)) * 16);
   // V-type (transposing read): lane = 32g + 16a + j addresses key row 8g + 4hh + j/4 (+16c) and the
   // 8-byte half (j>>1)&1 of logical chunk 4db + 2a + (j&1); it receives keys 16c+8g+4hh+(0..3) at
-  // column 32db + perm32(16a + j) of the slice.
+  // column 32db + perm32(16a + j).
   uint32_t voff[DB][2];
   {
     const int a = (lane >> 4) & 1, j = lane & 15;
@@ -446,8 +440,8 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
     const float inv = dead ? 0.f : 1.f / l_i;
     const float mu_n = mu_i * inv;
     if (qrow < L) {
-      T *Og = reinterpret_cast<T *>(p.o) + head + (size_t)qrow * D + slice * DV;
-      T *Otg = DUAL ? reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D + slice * DV : nullptr;
+      T *Og = reinterpret_cast<T *>(p.o) + head + (size_t)qrow * D;
+      T *Otg = DUAL ? reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D : nullptr;
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
 #pragma unroll
@@ -463,7 +457,7 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
           if constexpr (DUAL) store8<T>(Otg + d0, t8);
         }
       }
-      if (g == 0 && slice == 0) {  // every slice holds the same row statistics
+      if (g == 0) {
         p.M[(size_t)zh * L + qrow] = dead ? __builtin_inff() : m_i + __builtin_amdgcn_logf(l_i);
         if constexpr (DUAL) p.mu[(size_t)zh * L + qrow] = mu_n;
       }

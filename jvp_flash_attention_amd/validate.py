@@ -1,7 +1,7 @@
 """Accuracy and speed report for JVP attention on the current GPU.
 
     python -m jvp_flash_attention_amd.validate --dtype bfloat16 [--seq-lengths 32 64 ... 2048]
-                                               [--no-masks] [--json out.json]
+                                               [--no-masks] [--no-timing] [--json out.json]
 
 Counterpart of the reference's script ``tests/test_jvp_attention.py`` (run as a program there,
 README.md:111-113): for every sequence length, mask type (none / boolean / additive) and causal
@@ -10,6 +10,9 @@ with PyTorch's math SDPA under forward-mode AD (what the reference's own tests c
 primal, tangent, the loss ``mean((out - target)^2)`` and its q/k/v gradients; (2) times the dual
 forward the way the reference does (10 warm-up + 100 calls, input clones and ``make_dual``
 included, lines 129-143 and 770-780) next to math SDPA; (3) records the peak memory of one call.
+After the per-case lines it prints the reference's two tables (summary per case and method, lines 883-937;
+time by mask type, lines 940-976) and its speed-up statistics, and writes them with the rows into the JSON
+file (lines 1172-1227); the reference's PNG plots (lines 977-1091) are not drawn.
 Shapes default to the reference's (batch 2, 12 heads, head dim 64, lines 225-230); masks are its
 random masks with keep-probability 0.1 (lines 334-394).  TFLOP/s uses the reference's FLOP
 convention ``2 * (4 B H L^2 D + 5 B H L^2)``, halved when causal (lines 49-83).
@@ -125,8 +128,12 @@ def run(args):
                 def ours_kernel_only():
                     return JVPAttn.forward(q, k, v, qt, kt, vt, mask, 0.0, causal, None, True, True, False)
 
-                ms, ms_k = timed(ours), timed(ours_kernel_only)
-                ms_sdpa = timed(lambda: sdpa_dual(q, k, v, qt, kt, vt, mask, causal), 2, 10)
+                if args.no_timing:  # one call each: the accuracy half of the report only
+                    ms, ms_k = timed(ours, 0, 1), timed(ours_kernel_only, 0, 1)
+                    ms_sdpa = timed(lambda: sdpa_dual(q, k, v, qt, kt, vt, mask, causal), 0, 1)
+                else:
+                    ms, ms_k = timed(ours), timed(ours_kernel_only)
+                    ms_sdpa = timed(lambda: sdpa_dual(q, k, v, qt, kt, vt, mask, causal), 2, 10)
                 fl = 2 * flop_count(B, H, L, D, causal) / 2  # the convention already counts the JVP (x2 inside)
                 row = {"L": L, "mask": kind, "causal": causal, "ok": ok, **acc, "ms": ms, "ms_kernel_only": ms_k,
                        "ms_sdpa_math": ms_sdpa, "speedup": ms_sdpa / ms, "tflops": fl / (ms * 1e-3) / 1e12,
@@ -138,11 +145,54 @@ def run(args):
                       f"{ms:7.3f} ms ({ms_k:7.3f} kernel only) sdpa {ms_sdpa:8.3f} ms x{ms_sdpa / ms:5.1f} | "
                       f"{row['tflops']:6.1f} TFLOP/s | {row['mem_mb']:7.1f} MB vs {row['mem_mb_sdpa']:8.1f} MB", flush=True)
     n_ok = sum(r["ok"] for r in rows)
-    print(f"\naccuracy: {n_ok}/{len(rows)} passed; mean speed-up over math SDPA {sum(r['speedup'] for r in rows) / len(rows):.2f}x")
+    stats = summary_statistics(rows)
+    print(summary_table(rows))
+    print(mask_comparison_table(rows))
+    print(f"\naccuracy: {n_ok}/{len(rows)} passed; speed-up over math SDPA: mean {stats['speedup_mean']:.2f}x, "
+          f"min {stats['speedup_min']:.2f}x, max {stats['speedup_max']:.2f}x")
     if args.json:
         with open(args.json, "w") as f:
-            json.dump({"dtype": args.dtype, "bsz": B, "heads": H, "head_dim": D, "rows": rows}, f, indent=1)
+            json.dump({"dtype": args.dtype, "bsz": B, "heads": H, "head_dim": D, "tolerance": TOLERANCE[args.dtype],
+                       "passed": n_ok, "cases": len(rows), **stats, "rows": rows}, f, indent=1)
     return rows
+
+
+def summary_table(rows) -> str:
+    """The reference's summary table (its test file, lines 883-937): one line per case and method."""
+    out = ["", "=" * 110, "BENCHMARK SUMMARY", "=" * 110,
+           f"{'Seq Len':<10} {'Causal':<8} {'Mask':<10} {'Method':<10} {'Time (ms)':<12} {'Mem (MB)':<12} {'TFLOP/s':<12} "
+           f"{'Max Error':<12} {'Grad Check':<10}", "-" * 110]
+    for r in sorted(rows, key=lambda r: (r["L"], r["causal"], r["mask"])):
+        fl = r["tflops"] * r["ms"]  # TFLOP/s x ms: the case's FLOP count in units of 1e9
+        out.append(f"{r['L']:<10} {str(r['causal']):<8} {r['mask']:<10} {'sdpa':<10} {r['ms_sdpa_math']:<12.3f} "
+                   f"{r['mem_mb_sdpa']:<12.2f} {fl / r['ms_sdpa_math']:<12.2f} {'baseline':<12} {'N/A':<10}")
+        worst = max(r["primal"], r["tangent"])
+        out.append(f"{r['L']:<10} {str(r['causal']):<8} {r['mask']:<10} {'jvp_attn':<10} {r['ms']:<12.3f} "
+                   f"{r['mem_mb']:<12.2f} {r['tflops']:<12.2f} {worst:<12.2e} {'ok' if r['ok'] else 'FAIL':<10}")
+        out.append("")
+    return "\n".join(out)
+
+
+def mask_comparison_table(rows) -> str:
+    """The reference's mask-type table (lines 940-976): time by mask type, relative to no mask."""
+    out = ["", "=" * 80, "MASK TYPE PERFORMANCE COMPARISON", "=" * 80,
+           f"{'Seq Len':<10} {'Causal':<8} {'Method':<10} {'No Mask':<15} {'Boolean Mask':<15} {'Additive Mask':<15}", "-" * 80]
+    by = {}
+    for r in rows:
+        by.setdefault((r["L"], r["causal"]), {})[r["mask"]] = r["ms"]
+    for (L, causal), t in sorted(by.items()):
+        cell = lambda k: "N/A" if k not in t else (f"{t[k]:.2f} ms" + (f" ({t[k] / t['none']:.2f}x)" if k != "none" and "none" in t else ""))  # noqa: E731
+        out.append(f"{L:<10} {str(causal):<8} {'jvp_attn':<10} {cell('none'):<15} {cell('boolean'):<15} {cell('additive'):<15}")
+    return "\n".join(out)
+
+
+def summary_statistics(rows) -> dict:
+    """Speed-up over math SDPA (mean / min / max) and the worst errors, as the reference's closing statistics."""
+    sp = [r["speedup"] for r in rows] or [float("nan")]
+    return {"speedup_mean": sum(sp) / len(sp), "speedup_min": min(sp), "speedup_max": max(sp),
+            "max_primal_error": max((r["primal"] for r in rows), default=0.0),
+            "max_tangent_error": max((r["tangent"] for r in rows), default=0.0),
+            "max_grad_error": max((max(r["dq"], r["dk"], r["dv"]) for r in rows), default=0.0)}
 
 
 def main():
@@ -153,6 +203,7 @@ def main():
     ap.add_argument("--head-dim", type=int, default=64)
     ap.add_argument("--seq-lengths", type=int, nargs="+", default=[32, 64, 128, 256, 512, 1024, 2048])
     ap.add_argument("--no-masks", action="store_true")
+    ap.add_argument("--no-timing", action="store_true", help="one call per case instead of 10 + 100: accuracy only")
     ap.add_argument("--json", default=None)
     run(ap.parse_args())
 

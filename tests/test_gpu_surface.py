@@ -508,3 +508,26 @@ def test_config5_hvp_memory_is_linear_in_sequence_length():
 
     p1, p2 = peak(4096), peak(16384)
     assert p2 <= 4.5 * p1, (p1, p2)  # 4x the length: ~4x the memory (16x if anything were O(L^2))
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float16", "float32"])
+def test_validation_report_passes_every_case(dtype, tmp_path, capsys):
+    """``python -m jvp_flash_attention_amd.validate`` (the counterpart of the reference's test script): every case of
+    sequence length x mask type x causal flag within the reference's own tolerances against math SDPA, in the
+    three-way comparison (SDPA / fwAD / torch.func.jvp), with its tables and its JSON file written."""
+    import argparse
+    import json
+
+    from jvp_flash_attention_amd import validate
+
+    out = tmp_path / "report.json"
+    args = argparse.Namespace(dtype=dtype, bsz=2, model_dim=768, head_dim=64, seq_lengths=[32, 128, 512], no_masks=False,
+                              no_timing=True, json=str(out))
+    rows = validate.run(args)
+    assert len(rows) == 12  # 3 lengths x (no mask, causal, boolean mask, additive mask)
+    assert all(r["ok"] for r in rows), [(r["L"], r["mask"], r["causal"]) for r in rows if not r["ok"]]
+    text = capsys.readouterr().out
+    assert "BENCHMARK SUMMARY" in text and "MASK TYPE PERFORMANCE COMPARISON" in text and "accuracy: 12/12 passed" in text
+    rep = json.loads(out.read_text())
+    assert rep["passed"] == rep["cases"] == 12 and rep["dtype"] == dtype and len(rep["rows"]) == 12
+    assert rep["max_tangent_error"] < validate.TOLERANCE[dtype]
