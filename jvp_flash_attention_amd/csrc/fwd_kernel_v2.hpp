@@ -343,10 +343,14 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
       for (int e = 1; e < 16; ++e) mx = fmaxf(mx, S[e]);
       mx = pair_max(mx) * sl2;
     }
-    // lazy rescaling, decided per query row; the accumulators follow further down, in the one rare block
+    // lazy rescaling, decided per query row (rare); the accumulators follow further down, in the block
+    // that also re-centres them
     const bool up = mx > m_i + RESCALE_TAU;
-    const float alpha = up ? fast_exp2(m_i - mx) : 1.f;
-    m_i = up ? mx : m_i;
+    float alpha = 1.f;
+    if (__builtin_expect(__any(up), 0)) {
+      alpha = up ? fast_exp2(m_i - mx) : 1.f;
+      m_i = up ? mx : m_i;
+    }
     // V fragments of the first PV steps travel while the softmax runs
     static_for<(PD < NPV ? PD : NPV)>([&](auto ic) { issue_v(ic); });
 
@@ -362,10 +366,10 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) rs += S[e];
     // rare: some row's reference point moved, or (dual) this half tile outweighs what came before it four times
-    const bool outweighs = DUAL && rs > 4.f * l_i * alpha;
-    if (__builtin_expect(__any(up || outweighs), 0)) {
+    if (__builtin_expect(__any(up || (DUAL && rs > 4.f * l_i)), 0)) {
       float neg_shift = 0.f;
       if constexpr (DUAL) {
+        const bool outweighs = rs > 4.f * l_i * alpha;
         // both lanes of a query column must decide alike
         const bool move = rare_pair_max(outweighs ? 1.f : 0.f) > 0.f;
         float rc = 0.f;  // rowsum of P (S' - c) over this half tile, old reference

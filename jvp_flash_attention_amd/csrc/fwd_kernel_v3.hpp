@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     // ---- softmax state and units ----------------------------------------------------------------
     float mxa = NEG_INF, mxb = NEG_INF, mx = NEG_INF, alpha = 1.f, m_use = 0.f, rs = 0.f, rmu = 0.f;
     float pv[16], sv[16];
-    bool any_up = false, outweighs = false;
+    bool any_up = false, outweighs = false, up_l = false;
     auto unit = [&](auto uc) {
       constexpr int u = decltype(uc)::value;
       if constexpr (u == 0 || u == 1) {  // row maximum over registers 8u .. 8u+7
@@ -257,7 +257,8 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
         // lazy rescale, decided per query row: the reference point only moves when the row maximum
         // exceeds it by more than RESCALE_TAU (log2 units)
         const bool up = mx > m_i + RESCALE_TAU;
-        any_up = __any(up);
+        up_l = up;
+        if constexpr (!DUAL) any_up = __any(up);
         alpha = up ? fast_exp2(m_i - mx) : 1.f;
         m_i = up ? mx : m_i;
         anchor(alpha);
@@ -297,7 +298,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
           mu_i = __builtin_fmaf(mu_i, alpha, rmu);
           // this half tile holds over 4/5 of the row's weight so far: the reference of S' follows (rare)
           outweighs = 1.25f * rs > l_i;
-          any_up = any_up || __any(outweighs);
+          any_up = __any(up_l | outweighs);  // one test for both rare events (no branch inside the slot)
         }
       }
     };
