@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define JVPFA_ABI_VERSION 5
+#define JVPFA_ABI_VERSION 6
 
 enum jvpfa_dtype { JVPFA_BF16 = 0, JVPFA_FP16 = 1, JVPFA_FP32 = 2 };
 
@@ -92,9 +92,21 @@ typedef struct jvpfa_fwd_args {
    * (JA:2367-2378).  key_limit then counts the Lk keys; the tile lists are used when Lk equals p.L
    * (any Hk: they belong to the mask planes, which follow the query heads) and ignored otherwise. */
   int32_t Lk, Hk;
+  /* optional workspace for small grids, or NULL: jvpfa_fwd_split_workspace_bytes(&p, Lk) bytes of device memory,
+   * 16-byte aligned, contents don't-care.  When a launch would have fewer workgroups than the GPU has compute
+   * units (one long sequence, few heads), the key tiles of every query block are then split over up to 8
+   * workgroups that leave fp32 partial results there, and a second kernel merges them into o, ot, M, mu
+   * (bf16 / fp16, D = 128, no mask; ignored otherwise).  Results agree with the unsplit launch to rounding.
+   * No counterpart in the reference (one program per 32 query rows whatever the grid, JA:2474-2476). */
+  void *split_workspace;
+  uint64_t split_workspace_bytes;
 } jvpfa_fwd_args;
 
 int jvpfa_fwd(const jvpfa_fwd_args *args, void *hip_stream);
+
+/* Bytes of split_workspace with which jvpfa_fwd would split this problem on the current device; 0 if it would
+ * not (grid large enough, or a kernel that does not split). */
+size_t jvpfa_fwd_split_workspace_bytes(const jvpfa_problem *p, int32_t Lk);
 
 /*
  * Backward of  Loss = <go, o> + <gt, ot>.  Replaces the device work of

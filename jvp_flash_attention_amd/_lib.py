@@ -15,10 +15,10 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libjvpfa.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
-EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_bwd_workspace_bytes", "jvpfa_bwd_static", "jvpfa_bwd_static_max_rows", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
+EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_fwd_split_workspace_bytes", "jvpfa_bwd_workspace_bytes", "jvpfa_bwd_static", "jvpfa_bwd_static_max_rows", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
            "jvpfa_abi_version", "jvpfa_error_string")
 
 
@@ -43,6 +43,7 @@ class FwdArgs(C.Structure):
         ("key_limit", C.c_void_p),
         ("tiles_q", C.c_void_p),
         ("Lk", C.c_int32), ("Hk", C.c_int32),
+        ("split_workspace", C.c_void_p), ("split_workspace_bytes", C.c_uint64),
     ]
 
 
@@ -87,6 +88,8 @@ def load() -> C.CDLL:
         lib.jvpfa_bwd_static.restype = C.c_int
         lib.jvpfa_bwd_static_max_rows.argtypes = []
         lib.jvpfa_bwd_static_max_rows.restype = C.c_size_t
+        lib.jvpfa_fwd_split_workspace_bytes.argtypes = [C.POINTER(Problem), C.c_int32]
+        lib.jvpfa_fwd_split_workspace_bytes.restype = C.c_size_t
         lib.jvpfa_mask_tiles_bytes.argtypes = [C.POINTER(Problem)]
         lib.jvpfa_mask_tiles_bytes.restype = C.c_size_t
         lib.jvpfa_mask_tiles.argtypes = [C.POINTER(Problem), C.c_void_p, C.c_void_p, C.c_void_p]
@@ -178,6 +181,17 @@ def key_limit_hint(mask, mask_kind, Z, L):
                 pass
     # the kernels index the limits by batch entry: a mask shared by the batch ([1,1,1,L]) is spread over Z
     return lim if lim.shape[0] == Z else lim.expand(Z).contiguous()
+
+
+_split_enabled = True
+
+
+def set_split(enabled: bool) -> None:
+    """Switch the split of small launches over several workgroups per block on or off (default on): with it a
+    launch that would leave most compute units idle (one sequence, few heads) hands the library a workspace for
+    partial results, see ``split_workspace`` in ``include/jvpfa.h``."""
+    global _split_enabled
+    _split_enabled = bool(enabled)
 
 
 TILE_LISTS_MIN_L = 512  # below this a mask has too few tiles for skipping some to pay for the scan
@@ -295,6 +309,10 @@ class HipBackend:
             a.key_limit = _ptr(lim)
             tq, _ = tile_lists(q, mask, mask_kind, False) if k.shape[2] == q.shape[2] else (None, None)
             a.tiles_q = _ptr(tq)
+            nsplit = lib.jvpfa_fwd_split_workspace_bytes(C.byref(a.p), a.Lk) if _split_enabled else 0
+            if nsplit:
+                split_ws = torch.empty(nsplit, device=q.device, dtype=torch.uint8)
+                a.split_workspace, a.split_workspace_bytes = split_ws.data_ptr(), nsplit
             check(lib.jvpfa_fwd(C.byref(a), _stream(q)))
         return o, ot, M, mu
 

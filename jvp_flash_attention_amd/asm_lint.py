@@ -7,7 +7,9 @@ slots that the hardware needs
 
 1. between a vector-ALU write to a register (for instance ``v_accvgpr_read_b32`` bringing back a
    value the allocator parked in the accumulation file) and a matrix instruction that reads it, and
-2. between a matrix instruction and anything else that reads its result.
+2. between a matrix instruction and anything else that reads its result (a vector instruction reading a score
+   tile, or ``v_accvgpr_read_b32`` reading an accumulator: the compiler may schedule the epilogue's reads in front
+   of a wait that is not tied to the registers).
 
 The sources provide those slots themselves (``s_nop 1`` in front of the matrix instructions whose
 operands live long enough to be parked, ``tiles_ready()`` = ``s_nop 15; s_nop 3`` after each group).
@@ -72,7 +74,7 @@ def scan(isa_text: str, where: str = "") -> list[str]:
                     for pop, pops in hist[-2:]:
                         if pop.startswith("v_") and not pop.startswith("v_mfma") and pops and (_regs(pops[0]) & srcs):
                             out.append(f"{where} {kern}: '{pop} {pops[0]}' feeds '{t[:60]}' without idle slots")
-                pending |= {r for r in dst if r[0] == "v"}  # results in the accumulation file are only read by matrix instructions
+                pending |= dst  # vector registers, and accumulation registers (read back by v_accvgpr_read)
             else:
                 pending -= dst
         elif pending and op.startswith(("v_", "ds_write", "global_store", "buffer_store", "scratch_store")):

@@ -43,6 +43,9 @@ inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit, cons
   r.tiles_q = lists ? tiles_q : nullptr;
   r.tiles_k = lists ? tiles_k : nullptr;
   r.klimit = (masked && !r.tiles_q && !r.tiles_k) ? key_limit : nullptr;
+  r.chunks = 1;
+  r.chunk_tiles = 0;
+  r.part = nullptr;
   r.Z = p.Z;
   r.H = p.H;
   r.L = p.L;

@@ -3,6 +3,7 @@
 #include <stddef.h>
 
 #include "api_common.hpp"
+#include "split.hpp"
 
 namespace jvpfa {
 #define JVPFA_DECL(name) int name(const FwdParams &, bool, int, hipStream_t);
@@ -37,7 +38,22 @@ extern "C" int jvpfa_fwd(const jvpfa_fwd_args *a, void *hip_stream) {
   p.q = a->q; p.k = a->k; p.v = a->v;
   p.qt = a->qt; p.kt = a->kt; p.vt = a->vt;
   p.o = a->o; p.ot = a->ot; p.M = a->M; p.mu = a->mu;
+  if (a->split_workspace) {  // small grid: split the key tiles of every query block, if the workspace suffices
+    const SplitPlan sp = fwd_split_plan(a->p, p.pr.Lk);
+    if (sp.chunks > 1 && aligned16(a->split_workspace) &&
+        a->split_workspace_bytes >= fwd_part_floats(sp.chunks, (long long)a->p.Z * a->p.H * a->p.L, a->p.D) * sizeof(float)) {
+      p.pr.chunks = sp.chunks;
+      p.pr.chunk_tiles = sp.chunk_tiles;
+      p.pr.part = static_cast<float *>(a->split_workspace);
+    }
+  }
   return kFwd[slot(a->p)](p, dual, a->p.mask_kind, static_cast<hipStream_t>(hip_stream));
+}
+
+extern "C" size_t jvpfa_fwd_split_workspace_bytes(const jvpfa_problem *p, int32_t Lk) {
+  if (!p || check_problem(*p) != JVPFA_OK) return 0;
+  const SplitPlan sp = fwd_split_plan(*p, Lk > 0 ? Lk : p->L);
+  return sp.chunks > 1 ? fwd_part_floats(sp.chunks, (long long)p->Z * p->H * p->L, p->D) * sizeof(float) : 0;
 }
 
 extern "C" int jvpfa_abi_version(void) { return JVPFA_ABI_VERSION; }

@@ -6,6 +6,7 @@
 #include "fwd_kernel_v3.hpp"
 #include "fwd_kernel_wide.hpp"
 #include "launch.hpp"
+#include "split.hpp"
 
 namespace jvpfa {
 
@@ -44,9 +45,15 @@ static int launch_fwd3_one(const FwdParams &p, hipStream_t stream) {
   int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
   if (rc != 0) return rc;
   const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
-  const long long blocks = (long long)nqb * p.pr.Z * p.pr.H;
+  const long long blocks = (long long)nqb * p.pr.Z * p.pr.H * p.pr.chunks;
   if (blocks > 0x7fffffffLL) return -2;
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
+  if (p.pr.chunks > 1) {  // the chunks' partial results become o, ot, M, mu
+    const long long rows = (long long)p.pr.Z * p.pr.H * p.pr.L;
+    constexpr int RPB = 256 / (D / 8);
+    hipLaunchKernelGGL((fwd_merge_kernel<T, D, DUAL>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream,
+                       p.pr.part, p.pr.chunks, rows, reinterpret_cast<T *>(p.o), reinterpret_cast<T *>(p.ot), p.M, p.mu);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }
 

@@ -367,6 +367,9 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     for (int e = 0; e < 16; ++e) rs += S[e];
     // rare: some row's reference point moved, or (dual) this half tile outweighs what came before it four times
     if (__builtin_expect(__any(up || (DUAL && rs > 4.f * l_i)), 0)) {
+      // (the accumulations of the previous half tile finished long ago, behind this half tile's score products;
+      // the wait keeps that true wherever the compiler places this block)
+      asm volatile("s_nop 15\n\ts_nop 15");
       float neg_shift = 0.f;
       if constexpr (DUAL) {
         const bool outweighs = rs > 4.f * l_i * alpha;
@@ -484,7 +487,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   for (; t < ntiles; ++t) tile(t, std::true_type{});
 
   // ---- epilogue ---------------------------------------------------------------------------------
-  if constexpr (DUAL) asm volatile("s_nop 15\n\ts_nop 15");  // the last in-place accumulation has written its registers
+  if constexpr (DUAL) accs_ready(Oacc, Tacc);  // the last in-place accumulation has written its registers
   l_i += xor32(l_i);
   if constexpr (DUAL) mu_i += xor32(mu_i);
   const bool dead = !(l_i > 0.f);

@@ -57,8 +57,10 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   const Problem &pr = p.pr;
   const int L = pr.L;
   const int nqb = (L + Cfg::BM - 1) / Cfg::BM;
-  const int total = nqb * pr.Z * pr.H;
-  const int id = xcd_remap(blockIdx.x, nqb, pr.Z * pr.H);
+  // small grids: the key tiles of a query block are split over pr.chunks workgroups (see split.hpp)
+  const int chunks = pr.chunks;
+  const int chunk = chunks > 1 ? (int)(blockIdx.x % chunks) : 0;
+  const int id = xcd_remap(chunks > 1 ? blockIdx.x / chunks : blockIdx.x, nqb, pr.Z * pr.H);
   const int zh = id / nqb;
   const int qb = pr.causal ? nqb - 1 - id % nqb : id % nqb;
 
@@ -70,18 +72,33 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   const size_t head = (size_t)zh * L * D;
   // keys: Lk of them, in head h / (H / Hk) of the key/value tensors (L and h themselves for the
   // shapes the reference admits)
-  const int Lk = pr.Lk;
-  const size_t kvhead = ((size_t)(zh / pr.H) * pr.Hk + (zh % pr.H) / (pr.H / pr.Hk)) * Lk * D;
+  const int q0 = qb * Cfg::BM;
+  const int qrow = q0 + wave * 32 + r;
+  const int qld = qrow < L ? qrow : L - 1;
+  // This workgroup's keys: all of them, or the tiles of its chunk.  From here on key indices are counted from
+  // the chunk's first key k0: Lk is the number of keys left from there, and the causal limits move with it.
+  const int nt_all = ((pr.causal ? min(pr.Lk, q0 + Cfg::BM) : pr.Lk) + BN - 1) / BN;
+  const int t_first = chunks > 1 ? min(chunk * pr.chunk_tiles, nt_all) : 0;
+  const int ntiles = chunks > 1 ? min(nt_all - t_first, pr.chunk_tiles) : nt_all;  // 0: nothing for this chunk
+  const int k0 = t_first * BN;
+  const int Lk = pr.Lk - k0;
+  // partial results of a chunk: [chunk][row][O | T][D] floats, then [chunk][row][m, l, mu_acc, c]
+  const size_t nrows = (size_t)pr.Z * pr.H * L, prow = (size_t)chunk * nrows + (size_t)zh * L + qrow;
+  float *part_stat = pr.part + (size_t)chunks * nrows * 2 * D + prow * 4;
+  if (chunks > 1 && ntiles <= 0) {  // no tile falls to this chunk (short causal rows): it weighs nothing
+    if (qrow < L && g == 0) {
+      const f32x4 none = {-__builtin_inff(), 0.f, 0.f, 0.f};
+      *reinterpret_cast<f32x4 *>(part_stat) = none;
+    }
+    return;
+  }
+  const size_t kvhead = (((size_t)(zh / pr.H) * pr.Hk + (zh % pr.H) / (pr.H / pr.Hk)) * pr.Lk + k0) * D;
   const T *Qg = reinterpret_cast<const T *>(p.q) + head;
   const char *Kg = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.k) + kvhead);
   const char *Vg = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.v) + kvhead);
   const T *Qtg = DUAL ? reinterpret_cast<const T *>(p.qt) + head : nullptr;
   const char *Ktg = DUAL ? reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.kt) + kvhead) : nullptr;
   const char *Vtg = DUAL ? reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.vt) + kvhead) : nullptr;
-
-  const int q0 = qb * Cfg::BM;
-  const int qrow = q0 + wave * 32 + r;
-  const int qld = qrow < L ? qrow : L - 1;
 
   // ---- direct loads (see fwd_kernel_v2.hpp): instruction i of this wave fills chunks 64*(wave*IPW+i)..+63
   int ld_row[IPW];
@@ -142,9 +159,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
 
   const float sl2 = pr.scale * LOG2E;
   const bool neg_scale = !(sl2 > 0.f);
-  const int kend = pr.causal ? min(Lk, q0 + Cfg::BM) : Lk;
-  const int ntiles = (kend + BN - 1) / BN;
-  const int qlim = pr.causal ? qrow : 0x7fffffff;  // keys above this index are masked
+  const int qlim = pr.causal ? qrow - k0 : 0x7fffffff;  // keys above this index are masked
 
   // ---- next-tile loads, one instruction per super-step -------------------------------------------
   constexpr int NLOAD = IPW * Cfg::NTILE;
@@ -477,7 +492,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   // Iterations whose softmax needs the causal / sequence-end limits form the tail of the loop; they
   // get a loop of their own so that the common iteration is one straight-line block.
   int t_gen = (Lk >= 32) ? (Lk - 32) / BN + 1 : 0;
-  if (pr.causal) t_gen = min(t_gen, (q0 + 32) / BN);
+  if (pr.causal) t_gen = min(t_gen, max(q0 - k0 + 32, 0) / BN);
   t_gen = neg_scale ? 1 : max(1, t_gen);
   int t = 1;
   for (; t < min(t_gen, ntiles); ++t) {
@@ -502,11 +517,38 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   slot(B0{}, B1{}, B1{}, B1{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
        (ntiles - 1) * BN + 32);
   slot(B0{}, B1{}, B0{}, B1{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0);
-  asm volatile("s_nop 15\n\ts_nop 15");  // the last accumulation has written its registers
+  // the last accumulation has written its registers
+  if constexpr (DUAL) accs_ready(Oacc, Tacc);
+  else accs_ready(Oacc);
 
   // ---- epilogue ---------------------------------------------------------------------------------
   l_i += xor32(l_i);
   if constexpr (DUAL) mu_i += xor32(mu_i);
+  if (chunks > 1) {  // this chunk's share, left as it stands for the merge kernel
+    if (qrow < L) {
+      float *pa = pr.part + prow * 2 * D;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          float o8[8], t8[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            o8[e] = Oacc[db][8 * hf + e];
+            if constexpr (DUAL) t8[e] = Tacc[db][8 * hf + e];
+          }
+          const int d0 = 32 * db + 16 * hf + 8 * g;
+          store8<float>(pa + d0, o8);
+          if constexpr (DUAL) store8<float>(pa + D + d0, t8);
+        }
+      }
+      if (g == 0) {
+        const f32x4 st = {m_i, l_i, mu_i, c_i};
+        *reinterpret_cast<f32x4 *>(part_stat) = st;
+      }
+    }
+    return;
+  }
   const bool dead = !(l_i > 0.f);
   const float inv = dead ? 0.f : 1.f / l_i;
   const float mu_n = mu_i * inv;

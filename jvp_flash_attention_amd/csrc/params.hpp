@@ -20,6 +20,12 @@ struct Problem {
   // 1 + ceil(L/64) ints (count >= 1, then ascending indices of 64-wide tiles).  tiles_q: key tiles
   // per query block; tiles_k: query tiles per key block.
   const int *tiles_q, *tiles_k;
+  // Split of the streamed tiles of one block of owned rows over `chunks` workgroups (1 = no split), used when
+  // a launch would otherwise leave most compute units idle: workgroup c of a block takes the tiles
+  // c * chunk_tiles .. (c + 1) * chunk_tiles - 1 and writes fp32 partial results to `part`, which a merge
+  // kernel adds up.  Only the kernels for 16-bit element types, D = 128, without a mask.
+  int chunks, chunk_tiles;
+  float *part;
 };
 
 constexpr int TILE_BLOCK = 128, TILE_W = 64;  // geometry of the tile lists

@@ -130,6 +130,23 @@ __device__ __forceinline__ void mfma_acc(f32x16 &c, const f16x8 &a, const f16x8 
 }
 __device__ __forceinline__ void pin_acc(f32x16 &c) { asm volatile("" : "+a"(c)); }
 
+// 32 idle issue slots behind the last in-place accumulation, tied to the tiles: code the compiler generates to
+// read them (the epilogue) cannot be scheduled in front of the wait, which a bare asm statement would allow.
+template <int N> __device__ __forceinline__ void accs_ready(f32x16 (&o)[N]) {
+  static_assert(N == 1 || N == 2 || N == 4);
+  if constexpr (N == 1) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]));
+  if constexpr (N == 2) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]));
+  if constexpr (N == 4) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]));
+}
+template <int N> __device__ __forceinline__ void accs_ready(f32x16 (&o)[N], f32x16 (&t)[N]) {
+  static_assert(N == 1 || N == 2 || N == 4);
+  if constexpr (N == 1) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(t[0]));
+  if constexpr (N == 2) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]), "+a"(t[0]), "+a"(t[1]));
+  if constexpr (N == 4)
+    asm volatile("s_nop 15\n\ts_nop 15"
+                 : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(t[0]), "+a"(t[1]), "+a"(t[2]), "+a"(t[3]));
+}
+
 // 16 + 4 idle issue slots: the last matrix-core pass has written its registers when this returns
 __device__ __forceinline__ void tiles_ready(f32x16 &a) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a)); }
 __device__ __forceinline__ void tiles_ready(f32x16 &a, f32x16 &b) {

@@ -44,6 +44,28 @@ def test_a_result_read_before_the_wait_is_flagged():
     assert asm_lint.scan(EARLY_READ.replace("\tv_accvgpr_write_b32 a70, v33\n", ""), "unit") == []
 
 
+EARLY_ACCUMULATOR_READ = """
+_ZN5jvpfa4kernEv:
+	;;#ASMSTART
+	v_mfma_f32_32x32x16_bf16 a[0:15], v[64:67], v[16:19], a[0:15]
+	;;#ASMEND
+	v_accvgpr_read_b32 v5, a3
+	;;#ASMSTART
+	s_nop 15
+	s_nop 15
+	;;#ASMEND
+"""
+
+
+def test_an_accumulator_read_back_before_the_wait_is_flagged():
+    """What the compiler may do to an epilogue behind a wait that is not tied to the accumulators."""
+    found = asm_lint.scan(EARLY_ACCUMULATOR_READ, "unit")
+    assert len(found) == 1 and "before the wait" in found[0]
+    lines = EARLY_ACCUMULATOR_READ.split("\n")
+    moved = "\n".join(lines[:5] + lines[6:] + [lines[5]])  # the read behind the wait
+    assert asm_lint.scan(moved, "unit") == []
+
+
 def test_compiled_kernels_are_clean():
     """The ISA text that the build left behind for every kernel unit, or, without a build, two units
     compiled here (the D = 32 backward is where the allocator once parked a resident operand in the

@@ -5,6 +5,8 @@ Tolerances (the stated target): fp32 max-abs <= 1e-4; bf16 / fp16 relative error
 same, already rounded, inputs (it is itself pinned against PyTorch's math SDPA under
 ``torch.func.jvp`` in ``test_oracle.py``).
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -677,6 +679,48 @@ def test_results_are_the_same_from_run_to_run(D, heads, mode):
     for other in runs[1:]:
         for a_, b_ in zip(runs[0], other):
             assert torch.equal(a_, b_)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(1, 2, 1024, 1024, True), (1, 2, 1024, 1024, False), (1, 3, 333, 700, False),
+                                   (2, 1, 700, 700, True), (1, 1, 4096, 512, False)])
+@pytest.mark.parametrize("dual", [True, False])
+def test_small_launches_split_over_key_chunks(dt, shape, dual):
+    """Launches with far fewer query blocks than the GPU has compute units (D = 128, no mask): the key tiles of a
+    block are split over several workgroups and merged.  Against the oracle, and against the same launch without
+    the split (one ulp of the element type apart at most; M and mu, which stay fp32, to 1e-5)."""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H, L, Lk, causal = shape
+    D, dtype = 128, DTYPES[dt]
+    g = torch.Generator().manual_seed(L + Lk)
+    q, qt = [torch.randn(Z, H, L, D, generator=g).to(dtype) for _ in range(2)]
+    k, v, kt, vt = [torch.randn(Z, H, Lk, D, generator=g).to(dtype) for _ in range(4)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt)]
+    if not dual:
+        dev[3:] = [None, None, None]
+    be, scale = _lib.backend(), D**-0.5
+    print(f"case split Z{Z} H{H} L{L} Lk{Lk} causal={causal} {dt} dual={dual}", flush=True)
+    a = _lib.FwdArgs()
+    a.p = _lib.make_problem(dev[0], None, _lib.MASK_NONE, causal, scale)
+    assert _lib.load().jvpfa_fwd_split_workspace_bytes(C.byref(a.p), Lk) > 0  # this launch does split
+    got = be.fwd(*dev, None, _lib.MASK_NONE, causal, scale)
+    _lib.set_split(False)
+    try:
+        one = be.fwd(*dev, None, _lib.MASK_NONE, causal, scale)
+    finally:
+        _lib.set_split(True)
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt)]
+    ref = dense.forward(*f64, causal=causal, scale=scale) if dual else dense.forward(*f64[:3], causal=causal, scale=scale)
+    _tol_check("O", got[0], ref["O"], dtype)
+    assert np.abs(got[2].double().cpu().numpy() - ref["M"]).max() < 1e-4
+    assert (got[2] - one[2]).abs().max().item() <= 1e-5
+    ulp = 2.0**-7 if dtype == torch.bfloat16 else 2.0**-10
+    assert ((got[0].float() - one[0].float()).abs() <= ulp * one[0].float().abs().clamp_min(1.0)).all()
+    if dual:
+        _tol_check("O'", got[1], ref["Ot"], dtype)
+        assert np.abs(got[3].double().cpu().numpy() - ref["mu"]).max() < 1e-4 * max(1.0, np.abs(ref["mu"]).max())
+        assert ((got[1].float() - one[1].float()).abs() <= 2 * ulp * one[1].float().abs().clamp_min(1.0)).all()
 
 
 def test_c_abi_from_a_plain_cpp_program():
