@@ -192,6 +192,11 @@ def main():
     ap.add_argument("--fwd-only", action="store_true", help="time only the headline forward (for profiling)")
     ap.add_argument("--bwd-only", action="store_true",
                     help="run one forward, then time only the headline backward (for profiling); prints its own line")
+    ap.add_argument("--plain-only", action="store_true",
+                    help="time the headline shape without tangents (what attention() runs in first-order training): forward, "
+                         "then the backward of gO (for profiling); prints its own line")
+    ap.add_argument("--bwd6-only", action="store_true",
+                    help="run one forward, then time the backward that also returns dq', dk', dv' (for profiling)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, whose known traffic scales the rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings of the forward kernel")
@@ -231,6 +236,22 @@ def main():
                         args.steps, args.warmup)
         print(json.dumps({"workload": "bf16 B4 H16 L4096 D128 backward of (gO, gT) -> dq, dk, dv", "ms_per_step": ms_b,
                           "tflops_algorithmic": bwd_flops / (ms_b * 1e-3) / 1e12}), flush=True)
+        return
+    if args.plain_only:
+        ms_pf, _ = timed(lambda: be.fwd(q, k, v, None, None, None, None, _lib.MASK_NONE, False, scale), args.steps, args.warmup)
+        o, _, M, _ = be.fwd(q, k, v, None, None, None, None, _lib.MASK_NONE, False, scale)
+        ms_pb, _ = timed(lambda: be.bwd(q, k, v, None, None, None, o, None, M, None, go, None, None, _lib.MASK_NONE, False, scale),
+                         args.steps, args.warmup)
+        print(json.dumps({"workload": "bf16 B4 H16 L4096 D128 without tangents: forward (4 N flops), backward of gO (10 N)",
+                          "fwd_ms": ms_pf, "fwd_tflops": 4.0 * N / (ms_pf * 1e-3) / 1e12,
+                          "bwd_ms": ms_pb, "bwd_tflops": 10.0 * N / (ms_pb * 1e-3) / 1e12}), flush=True)
+        return
+    if args.bwd6_only:
+        o, ot, M, mu = fwd()
+        ms_b6, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, False, scale,
+                                        want_tangent_grads=True), args.steps, args.warmup)
+        print(json.dumps({"workload": "bf16 B4 H16 L4096 D128 backward of (gO, gT) -> dq, dk, dv, dq', dk', dv'", "ms_per_step": ms_b6,
+                          "tflops_algorithmic": bwd_flops * 15 / 12 / (ms_b6 * 1e-3) / 1e12}), flush=True)
         return
     if args.calibrate_copy:
         src = torch.empty(256 * 2**20, dtype=torch.uint8, device=dev).random_(0, 255)
