@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define JVPFA_ABI_VERSION 6
+#define JVPFA_ABI_VERSION 7
 
 enum jvpfa_dtype { JVPFA_BF16 = 0, JVPFA_FP16 = 1, JVPFA_FP32 = 2 };
 
@@ -36,7 +36,7 @@ enum jvpfa_mask_kind { JVPFA_MASK_NONE = 0, JVPFA_MASK_BOOL = 1, JVPFA_MASK_ADD 
 enum jvpfa_status {
   JVPFA_OK = 0,
   JVPFA_E_NULL = -1,      /* a required pointer is NULL */
-  JVPFA_E_SHAPE = -2,     /* Z,H,L < 1, D not in {32, 64, 128, 256}, or D = 256 with fp32 */
+  JVPFA_E_SHAPE = -2,     /* Z,H,L < 1, D not in {32, 64, 128, 256}, D = 256 with fp32 or with dropout, dropout_p outside [0, 1) */
   JVPFA_E_DTYPE = -3,     /* dtype / mask_kind out of range */
   JVPFA_E_ALIGN = -4,     /* a tensor pointer is not 16-byte aligned */
   JVPFA_E_CONFLICT = -5,  /* causal together with a mask (JA:2380-2381 raises ValueError) */
@@ -55,6 +55,14 @@ typedef struct jvpfa_problem {
   const void *mask;   /* bool: uint8, nonzero = attend (JA:241-245); additive: same dtype as q,
                          added to the scaled logits (SDPA semantics) */
   int64_t mask_stride[4]; /* element strides over (z, h, query, key); 0 broadcasts */
+  /* Dropout on the attention probabilities: 0 <= dropout_p < 1, 0 = none.  Entry (z, h, query, key) is kept or
+   * dropped by a counter-based hash of (dropout_seed, entry index) and kept entries are scaled by 1/(1 - p), as
+   * torch's scaled_dot_product_attention does; forward and backward of one call pair must get the same seed.
+   * jvpfa_dropout_keep() writes the keep pattern out.  The reference carries dead code for dropout and raises
+   * NotImplementedError (JA:94-122, JA:271-277, JA:2356-2357).  D <= 128; runs on the register-staged kernels
+   * for every element type (about 3x slower than without dropout for bf16 / fp16). */
+  float dropout_p;
+  uint64_t dropout_seed;
 } jvpfa_problem;
 
 /*
@@ -177,6 +185,13 @@ size_t jvpfa_bwd_static_max_rows(void);
  */
 size_t jvpfa_mask_tiles_bytes(const jvpfa_problem *p);
 int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t *tiles_q, int32_t *tiles_k, void *hip_stream);
+
+/*
+ * The keep pattern of dropout for this problem (only Z, H, L, dropout_p, dropout_seed are read) and Lk keys
+ * (0 = as L): keep[z][h][query][key] = 1 for a kept entry, 0 for a dropped one, Z*H*L*Lk bytes of device memory.
+ * For tests and for callers that want to reproduce a call with another implementation.
+ */
+int jvpfa_dropout_keep(const jvpfa_problem *p, int32_t Lk, uint8_t *keep, void *hip_stream);
 
 /* JVPFA_ABI_VERSION of the loaded library. */
 int jvpfa_abi_version(void);

@@ -15,10 +15,10 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libjvpfa.so")
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
-EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_fwd_split_workspace_bytes", "jvpfa_bwd_workspace_bytes", "jvpfa_bwd_static", "jvpfa_bwd_static_max_rows", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
+EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_fwd_split_workspace_bytes", "jvpfa_dropout_keep", "jvpfa_bwd_workspace_bytes", "jvpfa_bwd_static", "jvpfa_bwd_static_max_rows", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
            "jvpfa_abi_version", "jvpfa_error_string")
 
 
@@ -29,6 +29,8 @@ class Problem(C.Structure):
         ("sm_scale", C.c_float),
         ("mask", C.c_void_p),
         ("mask_stride", C.c_int64 * 4),
+        ("dropout_p", C.c_float),
+        ("dropout_seed", C.c_uint64),
     ]
 
 
@@ -90,6 +92,8 @@ def load() -> C.CDLL:
         lib.jvpfa_bwd_static_max_rows.restype = C.c_size_t
         lib.jvpfa_fwd_split_workspace_bytes.argtypes = [C.POINTER(Problem), C.c_int32]
         lib.jvpfa_fwd_split_workspace_bytes.restype = C.c_size_t
+        lib.jvpfa_dropout_keep.argtypes = [C.POINTER(Problem), C.c_int32, C.c_void_p, C.c_void_p]
+        lib.jvpfa_dropout_keep.restype = C.c_int
         lib.jvpfa_mask_tiles_bytes.argtypes = [C.POINTER(Problem)]
         lib.jvpfa_mask_tiles_bytes.restype = C.c_size_t
         lib.jvpfa_mask_tiles.argtypes = [C.POINTER(Problem), C.c_void_p, C.c_void_p, C.c_void_p]
@@ -114,9 +118,10 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
-def make_problem(q, mask, mask_kind, causal, sm_scale) -> Problem:
+def make_problem(q, mask, mask_kind, causal, sm_scale, dropout_p=0.0, dropout_seed=0) -> Problem:
     Z, H, L, D = q.shape
     p = Problem()
+    p.dropout_p, p.dropout_seed = float(dropout_p), int(dropout_seed) & (2**64 - 1)
     p.Z, p.H, p.L, p.D = Z, H, L, D
     p.dtype = DTYPES[q.dtype]
     p.causal = int(bool(causal))
@@ -271,24 +276,25 @@ class HipBackend:
 
     name = "hip"
 
-    def fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
+    def fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale, dropout_p=0.0, dropout_seed=0):
         """Returns (o, ot, M, mu); ot and mu are None for a plain forward."""
         if torch.compiler.is_compiling():
-            o, ot, M, mu = torch.ops.jvpfa.fwd(q, k, v, qt, kt, vt, mask, int(mask_kind), bool(causal), float(sm_scale))
+            o, ot, M, mu = torch.ops.jvpfa.fwd(q, k, v, qt, kt, vt, mask, int(mask_kind), bool(causal), float(sm_scale),
+                                               float(dropout_p), int(dropout_seed))
             return (o, ot, M, mu) if qt is not None else (o, None, M, None)
-        return self._fwd(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale)
+        return self._fwd(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale, dropout_p, dropout_seed)
 
     def bwd(self, q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
-            want_tangent_grads=False):
+            want_tangent_grads=False, dropout_p=0.0, dropout_seed=0):
         """Returns (dq, dk, dv, dqt, dkt, dvt); the last three are None unless requested."""
         if torch.compiler.is_compiling():
             out = torch.ops.jvpfa.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, int(mask_kind), bool(causal),
-                                      float(sm_scale), bool(want_tangent_grads))
+                                      float(sm_scale), bool(want_tangent_grads), float(dropout_p), int(dropout_seed))
             return tuple(out) if want_tangent_grads else (*out[:3], None, None, None)
         return self._bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
-                         want_tangent_grads)
+                         want_tangent_grads, dropout_p, dropout_seed)
 
-    def _fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
+    def _fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale, dropout_p=0.0, dropout_seed=0):
         _require_gpu(q, k, v, qt, kt, vt, mask)
         lib = load()
         dual = qt is not None
@@ -299,7 +305,7 @@ class HipBackend:
         mu = torch.empty((Z, H, L), device=q.device, dtype=torch.float32) if dual else None
         a = FwdArgs()
         a.struct_size = C.sizeof(FwdArgs)
-        a.p = make_problem(q, mask, mask_kind, causal, sm_scale)
+        a.p = make_problem(q, mask, mask_kind, causal, sm_scale, dropout_p, dropout_seed)
         a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
         a.qt, a.kt, a.vt = _ptr(qt), _ptr(kt), _ptr(vt)
         a.o, a.ot, a.M, a.mu = _ptr(o), _ptr(ot), _ptr(M), _ptr(mu)
@@ -317,7 +323,7 @@ class HipBackend:
         return o, ot, M, mu
 
     def _bwd(self, q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
-             want_tangent_grads=False):
+             want_tangent_grads=False, dropout_p=0.0, dropout_seed=0):
         _require_gpu(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask)
         lib = load()
         Z, H, L, _ = q.shape
@@ -328,7 +334,7 @@ class HipBackend:
         ws = torch.empty(lib.jvpfa_bwd_workspace_bytes(Z, H, L), device=q.device, dtype=torch.uint8)
         a = BwdArgs()
         a.struct_size = C.sizeof(BwdArgs)
-        a.p = make_problem(q, mask, mask_kind, causal, sm_scale)
+        a.p = make_problem(q, mask, mask_kind, causal, sm_scale, dropout_p, dropout_seed)
         a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
         a.qt, a.kt, a.vt = _ptr(qt), _ptr(kt), _ptr(vt)
         a.o, a.ot, a.M, a.mu = _ptr(o), _ptr(ot), _ptr(M), _ptr(mu)
@@ -346,6 +352,17 @@ class HipBackend:
         return dq, dk, dv, dqt, dkt, dvt
 
 
+    def dropout_keep(self, q, Lk, dropout_p, dropout_seed):
+        """The keep pattern (bool, shape (Z, H, L, Lk)) that a call with this dropout_p and seed applies."""
+        _require_gpu(q)
+        Z, H, L, _ = q.shape
+        keep = torch.empty((Z, H, L, Lk), device=q.device, dtype=torch.uint8)
+        prob = make_problem(q, None, MASK_NONE, False, 1.0, dropout_p, dropout_seed)
+        with torch.cuda.device(q.device):
+            check(load().jvpfa_dropout_keep(C.byref(prob), Lk, keep.data_ptr(), _stream(q)))
+        return keep.bool()
+
+
 _backend = HipBackend()
 _hip = _backend  # the operators below always mean the HIP library, whatever backend() has been pointed at
 
@@ -354,14 +371,14 @@ _T, _OT = torch.Tensor, Optional[torch.Tensor]
 
 @torch.library.custom_op("jvpfa::fwd", mutates_args=(), device_types="cuda")
 def _op_fwd(q: _T, k: _T, v: _T, qt: _OT, kt: _OT, vt: _OT, mask: _OT, mask_kind: int, causal: bool,
-            sm_scale: float) -> Tuple[_T, _T, _T, _T]:
-    o, ot, M, mu = _hip._fwd(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale)
+            sm_scale: float, dropout_p: float = 0.0, dropout_seed: int = 0) -> Tuple[_T, _T, _T, _T]:
+    o, ot, M, mu = _hip._fwd(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale, dropout_p, dropout_seed)
     # an operator returns tensors only: empty ones stand for the absent tangent outputs
     return o, (ot if ot is not None else q.new_empty(0)), M, (mu if mu is not None else M.new_empty(0))
 
 
 @_op_fwd.register_fake
-def _(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
+def _(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale, dropout_p=0.0, dropout_seed=0):
     Z, H, L, _ = q.shape
     stat = q.new_empty((Z, H, L), dtype=torch.float32)
     if qt is None:
@@ -372,13 +389,15 @@ def _(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale):
 @torch.library.custom_op("jvpfa::bwd", mutates_args=(), device_types="cuda")
 def _op_bwd(q: _T, k: _T, v: _T, qt: _OT, kt: _OT, vt: _OT, o: _T, ot: _OT, M: _T, mu: _OT, go: _OT, gt: _OT,
             mask: _OT, mask_kind: int, causal: bool, sm_scale: float,
-            want_tangent_grads: bool) -> Tuple[_T, _T, _T, _T, _T, _T]:
-    g = _hip._bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale, want_tangent_grads)
+            want_tangent_grads: bool, dropout_p: float = 0.0, dropout_seed: int = 0) -> Tuple[_T, _T, _T, _T, _T, _T]:
+    g = _hip._bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale, want_tangent_grads,
+                  dropout_p, dropout_seed)
     return tuple(t if t is not None else q.new_empty(0) for t in g)
 
 
 @_op_bwd.register_fake
-def _(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale, want_tangent_grads):
+def _(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale, want_tangent_grads,
+      dropout_p=0.0, dropout_seed=0):
     full = [torch.empty_like(t) for t in (q, k, v)]
     rest = [torch.empty_like(t) if want_tangent_grads else q.new_empty(0) for t in (q, k, v)]
     return (*full, *rest)

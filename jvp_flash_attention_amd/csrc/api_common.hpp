@@ -15,6 +15,8 @@ inline int check_problem(const jvpfa_problem &p) {
   if (p.dtype < JVPFA_BF16 || p.dtype > JVPFA_FP32) return JVPFA_E_DTYPE;
   if (p.D == 256 && p.dtype == JVPFA_FP32) return JVPFA_E_SHAPE;  // the fp32 tiles of D = 256 do not fit the LDS
   if (p.mask_kind < JVPFA_MASK_NONE || p.mask_kind > JVPFA_MASK_ADD) return JVPFA_E_DTYPE;
+  if (!(p.dropout_p >= 0.f && p.dropout_p < 1.f)) return JVPFA_E_SHAPE;
+  if (p.dropout_p > 0.f && p.D == 256) return JVPFA_E_SHAPE;  // the kernels with dropout stop at D = 128
   if (p.mask_kind != JVPFA_MASK_NONE) {
     if (p.causal) return JVPFA_E_CONFLICT;
     if (!p.mask) return JVPFA_E_NULL;
@@ -46,6 +48,16 @@ inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit, cons
   r.chunks = 1;
   r.chunk_tiles = 0;
   r.part = nullptr;
+  r.drop_thr = 0;
+  r.drop_s0 = r.drop_s1 = 0;
+  r.drop_rinv = 1.f;
+  if (p.dropout_p > 0.f) {
+    const double t = (double)p.dropout_p * 4294967296.0;
+    r.drop_thr = t < 1.0 ? 1u : (t > 4294967295.0 ? 4294967295u : (uint32_t)t);
+    r.drop_s0 = (uint32_t)p.dropout_seed;
+    r.drop_s1 = (uint32_t)(p.dropout_seed >> 32);
+    r.drop_rinv = 1.f / (1.f - p.dropout_p);
+  }
   r.Z = p.Z;
   r.H = p.H;
   r.L = p.L;

@@ -112,7 +112,7 @@ __device__ __forceinline__ void zero16(f32x16 &x) {
 // ------------------------------------------------------------------------------------------------
 // dq (MODE PLAIN / DUAL) or dq' (MODE TANGENT).  Scores are transposed (lane = query), as in the
 // forward, so ds is already the B operand of dQ^T += K^T dS^T.
-template <typename T, int D, int MODE, int MASK>
+template <typename T, int D, int MODE, int MASK, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
   using Cfg = BwdCfg<T, D, MODE>;
   constexpr int KK = D / 16, DB = D / 32;
@@ -254,6 +254,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
         if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
         if (diag) pv = (key0 + e <= qrow) ? pv : 0.f;
         if (ragged) pv = (key0 + e < Lk) ? pv : 0.f;
+        if constexpr (DROP) {  // gO V^T, gT V^T, gT V'^T reach the logits through the kept, rescaled entries only
+          const float ks = drop_scale(pr, ((uint64_t)zh * L + qld) * Lk + (key0 + e));
+          if constexpr (!TAN) dP[i] *= ks;
+          if constexpr (DUAL || TAN) At[i] *= ks;
+        }
         if constexpr (MODE == BWD_PLAIN) {
           S[i] = pv * (dP[i] - d1);
         } else if constexpr (DUAL) {
@@ -300,7 +305,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------------------------
 // dk, dv (MODE PLAIN / DUAL) or dk', dv' (MODE TANGENT).  Scores are S = Q K^T (lane = key,
 // registers = queries), so P and dS are the B operands of dV^T += gO^T P and dK^T += Q^T dS.
-template <typename T, int D, int MODE, int MASK>
+template <typename T, int D, int MODE, int MASK, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
   using Cfg = BwdCfg<T, D, MODE>;
   constexpr int KK = D / 16, DB = D / 32;
@@ -472,17 +477,23 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
       float pv = fast_exp2(s - sM[ql]);
       if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
       if (diag) pv = (krow <= qi) ? pv : 0.f;
+      float ks = 1.f;  // dropout: 1 / (1 - p) for a kept entry, 0 for a dropped one
+      if constexpr (DROP) {
+        ks = drop_scale(pr, (((uint64_t)z * pr.H + h) * L + (qi < L ? qi : L - 1)) * Lk + kld);
+        if constexpr (!TAN) dP[e] *= ks;
+        if constexpr (DUAL || TAN) At[e] *= ks;
+      }
       if constexpr (MODE == BWD_PLAIN) {
-        S[e] = pv;
+        S[e] = pv * ks;
         dP[e] = pv * (dP[e] - sd1[ql]);
       } else if constexpr (DUAL) {
         const float sp = Sp[e] * pr.scale, m_ = smu[ql], a_ = sa[ql];
-        S[e] = pv;
-        Pp[e] = pv * (sp - m_);
+        S[e] = pv * ks;
+        Pp[e] = pv * (sp - m_) * ks;
         Sp[e] = pv * (At[e] - a_);
         dP[e] = pv * (dP[e] - sd1[ql] + At[e] * (sp - m_) - a_ * sp - sd2[ql]);
       } else {
-        S[e] = pv;
+        S[e] = pv * ks;
         Sp[e] = pv * (At[e] - sa[ql]);
       }
     }

@@ -10,10 +10,10 @@
 
 namespace jvpfa {
 
-template <typename T, int D, int BN, bool DUAL, int MASK>
+template <typename T, int D, int BN, bool DUAL, int MASK, bool DROP = false>
 static int launch_fwd_one(const FwdParams &p, hipStream_t stream) {
   using Cfg = FwdCfg<T, D, BN, DUAL>;
-  auto kern = fwd_kernel<T, D, BN, DUAL, MASK>;
+  auto kern = fwd_kernel<T, D, BN, DUAL, MASK, DROP>;
   int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
   if (rc != 0) return rc;
   const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
@@ -83,6 +83,18 @@ static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
 
 template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
+  if (p.pr.drop_thr != 0) {
+    // dropout: every element type takes the register-staged kernel, the one family that carries it
+    if constexpr (D <= 128) {
+      constexpr int BNG = sizeof(T) == 4 ? 32 : 64;
+      switch (mask) {
+        case MASK_NONE: return launch_fwd_one<T, D, BNG, DUAL, MASK_NONE, true>(p, stream);
+        case MASK_BOOL: return launch_fwd_one<T, D, BNG, DUAL, MASK_BOOL, true>(p, stream);
+        case MASK_ADD: return launch_fwd_one<T, D, BNG, DUAL, MASK_ADD, true>(p, stream);
+      }
+    }
+    return -2;
+  }
   if constexpr (sizeof(T) == 2 && D == 256) {
     switch (mask) {
       case MASK_NONE: return launch_fwd_wide_one<T, D, DUAL, MASK_NONE>(p, stream);

@@ -29,7 +29,10 @@ template <typename T, int D, int BN, bool DUAL> struct FwdCfg {
   static constexpr size_t LDS_BYTES = (size_t)(DUAL ? 2 : 1) * (K_ELEMS + V_ELEMS) * sizeof(T);
 };
 
-template <typename T, int D, int BN, bool DUAL, int MASK>
+// DROP: dropout on the probabilities (the row sums l, mu stay those of the full softmax; what enters the
+// products with V, V' is P * keep / (1 - p)).  The reference has dead code for it and raises (its
+// jvp_attention.py:94-122, :271-277, :2356-2357).
+template <typename T, int D, int BN, bool DUAL, int MASK, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
   using Cfg = FwdCfg<T, D, BN, DUAL>;
   constexpr int NB = BN / 32;  // 32-key score blocks per tile
@@ -194,12 +197,17 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         float pv = fast_exp2(S[nb][e] - m_use);
-        S[nb][e] = pv;
         rs += pv;
+        float ks = 1.f;
+        if constexpr (DROP) {
+          const int key = j0 + 32 * nb + 16 * (e / 8) + 8 * g + (e % 8);
+          ks = drop_scale(pr, ((uint64_t)zh * L + qld) * Lk + key);
+        }
+        S[nb][e] = pv * ks;
         if constexpr (DUAL) {
           float ps = pv * (Sp[nb][e] * pr.scale);
-          Sp[nb][e] = ps;
           rmu += ps;
+          Sp[nb][e] = ps * ks;
         }
       }
     }

@@ -7,6 +7,7 @@
 // (jvp_attention.py:2383-2388, :241-251).
 #include <hip/hip_runtime.h>
 #include <stddef.h>
+#include <algorithm>
 
 #include "api_common.hpp"
 
@@ -101,6 +102,27 @@ static int launch_both(const jvpfa_problem &p, int *tq, int *tk, hipStream_t str
 }  // namespace jvpfa
 
 using namespace jvpfa;
+
+namespace jvpfa {
+__global__ __launch_bounds__(256) void dropout_keep_kernel(Problem pr, uint64_t n, uint8_t *keep) {
+  // a launch holds fewer than 2^32 threads, the pattern may hold more entries: each thread strides over the rest
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256)
+    keep[i] = drop_scale(pr, i) != 0.f;
+}
+}  // namespace jvpfa
+
+extern "C" int jvpfa_dropout_keep(const jvpfa_problem *p, int32_t Lk, uint8_t *keep, void *hip_stream) {
+  if (!p || !keep) return JVPFA_E_NULL;
+  if (p->Z < 1 || p->H < 1 || p->L < 1 || Lk < 0 || !(p->dropout_p >= 0.f && p->dropout_p < 1.f)) return JVPFA_E_SHAPE;
+  jvpfa_problem q = *p;
+  q.mask_kind = JVPFA_MASK_NONE;
+  const Problem pr = to_problem(q, nullptr, nullptr, nullptr, Lk, 0);
+  const uint64_t n = (uint64_t)p->Z * p->H * p->L * pr.Lk;  // the entry index is ((z H + h) L + i) Lk + j
+  if (n == 0) return JVPFA_OK;
+  const uint64_t blocks = std::min<uint64_t>((n + 255) / 256, 1u << 20);
+  hipLaunchKernelGGL(dropout_keep_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(hip_stream), pr, n, keep);
+  return hipGetLastError() == hipSuccess ? JVPFA_OK : JVPFA_E_LAUNCH;
+}
 
 extern "C" size_t jvpfa_mask_tiles_bytes(const jvpfa_problem *p) {
   if (!p || p->Z < 1 || p->H < 1 || p->L < 1) return 0;

@@ -26,7 +26,28 @@ struct Problem {
   // kernel adds up.  Only the kernels for 16-bit element types, D = 128, without a mask.
   int chunks, chunk_tiles;
   float *part;
+  // Dropout on the attention probabilities (0 in drop_thr: none).  Entry (z, h, query i, key j) is kept when
+  // drop_hash(((z H + h) L + i) Lk + j) >= drop_thr, and kept entries are scaled by drop_rinv = 1 / (1 - p); the
+  // same function of (seed, index) in the forward, both backward kernels and jvpfa_dropout_keep.
+  uint32_t drop_thr, drop_s0, drop_s1;
+  float drop_rinv;
 };
+
+// Counter-based keep decision: a 32-bit mix of the 64-bit entry index and the seed (two multiply-xorshift rounds).
+__host__ __device__ inline uint32_t drop_hash(uint64_t idx, uint32_t s0, uint32_t s1) {
+  uint32_t x = ((uint32_t)idx * 0x9E3779B1u) ^ s0;
+  x ^= (uint32_t)(idx >> 32) * 0x85EBCA77u + s1;
+  x ^= x >> 16;
+  x *= 0x7feb352du;
+  x ^= x >> 15;
+  x *= 0x846ca68bu;
+  x ^= x >> 16;
+  return x;
+}
+// 1 / (1 - p) for a kept entry, 0 for a dropped one
+__host__ __device__ inline float drop_scale(const Problem &pr, uint64_t idx) {
+  return drop_hash(idx, pr.drop_s0, pr.drop_s1) >= pr.drop_thr ? pr.drop_rinv : 0.f;
+}
 
 constexpr int TILE_BLOCK = 128, TILE_W = 64;  // geometry of the tile lists
 // first element of the list of (plane of (z, h), block)

@@ -56,7 +56,9 @@ inline size_t bwd_part_floats(int chunks, long long rows, long long kv_rows, int
 
 // The kernels that can split: 16-bit element types, D = 128, no mask (the software-pipelined forward and the
 // direct-to-LDS backward kernels).  Tiles are 64 wide, blocks 128 rows.
-template <typename P> inline bool split_capable(const P &p) { return p.dtype != 2 && p.D == 128 && p.mask_kind == 0; }
+template <typename P> inline bool split_capable(const P &p) {
+  return p.dtype != 2 && p.D == 128 && p.mask_kind == 0 && !(p.dropout_p > 0.f);
+}
 template <typename P> inline SplitPlan fwd_split_plan(const P &p, int Lk) {
   SplitPlan none = {1, 0};
   if (!split_capable(p)) return none;

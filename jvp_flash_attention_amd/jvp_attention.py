@@ -27,6 +27,11 @@ Differences from the reference, all deliberate:
 * k and v may have fewer heads than q (grouped heads: H a multiple of H_kv) and a length of their own
   (cross-attention); causal then means key index <= query index, as in SDPA.  The reference requires
   q, k, v of one shape (JA:2367-2378).
+* ``dropout_p`` > 0 works (the reference carries dead code for it and raises ``NotImplementedError``,
+  JA:94-122, JA:271-277, JA:2356-2357): dropout on the attention probabilities with SDPA's semantics (kept entries
+  scaled by 1/(1-p); the tangent O' sees the same pattern), the pattern a counter-based hash of a seed drawn from
+  torch's CPU generator per call (``torch.manual_seed`` makes it repeatable) and of the entry index, regenerated in
+  the backward.  Head dims up to 128; runs on the register-staged kernels (about 3x slower for bf16 / fp16).
 * ``attention`` notices dual inputs and then behaves like ``fwd_dual`` (the reference's ``attention``
   is ``JVPAttn.fwd`` and drops the tangent, its README.md:65-67).
 """
@@ -71,8 +76,9 @@ def is_blackwell() -> bool:
 
 def _validate(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dropout_p: float, causal: bool):
     """Argument checks of JA:2356-2392, with this build's shape limits."""
-    if dropout_p != 0.0:
-        raise NotImplementedError("Dropout is not currently supported in JVP attention.")
+    assert 0.0 <= dropout_p < 1.0, f"dropout_p must be in [0, 1), but got {dropout_p}"
+    if dropout_p != 0.0 and q.shape[-1] == 256:
+        raise NotImplementedError("Dropout is supported for HEAD_DIM_K up to 128 in JVP attention.")
     assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be (Z, H, N_CTX, HEAD_DIM)"
     Z, H, N_CTX, HEAD_DIM_Q = q.shape
     HEAD_DIM_K, HEAD_DIM_V = k.shape[-1], v.shape[-1]
@@ -153,6 +159,12 @@ def _unwrap(x):
     return x
 
 
+def _new_dropout_seed(dropout_p: float) -> int:
+    """A fresh seed for one forward call (0 without dropout), from torch's CPU generator: no device work, and
+    ``torch.manual_seed`` makes a run repeatable."""
+    return int(torch.randint(0, 2**62, (1,)).item()) if dropout_p > 0.0 else 0
+
+
 def _dense(t: Tensor | None) -> Tensor | None:
     return None if t is None else (t if t.is_contiguous() else t.contiguous())
 
@@ -165,17 +177,19 @@ class _DualCore(Function):
     """
 
     @staticmethod
-    def forward(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale):
-        o, o_t, M, mu = _lib.backend().fwd(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale)
+    def forward(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p=0.0, seed=0):
+        o, o_t, M, mu = _lib.backend().fwd(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale,
+                                           dropout_p, seed)
         return o, o_t, M, mu
 
     @staticmethod
     def setup_context(ctx, inputs, outputs):
-        q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale = inputs
+        q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p, seed = inputs
         o, o_t, M, mu = outputs
         ctx.mark_non_differentiable(M, mu)
         ctx.save_for_backward(q, k, v, q_t, k_t, v_t, o, o_t, M, mu)
         ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale = mask_tensor, MASK_TYPE, causal, sm_scale
+        ctx.dropout_p, ctx.philox_seed = dropout_p, seed
 
     @staticmethod
     @once_differentiable
@@ -185,8 +199,9 @@ class _DualCore(Function):
         dq, dk, dv, dqt, dkt, dvt = _lib.backend().bwd(
             q, k, v, q_t, k_t, v_t, o, o_t, M, mu, _dense(go), _dense(gt),
             ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale, want_tangent_grads=want_t,
+            dropout_p=ctx.dropout_p, dropout_seed=ctx.philox_seed,
         )
-        return dq, dk, dv, dqt, dkt, dvt, None, None, None, None
+        return dq, dk, dv, dqt, dkt, dvt, None, None, None, None, None, None
 
 
 class _PlainCore(Function):
@@ -195,17 +210,19 @@ class _PlainCore(Function):
     uses it while compiling."""
 
     @staticmethod
-    def forward(q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale):
-        o, _o_t, M, _mu = _lib.backend().fwd(q, k, v, None, None, None, mask_tensor, MASK_TYPE, causal, sm_scale)
+    def forward(q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p=0.0, seed=0):
+        o, _o_t, M, _mu = _lib.backend().fwd(q, k, v, None, None, None, mask_tensor, MASK_TYPE, causal, sm_scale,
+                                             dropout_p, seed)
         return o, M
 
     @staticmethod
     def setup_context(ctx, inputs, outputs):
-        q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale = inputs
+        q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p, seed = inputs
         o, M = outputs
         ctx.mark_non_differentiable(M)
         ctx.save_for_backward(q, k, v, o, M)
         ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale = mask_tensor, MASK_TYPE, causal, sm_scale
+        ctx.dropout_p, ctx.philox_seed = dropout_p, seed
 
     @staticmethod
     @once_differentiable
@@ -214,8 +231,9 @@ class _PlainCore(Function):
         dq, dk, dv, _, _, _ = _lib.backend().bwd(
             q, k, v, None, None, None, o, None, M, None, _dense(go), None,
             ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale,
+            dropout_p=ctx.dropout_p, dropout_seed=ctx.philox_seed,
         )
-        return dq, dk, dv, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None
 
 
 class _AttachTangent(Function):
@@ -247,11 +265,13 @@ class _AttachTangent(Function):
 
 class _DualCoreEager(Function):
     @staticmethod
-    def forward(ctx, q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale):
-        o, o_t, M, mu = _lib.backend().fwd(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale)
+    def forward(ctx, q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p=0.0, seed=0):
+        o, o_t, M, mu = _lib.backend().fwd(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale,
+                                           dropout_p, seed)
         ctx.mark_non_differentiable(M, mu)
         ctx.save_for_backward(q, k, v, q_t, k_t, v_t, o, o_t, M, mu)
         ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale = mask_tensor, MASK_TYPE, causal, sm_scale
+        ctx.dropout_p, ctx.philox_seed = dropout_p, seed
         return o, o_t, M, mu
 
     backward = _DualCore.backward
@@ -259,11 +279,13 @@ class _DualCoreEager(Function):
 
 class _PlainCoreEager(Function):
     @staticmethod
-    def forward(ctx, q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale):
-        o, _o_t, M, _mu = _lib.backend().fwd(q, k, v, None, None, None, mask_tensor, MASK_TYPE, causal, sm_scale)
+    def forward(ctx, q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p=0.0, seed=0):
+        o, _o_t, M, _mu = _lib.backend().fwd(q, k, v, None, None, None, mask_tensor, MASK_TYPE, causal, sm_scale,
+                                             dropout_p, seed)
         ctx.mark_non_differentiable(M)
         ctx.save_for_backward(q, k, v, o, M)
         ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale = mask_tensor, MASK_TYPE, causal, sm_scale
+        ctx.dropout_p, ctx.philox_seed = dropout_p, seed
         return o, M
 
     backward = _PlainCore.backward
@@ -388,11 +410,14 @@ class JVPAttn(Function):
             q_t = _dense(_unwrap(q_t))
             k_t = torch.zeros_like(k) if k_t is None else _dense(_unwrap(k_t))
             v_t = torch.zeros_like(v) if v_t is None else _dense(_unwrap(v_t))
-        o, o_t, M, _mu = _lib.backend().fwd(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale)
+        philox_seed = _new_dropout_seed(dropout_p)
+        o, o_t, M, _mu = _lib.backend().fwd(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale,
+                                            dropout_p, philox_seed)
         grid = JVPAttn.Grid((N_CTX + BLOCK_M - 1) // BLOCK_M, Z * H, 1)
         return JVPAttn.FwdOut(
             o,
-            JVPAttn.FwdOutCtxContrib(o_t, M, grid, HEAD_DIM_K, sm_scale, mask_tensor, MASK_TYPE, dropout_p, 0, False),
+            JVPAttn.FwdOutCtxContrib(o_t, M, grid, HEAD_DIM_K, sm_scale, mask_tensor, MASK_TYPE, dropout_p, philox_seed,
+                                     dropout_p > 0.0),
         )
 
     @staticmethod
@@ -428,12 +453,14 @@ class JVPAttn(Function):
         if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
             q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         if torch.compiler.is_compiling():
+            if dropout_p > 0.0:  # the seed is drawn on the host: such a call runs between two compiled pieces
+                return _fwd_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
             # the same computation through a Function the tracer can follow (no custom jvp, no
             # data-dependent mask checks); the kernels appear in the graph as jvpfa::fwd / jvpfa::bwd
             _validate(q, k, v, attn_mask, dropout_p, causal)
             scale = q.shape[-1] ** -0.5 if sm_scale is None else sm_scale
             mask_tensor, MASK_TYPE = _classify_mask(attn_mask, q, False)
-            o, _M = _PlainCore.apply(q, k, v, mask_tensor, MASK_TYPE, causal, scale)
+            o, _M = _PlainCore.apply(q, k, v, mask_tensor, MASK_TYPE, causal, scale, 0.0, 0)
             return o
         if fwAD._current_level < 0 and not _transforms_active():
             # no forward-mode level anywhere: nothing can ask for a tangent, so the plain Function
@@ -441,7 +468,8 @@ class JVPAttn(Function):
             _validate(q, k, v, attn_mask, dropout_p, causal)
             scale = q.shape[-1] ** -0.5 if sm_scale is None else sm_scale
             mask_tensor, MASK_TYPE = _classify_mask(attn_mask, q, True)
-            o, _M = _PlainCoreEager.apply(q, k, v, mask_tensor, MASK_TYPE, causal, scale)
+            o, _M = _PlainCoreEager.apply(q, k, v, mask_tensor, MASK_TYPE, causal, scale, dropout_p,
+                                          _new_dropout_seed(dropout_p))
             return o
         out: JVPAttn.FwdOut = JVPAttn.apply(
             q, k, v, None, None, None, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA
@@ -469,7 +497,7 @@ class JVPAttn(Function):
             # The tracer cannot follow the custom jvp that hands O' to forward-mode AD.  With a
             # forward-mode level active the call is therefore left out of the graph and runs as
             # ordinary Python between two compiled pieces; without one no tangent can exist.
-            if fwAD._current_level >= 0:
+            if fwAD._current_level >= 0 or dropout_p > 0.0:
                 return _fwd_dual_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
             return JVPAttn.fwd(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
         if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
@@ -489,7 +517,8 @@ class JVPAttn(Function):
         v_t = torch.zeros_like(v_p) if v_t is None else _dense(v_t)
         core, attach = (_DualCore, _AttachTangent) if _transforms_active() else (_DualCoreEager, _AttachTangentEager)
         o, o_t, _M, _mu = core.apply(
-            _dense(q_p), _dense(k_p), _dense(v_p), q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale
+            _dense(q_p), _dense(k_p), _dense(v_p), q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale,
+            dropout_p, _new_dropout_seed(dropout_p),
         )
         # NOTE: q, k, v are passed as dual tensors so that autograd calls jvp(), which hands back O'.
         return attach.apply(o, o_t, q, k, v)
@@ -515,8 +544,14 @@ class JVPAttn(Function):
         dq, dk, dv, _, _, _ = _lib.backend().bwd(
             q, k, v, None, None, None, o, None, M, None, do, None,
             ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale,
+            dropout_p=ctx.dropout_p, dropout_seed=ctx.philox_seed,
         )
         return JVPAttn.BwdOut(dq, dk, dv, None, None, None, None, None, None, None, None, None, None)
+
+
+@torch.compiler.disable
+def _fwd_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA):
+    return JVPAttn.fwd(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
 
 
 @torch.compiler.disable

@@ -20,6 +20,9 @@ Three independent statements of the same mathematics live here:
                (``:1384-1411``, ``:1415-1707``), plus the tangent-path backward
                the reference lacks.
 
+``dropout``    the keep pattern of the library's dropout (a hash of seed and entry index) in numpy; ``dense`` takes
+               the resulting matrix as ``keep_scale``.
+
 Pinning (what each function is checked against in ``tests/test_oracle.py``):
 
 * ``dense.forward`` / ``dense.backward`` vs ``sdpa_jvp`` (library routine) in
@@ -31,6 +34,9 @@ Pinning (what each function is checked against in ``tests/test_oracle.py``):
 * invariants: rows of P' sum to zero (constant V, V'=0 gives O'=0), O' is
   linear in the tangents, the gT=0 backward reduces to the reference's
   first-order backward formulas (``jvp_attention.py:1541-1553``, ``:1687-1697``);
+* ``dense`` with ``keep_scale`` vs torch's softmax times a fixed matrix under ``torch.func.jvp`` and
+  ``autograd.grad`` (SDPA's definition of dropout written out), all mask modes; ``dropout`` vs the bijectivity
+  and statistics the mix must have on the CPU, and bit for bit vs the pattern the library exports on the GPU;
 * ``tiled`` vs ``dense`` for every tile size that divides L and for ragged L.
 
 Parity unpinned by the reference itself: the tangent-path gradients

@@ -25,6 +25,13 @@ Backward for ``Loss = <gO, O> + <gT, O'>`` (the gT = 0 case is the reference's
     dS  = dS1 + dS2
     dQ = scale (dS K + dS' K')   dK = scale (dS^T Q + dS'^T Q')   dV = P^T gO + P'^T gT
     dQ' = scale dS' K            dK' = scale dS'^T Q              dV' = P^T gT
+
+Dropout (dead code in the reference, ``:94-122``, ``:271-277``, which raises for ``dropout_p > 0`` at
+``:2356-2357``; semantics here are SDPA's): a fixed matrix W = keep / (1 - p) multiplies the probabilities
+wherever they meet V or V' and nowhere else, so mu stays the undropped ``rowsum(P * S')``:
+
+    O = (P*W) V      O' = (P'*W) V + (P*W) V'
+    backward: gO V^T, A and B are multiplied by W; dV = (P*W)^T gO + (P'*W)^T gT; dV' = (P*W)^T gT
 """
 from __future__ import annotations
 
@@ -76,51 +83,53 @@ def _softmax(s, keep):
     return p, lse2[..., 0]
 
 
-def forward(q, k, v, qt=None, kt=None, vt=None, mask=None, causal=False, scale=None):
-    """Returns dict with O, M and (when tangents are given) O', mu, plus P, S' for reuse."""
+def forward(q, k, v, qt=None, kt=None, vt=None, mask=None, causal=False, scale=None, keep_scale=None):
+    """Returns dict with O, M and (when tangents are given) O', mu, plus P, S' for reuse.  ``keep_scale`` is
+    the dropout matrix W (broadcastable to Z, H, Lq, Lk), ``None`` for no dropout."""
     q, k, v = (np.asarray(x, dtype=np.float64) for x in (q, k, v))
     D, H = q.shape[-1], q.shape[1]
     k, v = _expand_heads(k, H), _expand_heads(v, H)
     scale = D**-0.5 if scale is None else scale
     s, keep = _logits(q, k, mask, causal, scale)
     p, M = _softmax(s, keep)
-    out = {"O": p @ v, "M": M, "P": p, "scale": scale}
+    w = 1.0 if keep_scale is None else np.broadcast_to(np.asarray(keep_scale, dtype=np.float64), p.shape)
+    out = {"O": (p * w) @ v, "M": M, "P": p, "scale": scale, "W": w}
     if qt is not None:
         qt, kt, vt = (np.asarray(x, dtype=np.float64) for x in (qt, kt, vt))
         kt, vt = _expand_heads(kt, H), _expand_heads(vt, H)
         sp = scale * (np.einsum("zhid,zhjd->zhij", qt, k) + np.einsum("zhid,zhjd->zhij", q, kt))
         mu = (p * sp).sum(-1, keepdims=True)
         pp = p * (sp - mu)
-        out.update({"Ot": pp @ v + p @ vt, "mu": mu[..., 0], "Sp": sp, "Pp": pp})
+        out.update({"Ot": (pp * w) @ v + (p * w) @ vt, "mu": mu[..., 0], "Sp": sp, "Pp": pp})
     return out
 
 
-def backward(q, k, v, qt, kt, vt, go, gt=None, mask=None, causal=False, scale=None):
+def backward(q, k, v, qt, kt, vt, go, gt=None, mask=None, causal=False, scale=None, keep_scale=None):
     """Six gradients of <gO,O> + <gT,O'>.  ``gt=None`` means gT = 0."""
     if qt is None:
         qt, kt, vt = (np.zeros_like(np.asarray(x, dtype=np.float64)) for x in (q, k, v))
-    f = forward(q, k, v, qt, kt, vt, mask=mask, causal=causal, scale=scale)
+    f = forward(q, k, v, qt, kt, vt, mask=mask, causal=causal, scale=scale, keep_scale=keep_scale)
     q, k, v, qt, kt, vt, go = (np.asarray(x, dtype=np.float64) for x in (q, k, v, qt, kt, vt, go))
     H, Hk = q.shape[1], k.shape[1]
     k, v, kt, vt = (_expand_heads(x, H) for x in (k, v, kt, vt))
-    p, sc = f["P"], f["scale"]
+    p, sc, w = f["P"], f["scale"], f["W"]
     T = lambda x: np.swapaxes(x, -1, -2)  # noqa: E731
     d1 = (go * f["O"]).sum(-1, keepdims=True)
-    ds = p * (go @ T(v) - d1)
-    dv = T(p) @ go
+    ds = p * (w * (go @ T(v)) - d1)
+    dv = T(p * w) @ go
     dsp = np.zeros_like(p)
     dvt = np.zeros_like(v)
     if gt is not None:
         gt = np.asarray(gt, dtype=np.float64)
         sp, mu = f["Sp"], f["mu"][..., None]
-        A = gt @ T(v)
-        B = gt @ T(vt)
+        A = w * (gt @ T(v))
+        B = w * (gt @ T(vt))
         a = (gt * f["O"]).sum(-1, keepdims=True)
         d2 = (gt * f["Ot"]).sum(-1, keepdims=True) - a * mu
         ds = ds + p * (B + A * (sp - mu) - a * sp - d2)
         dsp = p * (A - a)
-        dv = dv + T(f["Pp"]) @ gt
-        dvt = T(p) @ gt
+        dv = dv + T(f["Pp"] * w) @ gt
+        dvt = T(p * w) @ gt
     return {
         "dq": sc * (ds @ k + dsp @ kt),
         "dk": _reduce_heads(sc * (T(ds) @ q + T(dsp) @ qt), Hk),

@@ -125,6 +125,7 @@ def test_apply_returns_output_and_context_tuple_and_13_slot_backward():
         c = Ctx()
         c.saved_tensors = (q, k, v, o, ctx.M)
         c.mask_tensor, c.MASK_TYPE, c.causal, c.sm_scale = ctx.mask_tensor, 0, False, ctx.sm_scale
+        c.dropout_p, c.philox_seed, c.ENABLE_DROPOUT = ctx.dropout_p, ctx.philox_seed, ctx.ENABLE_DROPOUT  # JA:2696-2698
         res = JVPAttn.backward(c, go, None)
     assert isinstance(res, JVPAttn.BwdOut) and all(x is None for x in res[3:]) and all(x is not None for x in res[:3])
 
@@ -132,8 +133,13 @@ def test_apply_returns_output_and_context_tuple_and_13_slot_backward():
 def test_argument_errors_match_the_reference():
     q, k, v, *_ = _inputs()
     with oracle_backend():
-        with pytest.raises(NotImplementedError):
-            attention(q, k, v, dropout_p=0.1)
+        with pytest.raises(AssertionError):
+            attention(q, k, v, dropout_p=1.0)
+        with pytest.raises(AssertionError):
+            attention(q, k, v, dropout_p=-0.1)
+        with pytest.raises(NotImplementedError):  # dropout stops at head dim 128
+            x = torch.randn(1, 1, 16, 256, dtype=torch.float64)
+            attention(x, x, x, dropout_p=0.1)
         with pytest.raises(ValueError):
             attention(q, k, v, attn_mask=torch.ones(1, 2, 32, 32, dtype=torch.bool), causal=True)
         with pytest.raises(AssertionError):
@@ -305,3 +311,42 @@ def test_forget_mask_drops_what_was_remembered():
     _lib.forget_mask(mask)
     assert not ja._already_verified(mask)
     assert _lib.key_limit_hint(mask, _lib.MASK_BOOL, 2, L).tolist() == [L, 7]
+
+
+def test_dropout_draws_one_seed_per_call_and_replays_it_in_the_backward():
+    """dropout_p > 0 (the reference raises, jvp_attention.py:2356-2357): the forward draws a seed from torch's
+    CPU generator, the backward of the same call gets that seed again, and the results are those of SDPA's
+    dropout with that pattern, tangent and tangent-path gradients included."""
+    from oracle import dense, dropout
+
+    q, k, v, qt, kt, vt, go, gt = _inputs()
+    Z, H, L, _ = q.shape
+    with oracle_backend() as fake:
+        torch.manual_seed(11)
+        leaves = [t.clone().requires_grad_() for t in (q, k, v, qt, kt, vt)]
+        with fwAD.dual_level():
+            duals = [fwAD.make_dual(p, t) for p, t in zip(leaves[:3], leaves[3:])]
+            o, ot = fwAD.unpack_dual(attention(*duals, dropout_p=0.25))
+            ((o * go).sum() + (ot * gt).sum()).backward()
+        fwd_calls = [c for c in fake.calls if c[0] == "fwd"]
+        bwd_calls = [c for c in fake.calls if c[0] == "bwd"]
+        assert len(fwd_calls) == 1 and len(bwd_calls) == 1
+        p, seed = fwd_calls[0][-2:]
+        assert p == 0.25 and 0 <= seed < 2**62 and bwd_calls[0][-2:] == (p, seed)
+        W = dropout.keep_scale(Z, H, L, L, p, seed)
+        xs = [x.numpy() for x in (q, k, v, qt, kt, vt)]
+        f = dense.forward(*xs, keep_scale=W)
+        b = dense.backward(*xs, go.numpy(), gt.numpy(), keep_scale=W)
+        _close(o.detach(), torch.from_numpy(f["O"]))
+        _close(ot.detach(), torch.from_numpy(f["Ot"]))
+        for leaf, name in zip(leaves, ("dq", "dk", "dv", "dqt", "dkt", "dvt")):
+            _close(leaf.grad, torch.from_numpy(b[name]))
+        # same generator state, same pattern; another call, another pattern; plain path and apply() carry it too
+        torch.manual_seed(11)
+        o2 = attention(q, k, v, dropout_p=0.25)
+        _close(o2, o.detach())
+        o3 = attention(q, k, v, dropout_p=0.25)
+        assert (o3 - o2).abs().max() > 1e-3
+        out, ctx = JVPAttn.apply(q, k, v, None, None, None, None, 0.25, False, None, True, True)
+        assert ctx.dropout_p == 0.25 and ctx.ENABLE_DROPOUT and ctx.philox_seed == fake.calls[-1][-1]
+        assert torch.equal(attention(q, k, v, dropout_p=0.0), attention(q, k, v))

@@ -218,3 +218,66 @@ def test_config1_cpu_plumbing_fp32():
     assert (ot - ot_ref).abs().max() < 1e-4
     for name, ref in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
         assert (gr[name] - ref).abs().max() < 2e-4 * max(1.0, ref.abs().max().item()), name
+
+
+def _dropout_route(q, k, v, qt, kt, vt, go, gt, W, mask, causal):
+    """O, O' and the six gradients with a fixed dropout matrix W, by torch's softmax under ``torch.func.jvp`` and
+    ``autograd.grad``: SDPA's definition of dropout (``softmax(S) * keep / (1 - p) @ V``) written out, since the
+    library's own dropout draws a pattern nobody else can see."""
+    L, Lk = q.shape[-2], k.shape[-2]
+
+    def attn(a, b, c):
+        s = a @ b.transpose(-1, -2) * a.shape[-1] ** -0.5
+        if causal:
+            s = s.masked_fill(~torch.ones(L, Lk, dtype=torch.bool).tril(), -math.inf)
+        if mask is not None:
+            s = s.masked_fill(~mask, -math.inf) if mask.dtype == torch.bool else s + mask
+        return (torch.softmax(s, -1) * W) @ c
+
+    leaves = [t.detach().clone().requires_grad_(True) for t in (q, k, v, qt, kt, vt)]
+    o, ot = torch.func.jvp(attn, tuple(leaves[:3]), tuple(leaves[3:]))
+    loss = (o * go).sum() + ((ot * gt).sum() if gt is not None else 0.0)
+    grads = torch.autograd.grad(loss, leaves, allow_unused=True)
+    return o.detach(), ot.detach(), [torch.zeros_like(x) if g is None else g for g, x in zip(grads, leaves)]
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("with_gt", [True, False])
+def test_dense_with_dropout_matches_the_library_route(mode, with_gt):
+    from oracle import dropout
+
+    Z, H, L = 2, 2, 32
+    q, k, v, qt, kt, vt, go, gt = _inputs()
+    gt = gt if with_gt else None
+    mask, causal = _masks(Z, H, L)[mode]
+    W = dropout.keep_scale(Z, H, L, L, 0.3, seed=1234567890123)
+    assert 0.55 < (W != 0).mean() < 0.85 and np.allclose(W[W != 0], 1 / (1 - np.float32(0.3)))
+    o, ot, grads = _dropout_route(q, k, v, qt, kt, vt, go, gt, torch.from_numpy(W), mask, causal)
+    npm = None if mask is None else mask.numpy()
+    xs = [x.numpy() for x in (q, k, v, qt, kt, vt)]
+    f = dense.forward(*xs, mask=npm, causal=causal, keep_scale=W)
+    b = dense.backward(*xs, go.numpy(), None if gt is None else gt.numpy(), mask=npm, causal=causal, keep_scale=W)
+    assert np.abs(f["O"] - o.numpy()).max() < 1e-12
+    assert np.abs(f["Ot"] - ot.numpy()).max() < 1e-12
+    for name, ref in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        assert np.abs(b[name] - ref.numpy()).max() < 1e-11, name
+
+
+def test_dropout_pattern_properties():
+    """What the mathematics fixes about the pattern: the mix is a bijection of the low index word for a fixed
+    seed (so no value is favoured), the kept fraction is 1 - p, seeds and rows decorrelate, p = 0 keeps all."""
+    from oracle import dropout
+
+    idx = np.arange(1 << 16, dtype=np.uint64)
+    assert len(np.unique(dropout.mix(idx, 99))) == 1 << 16
+    for p in (0.1, 0.5, 0.9):
+        kp = dropout.keep(2, 3, 64, 128, p, seed=7)
+        assert abs(kp.mean() - (1 - p)) < 0.01
+        assert abs(kp[0, 0].mean(axis=-1) - (1 - p)).max() < 0.2  # every row has its own draw
+    a, b = dropout.keep(1, 1, 64, 64, 0.5, 1), dropout.keep(1, 1, 64, 64, 0.5, 2)
+    assert 0.4 < (a != b).mean() < 0.6
+    assert 0.4 < (a[..., 1:, :] != a[..., :-1, :]).mean() < 0.6
+    hi = dropout.mix(np.array([5, 5 + (1 << 32)], dtype=np.uint64), 3)
+    assert hi[0] != hi[1]  # the high index word takes part
+    assert dropout.keep(1, 1, 4, 4, 0.0, 5).all() and dropout.keep_scale(1, 1, 4, 4, 0.0, 5) is None
+    assert dropout.threshold(0.5) == 1 << 31 and dropout.threshold(1e-12) == 1
