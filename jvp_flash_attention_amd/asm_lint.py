@@ -11,6 +11,14 @@ slots that the hardware needs
    tile, or ``v_accvgpr_read_b32`` reading an accumulator: the compiler may schedule the epilogue's reads in front
    of a wait that is not tied to the registers).
 
+Likewise for the LDS reads issued through inline asm (``ds_read_b128``, ``ds_read_b64_tr_b16``): to the
+compiler the destination holds its value as soon as the statement is over, while the hardware delivers it
+some cycles later, and only the ``s_waitcnt lgkmcnt`` that the sources tie to the register (``lds_wait``)
+says when.  Under register pressure the allocator has been seen to give several such reads one destination
+and to copy each result away at once, in front of the wait: the copy holds whatever the register held before.
+
+3. No instruction may read a register while an inline-asm LDS read into it is still in flight.
+
 The sources provide those slots themselves (``s_nop 1`` in front of the matrix instructions whose
 operands live long enough to be parked, ``tiles_ready()`` = ``s_nop 15; s_nop 3`` after each group).
 ``scan()`` checks the ISA text of a translation unit for both; ``build()`` runs it on every kernel unit it
@@ -44,10 +52,11 @@ def scan(isa_text: str, where: str = "") -> list[str]:
     """Findings (one line each) in the ISA text of one translation unit."""
     out = []
     kern, inasm, hist, pending = "?", False, [], set()
+    flying: list[set] = []  # destinations of the inline-asm LDS reads in flight, oldest first
     for ln in isa_text.splitlines():
         t = ln.strip()
         if t.startswith("_Z") and ":" in t and "$" not in t.split(":")[0]:
-            kern, hist, pending = t.split(":")[0], [], set()
+            kern, hist, pending, flying = t.split(":")[0], [], set(), []
             continue
         if "ASMSTART" in t:
             inasm = True
@@ -64,6 +73,21 @@ def scan(isa_text: str, where: str = "") -> list[str]:
         ops = [x.strip() for x in t.split(None, 1)[1].split(",")] if " " in t else []
         if op == "s_nop" and ops and int(ops[0]) >= 15:
             pending = set()  # tiles_ready(): results of the group are readable from here on
+        if op.startswith("ds_read") and inasm:
+            flying.append(_regs(ops[0]))
+            hist.append((op, ops))
+            continue
+        if op == "s_waitcnt":
+            m = re.search(r"lgkmcnt\((\d+)\)", t)
+            if m:  # LDS reads return in order: the N youngest may still be in flight
+                n = int(m.group(1))
+                flying = flying[len(flying) - n:] if n and n < len(flying) else ([] if n == 0 else flying)
+        elif flying and op.startswith(("v_", "ds_", "global_", "buffer_", "scratch_")):
+            srcs = set()
+            for o in (ops[1:] if op.startswith("v_") else ops):
+                srcs |= _regs(o)
+            if any(srcs & f for f in flying):
+                out.append(f"{where} {kern}: '{t[:60]}' reads the destination of an LDS read that is still in flight")
         if op.startswith("v_mfma"):
             dst, srcs = _regs(ops[0]), set()
             for o in ops[1:4]:

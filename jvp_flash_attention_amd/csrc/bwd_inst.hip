@@ -9,8 +9,21 @@
 
 namespace jvpfa {
 
+// Which of the tangent-input gradients the dual kernels of the direct-to-LDS family produce on the way when
+// all six gradients are asked for (dq' costs the dq kernel one more product per tile and dk', dv' the dk/dv
+// kernel two, against a second pair of launches that forms the score tiles again): dq' wherever that family
+// runs; dk', dv' where the two extra accumulators fit (D <= 64; at D = 64 that kernel then has a compute unit
+// to itself instead of sharing it with a second workgroup and is still 4 - 9 % ahead; at D = 128 dK, dV, the
+// resident K, V, K' and the tiles already take 452 of the 512 registers and dK', dV' would add 128).
+template <typename T, int D> struct BwdFold {
+  static constexpr bool DQ = sizeof(T) == 2 && D <= 128;
+  static constexpr bool KV = sizeof(T) == 2 && D <= 64;
+};
+
+// six: all six gradients were asked for.  The dual launch then also writes what BwdFold says, and the tangent
+// launch skips the kernels whose outputs exist already.
 template <typename T, int D, int MODE, int MASK>
-static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
+static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
   using Cfg = BwdCfg<T, D, MODE>;
   const int nb = (p.pr.L + BWD_BLK - 1) / BWD_BLK;
   const long long blocks = (long long)nb * p.pr.Z * p.pr.H;
@@ -41,9 +54,29 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
     constexpr bool NG = MODE != BWD_DUAL;  // the GO template argument of the kernels without gO
     void (*kq)(const BwdParams), (*kkv)(const BwdParams);
     const bool grouped = p.pr.Hk != p.pr.H;  // a key/value head serves several query heads
+    using Fold = BwdFold<T, D>;
+    bool run_q = true, run_kv = true;
+    if constexpr (MODE == BWD_TANGENT) {
+      run_q = !(six && Fold::DQ);
+      run_kv = !(six && Fold::KV);
+    }
+    if constexpr (MODE == BWD_DUAL) {
+      if (six) {  // the variants that also write dq' (and dk', dv')
+        // (without gO the register cap of the two-workgroup twin makes the allocator copy LDS fragments out of
+        // their registers before they have arrived, which the build's lint refuses: that variant runs uncapped)
+        if constexpr (D == 64) kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, false, true> : bwd2_dq_kernel_2wg<T, D, MODE, MASK, true, true>;
+        else kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, false, true> : bwd2_dq_kernel<T, D, MODE, MASK, true, true>;
+        if constexpr (Fold::KV) {
+          if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, false, true, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true, true>;
+          else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, false, false, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, false, true>;
+        }
+      }
+    }
+    const bool plain_q = !(MODE == BWD_DUAL && six), plain_kv = !(MODE == BWD_DUAL && six && Fold::KV);
     if constexpr (D == 64) {  // the register-capped twins: two workgroups per compute unit (D = 32 needs no cap for that)
-      kq = no_go ? bwd2_dq_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dq_kernel_2wg<T, D, MODE, MASK, true>;
-      if constexpr (MASK == MASK_NONE || MODE != BWD_DUAL) {
+      if (plain_q) kq = no_go ? bwd2_dq_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dq_kernel_2wg<T, D, MODE, MASK, true>;
+      if (!plain_kv) {
+      } else if constexpr (MASK == MASK_NONE || MODE != BWD_DUAL) {
         if (grouped) kkv = no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, true, true>;
         else kkv = no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, true>;
       } else {  // the masked dual dk/dv kernel needs a few registers more than the cap leaves
@@ -51,15 +84,16 @@ static int launch_bwd_mode(const BwdParams &p, hipStream_t stream) {
         else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
       }
     } else {
-      kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG> : bwd2_dq_kernel<T, D, MODE, MASK, true>;
-      if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true>;
+      if (plain_q) kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG> : bwd2_dq_kernel<T, D, MODE, MASK, true>;
+      if (!plain_kv) {
+      } else if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true>;
       else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
     }
     int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
     if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);
     if (rc != 0) return rc;
-    hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
-    hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
+    if (run_kv) hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
+    if (run_q) hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
    }
   } else if constexpr (sizeof(T) == 2 && D == 256) {
@@ -112,9 +146,9 @@ static int launch_bwd_mask(const BwdParams &p, bool dual, bool tangent_grads, hi
   hipLaunchKernelGGL((bwd_prepass_kernel<T, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(BWD_NT), 0,
                      stream, p, rows, dual ? 1 : 0);
   if (hipGetLastError() != hipSuccess) return -6;
-  if (!dual) return launch_bwd_mode<T, D, BWD_PLAIN, MASK>(p, stream);
-  int rc = launch_bwd_mode<T, D, BWD_DUAL, MASK>(p, stream);
-  if (rc == 0 && tangent_grads) rc = launch_bwd_mode<T, D, BWD_TANGENT, MASK>(p, stream);
+  if (!dual) return launch_bwd_mode<T, D, BWD_PLAIN, MASK>(p, false, stream);
+  int rc = launch_bwd_mode<T, D, BWD_DUAL, MASK>(p, tangent_grads, stream);
+  if (rc == 0 && tangent_grads) rc = launch_bwd_mode<T, D, BWD_TANGENT, MASK>(p, true, stream);
   return rc;
 }
 

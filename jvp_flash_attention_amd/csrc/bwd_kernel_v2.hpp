@@ -134,10 +134,12 @@ __device__ __forceinline__ void zero_acc(f32x16 &x) {
 // dq (PLAIN / DUAL) or dq' (TANGENT): workgroup = 128 query rows, loop over 64-key tiles of
 // K, V (, K', V').  Scores are transposed (lane = query) so dS is the B operand of dQ^T += K^T dS^T.
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stubs (and has no buffer descriptor type)
-template <typename T, int D, int MODE, int MASK, bool GO>
+// SIX (dual mode only): dq' = scale dS' K as well, from the K fragments and the dS' tiles that dq already has.
+template <typename T, int D, int MODE, int MASK, bool GO, bool SIX>
 __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
+  static_assert(!SIX || DUAL, "dq' rides on the dual mode");
   JVPFA_BWD2_COMMON(Cfg, pr.Lk, pr.L, pr.H)  // owns query rows, streams key tiles
   const int qb = pr.causal ? nblk - 1 - id % nblk : id % nblk;
   const int q0 = qb * Cfg::BLK;
@@ -152,11 +154,13 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   }
   if constexpr (DUAL) load_bfrags<KK>(Qtf, reinterpret_cast<const T *>(p.qt) + head + (size_t)qld * D, g);
   if constexpr (DUAL || TAN) load_bfrags<KK>(gTf, reinterpret_cast<const T *>(p.gt) + head + (size_t)qld * D, g);
-  // the resident operands live in the accumulation register file from here on
+  // the resident operands live in the accumulation register file from here on (with dq' at D = 128 that
+  // file is full with the two accumulators and three of them: gO stays in vector registers)
+  constexpr bool GO_V = SIX && D == 128;
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) {
     pin_acc(Qf[kk]);
-    if constexpr (!TAN && has_go) pin_acc(gOf[kk]);
+    if constexpr (!TAN && has_go && !GO_V) pin_acc(gOf[kk]);
     if constexpr (DUAL) pin_acc(Qtf[kk]);
     if constexpr (DUAL || TAN) pin_acc(gTf[kk]);
   }
@@ -167,9 +171,12 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
   const float av = (DUAL || TAN) ? p.a[srow + qld] : 0.f;
   const float dsum = DUAL ? p.d2[srow + qld] : 0.f;
 
-  f32x16 acc[DB];
+  f32x16 acc[DB], accT[SIX ? DB : 1];
 #pragma unroll
-  for (int db = 0; db < DB; ++db) zero_acc(acc[db]);
+  for (int db = 0; db < DB; ++db) {
+    zero_acc(acc[db]);
+    if constexpr (SIX) zero_acc(accT[db]);
+  }
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
@@ -265,7 +272,8 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
       if constexpr (MODE == BWD_PLAIN) mma_vra<F>(dP, v_, gOf[kk]);
       if constexpr (TAN) mma_vra<F>(At, v_, gTf[kk]);
       if constexpr (DUAL) {
-        if constexpr (has_go) mma_vra<F>(dP, v_, gOf[kk]);
+        if constexpr (has_go && GO_V) mma_vrv<F>(dP, v_, gOf[kk]);
+        else if constexpr (has_go) mma_vra<F>(dP, v_, gOf[kk]);
         mma_vra<F>(Sp, k_, Qtf[kk]);
         mma_vra<F>(At, v_, gTf[kk]);
         mma_vra<false>(Sp, as_frag<T>(fkt[sl]), Qf[kk]);
@@ -352,6 +360,10 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
 #pragma unroll
         for (int u = 0; u < PW; ++u) mma(acc[PW * dp + u], as_frag<T>(tkt[sl][u]), dspf[c]);
       }
+      if constexpr (SIX) {
+#pragma unroll
+        for (int u = 0; u < PW; ++u) mma(accT[PW * dp + u], as_frag<T>(tk[sl][u]), dspf[c]);
+      }
     });
   };
 
@@ -420,23 +432,28 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) x[e] = acc[db][8 * hf + e] * pr.scale;
         store8<T>(out + 32 * db + 16 * hf + 8 * g, x);
+        if constexpr (SIX) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[e] = accT[db][8 * hf + e] * pr.scale;
+          store8<T>(reinterpret_cast<T *>(p.dqt) + head + (size_t)qrow * D + 32 * db + 16 * hf + 8 * g, x);
+        }
       }
     }
   }
 }
 #endif
-template <typename T, int D, int MODE, int MASK, bool GO>
+template <typename T, int D, int MODE, int MASK, bool GO, bool SIX = false>
 __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dq_body<T, D, MODE, MASK, GO>(p);
+  bwd2_dq_body<T, D, MODE, MASK, GO, SIX>(p);
 #endif
 }
 // The same code with the vector registers capped, for D = 64: together with the accumulation registers
 // the kernel then needs at most 256 registers and two workgroups share a compute unit.
-template <typename T, int D, int MODE, int MASK, bool GO>
+template <typename T, int D, int MODE, int MASK, bool GO, bool SIX = false>
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(160))) void bwd2_dq_kernel_2wg(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dq_body<T, D, MODE, MASK, GO>(p);
+  bwd2_dq_body<T, D, MODE, MASK, GO, SIX>(p);
 #endif
 }
 
@@ -447,10 +464,13 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(160))) void 
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stubs (and has no buffer descriptor type)
 // GROUPED: the key/value head serves several query heads (compiled apart, so that the common case of
 // one keeps its pointers loop-invariant).
-template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED>
+// SIX (dual mode only): dk' = scale dS'^T Q and dv' = P^T gT as well, from the fragments and tiles that dk, dv
+// already have (two more accumulators: fits for D <= 64).
+template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED, bool SIX>
 __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
+  static_assert(!SIX || (DUAL && D <= 64), "dk', dv' ride on the dual mode, where the accumulators fit");
   JVPFA_BWD2_COMMON(Cfg, pr.L, pr.Lk, pr.Hk)  // owns key rows (h: key/value head), streams query tiles
   const int kb = id % nblk;  // causal: the first key blocks have the longest query loops
   const int k0 = kb * Cfg::BLK;
@@ -468,6 +488,10 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
         for (int d0 = 8 * g; d0 < D; d0 += 16) {
           store8<T>(outk + d0, zero8);
           store8<T>(outv + d0, zero8);
+          if constexpr (SIX) {
+            store8<T>(reinterpret_cast<T *>(p.dkt) + head + (size_t)krow * D + d0, zero8);
+            store8<T>(reinterpret_cast<T *>(p.dvt) + head + (size_t)krow * D + d0, zero8);
+          }
         }
       }
       return;
@@ -493,11 +517,15 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
     }
   }
 
-  f32x16 dK[DB], dV[DB];
+  f32x16 dK[DB], dV[DB], dKt[SIX ? DB : 1], dVt[SIX ? DB : 1];
 #pragma unroll
   for (int db = 0; db < DB; ++db) {
     zero_acc(dK[db]);
     zero_acc(dV[db]);
+    if constexpr (SIX) {
+      zero_acc(dKt[db]);
+      zero_acc(dVt[db]);
+    }
   }
 
   const float sl2 = pr.scale * LOG2E;
@@ -785,6 +813,10 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
           if constexpr (has_go) mma(dV[db], as_frag<T>(tg[sl]), pf);
           mma(dK[db], as_frag<T>(tqt[sl]), dspf);
           mma(dV[db], as_frag<T>(tgt[sl]), ppf);
+          if constexpr (SIX) {
+            mma(dKt[db], as_frag<T>(tq[sl]), dspf);
+            mma(dVt[db], as_frag<T>(tgt[sl]), pf);
+          }
         } else {
           mma(dK[db], as_frag<T>(tq[sl]), dspf);
           mma(dV[db], as_frag<T>(tg[sl]), pf);
@@ -853,15 +885,25 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
         }
         store8<T>(outk + 32 * db + 16 * hf + 8 * g, xk);
         store8<T>(outv + 32 * db + 16 * hf + 8 * g, xv);
+        if constexpr (SIX) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            xk[e] = dKt[db][8 * hf + e] * pr.scale;
+            xv[e] = dVt[db][8 * hf + e];
+          }
+          const size_t o = head + (size_t)krow * D + 32 * db + 16 * hf + 8 * g;
+          store8<T>(reinterpret_cast<T *>(p.dkt) + o, xk);
+          store8<T>(reinterpret_cast<T *>(p.dvt) + o, xv);
+        }
       }
     }
   }
 }
 #endif
-template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED = false>
+template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED = false, bool SIX = false>
 __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED>(p);
+  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED, SIX>(p);
 #endif
 }
 // The same code with the vector registers capped, for D = 64: together with the accumulation registers
@@ -869,7 +911,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
 template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED = false>
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(144))) void bwd2_dkdv_kernel_2wg(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED>(p);
+  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED, false>(p);
 #endif
 }
 

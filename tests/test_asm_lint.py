@@ -81,3 +81,29 @@ def test_compiled_kernels_are_clean():
                 assert asm_lint.scan(f.read(), n) == []
     else:
         assert asm_lint.lint(["bwd_bf16_32", "fwd_bf16_64"]) == []
+
+
+COPY_BEFORE_ARRIVAL = """
+_ZN5jvpfa4kernEv:
+	;;#ASMSTART
+	ds_read_b64_tr_b16 v[64:65], v109 offset:4096
+	;;#ASMEND
+	;;#ASMSTART
+	ds_read_b64_tr_b16 v[66:67], v110 offset:4096
+	;;#ASMEND
+	v_mov_b64_e32 v[104:105], v[66:67]
+	;;#ASMSTART
+	s_waitcnt lgkmcnt(0)
+	;;#ASMEND
+	v_mov_b64_e32 v[102:103], v[64:65]
+"""
+
+
+def test_a_copy_of_an_lds_fragment_made_before_it_has_arrived_is_flagged():
+    found = asm_lint.scan(COPY_BEFORE_ARRIVAL, "unit")
+    assert len(found) == 1 and "still in flight" in found[0] and "v[104:105]" in found[0]
+    # a wait that leaves only the younger read in flight frees the older destination
+    partly = COPY_BEFORE_ARRIVAL.replace("\tv_mov_b64_e32 v[104:105], v[66:67]\n",
+                                         "\t;;#ASMSTART\n\ts_waitcnt lgkmcnt(1)\n\t;;#ASMEND\n\tv_mov_b64_e32 v[100:101], v[64:65]\n")
+    assert asm_lint.scan(partly, "unit") == []
+    assert len(asm_lint.scan(partly.replace("v[100:101], v[64:65]", "v[100:101], v[66:67]"), "unit")) == 1

@@ -398,6 +398,34 @@ def test_only_tangent_gradient_hvp_style():
         _tol_check(n, t, rb[n], torch.bfloat16)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("mode", ["causal", "bool_full"])
+def test_all_six_gradients_without_gO(dt, D, mode):
+    """gO absent and all six gradients asked for: the dual kernels that also write dq' (and dk', dv' for D = 32)
+    in their variant without gO, with grouped heads so that the dk/dv kernel adds up over the heads of a group."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    dtype = DTYPES[dt]
+    Z, H, Hk, L = 2, 4, 2, 200
+    q, k, v, qt, kt, vt, go, gt = _make(Z, H, L, D, dtype, 9)
+    k, v, kt, vt = (x[:, :Hk].contiguous() for x in (k, v, kt, vt))
+    mask = _mask(mode, Z, H, L, dtype)
+    causal = mode == "causal"
+    kind = _lib.MASK_NONE if mask is None else _lib.MASK_BOOL
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt)]
+    dmask = None if mask is None else mask.cuda()
+    print(f"six gradients without gO {dt} D{D} {mode}", flush=True)
+    o, ot, M, mu = be.fwd(*dev, dmask, kind, causal, D**-0.5)
+    grads = be.bwd(*dev, o, ot, M, mu, None, gt.cuda(), dmask, kind, causal, D**-0.5, want_tangent_grads=True)
+    rb = dense.backward(*f64, np.zeros(q.shape), gt.double().numpy(), mask=None if mask is None else mask.numpy(),
+                        causal=causal, scale=D**-0.5)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        _tol_check(n, t, rb[n], dtype)
+
+
 @pytest.mark.parametrize("dt", ["bf16", "fp32"])
 def test_single_key(dt):
     """L = 1: softmax is the constant 1, so O = v, O' = v' and dq = dk = dq' = dk' = 0 exactly.
