@@ -6,6 +6,7 @@
 #include "bwd_kernel_v2.hpp"
 #include "bwd_kernel_wide.hpp"
 #include "launch.hpp"
+#include "split.hpp"
 
 namespace jvpfa {
 
@@ -88,6 +89,16 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
       if (!plain_kv) {
       } else if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true>;
       else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
+    }
+    // a grid smaller than the GPU: both roles in one launch, side by side
+    const int cus = device_cus();
+    if (!grouped && !six && blocks < cus && kv_blocks < cus) {
+      void (*kb)(const BwdParams, int) = no_go ? bwd2_both_kernel<T, D, MODE, MASK, NG> : bwd2_both_kernel<T, D, MODE, MASK, true>;
+      constexpr size_t LDS = Cfg2::DKV_LDS > Cfg2::DQ_LDS ? Cfg2::DKV_LDS : Cfg2::DQ_LDS;
+      const int rcb = allow_lds(reinterpret_cast<const void *>(kb), LDS);
+      if (rcb != 0) return rcb;
+      hipLaunchKernelGGL(kb, dim3((unsigned)(kv_blocks + blocks)), dim3(Cfg2::NT), LDS, stream, p, (int)kv_blocks);
+      return hipGetLastError() == hipSuccess ? 0 : -6;
     }
     int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
     if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);

@@ -68,7 +68,7 @@ constexpr int bwd_spread(int nstep) { return 3 * nstep / 4; }
   const int L = pr.L;                                                                                               \
   /* a workgroup owns 128 of the OWN_ROWS rows of one (z, head out of OWN_HEADS) */                               \
   const int nblk = ((OWN_ROWS) + Cfg::BLK - 1) / Cfg::BLK;                                                          \
-  const int id = xcd_remap(blockIdx.x, nblk, pr.Z * (OWN_HEADS));                                                   \
+  const int id = xcd_remap(bid, nblk, pr.Z * (OWN_HEADS));                                                   \
   const int zh = id / nblk;                                                                                         \
   const int z = zh / (OWN_HEADS), h = zh % (OWN_HEADS);                                                             \
   const int tid = threadIdx.x;                                                                                      \
@@ -136,7 +136,7 @@ __device__ __forceinline__ void zero_acc(f32x16 &x) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stubs (and has no buffer descriptor type)
 // SIX (dual mode only): dq' = scale dS' K as well, from the K fragments and the dS' tiles that dq already has.
 template <typename T, int D, int MODE, int MASK, bool GO, bool SIX>
-__device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
+__device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
   static_assert(!SIX || DUAL, "dq' rides on the dual mode");
@@ -445,7 +445,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p) {
 template <typename T, int D, int MODE, int MASK, bool GO, bool SIX = false>
 __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dq_body<T, D, MODE, MASK, GO, SIX>(p);
+  bwd2_dq_body<T, D, MODE, MASK, GO, SIX>(p, blockIdx.x);
 #endif
 }
 // The same code with the vector registers capped, for D = 64: together with the accumulation registers
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
 template <typename T, int D, int MODE, int MASK, bool GO, bool SIX = false>
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(160))) void bwd2_dq_kernel_2wg(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dq_body<T, D, MODE, MASK, GO, SIX>(p);
+  bwd2_dq_body<T, D, MODE, MASK, GO, SIX>(p, blockIdx.x);
 #endif
 }
 
@@ -467,7 +467,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(160))) void 
 // SIX (dual mode only): dk' = scale dS'^T Q and dv' = P^T gT as well, from the fragments and tiles that dk, dv
 // already have (two more accumulators: fits for D <= 64).
 template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED, bool SIX>
-__device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
+__device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
   static_assert(!SIX || (DUAL && D <= 64), "dk', dv' ride on the dual mode, where the accumulators fit");
@@ -903,7 +903,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p) {
 template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED = false, bool SIX = false>
 __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED, SIX>(p);
+  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED, SIX>(p, blockIdx.x);
 #endif
 }
 // The same code with the vector registers capped, for D = 64: together with the accumulation registers
@@ -911,7 +911,20 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
 template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED = false>
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(144))) void bwd2_dkdv_kernel_2wg(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED, false>(p);
+  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED, false>(p, blockIdx.x);
+#endif
+}
+
+// Both roles in one launch, for grids smaller than the GPU: the first kv_blocks workgroups are dk/dv
+// workgroups, the others dq workgroups.  The two kernels do not depend on each other, so launched apart on a
+// stream each leaves the compute units it does not fill idle for its whole duration; together they run side
+// by side.  (For grids that fill the GPU the single launch measured the same as the two.)
+template <typename T, int D, int MODE, int MASK, bool GO>
+__global__ __launch_bounds__(256, 1) void bwd2_both_kernel(const BwdParams p, const int kv_blocks) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const int b = __builtin_amdgcn_readfirstlane(blockIdx.x);
+  if (b < kv_blocks) bwd2_dkdv_body<T, D, MODE, MASK, GO, false, false>(p, b);
+  else bwd2_dq_body<T, D, MODE, MASK, GO, false>(p, b - kv_blocks);
 #endif
 }
 

@@ -95,6 +95,11 @@ def _run_case(Z, H, L, D, dtype, mode, seed=0, tangent_std=1.0, plain=False, tan
     for n, t in zip(names, grads):
         if t is not None:
             _tol_check(n, t, rb[n], dtype)
+    if tangent_grads:  # the call for dq, dk, dv alone takes other kernels (small grids: both roles in one launch)
+        g3 = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, kind, causal, scale)
+        assert g3[3] is None and g3[4] is None and g3[5] is None
+        for n, t in zip(names[:3], g3[:3]):
+            _tol_check(n + "(three gradients)", t, rb[n], dtype)
     # first-order backward from gO only through the same saved state (reference's backward)
     rb1 = dense.backward(*f64[:7], None, mask=npm, causal=causal, scale=scale)
     g1 = be.bwd(dev[0], dev[1], dev[2], None, None, None, o, None, M, None, dev[6], None, dmask, kind, causal, scale)
