@@ -89,16 +89,15 @@ typedef struct jvpfa_fwd_args {
    * reference, which reads the full (Z,H,L,L) mask (JA:2383-2388).  Ignored without a mask. */
   const int32_t *key_limit;
   /* optional lists of the key tiles that hold an attended entry, written by jvpfa_mask_tiles() for
-   * this same mask, or NULL.  Tiles not listed are skipped instead of read and masked.  When set,
-   * key_limit is ignored.  Ignored (and key_limit used) for fp32, whose kernels visit every tile
-   * up to the key limit.  Ignored without a mask. */
+   * this same mask (and the same Lk), or NULL.  Tiles not listed are skipped instead of read and masked.
+   * When set, key_limit is ignored.  Ignored without a mask. */
   const int32_t *tiles_q;
   /* shape of k, v, kt, vt when it is not q's -- Lk keys (any length >= 1) and Hk key/value heads, Hk a divisor
    * of p.H; query head h reads key/value head h / (H / Hk).  0 means "as q" (p.L, p.H).  k, v and
    * their tangents are then (Z, Hk, Lk, D), the mask strides address (z, h, query, key) with Lk keys,
    * and causal means key index <= query index.  The reference requires q, k, v of one shape
-   * (JA:2367-2378).  key_limit then counts the Lk keys; the tile lists are used when Lk equals p.L
-   * (any Hk: they belong to the mask planes, which follow the query heads) and ignored otherwise. */
+     * (JA:2367-2378).  key_limit then counts the Lk keys; the tile lists must have been made for the same Lk
+   * (any Hk: they belong to the mask planes, which follow the query heads). */
   int32_t Lk, Hk;
   /* optional workspace for small grids, or NULL: jvpfa_fwd_split_workspace_bytes(&p, Lk) bytes of device memory,
    * 16-byte aligned, contents don't-care.  When a launch would have fewer workgroups than the GPU has compute
@@ -177,14 +176,16 @@ size_t jvpfa_bwd_static_max_rows(void);
  *   tiles_q  for every mask plane and block of 128 query rows: the 64-key tiles to visit
  *   tiles_k  for every mask plane and block of 128 keys: the 64-query tiles to visit
  * Either may be NULL (not both): the forward needs tiles_q only.
- * A mask plane is a (z, h) pair, with one plane along an axis whose mask stride is 0.  Each list
- * is 1 + ceil(L/64) int32 values: the count (at least 1), then the tile indices in ascending
- * order.  Both buffers are jvpfa_mask_tiles_bytes(p) bytes of device memory, 4-byte aligned.  The
- * lists describe the mask's contents: rebuild them when those change.  Only p->Z, H, L, dtype,
- * mask_kind, mask and mask_stride are read.
+ * A mask plane is a (z, h) pair, with one plane along an axis whose mask stride is 0.  The mask has p->L query
+ * rows and Lk keys (0 = as p->L).  A list of tiles_q is 1 + ceil(Lk/64) int32 values, one of tiles_k
+ * 1 + ceil(L/64): the count (at least 1), then the tile indices in ascending order.  The buffers are
+ * jvpfa_mask_tiles_bytes(p, Lk, 0) and jvpfa_mask_tiles_bytes(p, Lk, 1) bytes of device memory, 4-byte
+ * aligned.  The lists describe the mask's contents: rebuild them when those change.  Only p->Z, H, L, dtype,
+ * mask_kind, mask and mask_stride are read.  Every element type and head dim walks them (kernels with 32-wide
+ * tiles take a listed tile as two).
  */
-size_t jvpfa_mask_tiles_bytes(const jvpfa_problem *p);
-int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t *tiles_q, int32_t *tiles_k, void *hip_stream);
+size_t jvpfa_mask_tiles_bytes(const jvpfa_problem *p, int32_t Lk, int32_t keys_owned);
+int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t Lk, int32_t *tiles_q, int32_t *tiles_k, void *hip_stream);
 
 /*
  * The keep pattern of dropout for this problem (only Z, H, L, dropout_p, dropout_seed are read) and Lk keys

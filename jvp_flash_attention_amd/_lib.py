@@ -94,9 +94,9 @@ def load() -> C.CDLL:
         lib.jvpfa_fwd_split_workspace_bytes.restype = C.c_size_t
         lib.jvpfa_dropout_keep.argtypes = [C.POINTER(Problem), C.c_int32, C.c_void_p, C.c_void_p]
         lib.jvpfa_dropout_keep.restype = C.c_int
-        lib.jvpfa_mask_tiles_bytes.argtypes = [C.POINTER(Problem)]
+        lib.jvpfa_mask_tiles_bytes.argtypes = [C.POINTER(Problem), C.c_int32, C.c_int32]
         lib.jvpfa_mask_tiles_bytes.restype = C.c_size_t
-        lib.jvpfa_mask_tiles.argtypes = [C.POINTER(Problem), C.c_void_p, C.c_void_p, C.c_void_p]
+        lib.jvpfa_mask_tiles.argtypes = [C.POINTER(Problem), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.jvpfa_mask_tiles.restype = C.c_int
         lib.jvpfa_abi_version.argtypes = []
         lib.jvpfa_abi_version.restype = C.c_int
@@ -215,19 +215,18 @@ def set_tile_lists(enabled: bool, additive: bool | None = None) -> None:
         _tile_lists_additive = bool(additive)
 
 
-def tile_lists(q, mask, mask_kind, want_k):
-    """For a mask with a row per query (shape [*, *, L, L]): the lists of 64-wide tiles that hold an
+def tile_lists(q, mask, mask_kind, want_k, Lk=None):
+    """For a mask with a row per query (shape [*, *, L, Lk]): the lists of 64-wide tiles that hold an
     attended entry, made on the device by ``jvpfa_mask_tiles`` -- (tiles_q, tiles_k) int32 tensors,
     tiles_k only if ``want_k`` (the backward).  The kernels visit the listed tiles only, so block
     diagonal, banded or doubly padded masks cost time in proportion to their attended area.
-    (None, None) for masks that are not two-dimensional, short sequences, and the element types /
-    head dims whose kernels visit every tile.  Cached on the mask tensor, keyed by its version
-    counter, so that layers and the backward reuse one scan."""
+    (None, None) for masks that are not two-dimensional and for short sequences.  Cached on the mask
+    tensor, keyed by its version counter, so that layers and the backward reuse one scan."""
     Z, H, L, D = q.shape
-    if (not _tile_lists_enabled or mask is None or mask_kind == MASK_NONE or L < TILE_LISTS_MIN_L
-            or q.dtype == torch.float32):
+    Lk = L if Lk is None else Lk
+    if not _tile_lists_enabled or mask is None or mask_kind == MASK_NONE or max(L, Lk) < TILE_LISTS_MIN_L:
         return None, None
-    if mask.dim() != 4 or mask.shape[2] != L or mask.shape[3] != L:
+    if mask.dim() != 4 or mask.shape[2] != L or mask.shape[3] != Lk:
         return None, None
     if mask_kind == MASK_ADD and not _tile_lists_additive:
         return None, None
@@ -239,10 +238,12 @@ def tile_lists(q, mask, mask_kind, want_k):
     if tq is None or (want_k and tk is None):
         lib = load()
         prob = make_problem(q, mask, mask_kind, False, 1.0)
-        n = lib.jvpfa_mask_tiles_bytes(C.byref(prob)) // 4
-        new_q = torch.empty(n, device=q.device, dtype=torch.int32) if tq is None else None
-        new_k = torch.empty(n, device=q.device, dtype=torch.int32) if (want_k and tk is None) else None
-        check(lib.jvpfa_mask_tiles(C.byref(prob), _ptr(new_q), _ptr(new_k), _stream(q)))
+        new_q = new_k = None
+        if tq is None:
+            new_q = torch.empty(lib.jvpfa_mask_tiles_bytes(C.byref(prob), Lk, 0) // 4, device=q.device, dtype=torch.int32)
+        if want_k and tk is None:
+            new_k = torch.empty(lib.jvpfa_mask_tiles_bytes(C.byref(prob), Lk, 1) // 4, device=q.device, dtype=torch.int32)
+        check(lib.jvpfa_mask_tiles(C.byref(prob), Lk, _ptr(new_q), _ptr(new_k), _stream(q)))
         tq = new_q if tq is None else tq
         tk = new_k if new_k is not None else tk
         cached[1], cached[2] = tq, tk
@@ -313,7 +314,7 @@ class HipBackend:
         with torch.cuda.device(q.device):
             lim = key_limit_hint(mask, mask_kind, Z, k.shape[2])
             a.key_limit = _ptr(lim)
-            tq, _ = tile_lists(q, mask, mask_kind, False) if k.shape[2] == q.shape[2] else (None, None)
+            tq, _ = tile_lists(q, mask, mask_kind, False, k.shape[2])
             a.tiles_q = _ptr(tq)
             nsplit = lib.jvpfa_fwd_split_workspace_bytes(C.byref(a.p), a.Lk) if _split_enabled else 0
             if nsplit:
@@ -346,7 +347,7 @@ class HipBackend:
         with torch.cuda.device(q.device):
             lim = key_limit_hint(mask, mask_kind, Z, k.shape[2])
             a.key_limit = _ptr(lim)
-            tq, tk = tile_lists(q, mask, mask_kind, True) if k.shape[2] == q.shape[2] else (None, None)
+            tq, tk = tile_lists(q, mask, mask_kind, True, k.shape[2])
             a.tiles_q, a.tiles_k = _ptr(tq), _ptr(tk)
             check(lib.jvpfa_bwd(C.byref(a), _stream(q)))
         return dq, dk, dv, dqt, dkt, dvt

@@ -39,9 +39,8 @@ inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit, cons
   r.Lk = Lk > 0 ? Lk : p.L;
   r.Hk = Hk > 0 ? Hk : p.H;
   const bool masked = p.mask_kind != JVPFA_MASK_NONE;
-  // the tile lists are laid out for as many keys as queries and walked by the kernels for 16-bit
-  // element types; the key limit counts keys whatever the shape
-  const bool lists = masked && r.Lk == p.L && p.dtype != JVPFA_FP32;
+  // every kernel walks the tile lists when they are there; without them the key limit applies
+  const bool lists = masked;
   r.tiles_q = lists ? tiles_q : nullptr;
   r.tiles_k = lists ? tiles_k : nullptr;
   r.klimit = (masked && !r.tiles_q && !r.tiles_k) ? key_limit : nullptr;

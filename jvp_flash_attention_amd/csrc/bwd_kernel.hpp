@@ -172,7 +172,18 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
   const T *Ktg = DUAL ? reinterpret_cast<const T *>(p.kt) + kvhead : nullptr;
   const T *Vtg = DUAL ? reinterpret_cast<const T *>(p.vt) + kvhead : nullptr;
 
-  const int kend = pr.causal ? min(Lk, q0 + BWD_BLK) : Lk;
+  int kend = pr.causal ? min(Lk, q0 + BWD_BLK) : Lk;
+  // key tiles visited: up to kend (the causal diagonal, or the caller's key limit of a padded batch), or the
+  // caller's list of the tiles of this query block that hold an attended entry
+  TileWalk<BWD_T> walk;
+  {
+    const int *tl = nullptr;
+    if constexpr (MASK != MASK_NONE) {
+      if (pr.klimit) kend = min(kend, max(pr.klimit[z], 1));
+      if (pr.tiles_q) tl = pr.tiles_q + tile_list_offset_q(pr, z, h, qb);
+    }
+    walk.init(tl, 0, kend, Lk);
+  }
   // The next tile is fetched into registers while this one is computed and written to LDS behind the
   // barrier that follows; K (, K') is fetched once and written both ways.  (See the forward kernel for
   // where this is left out.)
@@ -189,9 +200,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
     }
   };
   if constexpr (AHEAD) {
-    if (kend > 0) fetch_tile(0);
+    if (walk.n > 0) fetch_tile(walk.at(0));
   }
-  for (int j0 = 0; j0 < kend; j0 += BWD_T) {
+  for (int it = 0; it < walk.n; ++it) {
+    const int j0 = walk.at(it);
     __syncthreads();
     if constexpr (AHEAD) {
       put_quads_rows(Kn, Cfg::LDN, rk, tid);
@@ -215,7 +227,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
     }
     __syncthreads();
     if constexpr (AHEAD) {
-      if (j0 + BWD_T < kend) fetch_tile(j0 + BWD_T);
+      if (it + 1 < walk.n) fetch_tile(walk.at(it + 1));
     }
 
     f32x16 S, dP, Sp, At;  // DUAL: dP also collects gT V'^T (the B term)
@@ -400,10 +412,24 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
     }
     fetch_stats(i0);
   };
-  if constexpr (AHEAD) {
-    if (istart < L) fetch_tile(istart);
+  // query tiles visited: all from istart on, or the caller's list of the tiles of this key block (and this
+  // query head's mask plane) that hold an attended entry
+  TileWalk<BWD_T> walk;
+  {
+    const int *tl = nullptr;
+    if constexpr (MASK != MASK_NONE) {
+      if (pr.tiles_k) tl = pr.tiles_k + tile_list_offset_k(pr, z, h, kb);
+    }
+    walk.init(tl, istart, L, L);
+    if constexpr (MASK != MASK_NONE) {
+      if (pr.klimit && k0 >= pr.klimit[z]) walk.n = 0;  // a key block the caller's hint declares fully masked: zeros
+    }
   }
-  for (int i0 = istart; i0 < L; i0 += BWD_T) {
+  if constexpr (AHEAD) {
+    if (walk.n > 0) fetch_tile(walk.at(0));
+  }
+  for (int it = 0; it < walk.n; ++it) {
+    const int i0 = walk.at(it);
     __syncthreads();
     if constexpr (AHEAD) {
       put_quads_rows(Qn, Cfg::LDN, rq, tid);
@@ -437,7 +463,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
     put_stats();
     __syncthreads();
     if constexpr (AHEAD) {
-      if (i0 + BWD_T < L) fetch_tile(i0 + BWD_T);
+      if (it + 1 < walk.n) fetch_tile(walk.at(it + 1));
     }
 
     f32x16 S, dP, Sp, At;  // DUAL: dP also collects V' gT^T (the B term)

@@ -199,7 +199,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
   // that hold an attended entry (ascending); tile_at(i) is the i-th one.
   const int *tlist = nullptr;
   if constexpr (MASK != MASK_NONE) {
-    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
+    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset_q(pr, z, h, qb);
   }
   const int tmax = (Lk + BT - 1) / BT - 1;  // index of the last tile of the sequence: bounds whatever a list holds
   const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1) : (kend + BT - 1) / BT;
@@ -571,7 +571,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
   auto set_list = [&](int hq_) {
     if constexpr (MASK != MASK_NONE) {
       if (pr.tiles_k) {
-        tlist = pr.tiles_k + tile_list_offset(pr, z, hq_, kb);
+        tlist = pr.tiles_k + tile_list_offset_k(pr, z, hq_, kb);
         ntiles = min(max(tlist[0], 1), tmax + 1);
       }
     }

@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   // the last key).
   const int *tlist = nullptr;
   if constexpr (MASK != MASK_NONE) {
-    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
+    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset_q(pr, z, h, qb);
   }
   const int tmax = (Lk + TILE_W - 1) / TILE_W - 1;  // bounds whatever a list holds
   int ntiles = (kend + BT - 1) / BT;
@@ -541,7 +541,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   auto set_list = [&](int hq) {
     if constexpr (MASK != MASK_NONE) {
       if (pr.tiles_k) {
-        tlist = pr.tiles_k + tile_list_offset(pr, z, hq, kb);
+        tlist = pr.tiles_k + tile_list_offset_k(pr, z, hq, kb);
         const int cnt = min(max(tlist[0], 1), tmax + 1);
         const int last = min(max(tlist[cnt], 0), tmax);
         ntiles = 2 * cnt - (last * TILE_W + BT >= L ? 1 : 0);

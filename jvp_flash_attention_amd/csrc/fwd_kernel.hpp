@@ -98,6 +98,17 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
 
   int kend = Lk;
   if (pr.causal) kend = min(Lk, q0 + Cfg::BM);
+  // key tiles visited: up to kend (the causal diagonal, or the caller's key limit of a padded batch), or the
+  // caller's list of the tiles of this query block that hold an attended entry
+  TileWalk<BN> walk;
+  {
+    const int *tl = nullptr;
+    if constexpr (MASK != MASK_NONE) {
+      if (pr.klimit) kend = min(kend, max(pr.klimit[z], 1));
+      if (pr.tiles_q) tl = pr.tiles_q + tile_list_offset_q(pr, z, h, qb);
+    }
+    walk.init(tl, 0, kend, Lk);
+  }
 
   // The next tile is fetched into registers while this one is computed and written to LDS behind the
   // barrier that follows.  Not for D >= 128 (no registers to spare) and not for 16-bit D = 32, where
@@ -116,9 +127,10 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
     }
   };
   if constexpr (AHEAD) {
-    if (kend > 0) fetch_tile(0);
+    if (walk.n > 0) fetch_tile(walk.at(0));
   }
-  for (int j0 = 0; j0 < kend; j0 += BN) {
+  for (int it = 0; it < walk.n; ++it) {
+    const int j0 = walk.at(it);
     __syncthreads();
     if constexpr (AHEAD) {
       put_rows(Ks, Cfg::LDK, rk, tid);
@@ -138,7 +150,7 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
     }
     __syncthreads();
     if constexpr (AHEAD) {
-      if (j0 + BN < kend) fetch_tile(j0 + BN);
+      if (it + 1 < walk.n) fetch_tile(walk.at(it + 1));
     }
 
     // ---- S^T = K Q^T and S'^T = K Q'^T + K' Q^T -------------------------------------------

@@ -197,7 +197,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   // out changes nothing).  tile_at(i) is the i-th tile visited.
   const int *tlist = nullptr;
   if constexpr (MASK != MASK_NONE) {
-    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
+    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset_q(pr, z, h, qb);
   }
   const int tmax = (Lk + BN - 1) / BN - 1;  // index of the last tile of the sequence: bounds whatever a list holds
   const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1) : (kend + BN - 1) / BN;

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
   // when it lies past the last key.
   const int *tlist = nullptr;
   if constexpr (MASK != MASK_NONE) {
-    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset(pr, z, h, qb);
+    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset_q(pr, z, h, qb);
   }
   const int tmax = (Lk + TILE_W - 1) / TILE_W - 1;  // bounds whatever a list holds
   int ntiles = (kend + BN - 1) / BN;

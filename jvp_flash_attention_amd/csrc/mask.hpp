@@ -86,4 +86,31 @@ template <typename T, int MASK> __device__ __forceinline__ float mask_bias_of(co
   return (float)m.f[e] * LOG2E;
 }
 
+// The streamed tiles (W = 32 or 64 rows) that a kernel outside the direct-to-LDS family visits: all of them from
+// `start` up to `end`, or those of a caller's list of 64-wide tiles (jvpfa_mask_tiles), each walked as 64 / W
+// pieces.  `len` is the length of the streamed axis: it bounds whatever a list holds, and a second piece that
+// would start past it is left out.
+template <int W> struct TileWalk {
+  static_assert(W == 32 || W == 64);
+  static constexpr int SUB = TILE_W / W;
+  const int *list = nullptr;
+  int n = 0, start = 0, tmax = 0;
+  __device__ __forceinline__ void init(const int *l, int start_, int end, int len) {
+    list = l;
+    start = start_;
+    tmax = (len + TILE_W - 1) / TILE_W - 1;
+    if (!l) {
+      n = end > start_ ? (end - start_ + W - 1) / W : 0;
+      return;
+    }
+    const int cnt = min(max(l[0], 1), tmax + 1);
+    const int last = min(max(l[cnt], 0), tmax);
+    n = SUB * cnt - ((SUB == 2 && last * TILE_W + W >= len) ? 1 : 0);
+  }
+  __device__ __forceinline__ int at(int it) const {
+    if (!list) return start + it * W;
+    return min(max(list[1 + it / SUB], 0), tmax) * TILE_W + (it % SUB) * W;
+  }
+};
+
 }  // namespace jvpfa

@@ -23,8 +23,10 @@ template <typename E, bool BOOL> __device__ __forceinline__ bool attended(E x) {
 // Every thread looks at 32 consecutive keys of one row of the current tile.
 template <typename E, bool BOOL, bool KEYS_OWNED>
 __global__ __launch_bounds__(256) void mask_tiles_kernel(const E *mask, int64_t s0, int64_t s1, int64_t s2,
-                                                         int64_t s3, int hm, int L, int *out) {
-  const int nblk = (L + TILE_BLOCK - 1) / TILE_BLOCK, nt = (L + TILE_W - 1) / TILE_W;
+                                                         int64_t s3, int hm, int Lq, int Lk, int *out) {
+  // owned: the axis cut into blocks of 128; streamed: the axis cut into tiles of 64
+  const int owned = KEYS_OWNED ? Lk : Lq, streamed = KEYS_OWNED ? Lq : Lk;
+  const int nblk = (owned + TILE_BLOCK - 1) / TILE_BLOCK, nt = (streamed + TILE_W - 1) / TILE_W;
   const int plane = blockIdx.x / nblk, blk = blockIdx.x % nblk;
   const E *base = mask + (int64_t)(plane / hm) * s0 + (int64_t)(plane % hm) * s1;
   int *list = out + ((size_t)plane * nblk + blk) * (size_t)(nt + 1);
@@ -45,9 +47,9 @@ __global__ __launch_bounds__(256) void mask_tiles_kernel(const E *mask, int64_t 
       const int row = KEYS_OWNED ? t * TILE_W + rsub : blk * TILE_BLOCK + rsub;
       const int key0 = (KEYS_OWNED ? blk * TILE_BLOCK : t * TILE_W) + 32 * part;
       any[u] = false;
-      if (t < nt && row < L && key0 < L) {
+      if (t < nt && row < Lq && key0 < Lk) {
         const E *rp = base + (int64_t)row * s2;
-        if (vec_ok && key0 + 32 <= L) {
+        if (vec_ok && key0 + 32 <= Lk) {
 #pragma unroll
           for (int v = 0; v < 32 / VEC; ++v) {
             const uint4 w = *reinterpret_cast<const uint4 *>(rp + key0 + v * VEC);
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(256) void mask_tiles_kernel(const E *mask, int64_t 
             }
           }
         } else {
-          const int n = min(32, L - key0);
+          const int n = min(32, Lk - key0);
           for (int i = 0; i < n; ++i) any[u] |= attended<E, BOOL>(rp[(int64_t)(key0 + i) * s3]);
         }
       }
@@ -83,22 +85,21 @@ __global__ __launch_bounds__(256) void mask_tiles_kernel(const E *mask, int64_t 
 }
 
 template <typename E, bool BOOL>
-static int launch_both(const jvpfa_problem &p, int *tq, int *tk, hipStream_t stream) {
+static int launch_both(const jvpfa_problem &p, int Lk, int *tq, int *tk, hipStream_t stream) {
   const int hm = p.mask_stride[1] ? p.H : 1, zm = p.mask_stride[0] ? p.Z : 1;
-  const int nblk = (p.L + TILE_BLOCK - 1) / TILE_BLOCK;
-  const long long blocks = (long long)zm * hm * nblk;
-  if (blocks > 0x7fffffffLL) return JVPFA_E_SHAPE;
+  const long long qblocks = (long long)zm * hm * ((p.L + TILE_BLOCK - 1) / TILE_BLOCK);
+  const long long kblocks = (long long)zm * hm * ((Lk + TILE_BLOCK - 1) / TILE_BLOCK);
+  if (qblocks > 0x7fffffffLL || kblocks > 0x7fffffffLL) return JVPFA_E_SHAPE;
   const E *m = static_cast<const E *>(p.mask);
   const int64_t *s = p.mask_stride;
   if (tq)
-    hipLaunchKernelGGL((mask_tiles_kernel<E, BOOL, false>), dim3((unsigned)blocks), dim3(256), 0, stream, m, s[0],
-                       s[1], s[2], s[3], hm, p.L, tq);
+    hipLaunchKernelGGL((mask_tiles_kernel<E, BOOL, false>), dim3((unsigned)qblocks), dim3(256), 0, stream, m, s[0],
+                       s[1], s[2], s[3], hm, p.L, Lk, tq);
   if (tk)
-    hipLaunchKernelGGL((mask_tiles_kernel<E, BOOL, true>), dim3((unsigned)blocks), dim3(256), 0, stream, m, s[0],
-                       s[1], s[2], s[3], hm, p.L, tk);
+    hipLaunchKernelGGL((mask_tiles_kernel<E, BOOL, true>), dim3((unsigned)kblocks), dim3(256), 0, stream, m, s[0],
+                       s[1], s[2], s[3], hm, p.L, Lk, tk);
   return hipGetLastError() == hipSuccess ? JVPFA_OK : JVPFA_E_LAUNCH;
 }
-
 }  // namespace jvpfa
 
 using namespace jvpfa;
@@ -124,26 +125,28 @@ extern "C" int jvpfa_dropout_keep(const jvpfa_problem *p, int32_t Lk, uint8_t *k
   return hipGetLastError() == hipSuccess ? JVPFA_OK : JVPFA_E_LAUNCH;
 }
 
-extern "C" size_t jvpfa_mask_tiles_bytes(const jvpfa_problem *p) {
-  if (!p || p->Z < 1 || p->H < 1 || p->L < 1) return 0;
+extern "C" size_t jvpfa_mask_tiles_bytes(const jvpfa_problem *p, int32_t Lk, int32_t keys_owned) {
+  if (!p || p->Z < 1 || p->H < 1 || p->L < 1 || Lk < 0) return 0;
   const size_t planes = (size_t)(p->mask_stride[0] ? p->Z : 1) * (p->mask_stride[1] ? p->H : 1);
-  const size_t nblk = (p->L + TILE_BLOCK - 1) / TILE_BLOCK, nt = (p->L + TILE_W - 1) / TILE_W;
+  const size_t lk = Lk > 0 ? Lk : p->L, owned = keys_owned ? lk : p->L, streamed = keys_owned ? p->L : lk;
+  const size_t nblk = (owned + TILE_BLOCK - 1) / TILE_BLOCK, nt = (streamed + TILE_W - 1) / TILE_W;
   return planes * nblk * (nt + 1) * sizeof(int32_t);
 }
 
-extern "C" int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t *tiles_q, int32_t *tiles_k, void *hip_stream) {
+extern "C" int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t Lk, int32_t *tiles_q, int32_t *tiles_k, void *hip_stream) {
   if (!p || (!tiles_q && !tiles_k)) return JVPFA_E_NULL;
-  if (p->Z < 1 || p->H < 1 || p->L < 1) return JVPFA_E_SHAPE;
+  if (p->Z < 1 || p->H < 1 || p->L < 1 || Lk < 0) return JVPFA_E_SHAPE;
   if (p->dtype < JVPFA_BF16 || p->dtype > JVPFA_FP32) return JVPFA_E_DTYPE;
   if (p->mask_kind != JVPFA_MASK_BOOL && p->mask_kind != JVPFA_MASK_ADD) return JVPFA_E_DTYPE;
   if (!p->mask) return JVPFA_E_NULL;
   for (int i = 0; i < 4; ++i)
     if (p->mask_stride[i] < 0) return JVPFA_E_SHAPE;
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  if (p->mask_kind == JVPFA_MASK_BOOL) return launch_both<uint8_t, true>(*p, tiles_q, tiles_k, stream);
+  const int lk = Lk > 0 ? Lk : p->L;
+  if (p->mask_kind == JVPFA_MASK_BOOL) return launch_both<uint8_t, true>(*p, lk, tiles_q, tiles_k, stream);
   switch (p->dtype) {
-    case JVPFA_BF16: return launch_both<__bf16, false>(*p, tiles_q, tiles_k, stream);
-    case JVPFA_FP16: return launch_both<_Float16, false>(*p, tiles_q, tiles_k, stream);
-    default: return launch_both<float, false>(*p, tiles_q, tiles_k, stream);
+    case JVPFA_BF16: return launch_both<__bf16, false>(*p, lk, tiles_q, tiles_k, stream);
+    case JVPFA_FP16: return launch_both<_Float16, false>(*p, lk, tiles_q, tiles_k, stream);
+    default: return launch_both<float, false>(*p, lk, tiles_q, tiles_k, stream);
   }
 }

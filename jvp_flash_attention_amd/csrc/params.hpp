@@ -50,12 +50,19 @@ __host__ __device__ inline float drop_scale(const Problem &pr, uint64_t idx) {
 }
 
 constexpr int TILE_BLOCK = 128, TILE_W = 64;  // geometry of the tile lists
-// first element of the list of (plane of (z, h), block)
-__host__ __device__ inline size_t tile_list_offset(const Problem &pr, int z, int h, int block) {
+// First element of the list of (plane of (z, h), block).  tiles_q: blocks of 128 query rows, each with up to
+// ceil(Lk / 64) key tiles; tiles_k: blocks of 128 keys, each with up to ceil(L / 64) query tiles.
+__host__ __device__ inline size_t tile_list_plane(const Problem &pr, int z, int h) {
   const int hm = pr.ms[1] ? pr.H : 1;
-  const size_t plane = (size_t)(pr.ms[0] ? z : 0) * hm + (pr.ms[1] ? h : 0);
-  const int nblk = (pr.L + TILE_BLOCK - 1) / TILE_BLOCK, nt = (pr.L + TILE_W - 1) / TILE_W;
-  return (plane * nblk + block) * (size_t)(nt + 1);
+  return (size_t)(pr.ms[0] ? z : 0) * hm + (pr.ms[1] ? h : 0);
+}
+__host__ __device__ inline size_t tile_list_offset_q(const Problem &pr, int z, int h, int block) {
+  const int nblk = (pr.L + TILE_BLOCK - 1) / TILE_BLOCK, nt = (pr.Lk + TILE_W - 1) / TILE_W;
+  return (tile_list_plane(pr, z, h) * nblk + block) * (size_t)(nt + 1);
+}
+__host__ __device__ inline size_t tile_list_offset_k(const Problem &pr, int z, int h, int block) {
+  const int nblk = (pr.Lk + TILE_BLOCK - 1) / TILE_BLOCK, nt = (pr.L + TILE_W - 1) / TILE_W;
+  return (tile_list_plane(pr, z, h) * nblk + block) * (size_t)(nt + 1);
 }
 
 struct FwdParams {

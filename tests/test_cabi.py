@@ -123,7 +123,7 @@ def test_tile_lists_are_only_made_for_masks_with_a_row_per_query():
     cases = [
         (q, torch.ones(2, 1, 1, 1024, dtype=torch.bool)),         # key padding: the key limit covers it
         (q[:, :, :256], full[:, :, :256, :256]),                   # too short to pay for the scan
-        (q.float(), full),                                          # fp32 kernels visit every tile
+        (q, full[:, :, :, :512]),                                   # not the shape of the scores (Lk = 1024)
         (q, None),
     ]
     for qq, m in cases:
@@ -145,16 +145,21 @@ def test_mask_tile_list_sizes_and_argument_checks():
     nblk, nt = 6, 11  # ceil(700/128) blocks of ceil(700/64) + 1 ints each
     for strides, planes in (((490000 * 4, 490000, 700, 1), 12), ((490000, 0, 700, 1), 3), ((0, 0, 700, 1), 1)):
         p.mask_stride = (C.c_int64 * 4)(*strides)
-        assert lib.jvpfa_mask_tiles_bytes(C.byref(p)) == planes * nblk * (nt + 1) * 4
+        assert lib.jvpfa_mask_tiles_bytes(C.byref(p), 0, 0) == planes * nblk * (nt + 1) * 4
+        assert lib.jvpfa_mask_tiles_bytes(C.byref(p), 0, 1) == planes * nblk * (nt + 1) * 4
+        # 200 keys: 4 key tiles per block of query rows; 2 blocks of keys with 11 query tiles each
+        assert lib.jvpfa_mask_tiles_bytes(C.byref(p), 200, 0) == planes * nblk * (4 + 1) * 4
+        assert lib.jvpfa_mask_tiles_bytes(C.byref(p), 200, 1) == planes * 2 * (nt + 1) * 4
     buf = (C.c_int32 * 16)()
-    assert lib.jvpfa_mask_tiles(C.byref(p), buf, None, None) == -1  # no mask pointer
+    assert lib.jvpfa_mask_tiles(C.byref(p), 0, buf, None, None) == -1  # no mask pointer
     p.mask = C.addressof(buf)
-    assert lib.jvpfa_mask_tiles(C.byref(p), None, None, None) == -1  # no output at all
+    assert lib.jvpfa_mask_tiles(C.byref(p), 0, None, None, None) == -1  # no output at all
+    assert lib.jvpfa_mask_tiles(C.byref(p), -5, buf, None, None) == -2
     p.mask_kind = _lib.MASK_NONE
-    assert lib.jvpfa_mask_tiles(C.byref(p), buf, None, None) == -3
+    assert lib.jvpfa_mask_tiles(C.byref(p), 0, buf, None, None) == -3
     p.mask_kind, p.L = _lib.MASK_BOOL, 0
-    assert lib.jvpfa_mask_tiles(C.byref(p), buf, None, None) == -2
-    assert lib.jvpfa_mask_tiles_bytes(C.byref(p)) == 0
+    assert lib.jvpfa_mask_tiles(C.byref(p), 0, buf, None, None) == -2
+    assert lib.jvpfa_mask_tiles_bytes(C.byref(p), 0, 0) == 0
     # the backward takes both lists or none
     b = _lib.BwdArgs()
     b.struct_size = C.sizeof(_lib.BwdArgs)

@@ -160,15 +160,16 @@ def test_masks_over_several_tiles_interior_and_edge(D, mode):
     _run_case(1, 2, 328, D, torch.bfloat16, mode, seed=12)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("kind", ["bool", "bias"])
-def test_key_padding_with_skipped_tiles(D, kind):
+def test_key_padding_with_skipped_tiles(D, kind, dt):
     """Long enough for the host to pass the key-limit hint: key tiles past the longest valid length of a
     batch entry are skipped (forward, dq) and fully padded key blocks return zero gradients (dk/dv)."""
     from jvp_flash_attention_amd import _lib
 
     Z, H, L = 3, 2, 640
-    dtype = torch.bfloat16
+    dtype = DTYPES[dt]
     q, k, v, qt, kt, vt, go, gt = _make(Z, H, L, D, dtype, 21)
     lens = [640, 200, 65]
     keep = torch.arange(L)[None, :] < torch.tensor(lens)[:, None]
@@ -256,17 +257,18 @@ def test_mask_tile_lists_match_a_numpy_scan(kind, as_bias, L):
             assert row[0] == len(want) and row[1:1 + row[0]] == want
 
 
-@pytest.mark.parametrize("D", [32, 64, 128, 256])
+@pytest.mark.parametrize("dt,D", [("bf16", 32), ("bf16", 64), ("bf16", 128), ("bf16", 256),
+                                  ("fp32", 32), ("fp32", 64), ("fp32", 128)])
 @pytest.mark.parametrize("kind", ["blockdiag", "band", "pad2d", "lower"])
 @pytest.mark.parametrize("as_bias", [False, True])
-def test_structured_masks_with_skipped_tiles(D, kind, as_bias):
+def test_structured_masks_with_skipped_tiles(dt, D, kind, as_bias):
     """Masks with whole tiles masked: the host scans them into tile lists and the kernels visit the
     listed tiles only.  Checked against the oracle, and bit for bit against the same kernels made to
     visit every tile (a fully masked tile contributes exact zeros)."""
     from jvp_flash_attention_amd import _lib
 
     Z, H, L = 2, 2, 700
-    dtype = torch.bfloat16
+    dtype = DTYPES[dt]
     q, k, v, qt, kt, vt, go, gt = _make(Z, H, L, D, dtype, 31)
     keep = _structured_keep(kind, Z, H, L)
     mask = torch.where(keep, 0.0, float("-inf")).to(dtype) if as_bias else keep
@@ -275,7 +277,7 @@ def test_structured_masks_with_skipped_tiles(D, kind, as_bias):
     dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
     be = _lib.backend()
     scale = D**-0.5
-    print(f"case structured {kind} D{D} bias={as_bias}", flush=True)
+    print(f"case structured {dt} {kind} D{D} bias={as_bias}", flush=True)
 
     def run(dmask):
         o, ot, M, mu = be.fwd(*dev[:6], dmask, mk, False, scale)
@@ -298,6 +300,71 @@ def test_structured_masks_with_skipped_tiles(D, kind, as_bias):
     npm = keep.numpy()
     ref = dense.forward(*f64[:6], mask=npm, causal=False, scale=scale)
     rb = dense.backward(*f64, mask=npm, causal=False, scale=scale)
+    _tol_check("O", with_lists[0], ref["O"], dtype)
+    _tol_check("O'", with_lists[1], ref["Ot"], dtype)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), with_lists[4:10]):
+        _tol_check(n, t, rb[n], dtype)
+
+
+def _numpy_tile_lists_rect(keep, Lq, Lk):
+    """(tiles_q, tiles_k) from a (P, Lq, Lk) boolean array: per block of 128 query rows the 64-key tiles, per
+    block of 128 keys the 64-query tiles."""
+    tq, tk = [], []
+    for pl in keep:
+        for b in range((Lq + 127) // 128):
+            rows = pl[128 * b:128 * b + 128]
+            tq.append([t for t in range((Lk + 63) // 64) if rows[:, 64 * t:64 * t + 64].any()] or [0])
+        for b in range((Lk + 127) // 128):
+            cols = pl[:, 128 * b:128 * b + 128]
+            tk.append([t for t in range((Lq + 63) // 64) if cols[64 * t:64 * t + 64].any()] or [0])
+    return tq, tk
+
+
+@pytest.mark.parametrize("dt,D", [("bf16", 64), ("fp16", 128), ("bf16", 256), ("fp32", 64)])
+@pytest.mark.parametrize("Lq,Lk", [(300, 900), (900, 300), (520, 97)])
+def test_structured_masks_with_as_many_keys_as_they_like(dt, D, Lq, Lk):
+    """Tile lists of a mask whose two axes differ in length (cross attention over packed or windowed memory):
+    the lists against a numpy scan, the kernels with lists bit for bit against every tile, and against the
+    oracle; 4 query heads over 2 key/value heads."""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H, Hk = 2, 4, 2
+    dtype = DTYPES[dt]
+    g = torch.Generator().manual_seed(Lq + Lk)
+    q, qt, go, gt = (torch.randn(Z, H, Lq, D, generator=g).to(dtype) for _ in range(4))
+    k, v, kt, vt = (torch.randn(Z, Hk, Lk, D, generator=g).to(dtype) for _ in range(4))
+    # a slanted band (each query sees a window of keys around its own relative position), different per batch entry
+    i, j = torch.arange(Lq)[:, None].float() / Lq, torch.arange(Lk)[None, :].float() / Lk
+    keep = torch.stack([(i - j).abs() <= w for w in (0.08, 0.2)]).view(Z, 1, Lq, Lk)
+    keep[1, 0, 10:150] = False  # query rows that attend nothing: zeros
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    be, scale = _lib.backend(), D**-0.5
+    print(f"case rectangular lists {dt} D{D} Lq{Lq} Lk{Lk}", flush=True)
+
+    def run(dmask):
+        o, ot, M, mu = be.fwd(*dev[:6], dmask, _lib.MASK_BOOL, False, scale)
+        grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, _lib.MASK_BOOL, False, scale, want_tangent_grads=True)
+        return [o, ot, M, mu, *grads]
+
+    dmask = keep.cuda()
+    with_lists = run(dmask)
+    tq, tk = getattr(dmask, "_jvpfa_tiles")[1:3]
+    rq, rk = _numpy_tile_lists_rect(keep.reshape(-1, Lq, Lk).numpy(), Lq, Lk)
+    for got, ref, nt in ((tq, rq, (Lk + 63) // 64), (tk, rk, (Lq + 63) // 64)):
+        got = got.cpu().view(-1, nt + 1).tolist()
+        assert len(got) == len(ref)
+        for row, want in zip(got, ref):
+            assert row[0] == len(want) and row[1:1 + row[0]] == want
+    _lib.set_tile_lists(False)
+    try:
+        every_tile = run(keep.cuda())
+    finally:
+        _lib.set_tile_lists(True)
+    for a, b in zip(with_lists, every_tile):
+        assert torch.equal(a, b)
+    ref = dense.forward(*f64[:6], mask=keep.numpy(), causal=False, scale=scale)
+    rb = dense.backward(*f64, mask=keep.numpy(), causal=False, scale=scale)
     _tol_check("O", with_lists[0], ref["O"], dtype)
     _tol_check("O'", with_lists[1], ref["Ot"], dtype)
     for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), with_lists[4:10]):
