@@ -36,7 +36,7 @@ enum jvpfa_mask_kind { JVPFA_MASK_NONE = 0, JVPFA_MASK_BOOL = 1, JVPFA_MASK_ADD 
 enum jvpfa_status {
   JVPFA_OK = 0,
   JVPFA_E_NULL = -1,      /* a required pointer is NULL */
-  JVPFA_E_SHAPE = -2,     /* Z,H,L < 1, D not in {32, 64, 128, 256}, D = 256 with fp32 or with dropout, dropout_p outside [0, 1) */
+  JVPFA_E_SHAPE = -2,     /* Z,H,L < 1, D not in {32, 64, 128, 256}, D = 256 with dropout, dropout_p outside [0, 1) */
   JVPFA_E_DTYPE = -3,     /* dtype / mask_kind out of range */
   JVPFA_E_ALIGN = -4,     /* a tensor pointer is not 16-byte aligned */
   JVPFA_E_CONFLICT = -5,  /* causal together with a mask (JA:2380-2381 raises ValueError) */
@@ -47,7 +47,7 @@ enum jvpfa_status {
 
 /* Shape, numeric type and masking shared by forward and backward. */
 typedef struct jvpfa_problem {
-  int32_t Z, H, L, D; /* D in {32, 64, 128, 256} (JA:2371-2374); 256 for bf16 / fp16 only */
+  int32_t Z, H, L, D; /* D in {32, 64, 128, 256} (JA:2371-2374) */
   int32_t dtype;      /* enum jvpfa_dtype: element type of q,k,v,o and their tangents/gradients */
   int32_t causal;     /* 0/1; lower-triangular (query index >= key index), JA:253-258 */
   int32_t mask_kind;  /* enum jvpfa_mask_kind */

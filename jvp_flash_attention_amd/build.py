@@ -25,7 +25,7 @@ FLAGS = [
 ]
 
 TYPES = {"bf16": "__bf16", "fp16": "_Float16", "fp32": "float"}
-DIMS = (32, 64, 128, 256)  # 256: 16-bit element types only
+DIMS = (32, 64, 128, 256)
 
 
 def units():
@@ -37,8 +37,6 @@ def units():
             continue
         for tag, ctype in TYPES.items():
             for d in DIMS:
-                if d == 256 and tag == "fp32":
-                    continue
                 name = f"{kind}_{tag}_{d}"
                 out.append((name, src, [f"-DJVPFA_T={ctype}", f"-DJVPFA_D={d}", f"-DJVPFA_NAME={name}"]))
     for api in ("api_fwd", "api_bwd", "mask_tiles"):

@@ -12,11 +12,11 @@ namespace jvpfa {
 #define JVPFA_DECL(name) int name(const BwdParams &, int, bool, bool, hipStream_t);
 JVPFA_DECL(bwd_bf16_32) JVPFA_DECL(bwd_bf16_64) JVPFA_DECL(bwd_bf16_128) JVPFA_DECL(bwd_bf16_256)
 JVPFA_DECL(bwd_fp16_32) JVPFA_DECL(bwd_fp16_64) JVPFA_DECL(bwd_fp16_128) JVPFA_DECL(bwd_fp16_256)
-JVPFA_DECL(bwd_fp32_32) JVPFA_DECL(bwd_fp32_64) JVPFA_DECL(bwd_fp32_128)
+JVPFA_DECL(bwd_fp32_32) JVPFA_DECL(bwd_fp32_64) JVPFA_DECL(bwd_fp32_128) JVPFA_DECL(bwd_fp32_256)
 #undef JVPFA_DECL
 typedef int (*bwd_launcher)(const BwdParams &, int, bool, bool, hipStream_t);
 static const bwd_launcher kBwd[12] = {bwd_bf16_32, bwd_bf16_64, bwd_bf16_128, bwd_bf16_256, bwd_fp16_32, bwd_fp16_64,
-                                      bwd_fp16_128, bwd_fp16_256, bwd_fp32_32, bwd_fp32_64, bwd_fp32_128, nullptr};
+                                      bwd_fp16_128, bwd_fp16_256, bwd_fp32_32, bwd_fp32_64, bwd_fp32_128, bwd_fp32_256};
 
 // Each row statistic is padded to a multiple of 4 floats so the three arrays stay 16-byte aligned.
 static inline size_t stat_floats(int Z, int H, int L) { return (((size_t)Z * H * L) + 3) & ~(size_t)3; }

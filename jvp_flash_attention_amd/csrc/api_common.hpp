@@ -13,7 +13,6 @@ inline int check_problem(const jvpfa_problem &p) {
   if (p.Z < 1 || p.H < 1 || p.L < 1) return JVPFA_E_SHAPE;
   if (p.D != 32 && p.D != 64 && p.D != 128 && p.D != 256) return JVPFA_E_SHAPE;
   if (p.dtype < JVPFA_BF16 || p.dtype > JVPFA_FP32) return JVPFA_E_DTYPE;
-  if (p.D == 256 && p.dtype == JVPFA_FP32) return JVPFA_E_SHAPE;  // the fp32 tiles of D = 256 do not fit the LDS
   if (p.mask_kind < JVPFA_MASK_NONE || p.mask_kind > JVPFA_MASK_ADD) return JVPFA_E_DTYPE;
   if (!(p.dropout_p >= 0.f && p.dropout_p < 1.f)) return JVPFA_E_SHAPE;
   if (p.dropout_p > 0.f && p.D == 256) return JVPFA_E_SHAPE;  // the kernels with dropout stop at D = 128

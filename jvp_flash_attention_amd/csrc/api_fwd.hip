@@ -9,11 +9,11 @@ namespace jvpfa {
 #define JVPFA_DECL(name) int name(const FwdParams &, bool, int, hipStream_t);
 JVPFA_DECL(fwd_bf16_32) JVPFA_DECL(fwd_bf16_64) JVPFA_DECL(fwd_bf16_128) JVPFA_DECL(fwd_bf16_256)
 JVPFA_DECL(fwd_fp16_32) JVPFA_DECL(fwd_fp16_64) JVPFA_DECL(fwd_fp16_128) JVPFA_DECL(fwd_fp16_256)
-JVPFA_DECL(fwd_fp32_32) JVPFA_DECL(fwd_fp32_64) JVPFA_DECL(fwd_fp32_128)
+JVPFA_DECL(fwd_fp32_32) JVPFA_DECL(fwd_fp32_64) JVPFA_DECL(fwd_fp32_128) JVPFA_DECL(fwd_fp32_256)
 #undef JVPFA_DECL
 typedef int (*fwd_launcher)(const FwdParams &, bool, int, hipStream_t);
 static const fwd_launcher kFwd[12] = {fwd_bf16_32, fwd_bf16_64, fwd_bf16_128, fwd_bf16_256, fwd_fp16_32, fwd_fp16_64,
-                                      fwd_fp16_128, fwd_fp16_256, fwd_fp32_32, fwd_fp32_64, fwd_fp32_128, nullptr};
+                                      fwd_fp16_128, fwd_fp16_256, fwd_fp32_32, fwd_fp32_64, fwd_fp32_128, fwd_fp32_256};
 }  // namespace jvpfa
 
 using namespace jvpfa;
@@ -62,7 +62,7 @@ extern "C" const char *jvpfa_error_string(int status) {
   switch (status) {
     case JVPFA_OK: return "ok";
     case JVPFA_E_NULL: return "a required pointer is NULL";
-    case JVPFA_E_SHAPE: return "unsupported shape (Z,H,L >= 1 and D in {32,64,128,256} required; 256 not with fp32 nor with dropout; dropout_p in [0,1))";
+    case JVPFA_E_SHAPE: return "unsupported shape (Z,H,L >= 1 and D in {32,64,128,256} required; 256 not with dropout; dropout_p in [0,1))";
     case JVPFA_E_DTYPE: return "dtype or mask kind out of range";
     case JVPFA_E_ALIGN: return "tensor pointer not 16-byte aligned";
     case JVPFA_E_CONFLICT: return "causal attention does not take a mask";

@@ -71,9 +71,15 @@ template <typename T, int D, int MODE> struct BwdCfg {
   static constexpr int T_ELEMS = D * LDT;
   // dq:   PLAIN K,V,K^T | DUAL K,K',V,V',K^T,K'^T | TANGENT K,V,K^T
   // dkdv: PLAIN Q,gO,Q^T,gO^T | DUAL Q,Q',gO,gT + 4 transposed | TANGENT Q,gT,Q^T,gT^T
-  static constexpr int DQ_NAT = MODE == BWD_DUAL ? 4 : 2;
+  // Rows of 1024 bytes (fp32, D = 256): a wave's own rows of four operands would be the whole register file
+  // (4 x 128 registers) and eight 32-row tiles twice the LDS, so there the own rows are read from global
+  // memory where they are used (the same 32 bytes per lane every tile: cache hits) and only the tiles whose
+  // fragments run along the streamed index are staged (dq: K, K' both ways; dk/dv: the four transposed ones);
+  // the other row-wise fragments also come straight from global memory.
+  static constexpr bool SB = sizeof(T) == 4 && D == 256;
+  static constexpr int DQ_NAT = SB ? (MODE == BWD_DUAL ? 2 : 1) : (MODE == BWD_DUAL ? 4 : 2);
   static constexpr int DQ_TR = MODE == BWD_DUAL ? 2 : 1;
-  static constexpr int DKV_NAT = MODE == BWD_DUAL ? 4 : 2;
+  static constexpr int DKV_NAT = SB ? 0 : (MODE == BWD_DUAL ? 4 : 2);
   static constexpr int DKV_TR = MODE == BWD_DUAL ? 4 : 2;
   static constexpr size_t DQ_LDS = (size_t)(DQ_NAT * N_ELEMS + DQ_TR * T_ELEMS) * sizeof(T);
   static constexpr size_t DKV_LDS = (size_t)(DKV_NAT * N_ELEMS + DKV_TR * T_ELEMS) * sizeof(T) + 5 * BWD_T * sizeof(float);
@@ -104,6 +110,17 @@ __device__ __forceinline__ void gemm_tile(f32x16 &acc, const T *tile, int ld, in
   }
 }
 
+// The same with the B fragments (the lane's own row) read from global memory where they are used; `tile` may
+// be an LDS tile or rows of global memory (then `ld` is the row length and `arow` an index clamped by the caller).
+template <int KK, typename T>
+__device__ __forceinline__ void gemm_tile(f32x16 &acc, const T *tile, int ld, int arow, int g, const T *brow) {
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    mma(acc, lds_frag(tile + (size_t)arow * ld + 16 * kk + 8 * g), ld8<T>(brow + 16 * kk + 8 * g));
+    if (kk % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 __device__ __forceinline__ void zero16(f32x16 &x) {
 #pragma unroll
   for (int e = 0; e < 16; ++e) x[e] = 0.f;
@@ -120,12 +137,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
   constexpr float NEG_INF = -__builtin_inff();
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  constexpr bool SB = Cfg::SB;    // V, V' are not staged (see BwdCfg)
   T *Kn = reinterpret_cast<T *>(smem_raw);
   T *Vn = Kn + Cfg::N_ELEMS;
-  T *KT = Vn + Cfg::N_ELEMS;
+  T *KT = SB ? Vn : Vn + Cfg::N_ELEMS;
   T *Ktn = KT + Cfg::T_ELEMS;     // DUAL only from here on
   T *Vtn = Ktn + Cfg::N_ELEMS;
-  T *KtT = Vtn + Cfg::N_ELEMS;
+  T *KtT = SB ? Vtn : Vtn + Cfg::N_ELEMS;
 
   const Problem &pr = p.pr;
   const int L = pr.L;
@@ -145,13 +163,21 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
   const int qld = qrow < L ? qrow : L - 1;
   const bool has_go = p.go != nullptr;
 
-  Frag<T> Qf[KK], gOf[TAN ? 1 : KK], Qtf[DUAL ? KK : 1], gTf[(DUAL || TAN) ? KK : 1];
-  load_row_frags<KK>(Qf, reinterpret_cast<const T *>(p.q) + head + (size_t)qld * D, g);
-  if constexpr (!TAN) {
-    if (has_go) load_row_frags<KK>(gOf, reinterpret_cast<const T *>(p.go) + head + (size_t)qld * D, g);
+  // this lane's own row of the tensors that are B operands: resident fragments, or (SB) pointers to read through
+  const T *Qrow = reinterpret_cast<const T *>(p.q) + head + (size_t)qld * D;
+  const T *gOrow = (!TAN && has_go) ? reinterpret_cast<const T *>(p.go) + head + (size_t)qld * D : nullptr;
+  const T *Qtrow = DUAL ? reinterpret_cast<const T *>(p.qt) + head + (size_t)qld * D : nullptr;
+  const T *gTrow = (DUAL || TAN) ? reinterpret_cast<const T *>(p.gt) + head + (size_t)qld * D : nullptr;
+  constexpr int KR = SB ? 1 : KK;
+  Frag<T> Qf[KR], gOf[TAN ? 1 : KR], Qtf[DUAL ? KR : 1], gTf[(DUAL || TAN) ? KR : 1];
+  if constexpr (!SB) {
+    load_row_frags<KK>(Qf, Qrow, g);
+    if constexpr (!TAN) {
+      if (has_go) load_row_frags<KK>(gOf, gOrow, g);
+    }
+    if constexpr (DUAL) load_row_frags<KK>(Qtf, Qtrow, g);
+    if constexpr (DUAL || TAN) load_row_frags<KK>(gTf, gTrow, g);
   }
-  if constexpr (DUAL) load_row_frags<KK>(Qtf, reinterpret_cast<const T *>(p.qt) + head + (size_t)qld * D, g);
-  if constexpr (DUAL || TAN) load_row_frags<KK>(gTf, reinterpret_cast<const T *>(p.gt) + head + (size_t)qld * D, g);
 
   const float Mq = qrow < L ? p.M[srow + qld] : __builtin_inff();
   const float d1 = (MODE == BWD_PLAIN) ? p.d1[srow + qld] : 0.f;  // BWD_DUAL: d2 already holds d1 + d2
@@ -217,11 +243,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
     } else {
       const int nvalid = Lk - j0;
       copy_rows<T, BWD_T, D, BWD_NT>(Kn, Cfg::LDN, Kg + (size_t)j0 * D, nvalid, tid);
-      copy_rows<T, BWD_T, D, BWD_NT>(Vn, Cfg::LDN, Vg + (size_t)j0 * D, nvalid, tid);
+      if constexpr (!SB) copy_rows<T, BWD_T, D, BWD_NT>(Vn, Cfg::LDN, Vg + (size_t)j0 * D, nvalid, tid);
       copy_rows_transposed<T, BWD_T, D, BWD_NT>(KT, Cfg::LDT, Kg + (size_t)j0 * D, nvalid, tid);
       if constexpr (DUAL) {
         copy_rows<T, BWD_T, D, BWD_NT>(Ktn, Cfg::LDN, Ktg + (size_t)j0 * D, nvalid, tid);
-        copy_rows<T, BWD_T, D, BWD_NT>(Vtn, Cfg::LDN, Vtg + (size_t)j0 * D, nvalid, tid);
+        if constexpr (!SB) copy_rows<T, BWD_T, D, BWD_NT>(Vtn, Cfg::LDN, Vtg + (size_t)j0 * D, nvalid, tid);
         copy_rows_transposed<T, BWD_T, D, BWD_NT>(KtT, Cfg::LDT, Ktg + (size_t)j0 * D, nvalid, tid);
       }
     }
@@ -232,6 +258,26 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
 
     f32x16 S, dP, Sp, At;  // DUAL: dP also collects gT V'^T (the B term)
     zero16(S);
+    if constexpr (SB) {
+      // V, V' fragments from global memory: this lane's key row, clamped (a key past the end has p = 0 and
+      // must meet finite values)
+      const int vrow = min(j0 + pr32, Lk - 1);
+      gemm_tile<KK>(S, Kn, Cfg::LDN, pr32, g, Qrow);
+      if constexpr (!TAN) {
+        zero16(dP);
+        if (has_go) gemm_tile<KK>(dP, Vg, D, vrow, g, gOrow);
+      }
+      if constexpr (DUAL) {
+        zero16(Sp);
+        gemm_tile<KK>(Sp, Kn, Cfg::LDN, pr32, g, Qtrow);
+        gemm_tile<KK>(Sp, Ktn, Cfg::LDN, pr32, g, Qrow);
+        gemm_tile<KK>(dP, Vtg, D, vrow, g, gTrow);
+      }
+      if constexpr (DUAL || TAN) {
+        zero16(At);
+        gemm_tile<KK>(At, Vg, D, vrow, g, gTrow);
+      }
+    } else {
     gemm_tile<KK>(S, Kn, Cfg::LDN, pr32, g, Qf);
     if constexpr (!TAN) {
       zero16(dP);
@@ -246,6 +292,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
     if constexpr (DUAL || TAN) {
       zero16(At);
       gemm_tile<KK>(At, Vn, Cfg::LDN, pr32, g, gTf);
+    }
     }
 
     const bool diag = pr.causal && (j0 + BWD_T - 1 > q0 + wave * 32);
@@ -355,12 +402,21 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
   const int kld = krow < Lk ? krow : Lk - 1;
   const bool has_go = p.go != nullptr;
 
-  Frag<T> Kf[KK], Vf[KK], Ktf[DUAL ? KK : 1], Vtf[DUAL ? KK : 1];
-  load_row_frags<KK>(Kf, reinterpret_cast<const T *>(p.k) + kvhead + (size_t)kld * D, g);
-  load_row_frags<KK>(Vf, reinterpret_cast<const T *>(p.v) + kvhead + (size_t)kld * D, g);
-  if constexpr (DUAL) {
-    load_row_frags<KK>(Ktf, reinterpret_cast<const T *>(p.kt) + kvhead + (size_t)kld * D, g);
-    load_row_frags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + kvhead + (size_t)kld * D, g);
+  // this lane's own key row of K, V (, K', V'): resident fragments, or (SB, see BwdCfg) pointers to read through
+  constexpr bool SB = Cfg::SB;
+  const T *Krow = reinterpret_cast<const T *>(p.k) + kvhead + (size_t)kld * D;
+  const T *Vrow = reinterpret_cast<const T *>(p.v) + kvhead + (size_t)kld * D;
+  const T *Ktrow = DUAL ? reinterpret_cast<const T *>(p.kt) + kvhead + (size_t)kld * D : nullptr;
+  const T *Vtrow = DUAL ? reinterpret_cast<const T *>(p.vt) + kvhead + (size_t)kld * D : nullptr;
+  constexpr int KR = SB ? 1 : KK;
+  Frag<T> Kf[KR], Vf[KR], Ktf[DUAL ? KR : 1], Vtf[DUAL ? KR : 1];
+  if constexpr (!SB) {
+    load_row_frags<KK>(Kf, Krow, g);
+    load_row_frags<KK>(Vf, Vrow, g);
+    if constexpr (DUAL) {
+      load_row_frags<KK>(Ktf, Ktrow, g);
+      load_row_frags<KK>(Vtf, Vtrow, g);
+    }
   }
 
   f32x16 dK[DB], dV[DB];
@@ -446,16 +502,16 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
       }
     } else {
       const int nvalid = L - i0;
-      copy_rows<T, BWD_T, D, BWD_NT>(Qn, Cfg::LDN, Qg + (size_t)i0 * D, nvalid, tid);
+      if constexpr (!SB) copy_rows<T, BWD_T, D, BWD_NT>(Qn, Cfg::LDN, Qg + (size_t)i0 * D, nvalid, tid);
       copy_rows_transposed<T, BWD_T, D, BWD_NT>(QT, Cfg::LDT, Qg + (size_t)i0 * D, nvalid, tid);
       if (Gg) {
-        copy_rows<T, BWD_T, D, BWD_NT>(Gn, Cfg::LDN, Gg + (size_t)i0 * D, nvalid, tid);
+        if constexpr (!SB) copy_rows<T, BWD_T, D, BWD_NT>(Gn, Cfg::LDN, Gg + (size_t)i0 * D, nvalid, tid);
         copy_rows_transposed<T, BWD_T, D, BWD_NT>(GT, Cfg::LDT, Gg + (size_t)i0 * D, nvalid, tid);
       }
       if constexpr (DUAL) {
-        copy_rows<T, BWD_T, D, BWD_NT>(Qtn, Cfg::LDN, Qtg + (size_t)i0 * D, nvalid, tid);
+        if constexpr (!SB) copy_rows<T, BWD_T, D, BWD_NT>(Qtn, Cfg::LDN, Qtg + (size_t)i0 * D, nvalid, tid);
         copy_rows_transposed<T, BWD_T, D, BWD_NT>(QtT, Cfg::LDT, Qtg + (size_t)i0 * D, nvalid, tid);
-        copy_rows<T, BWD_T, D, BWD_NT>(GTn, Cfg::LDN, gTg + (size_t)i0 * D, nvalid, tid);
+        if constexpr (!SB) copy_rows<T, BWD_T, D, BWD_NT>(GTn, Cfg::LDN, gTg + (size_t)i0 * D, nvalid, tid);
         copy_rows_transposed<T, BWD_T, D, BWD_NT>(GTT, Cfg::LDT, gTg + (size_t)i0 * D, nvalid, tid);
       }
       fetch_stats(i0);
@@ -468,6 +524,28 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
 
     f32x16 S, dP, Sp, At;  // DUAL: dP also collects V' gT^T (the B term)
     zero16(S);
+    if constexpr (SB) {
+      // row-wise fragments of Q, G (, Q', gT) from global memory: this lane's query row, clamped (a query past
+      // the end has p = 0 and must meet finite values)
+      const int qr = min(i0 + pr32, L - 1);
+      gemm_tile<KK>(S, Qg, D, qr, g, Krow);
+      if constexpr (!TAN) {
+        zero16(dP);
+        if (has_go) gemm_tile<KK>(dP, Gg, D, qr, g, Vrow);
+      }
+      if constexpr (DUAL) {
+        zero16(Sp);
+        gemm_tile<KK>(Sp, Qtg, D, qr, g, Krow);
+        gemm_tile<KK>(Sp, Qg, D, qr, g, Ktrow);
+        zero16(At);
+        gemm_tile<KK>(At, gTg, D, qr, g, Vrow);
+        gemm_tile<KK>(dP, gTg, D, qr, g, Vtrow);
+      }
+      if constexpr (TAN) {
+        zero16(At);
+        gemm_tile<KK>(At, Gg, D, qr, g, Vrow);
+      }
+    } else {
     gemm_tile<KK>(S, Qn, Cfg::LDN, pr32, g, Kf);
     if constexpr (!TAN) {
       zero16(dP);
@@ -484,6 +562,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
     if constexpr (TAN) {
       zero16(At);
       gemm_tile<KK>(At, Gn, Cfg::LDN, pr32, g, Vf);
+    }
     }
 
     const bool diag = pr.causal && (i0 < k0 + wave * 32 + 31);  // some query may precede a key

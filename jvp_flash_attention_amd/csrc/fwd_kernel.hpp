@@ -75,11 +75,18 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
   const int qrow = q0 + wave * 32 + r; // this lane's query row
   const int qld = qrow < L ? qrow : L - 1;
 
-  Frag<T> Qf[KK], Qtf[DUAL ? KK : 1];
+  // Rows of 1024 bytes (fp32, D = 256): Q, Q' resident would be 256 registers next to 256 of accumulators, so
+  // there the lane's fragments are read from global memory where they are used (the same 32 bytes per lane on
+  // every tile: cache hits)
+  constexpr bool SB = sizeof(T) == 4 && D == 256;
+  const T *Qrow = Qg + (size_t)qld * D + 8 * g, *Qtrow = DUAL ? Qtg + (size_t)qld * D + 8 * g : nullptr;
+  Frag<T> Qf[SB ? 1 : KK], Qtf[(DUAL && !SB) ? KK : 1];
+  if constexpr (!SB) {
 #pragma unroll
-  for (int kk = 0; kk < KK; ++kk) {
-    Qf[kk] = ld8<T>(Qg + (size_t)qld * D + 16 * kk + 8 * g);
-    if constexpr (DUAL) Qtf[kk] = ld8<T>(Qtg + (size_t)qld * D + 16 * kk + 8 * g);
+    for (int kk = 0; kk < KK; ++kk) {
+      Qf[kk] = ld8<T>(Qrow + 16 * kk);
+      if constexpr (DUAL) Qtf[kk] = ld8<T>(Qtrow + 16 * kk);
+    }
   }
 
   f32x16 Oacc[DB], Tacc[DUAL ? DB : 1];
@@ -165,11 +172,22 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
         Frag<T> a = lds_frag(Ks + (32 * nb + pr32) * Cfg::LDK + 16 * kk + 8 * g);
+        if constexpr (SB) {
+          const Frag<T> qf = ld8<T>(Qrow + 16 * kk);
+          mma(S[nb], a, qf);
+          if constexpr (DUAL) {
+            mma(Sp[nb], a, ld8<T>(Qtrow + 16 * kk));
+            Frag<T> a2 = lds_frag(Kts + (32 * nb + pr32) * Cfg::LDK + 16 * kk + 8 * g);
+            mma(Sp[nb], a2, qf);
+          }
+          if (kk % 4 == 3) __builtin_amdgcn_sched_barrier(0);  // bound the fragment reads in flight
+        } else {
         mma(S[nb], a, Qf[kk]);
         if constexpr (DUAL) {
           mma(Sp[nb], a, Qtf[kk]);
           Frag<T> a2 = lds_frag(Kts + (32 * nb + pr32) * Cfg::LDK + 16 * kk + 8 * g);
           mma(Sp[nb], a2, Qf[kk]);
+        }
         }
       }
     }

@@ -23,7 +23,7 @@ Differences from the reference, all deliberate:
   functions of O' (Hessian-vector products) reach q, k, v and the input tangents.  The
   reference's tangent is a constant (JA:2399, JA:2828) and its backward ignores it (JA:2831).
 * Any sequence length L >= 1 and head dims {32, 64, 128, 256} (the reference: L a multiple of 32,
-  JA:2371-2378, JA:2892); D = 256 for bf16 / fp16 only.
+  JA:2371-2378, JA:2892).
 * k and v may have fewer heads than q (grouped heads: H a multiple of H_kv) and a length of their own
   (cross-attention); causal then means key index <= query index, as in SDPA.  The reference requires
   q, k, v of one shape (JA:2367-2378).
@@ -49,7 +49,7 @@ from . import _lib
 
 MASK_CONST = -100.0  # JA:48-50: value float masks use for "masked"; far below any real logit
 MIN_SEQUENCE_LENGTH = 32  # JA:51; kept for importers, not a limit of these kernels
-SUPPORTED_HEAD_DIMS = (32, 64, 128, 256)  # 256: bf16 / fp16 only
+SUPPORTED_HEAD_DIMS = (32, 64, 128, 256)
 BLOCK_M = 128  # query rows per workgroup of the forward kernel (only reported through Grid)
 
 
@@ -92,9 +92,6 @@ def _validate(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dropout
     assert k.shape == v.shape and k.shape[0] == Z and H % k.shape[1] == 0, (
         "JVP attention requires k and v of one shape (Z, H_kv, N_CTX_kv, HEAD_DIM) with H a multiple of H_kv,"
         f" but got q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}"
-    )
-    assert not (HEAD_DIM_K == 256 and q.dtype == torch.float32), (
-        "JVP attention supports HEAD_DIM_K=256 for bfloat16 and float16 only"
     )
     assert N_CTX >= 1, f"JVP attention requires N_CTX >= 1, but got N_CTX={N_CTX}"
     assert q.dtype in _lib.DTYPES and k.dtype == q.dtype and v.dtype == q.dtype, (

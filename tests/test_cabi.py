@@ -74,7 +74,7 @@ def _fwd_args(**kw):
         (dict(struct_size=4), -7),
         (dict(q=None), -1),
         (dict(p_D=48), -2),
-        (dict(p_D=256, p_dtype=2), -2),     # D = 256 exists for the 16-bit element types only
+        (dict(p_D=256, p_dropout_p=0.1), -2),  # dropout stops at D = 128
         (dict(p_L=0), -2),
         (dict(p_dtype=5), -3),
         (dict(p_mask_kind=1), -1),          # mask kind set, mask pointer NULL

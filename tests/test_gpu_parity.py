@@ -114,16 +114,18 @@ def test_dual_fwd_bwd_dense_and_causal(dt, D, mode):
     _run_case(2, 2, 256, D, DTYPES[dt], mode)
 
 
-@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
 @pytest.mark.parametrize("mode", ["none", "causal", "keypad", "bias", "bool_full"])
 def test_head_dim_256(dt, mode):
-    # the largest head dim the reference admits (its jvp_attention.py:2371-2374); 16-bit element types only here
+    # the largest head dim the reference admits (its jvp_attention.py:2371-2374)
     _run_case(1, 2, 200, 256, DTYPES[dt], mode, seed=17)
 
 
-def test_head_dim_256_in_fp32_is_refused():
-    with pytest.raises(RuntimeError, match="unsupported shape"):
-        _run_case(1, 1, 64, 256, torch.float32, "none")
+def test_head_dim_256_in_fp32_plain_and_at_a_benchmark_length():
+    """fp32 at D = 256 reads its own rows' fragments from global memory instead of keeping them in registers:
+    the plain path, and a length with many interior tiles (causal, so that both loops' edges are crossed)."""
+    _run_case(1, 2, 200, 256, torch.float32, "none", seed=18, plain=True)
+    _run_case(1, 1, 1024, 256, torch.float32, "causal", seed=19)
 
 
 @pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
@@ -258,7 +260,7 @@ def test_mask_tile_lists_match_a_numpy_scan(kind, as_bias, L):
 
 
 @pytest.mark.parametrize("dt,D", [("bf16", 32), ("bf16", 64), ("bf16", 128), ("bf16", 256),
-                                  ("fp32", 32), ("fp32", 64), ("fp32", 128)])
+                                  ("fp32", 32), ("fp32", 64), ("fp32", 128), ("fp32", 256)])
 @pytest.mark.parametrize("kind", ["blockdiag", "band", "pad2d", "lower"])
 @pytest.mark.parametrize("as_bias", [False, True])
 def test_structured_masks_with_skipped_tiles(dt, D, kind, as_bias):
@@ -379,7 +381,7 @@ def test_random_configurations(seed):
 
     rng = np.random.default_rng(1000 + seed)
     dt = ["bf16", "fp16", "fp32"][rng.integers(3)]
-    D = [32, 64, 128, 256][rng.integers(4)] if dt != "fp32" else [32, 64, 128][rng.integers(3)]
+    D = [32, 64, 128, 256][rng.integers(4)] if dt != "fp32" else [32, 64, 128, 256][int(rng.integers(3)) + (seed % 5 == 4)]
     Z, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
     long_case = seed % 3 == 0
     L = int(rng.integers(513, 900)) if long_case else int(rng.integers(1, 300))
@@ -626,7 +628,7 @@ def test_grouped_heads_and_a_key_length_of_its_own(dt, D, shape, mode):
     _run_kv_shape_case(dt, D, shape, mode)
 
 
-@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
 @pytest.mark.parametrize("shape", [(4, 2, 96, 96), (2, 1, 70, 200), (2, 2, 200, 70), (1, 1, 1, 3), (1, 1, 33, 31), (2, 2, 5, 2)])
 @pytest.mark.parametrize("mode", ["none", "causal", "bool", "bias"])
 def test_head_dim_256_with_grouped_heads_key_lengths_and_tiny_shapes(dt, shape, mode):
