@@ -36,7 +36,7 @@ enum jvpfa_mask_kind { JVPFA_MASK_NONE = 0, JVPFA_MASK_BOOL = 1, JVPFA_MASK_ADD 
 enum jvpfa_status {
   JVPFA_OK = 0,
   JVPFA_E_NULL = -1,      /* a required pointer is NULL */
-  JVPFA_E_SHAPE = -2,     /* Z,H,L < 1, D not in {32, 64, 128, 256}, D = 256 with dropout, dropout_p outside [0, 1) */
+  JVPFA_E_SHAPE = -2,     /* Z,H,L < 1, D not in {32, 64, 128, 256}, dropout_p outside [0, 1) */
   JVPFA_E_DTYPE = -3,     /* dtype / mask_kind out of range */
   JVPFA_E_ALIGN = -4,     /* a tensor pointer is not 16-byte aligned */
   JVPFA_E_CONFLICT = -5,  /* causal together with a mask (JA:2380-2381 raises ValueError) */
@@ -59,7 +59,7 @@ typedef struct jvpfa_problem {
    * dropped by a counter-based hash of (dropout_seed, entry index) and kept entries are scaled by 1/(1 - p), as
    * torch's scaled_dot_product_attention does; forward and backward of one call pair must get the same seed.
    * jvpfa_dropout_keep() writes the keep pattern out.  The reference carries dead code for dropout and raises
-   * NotImplementedError (JA:94-122, JA:271-277, JA:2356-2357).  D <= 128; runs on the register-staged kernels
+   * NotImplementedError (JA:94-122, JA:271-277, JA:2356-2357).  Runs on the register-staged kernels
    * for every element type (about 3x slower than without dropout for bf16 / fp16). */
   float dropout_p;
   uint64_t dropout_seed;

@@ -15,7 +15,6 @@ inline int check_problem(const jvpfa_problem &p) {
   if (p.dtype < JVPFA_BF16 || p.dtype > JVPFA_FP32) return JVPFA_E_DTYPE;
   if (p.mask_kind < JVPFA_MASK_NONE || p.mask_kind > JVPFA_MASK_ADD) return JVPFA_E_DTYPE;
   if (!(p.dropout_p >= 0.f && p.dropout_p < 1.f)) return JVPFA_E_SHAPE;
-  if (p.dropout_p > 0.f && p.D == 256) return JVPFA_E_SHAPE;  // the kernels with dropout stop at D = 128
   if (p.mask_kind != JVPFA_MASK_NONE) {
     if (p.causal) return JVPFA_E_CONFLICT;
     if (!p.mask) return JVPFA_E_NULL;

@@ -62,7 +62,7 @@ extern "C" const char *jvpfa_error_string(int status) {
   switch (status) {
     case JVPFA_OK: return "ok";
     case JVPFA_E_NULL: return "a required pointer is NULL";
-    case JVPFA_E_SHAPE: return "unsupported shape (Z,H,L >= 1 and D in {32,64,128,256} required; 256 not with dropout; dropout_p in [0,1))";
+    case JVPFA_E_SHAPE: return "unsupported shape (Z,H,L >= 1 and D in {32,64,128,256} and dropout_p in [0,1) required)";
     case JVPFA_E_DTYPE: return "dtype or mask kind out of range";
     case JVPFA_E_ALIGN: return "tensor pointer not 16-byte aligned";
     case JVPFA_E_CONFLICT: return "causal attention does not take a mask";

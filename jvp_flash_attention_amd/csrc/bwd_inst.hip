@@ -35,17 +35,14 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
   if (kv_blocks > 0x7fffffffLL) return -2;
   if (p.pr.drop_thr != 0) {
     // dropout: every element type takes the register-staged kernels, the one family that carries it
-    if constexpr (D <= 128) {
-      auto kq = bwd_dq_kernel<T, D, MODE, MASK, true>;
-      auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK, true>;
-      int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);
-      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg::DKV_LDS);
-      if (rc != 0) return rc;
-      hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
-      hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DQ_LDS, stream, p);
-      return hipGetLastError() == hipSuccess ? 0 : -6;
-    }
-    return -2;
+    auto kq = bwd_dq_kernel<T, D, MODE, MASK, true>;
+    auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK, true>;
+    int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);
+    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg::DKV_LDS);
+    if (rc != 0) return rc;
+    hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+    hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DQ_LDS, stream, p);
+    return hipGetLastError() == hipSuccess ? 0 : -6;
   }
   if constexpr (sizeof(T) == 2 && D <= 128) {  // direct-to-LDS, double-buffered kernels
    {

@@ -71,12 +71,13 @@ template <typename T, int D, int MODE> struct BwdCfg {
   static constexpr int T_ELEMS = D * LDT;
   // dq:   PLAIN K,V,K^T | DUAL K,K',V,V',K^T,K'^T | TANGENT K,V,K^T
   // dkdv: PLAIN Q,gO,Q^T,gO^T | DUAL Q,Q',gO,gT + 4 transposed | TANGENT Q,gT,Q^T,gT^T
-  // Rows of 1024 bytes (fp32, D = 256): a wave's own rows of four operands would be the whole register file
-  // (4 x 128 registers) and eight 32-row tiles twice the LDS, so there the own rows are read from global
+  // D = 256 (fp32: rows of 1024 bytes; 16-bit types come here with dropout only): a wave's own rows of four
+  // operands would be the whole register file (fp32: 4 x 128 registers, next to 128 - 256 of accumulators) and
+  // eight 32-row fp32 tiles twice the LDS, so there the own rows are read from global
   // memory where they are used (the same 32 bytes per lane every tile: cache hits) and only the tiles whose
   // fragments run along the streamed index are staged (dq: K, K' both ways; dk/dv: the four transposed ones);
   // the other row-wise fragments also come straight from global memory.
-  static constexpr bool SB = sizeof(T) == 4 && D == 256;
+  static constexpr bool SB = D == 256;
   static constexpr int DQ_NAT = SB ? (MODE == BWD_DUAL ? 2 : 1) : (MODE == BWD_DUAL ? 4 : 2);
   static constexpr int DQ_TR = MODE == BWD_DUAL ? 2 : 1;
   static constexpr int DKV_NAT = SB ? 0 : (MODE == BWD_DUAL ? 4 : 2);

@@ -85,15 +85,13 @@ template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
   if (p.pr.drop_thr != 0) {
     // dropout: every element type takes the register-staged kernel, the one family that carries it
-    if constexpr (D <= 128) {
-      constexpr int BNG = sizeof(T) == 4 ? 32 : 64;
-      switch (mask) {
-        case MASK_NONE: return launch_fwd_one<T, D, BNG, DUAL, MASK_NONE, true>(p, stream);
-        case MASK_BOOL: return launch_fwd_one<T, D, BNG, DUAL, MASK_BOOL, true>(p, stream);
-        case MASK_ADD: return launch_fwd_one<T, D, BNG, DUAL, MASK_ADD, true>(p, stream);
-      }
+    constexpr int BNG = (sizeof(T) == 4 || D > 128) ? 32 : 64;
+    switch (mask) {
+      case MASK_NONE: return launch_fwd_one<T, D, BNG, DUAL, MASK_NONE, true>(p, stream);
+      case MASK_BOOL: return launch_fwd_one<T, D, BNG, DUAL, MASK_BOOL, true>(p, stream);
+      case MASK_ADD: return launch_fwd_one<T, D, BNG, DUAL, MASK_ADD, true>(p, stream);
     }
-    return -2;
+    return -3;
   }
   if constexpr (sizeof(T) == 2 && D == 256) {
     switch (mask) {

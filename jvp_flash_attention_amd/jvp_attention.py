@@ -31,7 +31,7 @@ Differences from the reference, all deliberate:
   JA:94-122, JA:271-277, JA:2356-2357): dropout on the attention probabilities with SDPA's semantics (kept entries
   scaled by 1/(1-p); the tangent O' sees the same pattern), the pattern a counter-based hash of a seed drawn from
   torch's CPU generator per call (``torch.manual_seed`` makes it repeatable) and of the entry index, regenerated in
-  the backward.  Head dims up to 128; runs on the register-staged kernels (about 3x slower for bf16 / fp16).
+  the backward.  Runs on the register-staged kernels (about 3x slower for bf16 / fp16).
 * ``attention`` notices dual inputs and then behaves like ``fwd_dual`` (the reference's ``attention``
   is ``JVPAttn.fwd`` and drops the tangent, its README.md:65-67).
 """
@@ -77,8 +77,6 @@ def is_blackwell() -> bool:
 def _validate(q: Tensor, k: Tensor, v: Tensor, attn_mask: Tensor | None, dropout_p: float, causal: bool):
     """Argument checks of JA:2356-2392, with this build's shape limits."""
     assert 0.0 <= dropout_p < 1.0, f"dropout_p must be in [0, 1), but got {dropout_p}"
-    if dropout_p != 0.0 and q.shape[-1] == 256:
-        raise NotImplementedError("Dropout is supported for HEAD_DIM_K up to 128 in JVP attention.")
     assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be (Z, H, N_CTX, HEAD_DIM)"
     Z, H, N_CTX, HEAD_DIM_Q = q.shape
     HEAD_DIM_K, HEAD_DIM_V = k.shape[-1], v.shape[-1]

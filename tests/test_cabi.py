@@ -74,7 +74,7 @@ def _fwd_args(**kw):
         (dict(struct_size=4), -7),
         (dict(q=None), -1),
         (dict(p_D=48), -2),
-        (dict(p_D=256, p_dropout_p=0.1), -2),  # dropout stops at D = 128
+        (dict(p_dropout_p=1.0), -2),        # dropout_p must be below 1
         (dict(p_L=0), -2),
         (dict(p_dtype=5), -3),
         (dict(p_mask_kind=1), -1),          # mask kind set, mask pointer NULL
