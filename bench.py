@@ -120,13 +120,13 @@ def hvp_sweep(be, _lib):
 def shape_rows(be, _lib):
     """Shapes next to the headline one, no mask: the other benchmark configurations' shapes, D = 32 and
     D = 256 (the smallest and the largest head dim the reference admits), 16 query heads over 4 key/value heads, and 4096 queries over 512 keys (the last two are
-    shapes the reference refuses).  Dual forward and dual backward, counted as 12 and 24 flops per
+    shapes the reference refuses), fp32 at D = 256, and the headline shape with dropout.  Dual forward and dual backward, counted as 12 and 24 flops per
     (query, key, d) triple."""
     import torch
 
     dev = torch.device("cuda:0")
     rows = {}
-    for name, (Zs, Hs, Hk, Lq, Lk, Ds, dtype) in {
+    for name, (Zs, Hs, Hk, Lq, Lk, Ds, dtype, *drop) in {
         "bf16_B4_H16_L2048_D32": (4, 16, 16, 2048, 2048, 32, torch.bfloat16),
         "bf16_B4_H16_L2048_D64_config2": (4, 16, 16, 2048, 2048, 64, torch.bfloat16),
         "bf16_B4_H16_L2048_D256": (4, 16, 16, 2048, 2048, 256, torch.bfloat16),
@@ -134,15 +134,19 @@ def shape_rows(be, _lib):
         "fp32_B4_H8_L1024_D64_config4_nomask": (4, 8, 8, 1024, 1024, 64, torch.float32),
         "bf16_B4_H16_over_4_kv_heads_L4096_D128": (4, 16, 4, 4096, 4096, 128, torch.bfloat16),
         "bf16_B4_H16_Lq4096_Lk512_D128": (4, 16, 16, 4096, 512, 128, torch.bfloat16),
+        "fp32_B4_H8_L1024_D256": (4, 8, 8, 1024, 1024, 256, torch.float32),
+        "bf16_B4_H16_L4096_D128_dropout_0.1": (4, 16, 16, 4096, 4096, 128, torch.bfloat16, 0.1),
     }.items():
+        dp = drop[0] if drop else 0.0
         g = torch.Generator(device=dev).manual_seed(11)
         mk = lambda h, l: torch.randn(Zs, h, l, Ds, generator=g, device=dev).to(dtype)  # noqa: E731
         q, qt, go, gt = [mk(Hs, Lq) for _ in range(4)]
         k, v, kt, vt = [mk(Hk, Lk) for _ in range(4)]
         scale = Ds**-0.5
-        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale), 10, 3)
-        o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale)
-        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, False, scale), 5, 2)
+        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale, dp, 7), 10, 3)
+        o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale, dp, 7)
+        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, False, scale,
+                                       dropout_p=dp, dropout_seed=7), 5, 2)
         n = float(Zs) * Hs * Lq * Lk * Ds
         rows[name] = {"fwd_ms": ms_f, "fwd_tflops": 12 * n / (ms_f * 1e-3) / 1e12,
                       "bwd_ms": ms_b, "bwd_tflops": 24 * n / (ms_b * 1e-3) / 1e12}
