@@ -34,7 +34,24 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
   const long long kv_blocks = (long long)((p.pr.Lk + BWD_BLK - 1) / BWD_BLK) * p.pr.Z * p.pr.Hk;
   if (kv_blocks > 0x7fffffffLL) return -2;
   if (p.pr.drop_thr != 0) {
-    // dropout: every element type takes the register-staged kernels, the one family that carries it
+    // dropout: the direct-to-LDS kernels carry it where there is no explicit mask; everything else takes the
+    // register-staged kernels
+    if constexpr (sizeof(T) == 2 && D <= 128 && MASK == MASK_NONE) {
+      using Cfg2 = Bwd2Cfg<T, D, MODE>;
+      const bool no_go = MODE == BWD_DUAL && p.go == nullptr;
+      constexpr bool NG = MODE != BWD_DUAL;
+      const bool grouped = p.pr.Hk != p.pr.H;
+      void (*kq)(const BwdParams) = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG, false, true> : bwd2_dq_kernel<T, D, MODE, MASK, true, false, true>;
+      void (*kkv)(const BwdParams);
+      if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true, false, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true, false, true>;
+      else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, false, false, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, false, false, true>;
+      int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
+      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);
+      if (rc != 0) return rc;
+      hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
+      hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
+      return hipGetLastError() == hipSuccess ? 0 : -6;
+    }
     auto kq = bwd_dq_kernel<T, D, MODE, MASK, true>;
     auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK, true>;
     int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);

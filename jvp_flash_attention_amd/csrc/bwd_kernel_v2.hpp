@@ -135,7 +135,9 @@ __device__ __forceinline__ void zero_acc(f32x16 &x) {
 // K, V (, K', V').  Scores are transposed (lane = query) so dS is the B operand of dQ^T += K^T dS^T.
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stubs (and has no buffer descriptor type)
 // SIX (dual mode only): dq' = scale dS' K as well, from the K fragments and the dS' tiles that dq already has.
-template <typename T, int D, int MODE, int MASK, bool GO, bool SIX>
+// DROP: dropout (see bwd_kernel.hpp): gO V^T, gT V^T and gT V'^T reach the logits through the kept, rescaled
+// entries only.
+template <typename T, int D, int MODE, int MASK, bool GO, bool SIX, bool DROP = false>
 __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
@@ -298,6 +300,11 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
           if constexpr (MASK == MASK_BOOL) keep[e] = mask_keep_of<T, MASK>(mah[hf], e);
         }
       }
+      uint32_t dlo = 0, dhi = 0;
+      if constexpr (DROP) {
+        const uint64_t base = ((uint64_t)zh * L + qld) * Lk + (uint32_t)key0;
+        dlo = (uint32_t)base, dhi = (uint32_t)(base >> 32);
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int i = 8 * hf + e;
@@ -306,6 +313,11 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
         float pv = fast_exp2(s - Mq);
         if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
         if constexpr (EDGE) pv = (key0 + e <= klim) ? pv : 0.f;
+        if constexpr (DROP) {
+          const float ks = drop_scale_at(pr, dlo, dhi, e);
+          if constexpr (!TAN) dP[i] *= ks;
+          if constexpr (DUAL || TAN) At[i] *= ks;
+        }
         if constexpr (MODE == BWD_PLAIN) {
           S[i] = pv * (dP[i] - d1);
         } else if constexpr (DUAL) {
@@ -442,10 +454,10 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
   }
 }
 #endif
-template <typename T, int D, int MODE, int MASK, bool GO, bool SIX = false>
+template <typename T, int D, int MODE, int MASK, bool GO, bool SIX = false, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwd2_dq_kernel(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dq_body<T, D, MODE, MASK, GO, SIX>(p, blockIdx.x);
+  bwd2_dq_body<T, D, MODE, MASK, GO, SIX, DROP>(p, blockIdx.x);
 #endif
 }
 // The same code with the vector registers capped, for D = 64: together with the accumulation registers
@@ -466,7 +478,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(160))) void 
 // one keeps its pointers loop-invariant).
 // SIX (dual mode only): dk' = scale dS'^T Q and dv' = P^T gT as well, from the fragments and tiles that dk, dv
 // already have (two more accumulators: fits for D <= 64).
-template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED, bool SIX>
+template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED, bool SIX, bool DROP = false>
 __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
@@ -774,12 +786,18 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
           float pv = fast_exp2(s - stat(0, e));
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
           if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
-          S[e] = pv;
+          float ks = 1.f;  // dropout: 1 / (1 - p) for a kept entry, 0 for a dropped one
+          if constexpr (DROP) {
+            ks = drop_scale(pr, (((uint64_t)z * pr.H + hq) * L + min(qi, L - 1)) * Lk + kld);
+            if constexpr (!TAN) dP[e] *= ks;
+            if constexpr (DUAL || TAN) At[e] *= ks;
+          }
+          S[e] = pv * ks;
           if constexpr (MODE == BWD_PLAIN) {
             dP[e] = pv * (dP[e] - stat(1, e));
           } else if constexpr (DUAL) {
             const float sp = Sp[e] * pr.scale, m_ = stat(1, e), am = At[e] - stat(2, e);
-            Pp[e - 8 * c] = pv * (sp - m_);
+            Pp[e - 8 * c] = pv * (sp - m_) * ks;
             Sp[e] = pv * am;
             dP[e] = pv * (dP[e] + am * sp - At[e] * m_ - stat(3, e));
           } else {
@@ -900,10 +918,10 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
   }
 }
 #endif
-template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED = false, bool SIX = false>
+template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED = false, bool SIX = false, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED, SIX>(p, blockIdx.x);
+  bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED, SIX, DROP>(p, blockIdx.x);
 #endif
 }
 // The same code with the vector registers capped, for D = 64: together with the accumulation registers

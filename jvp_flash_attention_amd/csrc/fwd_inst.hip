@@ -24,10 +24,10 @@ static int launch_fwd_one(const FwdParams &p, hipStream_t stream) {
 }
 
 // 16-bit element types with D = 64 or 128 take the direct-to-LDS, double-buffered kernel.
-template <typename T, int D, bool DUAL, int MASK>
+template <typename T, int D, bool DUAL, int MASK, bool DROP = false>
 static int launch_fwd2_one(const FwdParams &p, hipStream_t stream) {
   using Cfg = Fwd2Cfg<T, D, DUAL>;
-  auto kern = fwd2_kernel<T, D, DUAL, MASK>;
+  auto kern = fwd2_kernel<T, D, DUAL, MASK, DROP>;
   int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
   if (rc != 0) return rc;
   const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
@@ -84,7 +84,11 @@ static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
 template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
   if (p.pr.drop_thr != 0) {
-    // dropout: every element type takes the register-staged kernel, the one family that carries it
+    // dropout: the direct-to-LDS kernel carries it where there is no explicit mask; everything else takes the
+    // register-staged kernel
+    if constexpr (sizeof(T) == 2 && D <= 128) {
+      if (mask == MASK_NONE) return launch_fwd2_one<T, D, DUAL, MASK_NONE, true>(p, stream);
+    }
     constexpr int BNG = (sizeof(T) == 4 || D > 128) ? 32 : 64;
     switch (mask) {
       case MASK_NONE: return launch_fwd_one<T, D, BNG, DUAL, MASK_NONE, true>(p, stream);

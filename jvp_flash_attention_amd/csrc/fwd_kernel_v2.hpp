@@ -35,7 +35,9 @@ template <typename T, int D, bool DUAL> struct Fwd2Cfg {
   static constexpr int IPW = TILEB / 1024 / NW;       // direct-load instructions per wave per tile
 };
 
-template <typename T, int D, bool DUAL, int MASK>
+// DROP: dropout on the probabilities (see fwd_kernel.hpp): what enters the products with V, V' is
+// P * keep / (1 - p); the row sums l, mu stay those of the full softmax.
+template <typename T, int D, bool DUAL, int MASK, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   using Cfg = Fwd2Cfg<T, D, DUAL>;
   constexpr int BN = Cfg::BN, CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW;
@@ -404,6 +406,16 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     }
     l_i += rs;
     if constexpr (DUAL) mu_i += rmu;
+    if constexpr (DROP) {  // entry index ((z H + h) L + query) Lk + key; register e holds key jh + 16(e/8) + 8g + e%8
+      const uint64_t base = ((uint64_t)zh * L + qld) * Lk + (uint32_t)(jh + 8 * g);
+      const uint32_t blo = (uint32_t)base, bhi = (uint32_t)(base >> 32);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float ks = drop_scale_at(pr, blo, bhi, 16 * (e / 8) + (e % 8));
+        S[e] *= ks;
+        if constexpr (DUAL) Sp[e] *= ks;
+      }
+    }
     Frag<T> pf[2], psf[2];
 #pragma unroll
     for (int c = 0; c < 2; ++c) {

@@ -49,6 +49,13 @@ __host__ __device__ inline float drop_scale(const Problem &pr, uint64_t idx) {
   return drop_hash(idx, pr.drop_s0, pr.drop_s1) >= pr.drop_thr ? pr.drop_rinv : 0.f;
 }
 
+// The same for entry base + off, base a 64-bit index and off a small offset: the carry into the high word is
+// taken from the low-word sum.
+__device__ __forceinline__ float drop_scale_at(const Problem &pr, uint32_t base_lo, uint32_t base_hi, uint32_t off) {
+  const uint32_t lo = base_lo + off, hi = base_hi + (lo < base_lo ? 1u : 0u);
+  return drop_hash(((uint64_t)hi << 32) | lo, pr.drop_s0, pr.drop_s1) >= pr.drop_thr ? pr.drop_rinv : 0.f;
+}
+
 constexpr int TILE_BLOCK = 128, TILE_W = 64;  // geometry of the tile lists
 // First element of the list of (plane of (z, h), block).  tiles_q: blocks of 128 query rows, each with up to
 // ceil(Lk / 64) key tiles; tiles_k: blocks of 128 keys, each with up to ceil(L / 64) query tiles.
