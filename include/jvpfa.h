@@ -59,8 +59,7 @@ typedef struct jvpfa_problem {
    * dropped by a counter-based hash of (dropout_seed, entry index) and kept entries are scaled by 1/(1 - p), as
    * torch's scaled_dot_product_attention does; forward and backward of one call pair must get the same seed.
    * jvpfa_dropout_keep() writes the keep pattern out.  The reference carries dead code for dropout and raises
-   * NotImplementedError (JA:94-122, JA:271-277, JA:2356-2357).  bf16 / fp16 without an explicit mask: +15 % or so;
-   * with a mask the call leaves the direct-to-LDS kernels (about 3x slower than without dropout). */
+   * NotImplementedError (JA:94-122, JA:271-277, JA:2356-2357).  Costs bf16 / fp16 calls 13 - 22 % (D <= 128), fp32 2 - 6 %. */
   float dropout_p;
   uint64_t dropout_seed;
 } jvpfa_problem;

@@ -34,9 +34,9 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
   const long long kv_blocks = (long long)((p.pr.Lk + BWD_BLK - 1) / BWD_BLK) * p.pr.Z * p.pr.Hk;
   if (kv_blocks > 0x7fffffffLL) return -2;
   if (p.pr.drop_thr != 0) {
-    // dropout: the direct-to-LDS kernels carry it where there is no explicit mask; everything else takes the
-    // register-staged kernels
-    if constexpr (sizeof(T) == 2 && D <= 128 && MASK == MASK_NONE) {
+    // dropout: the direct-to-LDS kernels carry it for the 16-bit types up to D = 128, the register-staged ones
+    // for fp32 and for D = 256
+    if constexpr (sizeof(T) == 2 && D <= 128) {
       using Cfg2 = Bwd2Cfg<T, D, MODE>;
       const bool no_go = MODE == BWD_DUAL && p.go == nullptr;
       constexpr bool NG = MODE != BWD_DUAL;
@@ -51,15 +51,16 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
       hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
       hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
       return hipGetLastError() == hipSuccess ? 0 : -6;
+    } else {
+      auto kq = bwd_dq_kernel<T, D, MODE, MASK, true>;
+      auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK, true>;
+      int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);
+      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg::DKV_LDS);
+      if (rc != 0) return rc;
+      hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
+      hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DQ_LDS, stream, p);
+      return hipGetLastError() == hipSuccess ? 0 : -6;
     }
-    auto kq = bwd_dq_kernel<T, D, MODE, MASK, true>;
-    auto kkv = bwd_dkdv_kernel<T, D, MODE, MASK, true>;
-    int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg::DQ_LDS);
-    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg::DKV_LDS);
-    if (rc != 0) return rc;
-    hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(BWD_NT), Cfg::DKV_LDS, stream, p);
-    hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(BWD_NT), Cfg::DQ_LDS, stream, p);
-    return hipGetLastError() == hipSuccess ? 0 : -6;
   }
   if constexpr (sizeof(T) == 2 && D <= 128) {  // direct-to-LDS, double-buffered kernels
    {

@@ -84,16 +84,21 @@ static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
 template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
   if (p.pr.drop_thr != 0) {
-    // dropout: the direct-to-LDS kernel carries it where there is no explicit mask; everything else takes the
-    // register-staged kernel
+    // dropout: the direct-to-LDS kernel carries it for the 16-bit types up to D = 128, the register-staged one
+    // for fp32 and for D = 256
     if constexpr (sizeof(T) == 2 && D <= 128) {
-      if (mask == MASK_NONE) return launch_fwd2_one<T, D, DUAL, MASK_NONE, true>(p, stream);
-    }
-    constexpr int BNG = (sizeof(T) == 4 || D > 128) ? 32 : 64;
-    switch (mask) {
-      case MASK_NONE: return launch_fwd_one<T, D, BNG, DUAL, MASK_NONE, true>(p, stream);
-      case MASK_BOOL: return launch_fwd_one<T, D, BNG, DUAL, MASK_BOOL, true>(p, stream);
-      case MASK_ADD: return launch_fwd_one<T, D, BNG, DUAL, MASK_ADD, true>(p, stream);
+      switch (mask) {
+        case MASK_NONE: return launch_fwd2_one<T, D, DUAL, MASK_NONE, true>(p, stream);
+        case MASK_BOOL: return launch_fwd2_one<T, D, DUAL, MASK_BOOL, true>(p, stream);
+        case MASK_ADD: return launch_fwd2_one<T, D, DUAL, MASK_ADD, true>(p, stream);
+      }
+    } else {
+      constexpr int BNG = (sizeof(T) == 4 || D > 128) ? 32 : 64;
+      switch (mask) {
+        case MASK_NONE: return launch_fwd_one<T, D, BNG, DUAL, MASK_NONE, true>(p, stream);
+        case MASK_BOOL: return launch_fwd_one<T, D, BNG, DUAL, MASK_BOOL, true>(p, stream);
+        case MASK_ADD: return launch_fwd_one<T, D, BNG, DUAL, MASK_ADD, true>(p, stream);
+      }
     }
     return -3;
   }
