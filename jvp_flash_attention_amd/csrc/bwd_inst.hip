@@ -5,6 +5,7 @@
 #include "bwd_kernel.hpp"
 #include "bwd_kernel_v2.hpp"
 #include "bwd_kernel_wide.hpp"
+#include "bwd_kernel_pair.hpp"
 #include "launch.hpp"
 #include "split.hpp"
 
@@ -122,36 +123,32 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
     if (run_q) hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
    }
-  } else if constexpr (sizeof(T) == 2 && D == 256) {
-    // dq: two workgroups per query block, each with 128 of its columns, on the direct-to-LDS pipeline
-    using CfgW = BwdWideCfg<T, D, 128, MODE>;
-    const bool no_go = MODE == BWD_DUAL && p.go == nullptr;
-    constexpr bool NG = MODE != BWD_DUAL;
-    void (*kq)(const BwdParams) = no_go ? bwdw_dq_kernel<T, D, 128, MODE, MASK, NG> : bwdw_dq_kernel<T, D, 128, MODE, MASK, true>;
-    if (blocks * CfgW::NS > 0x7fffffffLL) return -2;
-    int rc = allow_lds(reinterpret_cast<const void *>(kq), CfgW::DQ_LDS);
+  } else if constexpr (sizeof(T) == 2 && D == 256 && MODE == BWD_DUAL) {
+    // pairs of waves that share 32 rows and split the resident operands: every product formed once
+    using CfgP = BwdPairCfg<T, D>;
+    const bool no_go = p.go == nullptr;
+    const long long qblocks = (long long)((p.pr.L + CfgP::BLK - 1) / CfgP::BLK) * p.pr.Z * p.pr.H;
+    const long long kblocks = (long long)((p.pr.Lk + CfgP::BLK - 1) / CfgP::BLK) * p.pr.Z * p.pr.Hk;
+    if (qblocks > 0x7fffffffLL || kblocks > 0x7fffffffLL) return -2;
+    void (*kq)(const BwdParams) = no_go ? bwdp_dq_kernel<T, D, MASK, false> : bwdp_dq_kernel<T, D, MASK, true>;
+    void (*kkv)(const BwdParams) = no_go ? bwdp_dkdv_kernel<T, D, MASK, false> : bwdp_dkdv_kernel<T, D, MASK, true>;
+    int rc = allow_lds(reinterpret_cast<const void *>(kq), CfgP::DQ_LDS);
+    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), CfgP::DKV_LDS);
     if (rc != 0) return rc;
-    // dk/dv on the same pipeline: dV from K, K' alone, then dK in two column halves (dual); both in two
-    // column halves (otherwise)
-    using CfgK = BwdWideKvCfg<T, D, 128, MODE>;
-    if (kv_blocks * CfgK::NS > 0x7fffffffLL) return -2;
-    if constexpr (MODE == BWD_DUAL) {
-      void (*kv)(const BwdParams) = no_go ? bwdw_dkdv_kernel<T, D, 128, MODE, MASK, NG, WIDE_DV>
-                                          : bwdw_dkdv_kernel<T, D, 128, MODE, MASK, true, WIDE_DV>;
-      void (*kk)(const BwdParams) = no_go ? bwdw_dkdv_kernel<T, D, 128, MODE, MASK, NG, WIDE_DK>
-                                          : bwdw_dkdv_kernel<T, D, 128, MODE, MASK, true, WIDE_DK>;
-      rc = allow_lds(reinterpret_cast<const void *>(kv), CfgK::DKV_LDS);
-      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kk), CfgK::DKV_LDS);
-      if (rc != 0) return rc;
-      hipLaunchKernelGGL(kv, dim3((unsigned)kv_blocks), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
-      hipLaunchKernelGGL(kk, dim3((unsigned)(kv_blocks * CfgK::NS)), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
-    } else {
-      auto kkv = bwdw_dkdv_kernel<T, D, 128, MODE, MASK, true, WIDE_BOTH>;
-      rc = allow_lds(reinterpret_cast<const void *>(kkv), CfgK::DKV_LDS);
-      if (rc != 0) return rc;
-      hipLaunchKernelGGL(kkv, dim3((unsigned)(kv_blocks * CfgK::NS)), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
-    }
-    hipLaunchKernelGGL(kq, dim3((unsigned)(blocks * CfgW::NS)), dim3(CfgW::NT), CfgW::DQ_LDS, stream, p);
+    hipLaunchKernelGGL(kkv, dim3((unsigned)kblocks), dim3(CfgP::NT), CfgP::DKV_LDS, stream, p);
+    hipLaunchKernelGGL(kq, dim3((unsigned)qblocks), dim3(CfgP::NT), CfgP::DQ_LDS, stream, p);
+    return hipGetLastError() == hipSuccess ? 0 : -6;
+  } else if constexpr (sizeof(T) == 2 && D == 256) {
+    // without tangents in the launch two operands stay resident and one workgroup holds all 256 columns
+    using CfgW = BwdWideCfg<T, D, MODE>;
+    using CfgK = BwdWideKvCfg<T, D, MODE>;
+    auto kq = bwdw_dq_kernel<T, D, MODE, MASK>;
+    auto kkv = bwdw_dkdv_kernel<T, D, MODE, MASK>;
+    int rc = allow_lds(reinterpret_cast<const void *>(kq), CfgW::DQ_LDS);
+    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), CfgK::DKV_LDS);
+    if (rc != 0) return rc;
+    hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
+    hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(CfgW::NT), CfgW::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
   } else {
     auto kq = bwd_dq_kernel<T, D, MODE, MASK>;

@@ -1,31 +1,29 @@
-// Backward kernels for 16-bit element types with D = 256, on the memory pipeline of bwd_kernel_v2.hpp.
+// Backward kernels for 16-bit element types with D = 256 and no tangents in the launch (BWD_PLAIN: dq / dk, dv;
+// BWD_TANGENT: dq' / dk', dv'), on the memory pipeline of bwd_kernel_v2.hpp.  (The dual mode has four resident
+// operands instead of two and is built differently: bwd_kernel_pair.hpp.)
 //
-// With D = 256 the operands that stay in registers are the whole accumulation file (dq: Q, gO, Q',
-// gT; dk: K, V, K', V': 4 x 64 registers), so the accumulators live in ordinary vector registers and
-// cover DV = 128 columns: two workgroups per block of 128 rows recompute the score tiles over all of
-// D and each accumulates half of the output.  (dV needs S and S' only: in the dual mode it is a launch
-// of its own with K, K' resident and all 256 columns.)  Streamed tiles are 32 rows of 512 bytes: two
-// stages of four 16 KB tiles fill 128 KB of LDS; a tile is read both ways from its one row-major copy.
-// The inline-asm matrix instructions are the guarded form (see mma_vra): with the accumulation file
-// full the allocator moves resident operands through a spare register right before their use.
+// The operands that stay in registers are 2 x 64 registers of the accumulation file (dq: Q and gO or gT; dk/dv:
+// K and V); the accumulators cover all 256 columns (dq: 128 registers; dk and dv: 2 x 128).  Streamed tiles are
+// 32 rows of 512 bytes: two stages of two 16 KB tiles; a tile is read both ways from its one row-major copy.
+// The inline-asm matrix instructions are the guarded form (see mma_vra): with the accumulation file full the
+// allocator moves resident operands through a spare register right before their use.
 //
-// First kernel: dq (PLAIN / DUAL) or dq' (TANGENT).
+// First kernel: dq (PLAIN) or dq' (TANGENT).
 #pragma once
 #include "bwd_kernel_v2.hpp"
 
 namespace jvpfa {
 
-template <typename T, int D, int DV, int MODE> struct BwdWideCfg {
-  static_assert(sizeof(T) == 2 && D == 256 && DV == 128);
+template <typename T, int D, int MODE> struct BwdWideCfg {
+  static_assert(sizeof(T) == 2 && D == 256 && (MODE == BWD_PLAIN || MODE == BWD_TANGENT));
   static constexpr int NW = 4;
   static constexpr int NT = NW * WAVE;
-  static constexpr int BLK = NW * 32;                 // query rows owned by a workgroup
-  static constexpr int BT = 32;                       // keys of a streamed tile
-  static constexpr int NS = D / DV;                   // workgroups per query block
+  static constexpr int BLK = NW * 32;                 // rows owned by a workgroup
+  static constexpr int BT = 32;                       // rows of a streamed tile
   static constexpr int CH = D * sizeof(T) / 16;       // 32 chunks of 16 bytes per row
   static constexpr int ROWB = D * sizeof(T);
   static constexpr int TILEB = BT * ROWB;
-  static constexpr int NTILE = MODE == BWD_DUAL ? 4 : 2;
+  static constexpr int NTILE = 2;
   static constexpr int STAGEB = NTILE * TILEB;
   static constexpr int IPW = TILEB / 1024 / NW;
   static constexpr size_t DQ_LDS = 2 * (size_t)STAGEB;
@@ -39,23 +37,21 @@ template <typename T, int D, int DV, int MODE> struct BwdWideCfg {
 __device__ __forceinline__ int swz_w(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
 #if defined(__HIP_DEVICE_COMPILE__)
-template <typename T, int D, int DV, int MODE, int MASK, bool GO>
+template <typename T, int D, int MODE, int MASK>
 __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
-  using Cfg = BwdWideCfg<T, D, DV, MODE>;
-  constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
-  constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT, NS = Cfg::NS;
-  constexpr int KK = D / 16, DB = DV / 32;
+  using Cfg = BwdWideCfg<T, D, MODE>;
+  constexpr bool TAN = MODE == BWD_TANGENT;
+  constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT;
+  constexpr int KK = D / 16, DB = D / 32;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem_raw;
   const Problem &pr = p.pr;
   const int L = pr.L;
   const int nblk = (L + Cfg::BLK - 1) / Cfg::BLK;
-  // the workgroups of one query block follow each other, so they stream the same key tiles from L2
-  const int id = xcd_remap(blockIdx.x, nblk * NS, pr.Z * pr.H);
-  const int zh = id / (nblk * NS);
-  const int rem = id % (nblk * NS);
-  const int slice = rem % NS;
-  const int qb = pr.causal ? nblk - 1 - rem / NS : rem / NS;
+  const int id = xcd_remap(blockIdx.x, nblk, pr.Z * pr.H);
+  const int zh = id / nblk;
+  const int rem = id % nblk;
+  const int qb = pr.causal ? nblk - 1 - rem : rem;
   const int z = zh / pr.H, h = zh % pr.H;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
@@ -65,7 +61,6 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   const int q0 = qb * Cfg::BLK;
   const int qrow = q0 + wave * 32 + r;
   const int qld = qrow < L ? qrow : L - 1;
-  constexpr bool has_go = GO;
 
   // direct loads: instruction i of this wave fills LDS chunks 64*(wave*IPW+i) .. +63 of a tile
   uint32_t ld_o[IPW];
@@ -76,7 +71,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
     ld_o[i] = row * ROWB + (((lc % CH) ^ swz_w(row)) * 16);
   }
   uint32_t ld_dst = 0;
-  __amdgpu_buffer_rsrc_t ld_rs[4];
+  __amdgpu_buffer_rsrc_t ld_rs[2];
   // buffer loads: descriptor = (start of the tile, bytes left in the head); rows past the end of the
   // sequence and tiles that do not exist are out of range and read as zeros
   auto tile_rsrc = [&](const char *base, int j, bool exists) {
@@ -96,41 +91,33 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) noff[kk] = pr32 * ROWB + (((2 * kk + g) ^ x) * 16);
   }
-  // transposed fragment of this workgroup's columns (see fwd_kernel_v2.hpp for the lane pattern)
-  uint32_t toff[DB][2];
+  // transposed fragment (see fwd_kernel_v2.hpp for the lane pattern): d-block db is at toff[db % 4] + 256 * (db / 4)
+  uint32_t toff[4][2];
   {
     const int a_ = (lane >> 4) & 1, j_ = lane & 15;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+    for (int db = 0; db < 4; ++db) {
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
         const int row = 8 * g + 4 * hh + (j_ >> 2);
         const int ch = (4 * db + 2 * a_ + (j_ & 1)) ^ swz_w(row);
-        toff[db][hh] = row * ROWB + (16 * slice + ch) * 16 + 8 * ((j_ >> 1) & 1);
+        toff[db][hh] = row * ROWB + ch * 16 + 8 * ((j_ >> 1) & 1);
       }
     }
   }
 
-  Frag<T> Qf[KK], gOf[TAN ? 1 : KK], Qtf[DUAL ? KK : 1], gTf[(DUAL || TAN) ? KK : 1];
+  // resident: Q and gO (PLAIN) or gT (TANGENT)
+  Frag<T> Qf[KK], Gf[KK];
   load_bfrags<KK>(Qf, reinterpret_cast<const T *>(p.q) + head + (size_t)qld * D, g);
-  if constexpr (!TAN) {
-    if constexpr (has_go) load_bfrags<KK>(gOf, reinterpret_cast<const T *>(p.go) + head + (size_t)qld * D, g);
-  }
-  if constexpr (DUAL) load_bfrags<KK>(Qtf, reinterpret_cast<const T *>(p.qt) + head + (size_t)qld * D, g);
-  if constexpr (DUAL || TAN) load_bfrags<KK>(gTf, reinterpret_cast<const T *>(p.gt) + head + (size_t)qld * D, g);
+  load_bfrags<KK>(Gf, reinterpret_cast<const T *>(TAN ? p.gt : p.go) + head + (size_t)qld * D, g);
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) {
     pin_acc(Qf[kk]);
-    if constexpr (!TAN && has_go) pin_acc(gOf[kk]);
-    if constexpr (DUAL) pin_acc(Qtf[kk]);
-    if constexpr (DUAL || TAN) pin_acc(gTf[kk]);
+    pin_acc(Gf[kk]);
   }
 
   const float Mq = qrow < L ? p.M[srow + qld] : __builtin_inff();
-  const float d1 = (MODE == BWD_PLAIN) ? p.d1[srow + qld] : 0.f;
-  const float mu = DUAL ? p.mu[srow + qld] : 0.f;
-  const float av = (DUAL || TAN) ? p.a[srow + qld] : 0.f;
-  const float dsum = DUAL ? p.d2[srow + qld] : 0.f;
+  const float sub = TAN ? p.a[srow + qld] : p.d1[srow + qld];  // what the row takes off dP (PLAIN) or A (TANGENT)
 
   f32x16 acc[DB];
 #pragma unroll
@@ -144,8 +131,6 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   const size_t kvhead = ((size_t)z * pr.Hk + h / (pr.H / pr.Hk)) * Lk * D;
   const char *Kb = reinterpret_cast<const char *>(p.k) + kvhead * sizeof(T);
   const char *Vb = reinterpret_cast<const char *>(p.v) + kvhead * sizeof(T);
-  const char *Ktb = DUAL ? reinterpret_cast<const char *>(p.kt) + kvhead * sizeof(T) : nullptr;
-  const char *Vtb = DUAL ? reinterpret_cast<const char *>(p.vt) + kvhead * sizeof(T) : nullptr;
 
   int kend = pr.causal ? min(Lk, q0 + Cfg::BLK) : Lk;
   if constexpr (MASK != MASK_NONE) {
@@ -167,19 +152,14 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   }
   auto list_slot = [&](int t) { return tlist ? tlist + 1 + (t >> 1) : reinterpret_cast<const int *>(p.q); };
   auto key_of = [&](int entry, int t) { return tlist ? min(max(entry, 0), tmax) * TILE_W + (t & 1) * BT : t * BT; };
-  // tile slots in a stage: 0 K, 1 V, 2 K', 3 V'
+  // tile slots in a stage: 0 K, 1 V
   constexpr int NLOAD = IPW * Cfg::NTILE;
-  constexpr int NACC = DUAL ? 2 : 1;
   constexpr int NPV = 2 * (DB / 2);  // accumulation steps: (16-key chunk c, pair of d-blocks)
   constexpr int NSTEP = KK + NPV;
   auto prepare_loads = [&](int stage, int j0, bool on) {
     ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
     ld_rs[0] = tile_rsrc(Kb, j0, on);
     ld_rs[1] = tile_rsrc(Vb, j0, on);
-    if constexpr (DUAL) {
-      ld_rs[2] = tile_rsrc(Ktb, j0, on);
-      ld_rs[3] = tile_rsrc(Vtb, j0, on);
-    }
   };
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
@@ -195,46 +175,28 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   // EDGE: the tile may cross the causal diagonal or the end of the sequence
   auto tile_body = [&](auto EDGEc, uint32_t sbase, int j0) {
     constexpr bool EDGE = decltype(EDGEc)::value;
-    // ---- recompute: S, (S', dP, A, B) ----------------------------------------------------------
-    FragN fk[2], fv[2], fkt[2], fvt[2];
+    // ---- recompute: S and dP = V gO^T (PLAIN) or A = V gT^T (TANGENT) ----------------------------
+    FragN fk[2], fv[2];
     auto issue_n = [&](auto kkc) {
       constexpr int kk = decltype(kkc)::value, sl = kk % 2, HI = (kk / 8) * 256;
       const uint32_t ad = sbase + noff[kk % 8];
       fk[sl].v = lds_b128<HI>(ad);
       fv[sl].v = lds_b128<HI + TILEB>(ad);
-      if constexpr (DUAL) {
-        fkt[sl].v = lds_b128<HI + 2 * TILEB>(ad);
-        fvt[sl].v = lds_b128<HI + 3 * TILEB>(ad);
-      }
     };
-    constexpr int NRN = DUAL ? 4 : 2;
-    constexpr bool GD = DUAL;  // the accumulation file is full: see mma_vra
-    f32x16 S, dP, Sp, At;  // DUAL: dP also collects V' gT^T (the B term)
+    f32x16 S, G;
     issue_n(std::integral_constant<int, 0>{});
     static_for<KK>([&](auto kkc) {
       constexpr int kk = decltype(kkc)::value, sl = kk % 2;
       constexpr bool F = kk == 0;
       if constexpr (kk + 1 < KK) issue_n(std::integral_constant<int, kk + 1>{});
-      if constexpr (DUAL) lds_wait<(kk + 1 < KK) ? NRN : 0>(fk[sl], fv[sl], fkt[sl], fvt[sl]);
-      else lds_wait<(kk + 1 < KK) ? NRN : 0>(fk[sl], fv[sl]);
+      lds_wait<(kk + 1 < KK) ? 2 : 0>(fk[sl], fv[sl]);
       load_step(std::integral_constant<int, kk>{});
-      const Frag<T> k_ = as_frag<T>(fk[sl]), v_ = as_frag<T>(fv[sl]);
-      mma_vra<F, GD>(S, k_, Qf[kk]);
-      if constexpr (MODE == BWD_PLAIN) mma_vra<F, GD>(dP, v_, gOf[kk]);
-      if constexpr (TAN) mma_vra<F, GD>(At, v_, gTf[kk]);
-      if constexpr (DUAL) {
-        if constexpr (has_go) mma_vra<F, GD>(dP, v_, gOf[kk]);
-        mma_vra<F, GD>(Sp, k_, Qtf[kk]);
-        mma_vra<F, GD>(At, v_, gTf[kk]);
-        mma_vra<false, GD>(Sp, as_frag<T>(fkt[sl]), Qf[kk]);
-        mma_vra<F && !has_go, GD>(dP, as_frag<T>(fvt[sl]), gTf[kk]);
-      }
+      mma_vra<F, true>(S, as_frag<T>(fk[sl]), Qf[kk]);
+      mma_vra<F, true>(G, as_frag<T>(fv[sl]), Gf[kk]);
     });
-    if constexpr (DUAL) tiles_ready(S, dP, Sp, At);
-    else if constexpr (TAN) tiles_ready(S, At);
-    else tiles_ready(S, dP);
+    tiles_ready(S, G);
 
-    // ---- P and the score gradients -------------------------------------------------------------
+    // ---- P and the score gradient ---------------------------------------------------------------
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
       const int key0 = j0 + 16 * hf + 8 * g;
@@ -255,54 +217,32 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
         float pv = fast_exp2(s - Mq);
         if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
         if constexpr (EDGE) pv = (key0 + e <= klim) ? pv : 0.f;
-        if constexpr (MODE == BWD_PLAIN) {
-          S[i] = pv * (dP[i] - d1);
-        } else if constexpr (DUAL) {
-          const float sp = Sp[i] * pr.scale, am = At[i] - av;
-          Sp[i] = pv * am;
-          S[i] = pv * (dP[i] + am * sp - At[i] * mu - dsum);
-        } else {
-          S[i] = pv * (At[i] - av);
-        }
+        S[i] = pv * (G[i] - sub);
       }
     }
-    Frag<T> dsf[2], dspf[2];
+    Frag<T> dsf[2];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      dsf[c] = to_frag<T>(S, c);
-      if constexpr (DUAL) dspf[c] = to_frag<T>(Sp, c);
-    }
+    for (int c = 0; c < 2; ++c) dsf[c] = to_frag<T>(S, c);
 
-    // ---- dQ^T += K^T dS^T (+ K'^T dS'^T) on this workgroup's columns -----------------------------
-    FragT tk[2][2], tkt[2][2];  // [ring slot][d-block of the pair]
+    // ---- dQ^T += K^T dS^T -------------------------------------------------------------------------
+    FragT tk[2][2];  // [ring slot][d-block of the pair]
     auto issue_t = [&](auto ic) {
       constexpr int i = decltype(ic)::value, c = i / (DB / 2), dp = i % (DB / 2), sl = i % 2;
-      constexpr int TO = c * 16 * ROWB;
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const uint32_t a0 = sbase + toff[2 * dp + u][0], a1 = sbase + toff[2 * dp + u][1];
+      static_for<2>([&](auto uc) {
+        constexpr int u = decltype(uc)::value, db = 2 * dp + u, TO = c * 16 * ROWB + (db / 4) * 256;
+        const uint32_t a0 = sbase + toff[db % 4][0], a1 = sbase + toff[db % 4][1];
         tk[sl][u].lo = lds_tr64<TO>(a0);
         tk[sl][u].hi = lds_tr64<TO>(a1);
-        if constexpr (DUAL) {
-          tkt[sl][u].lo = lds_tr64<TO + 2 * TILEB>(a0);
-          tkt[sl][u].hi = lds_tr64<TO + 2 * TILEB>(a1);
-        }
-      }
+      });
     };
-    constexpr int NRT = 4 * NACC;
     issue_t(std::integral_constant<int, 0>{});
     static_for<NPV>([&](auto ic) {
       constexpr int i = decltype(ic)::value, c = i / (DB / 2), dp = i % (DB / 2), sl = i % 2;
       if constexpr (i + 1 < NPV) issue_t(std::integral_constant<int, i + 1>{});
-      if constexpr (DUAL) lds_wait<(i + 1 < NPV) ? NRT : 0>(tk[sl][0], tk[sl][1], tkt[sl][0], tkt[sl][1]);
-      else lds_wait<(i + 1 < NPV) ? NRT : 0>(tk[sl][0], tk[sl][1]);
+      lds_wait<(i + 1 < NPV) ? 4 : 0>(tk[sl][0], tk[sl][1]);
       load_step(std::integral_constant<int, KK + i>{});
       mma(acc[2 * dp], as_frag<T>(tk[sl][0]), dsf[c]);
       mma(acc[2 * dp + 1], as_frag<T>(tk[sl][1]), dsf[c]);
-      if constexpr (DUAL) {
-        mma(acc[2 * dp], as_frag<T>(tkt[sl][0]), dspf[c]);
-        mma(acc[2 * dp + 1], as_frag<T>(tkt[sl][1]), dspf[c]);
-      }
     });
   };
 
@@ -353,7 +293,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the redirected loads of the last iteration must not outlive the kernel
 
   if (qrow < L) {
-    T *out = reinterpret_cast<T *>(TAN ? p.dqt : p.dq) + head + (size_t)qrow * D + slice * DV;
+    T *out = reinterpret_cast<T *>(TAN ? p.dqt : p.dq) + head + (size_t)qrow * D;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
 #pragma unroll
@@ -367,51 +307,35 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   }
 }
 #else
-template <typename T, int D, int DV, int MODE, int MASK, bool GO>
+template <typename T, int D, int MODE, int MASK>
 __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {}
 #endif
 
 // ------------------------------------------------------------------------------------------------
-// dk, dv (PLAIN / DUAL) or dk', dv' (TANGENT) for D = 256: workgroup = 128 keys of a head, loop over
-// 32-query tiles of Q, G (, Q', gT) with their row statistics.  What a launch produces:
-//   WIDE_DV    (DUAL) dV, all 256 columns: it needs S and S' only, so K, K' are resident (2 x 64
-//              registers) next to the accumulators (128)
-//   WIDE_DK    (DUAL) 128 columns of dK, two workgroups per key block: K, V, K', V' resident (the
-//              whole accumulation file), the accumulators in ordinary registers
-//   WIDE_BOTH  (PLAIN, TANGENT) 128 columns of dK and of dV, two workgroups per key block
-// With grouped heads the query heads that read this key/value head are visited one after another.
-enum WidePart { WIDE_BOTH = 0, WIDE_DV = 1, WIDE_DK = 2 };
-
-template <typename T, int D, int DV, int MODE> struct BwdWideKvCfg : BwdWideCfg<T, D, DV, MODE> {
-  static constexpr int NSTAT = MODE == BWD_DUAL ? 4 : 2;
+// dk, dv (PLAIN) or dk', dv' (TANGENT) for D = 256: workgroup = 128 keys of a head, K and V resident,
+// loop over 32-query tiles of Q and gO (PLAIN) or gT (TANGENT) with their row statistics.  With grouped
+// heads the query heads that read this key/value head are visited one after another.
+template <typename T, int D, int MODE> struct BwdWideKvCfg : BwdWideCfg<T, D, MODE> {
+  static constexpr int NSTAT = 2;
   static constexpr int STATB = NSTAT * 64 * 4;  // 64 floats per statistic and stage (32 used)
-  static constexpr size_t DKV_LDS = 2 * (size_t)BwdWideCfg<T, D, DV, MODE>::STAGEB + 2 * (size_t)STATB;
+  static constexpr size_t DKV_LDS = 2 * (size_t)BwdWideCfg<T, D, MODE>::STAGEB + 2 * (size_t)STATB;
 };
 
 #if defined(__HIP_DEVICE_COMPILE__)
-template <typename T, int D, int DV, int MODE, int MASK, bool GO, int PART>
+template <typename T, int D, int MODE, int MASK>
 __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
-  using Cfg = BwdWideKvCfg<T, D, DV, MODE>;
-  constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
-  static_assert(DUAL ? (PART == WIDE_DV || PART == WIDE_DK) : PART == WIDE_BOTH);
-  constexpr bool WANT_DK = PART != WIDE_DV, WANT_DV = PART != WIDE_DK;
-  constexpr bool NEED_V = !DUAL || WANT_DK;  // V (, V') enter only through dP, A, B
-  constexpr int NSL = PART == WIDE_DV ? 1 : Cfg::NS;  // workgroups per key block
+  using Cfg = BwdWideKvCfg<T, D, MODE>;
+  constexpr bool TAN = MODE == BWD_TANGENT;
   constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT;
-  constexpr int KK = D / 16;
-  constexpr int DBK = WANT_DK ? DV / 32 : 1;                             // d-blocks of the dK accumulator
-  constexpr int DBV = WANT_DV ? (PART == WIDE_DV ? D / 32 : DV / 32) : 1;  // ... of the dV accumulator
-  constexpr int DBS = PART == WIDE_DV ? D / 32 : DV / 32;                // d-blocks visited by a step
+  constexpr int KK = D / 16, DB = D / 32;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem_raw;
   const Problem &pr = p.pr;
   const int L = pr.L, Lk = pr.Lk;  // queries, keys
   const int nblk = (Lk + Cfg::BLK - 1) / Cfg::BLK;
-  const int id = xcd_remap(blockIdx.x, nblk * NSL, pr.Z * pr.Hk);
-  const int zh = id / (nblk * NSL);
-  const int rem = id % (nblk * NSL);
-  const int slice = rem % NSL;
-  const int kb = rem / NSL;  // causal: the first key blocks have the longest query loops
+  const int id = xcd_remap(blockIdx.x, nblk, pr.Z * pr.Hk);
+  const int zh = id / nblk;
+  const int kb = id % nblk;  // causal: the first key blocks have the longest query loops
   const int z = zh / pr.Hk, hk = zh % pr.Hk, group = pr.H / pr.Hk;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
@@ -420,18 +344,17 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   const int k0 = kb * Cfg::BLK;
   const int krow = k0 + wave * 32 + r;
   const int kld = krow < Lk ? krow : Lk - 1;
-  constexpr bool has_go = GO;
-  T *outk = reinterpret_cast<T *>(TAN ? p.dkt : p.dk) + head + (size_t)krow * D + slice * DV;
-  T *outv = reinterpret_cast<T *>(TAN ? p.dvt : p.dv) + head + (size_t)krow * D + (PART == WIDE_DV ? 0 : slice * DV);
+  T *outk = reinterpret_cast<T *>(TAN ? p.dkt : p.dk) + head + (size_t)krow * D;
+  T *outv = reinterpret_cast<T *>(TAN ? p.dvt : p.dv) + head + (size_t)krow * D;
   if constexpr (MASK != MASK_NONE) {
     // a key block that the caller's hint declares fully masked has zero gradients
     if (pr.klimit && k0 >= pr.klimit[z]) {
       if (krow < Lk) {
         float zero8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int d0 = 8 * g; d0 < 32 * DBS; d0 += 16) {
-          if constexpr (WANT_DK) store8<T>(outk + d0, zero8);
-          if constexpr (WANT_DV) store8<T>(outv + d0, zero8);
+        for (int d0 = 8 * g; d0 < D; d0 += 16) {
+          store8<T>(outk + d0, zero8);
+          store8<T>(outv + d0, zero8);
         }
       }
       return;
@@ -447,7 +370,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
     ld_o[i] = row * ROWB + (((lc % CH) ^ swz_w(row)) * 16);
   }
   uint32_t ld_dst = 0;
-  __amdgpu_buffer_rsrc_t ld_rs[4];
+  __amdgpu_buffer_rsrc_t ld_rs[2];
   auto tile_rsrc = [&](const char *base, int j, bool exists) {
     const int rows = exists ? max(L - j, 0) : 0;
     return __builtin_amdgcn_make_buffer_rsrc((void *)(base + (size_t)j * ROWB), 0, rows * ROWB, 0x00020000);
@@ -463,7 +386,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) noff[kk] = pr32 * ROWB + (((2 * kk + g) ^ x) * 16);
   }
-  // transposed fragment: d-block db of this launch's columns is at toff[db % 4] + 256 * (db / 4)
+  // transposed fragment: d-block db is at toff[db % 4] + 256 * (db / 4)
   uint32_t toff[4][2];
   {
     const int a_ = (lane >> 4) & 1, j_ = lane & 15;
@@ -473,36 +396,27 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
       for (int hh = 0; hh < 2; ++hh) {
         const int row = 8 * g + 4 * hh + (j_ >> 2);
         const int ch = (4 * db + 2 * a_ + (j_ & 1)) ^ swz_w(row);
-        toff[db][hh] = row * ROWB + (16 * (PART == WIDE_DV ? 0 : slice) + ch) * 16 + 8 * ((j_ >> 1) & 1);
+        toff[db][hh] = row * ROWB + ch * 16 + 8 * ((j_ >> 1) & 1);
       }
     }
   }
   const uint32_t stat0 = lds0 + 2 * Cfg::STAGEB;  // row statistics, two stages of NSTAT x 64 floats
 
-  Frag<T> Kf[KK], Vf[NEED_V ? KK : 1], Ktf[DUAL ? KK : 1], Vtf[DUAL && NEED_V ? KK : 1];
+  Frag<T> Kf[KK], Vf[KK];
   load_bfrags<KK>(Kf, reinterpret_cast<const T *>(p.k) + head + (size_t)kld * D, g);
-  if constexpr (NEED_V) load_bfrags<KK>(Vf, reinterpret_cast<const T *>(p.v) + head + (size_t)kld * D, g);
-  if constexpr (DUAL) {
-    load_bfrags<KK>(Ktf, reinterpret_cast<const T *>(p.kt) + head + (size_t)kld * D, g);
-    if constexpr (NEED_V) load_bfrags<KK>(Vtf, reinterpret_cast<const T *>(p.vt) + head + (size_t)kld * D, g);
-  }
+  load_bfrags<KK>(Vf, reinterpret_cast<const T *>(p.v) + head + (size_t)kld * D, g);
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) {
     pin_acc(Kf[kk]);
-    if constexpr (NEED_V) pin_acc(Vf[kk]);
-    if constexpr (DUAL) {
-      pin_acc(Ktf[kk]);
-      if constexpr (NEED_V) pin_acc(Vtf[kk]);
-    }
+    pin_acc(Vf[kk]);
   }
-  // the accumulation file is full (or nearly) in every variant: see mma_vra
-  constexpr bool GD = true;
 
-  f32x16 dK[DBK], dV[DBV];
+  f32x16 dK[DB], dV[DB];
 #pragma unroll
-  for (int db = 0; db < DBK; ++db) zero_acc(dK[db]);
-#pragma unroll
-  for (int db = 0; db < DBV; ++db) zero_acc(dV[db]);
+  for (int db = 0; db < DB; ++db) {
+    zero_acc(dK[db]);
+    zero_acc(dV[db]);
+  }
 
   const float sl2 = pr.scale * LOG2E;
   bool mask_small = true;
@@ -512,23 +426,18 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
     mask_small = pr.ms[2] >= 0 && pr.ms[3] >= 0 && 8 * pr.ms[2] + (int64_t)Lk * pr.ms[3] < lim;
     mlane = (uint32_t)(8 * g * pr.ms[2] + (int64_t)kld * pr.ms[3]);
   }
-  // tile slots 0 Q, 1 G (gO; gT in TANGENT; gT again in DUAL without gO), 2 Q', 3 gT, and the
-  // statistics slots PLAIN M, d1 | DUAL M, mu, a, d2 (= d1 + d2) | TANGENT M, a
+  // tile slots 0 Q, 1 G (gO; gT in TANGENT), and the statistics slots PLAIN M, d1 | TANGENT M, a
   // h is the query head being visited; what depends on it is set per head
   int h = hk * group;
-  const char *Qb = nullptr, *gTb = nullptr, *Gb = nullptr, *Qtb = nullptr;
-  const float *st_p[4] = {nullptr, nullptr, nullptr, nullptr};
+  const char *Qb = nullptr, *Gb = nullptr;
+  const float *st_p[2] = {nullptr, nullptr};
   auto set_query_head = [&](int hq) {
     h = hq;
     const size_t qhead = ((size_t)z * pr.H + hq) * L * D * sizeof(T), srow = ((size_t)z * pr.H + hq) * L;
     Qb = reinterpret_cast<const char *>(p.q) + qhead;
-    gTb = (DUAL || TAN) ? reinterpret_cast<const char *>(p.gt) + qhead : nullptr;
-    Gb = TAN ? gTb : (has_go ? reinterpret_cast<const char *>(p.go) + qhead : gTb);
-    Qtb = DUAL ? reinterpret_cast<const char *>(p.qt) + qhead : nullptr;
+    Gb = reinterpret_cast<const char *>(TAN ? p.gt : p.go) + qhead;
     st_p[0] = p.M + srow;
-    st_p[1] = MODE == BWD_PLAIN ? p.d1 + srow : (DUAL ? p.mu + srow : p.a + srow);
-    st_p[2] = DUAL ? p.a + srow : nullptr;
-    st_p[3] = DUAL ? p.d2 + srow : nullptr;
+    st_p[1] = (TAN ? p.a : p.d1) + srow;
   };
 
   const int istart = pr.causal ? (k0 / BT) * BT : 0;
@@ -553,7 +462,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
     return tlist ? min(max(entry, 0), tmax) * TILE_W + (t & 1) * BT : istart + t * BT;
   };
   constexpr int NLOAD = IPW * Cfg::NTILE;
-  constexpr int NPV = 2 * DBS;  // accumulation steps: (16-query chunk c, d-block db)
+  constexpr int NPV = 2 * DB;  // accumulation steps: (16-query chunk c, d-block db)
   constexpr int NSTEP = KK + NPV;
   int st_row = 0;
   uint32_t st_dst = 0;
@@ -561,10 +470,6 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
     ld_dst = lds0 + stage * Cfg::STAGEB + (wave * IPW) * 1024;
     ld_rs[0] = tile_rsrc(Qb, i0, on);
     ld_rs[1] = tile_rsrc(Gb, i0, on);
-    if constexpr (DUAL) {
-      ld_rs[2] = tile_rsrc(Qtb, i0, on);
-      ld_rs[3] = tile_rsrc(gTb, i0, on);
-    }
     i0 = on ? i0 : istart;
     st_row = min(i0 + lane, L - 1);
     st_dst = stat0 + stage * Cfg::STATB;
@@ -613,19 +518,14 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   // ih: first query of this tile; ihn: of the tile that follows it
   auto tile_body = [&](auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn) {
     constexpr bool EDGE = decltype(EDGEc)::value;
-    // ---- recompute ------------------------------------------------------------------------------
-    FragN fq[2], fg[2], fqt[2], fgt[2];
+    // ---- recompute: S and dP = gO V^T (PLAIN) or A = gT V^T (TANGENT) -----------------------------
+    FragN fq[2], fg[2];
     auto issue_n = [&](auto kkc) {
       constexpr int kk = decltype(kkc)::value, sl = kk % 2, HI = (kk / 8) * 256;
       const uint32_t ad = sbase + noff[kk % 8];
       fq[sl].v = lds_b128<HI>(ad);
-      if constexpr (NEED_V) fg[sl].v = lds_b128<HI + TILEB>(ad);
-      if constexpr (DUAL) {
-        fqt[sl].v = lds_b128<HI + 2 * TILEB>(ad);
-        if constexpr (NEED_V) fgt[sl].v = lds_b128<HI + 3 * TILEB>(ad);
-      }
+      fg[sl].v = lds_b128<HI + TILEB>(ad);
     };
-    constexpr int NRN = (DUAL ? 2 : 1) * (NEED_V ? 2 : 1);
     T mraw_a[MASK == MASK_ADD ? 16 : 1];
     uint8_t mraw_b[MASK == MASK_BOOL ? 16 : 1];
     if constexpr (MASK != MASK_NONE) {
@@ -636,36 +536,18 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
       }
       fetch_mask_tile(ihn);
     }
-    f32x16 S, dP, Sp, At;  // DUAL: dP also collects gT V'^T (the B term)
+    f32x16 S, G;
     issue_n(std::integral_constant<int, 0>{});
     static_for<KK>([&](auto kkc) {
       constexpr int kk = decltype(kkc)::value, sl = kk % 2;
       constexpr bool F = kk == 0;
       if constexpr (kk + 1 < KK) issue_n(std::integral_constant<int, kk + 1>{});
-      constexpr int younger_n = (kk + 1 < KK) ? NRN : 0;
-      if constexpr (DUAL && NEED_V) lds_wait<younger_n>(fq[sl], fg[sl], fqt[sl], fgt[sl]);
-      else if constexpr (DUAL) lds_wait<younger_n>(fq[sl], fqt[sl]);
-      else lds_wait<younger_n>(fq[sl], fg[sl]);
+      lds_wait<(kk + 1 < KK) ? 2 : 0>(fq[sl], fg[sl]);
       load_step(std::integral_constant<int, kk>{});
-      const Frag<T> q_ = as_frag<T>(fq[sl]);
-      mma_vra<F, GD>(S, q_, Kf[kk]);
-      if constexpr (MODE == BWD_PLAIN) mma_vra<F, GD>(dP, as_frag<T>(fg[sl]), Vf[kk]);
-      if constexpr (TAN) mma_vra<F, GD>(At, as_frag<T>(fg[sl]), Vf[kk]);
-      if constexpr (DUAL) {
-        mma_vra<F, GD>(Sp, as_frag<T>(fqt[sl]), Kf[kk]);
-        mma_vra<false, GD>(Sp, q_, Ktf[kk]);
-        if constexpr (NEED_V) {
-          const Frag<T> gt_ = as_frag<T>(fgt[sl]);
-          if constexpr (has_go) mma_vra<F, GD>(dP, as_frag<T>(fg[sl]), Vf[kk]);
-          mma_vra<F, GD>(At, gt_, Vf[kk]);
-          mma_vra<F && !has_go, GD>(dP, gt_, Vtf[kk]);
-        }
-      }
+      mma_vra<F, true>(S, as_frag<T>(fq[sl]), Kf[kk]);
+      mma_vra<F, true>(G, as_frag<T>(fg[sl]), Vf[kk]);
     });
-    if constexpr (DUAL && NEED_V) tiles_ready(S, dP, Sp, At);
-    else if constexpr (DUAL) tiles_ready(S, Sp);
-    else if constexpr (TAN) tiles_ready(S, At);
-    else tiles_ready(S, dP);
+    tiles_ready(S, G);
 
     // ---- row statistics of the 32 queries: register e belongs to query 16(e/8) + 8g + e%8, read one
     // quad of registers at a time, one quad ahead
@@ -679,43 +561,25 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
       });
     };
     const int qmin = pr.causal ? krow : 0;  // queries below this index do not see this key
-    FragT tq[2], tg[2], tqt[2], tgt[2];
-    // one step: transposed fragments of d-block db of chunk c; Q, Q' feed dK, G, gT feed dV
+    FragT tq[2], tg[2];
+    // one step: transposed fragments of d-block db of chunk c; Q feeds dK, G feeds dV
     auto issue_t = [&](auto ic) {
-      constexpr int i = decltype(ic)::value, c = i / DBS, db = i % DBS, sl = i % 2;
+      constexpr int i = decltype(ic)::value, c = i / DB, db = i % DB, sl = i % 2;
       constexpr int TO = c * 16 * ROWB + (db / 4) * 256;
       const uint32_t a0 = sbase + toff[db % 4][0], a1 = sbase + toff[db % 4][1];
-      if constexpr (WANT_DK) {
-        tq[sl].lo = lds_tr64<TO>(a0);
-        tq[sl].hi = lds_tr64<TO>(a1);
-      }
-      if constexpr (WANT_DV && (!DUAL || has_go)) {
-        tg[sl].lo = lds_tr64<TO + TILEB>(a0);
-        tg[sl].hi = lds_tr64<TO + TILEB>(a1);
-      }
-      if constexpr (DUAL && WANT_DK) {
-        tqt[sl].lo = lds_tr64<TO + 2 * TILEB>(a0);
-        tqt[sl].hi = lds_tr64<TO + 2 * TILEB>(a1);
-      }
-      if constexpr (DUAL && WANT_DV) {
-        tgt[sl].lo = lds_tr64<TO + 3 * TILEB>(a0);
-        tgt[sl].hi = lds_tr64<TO + 3 * TILEB>(a1);
-      }
+      tq[sl].lo = lds_tr64<TO>(a0);
+      tq[sl].hi = lds_tr64<TO>(a1);
+      tg[sl].lo = lds_tr64<TO + TILEB>(a0);
+      tg[sl].hi = lds_tr64<TO + TILEB>(a1);
     };
-    // LDS reads of a step (each FragT is two)
-    constexpr int NRT = 2 * ((WANT_DK ? 1 : 0) + ((WANT_DV && (!DUAL || has_go)) ? 1 : 0) + ((DUAL && WANT_DK) ? 1 : 0) +
-                             ((DUAL && WANT_DV) ? 1 : 0));
     issue_s(std::integral_constant<int, 0>{});
     static_for<2>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
-      f32x8 Pp;  // P * (S' - mu) of this chunk
       static_for<2>([&](auto hc) {
         constexpr int c4 = 2 * c + decltype(hc)::value, sl = c4 % 2;
         if constexpr (c4 + 1 < 4) issue_s(std::integral_constant<int, c4 + 1>{});
         // waits also cover the transposed fragments issued before (LDS reads complete in order)
-        constexpr int younger = (c4 + 1 < 4) ? Cfg::NSTAT : 0;
-        if constexpr (Cfg::NSTAT == 4) lds_wait4<younger>(stq[sl][0], stq[sl][1], stq[sl][2], stq[sl][3]);
-        else lds_wait<younger>(stq[sl][0], stq[sl][1]);
+        lds_wait<(c4 + 1 < 4) ? Cfg::NSTAT : 0>(stq[sl][0], stq[sl][1]);
         auto stat = [&](int s_, int e) { return __uint_as_float(stq[sl][s_][e % 4]); };
 #pragma unroll
         for (int e = 4 * c4; e < 4 * c4 + 4; ++e) {
@@ -728,54 +592,18 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
           if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
           S[e] = pv;
-          if constexpr (MODE == BWD_PLAIN) {
-            dP[e] = pv * (dP[e] - stat(1, e));
-          } else if constexpr (DUAL) {
-            const float sp = Sp[e] * pr.scale, m_ = stat(1, e);
-            if constexpr (WANT_DV) Pp[e - 8 * c] = pv * (sp - m_);
-            if constexpr (WANT_DK) {
-              const float am = At[e] - stat(2, e);
-              Sp[e] = pv * am;
-              dP[e] = pv * (dP[e] + am * sp - At[e] * m_ - stat(3, e));
-            }
-          } else {
-            Sp[e] = pv * (At[e] - stat(1, e));
-          }
+          G[e] = pv * (G[e] - stat(1, e));
         }
       });
-      Frag<T> pf, dsf, dspf, ppf;
-      if constexpr (WANT_DV) pf = to_frag<T>(S, c);
-      if constexpr (!TAN && WANT_DK) dsf = to_frag<T>(dP, c);
-      if constexpr ((DUAL && WANT_DK) || TAN) dspf = to_frag<T>(Sp, c);
-      if constexpr (DUAL && WANT_DV) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ppf[e] = (T)Pp[e];
-      }
-      issue_t(std::integral_constant<int, c * DBS>{});
-      static_for<DBS>([&](auto dbc) {
-        constexpr int db = decltype(dbc)::value, i = c * DBS + db, sl = i % 2;
-        if constexpr (db + 1 < DBS) issue_t(std::integral_constant<int, i + 1>{});
-        constexpr int younger = (db + 1 < DBS) ? NRT : 0;
-        if constexpr (MODE != BWD_DUAL) lds_wait<younger>(tq[sl], tg[sl]);
-        else if constexpr (WANT_DK) lds_wait<younger>(tq[sl], tqt[sl]);
-        else if constexpr (has_go) lds_wait<younger>(tg[sl], tgt[sl]);
-        else lds_wait<younger>(tgt[sl].lo, tgt[sl].hi);
+      const Frag<T> pf = to_frag<T>(S, c), dsf = to_frag<T>(G, c);
+      issue_t(std::integral_constant<int, c * DB>{});
+      static_for<DB>([&](auto dbc) {
+        constexpr int db = decltype(dbc)::value, i = c * DB + db, sl = i % 2;
+        if constexpr (db + 1 < DB) issue_t(std::integral_constant<int, i + 1>{});
+        lds_wait<(db + 1 < DB) ? 4 : 0>(tq[sl], tg[sl]);
         load_step(std::integral_constant<int, KK + i>{});
-        if constexpr (MODE == BWD_PLAIN) {
-          mma(dK[db], as_frag<T>(tq[sl]), dsf);
-          mma(dV[db], as_frag<T>(tg[sl]), pf);
-        } else if constexpr (DUAL) {
-          if constexpr (WANT_DK) {
-            mma(dK[db], as_frag<T>(tq[sl]), dsf);
-            mma(dK[db], as_frag<T>(tqt[sl]), dspf);
-          } else {
-            if constexpr (has_go) mma(dV[db], as_frag<T>(tg[sl]), pf);
-            mma(dV[db], as_frag<T>(tgt[sl]), ppf);
-          }
-        } else {
-          mma(dK[db], as_frag<T>(tq[sl]), dspf);
-          mma(dV[db], as_frag<T>(tg[sl]), pf);
-        }
+        mma(dK[db], as_frag<T>(tq[sl]), dsf);
+        mma(dV[db], as_frag<T>(tg[sl]), pf);
       });
     });
   };
@@ -818,34 +646,24 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   }
 
   if (krow < Lk) {
-    if constexpr (WANT_DK) {
 #pragma unroll
-      for (int db = 0; db < DBK; ++db) {
+    for (int db = 0; db < DB; ++db) {
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-          float x[8];
+      for (int hf = 0; hf < 2; ++hf) {
+        float x[8], y[8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) x[e] = dK[db][8 * hf + e] * pr.scale;
-          store8<T>(outk + 32 * db + 16 * hf + 8 * g, x);
+        for (int e = 0; e < 8; ++e) {
+          x[e] = dK[db][8 * hf + e] * pr.scale;
+          y[e] = dV[db][8 * hf + e];
         }
-      }
-    }
-    if constexpr (WANT_DV) {
-#pragma unroll
-      for (int db = 0; db < DBV; ++db) {
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-          float x[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) x[e] = dV[db][8 * hf + e];
-          store8<T>(outv + 32 * db + 16 * hf + 8 * g, x);
-        }
+        store8<T>(outk + 32 * db + 16 * hf + 8 * g, x);
+        store8<T>(outv + 32 * db + 16 * hf + 8 * g, y);
       }
     }
   }
 }
 #else
-template <typename T, int D, int DV, int MODE, int MASK, bool GO, int PART>
+template <typename T, int D, int MODE, int MASK>
 __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {}
 #endif
 
