@@ -121,6 +121,20 @@ def test_head_dim_256(dt, mode):
     _run_case(1, 2, 200, 256, DTYPES[dt], mode, seed=17)
 
 
+@pytest.mark.parametrize("L", [65, 130, 333])
+@pytest.mark.parametrize("mode", ["none", "causal", "keypad", "bool_full"])
+def test_head_dim_256_lengths_across_the_64_row_workgroups(L, mode):
+    """The dual backward at D = 256 runs workgroups of 64 rows (two pairs of waves that hand each other score
+    tiles through LDS), the other D = 256 kernels 128 rows: lengths that end inside either kind of block."""
+    _run_case(1, 2, L, 256, torch.bfloat16, mode, seed=23)
+
+
+def test_head_dim_256_tiles_away_from_every_edge():
+    _run_case(1, 1, 1100, 256, torch.bfloat16, "causal", seed=24)
+    _run_case(1, 1, 520, 256, torch.float16, "bias", seed=25)
+    _run_case(1, 1, 520, 256, torch.float16, "none", seed=26, plain=True)
+
+
 def test_head_dim_256_in_fp32_plain_and_at_a_benchmark_length():
     """fp32 at D = 256 reads its own rows' fragments from global memory instead of keeping them in registers:
     the plain path, and a length with many interior tiles (causal, so that both loops' edges are crossed)."""
@@ -632,8 +646,8 @@ def test_grouped_heads_and_a_key_length_of_its_own(dt, D, shape, mode):
 @pytest.mark.parametrize("shape", [(4, 2, 96, 96), (2, 1, 70, 200), (2, 2, 200, 70), (1, 1, 1, 3), (1, 1, 33, 31), (2, 2, 5, 2)])
 @pytest.mark.parametrize("mode", ["none", "causal", "bool", "bias"])
 def test_head_dim_256_with_grouped_heads_key_lengths_and_tiny_shapes(dt, shape, mode):
-    """The D = 256 forward (two workgroups per query block, 32-key tiles) and the split dk/dv launches
-    on the shapes of the test above, down to a single query."""
+    """The D = 256 kernels (two forward passes over 32-key tiles; a backward whose workgroups are two pairs
+    of waves that share 32 rows) on the shapes of the test above, down to a single query."""
     if mode == "causal" and shape == (1, 1, 1, 3):
         pytest.skip("one query sees one key under the causal rule: every gradient of q is exactly zero")
     _run_kv_shape_case(dt, 256, shape, mode)
