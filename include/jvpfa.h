@@ -47,7 +47,8 @@ enum jvpfa_status {
 
 /* Shape, numeric type and masking shared by forward and backward. */
 typedef struct jvpfa_problem {
-  int32_t Z, H, L, D; /* D in {32, 64, 128, 256} (JA:2371-2374) */
+  int32_t Z, H, L, D; /* D in {32, 64, 128, 256}; the reference also admits 16 (JA:2371-2374): a caller pads
+                       * q, k, v (and tangents, gradients) with zero columns to 32 and drops them from the results */
   int32_t dtype;      /* enum jvpfa_dtype: element type of q,k,v,o and their tangents/gradients */
   int32_t causal;     /* 0/1; lower-triangular (query index >= key index), JA:253-258 */
   int32_t mask_kind;  /* enum jvpfa_mask_kind */

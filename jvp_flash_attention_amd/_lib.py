@@ -268,6 +268,20 @@ def _stream(t) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+# The reference admits a head dim of 16 (jvp_flash_attention/jvp_attention.py:2371-2374); the matrix instructions
+# here contract over 16 and produce 32 columns, so the kernels start at 32 and a head dim of 16 runs on them with
+# zero columns appended (one copy of each operand per call).
+PADDED_HEAD_DIM = 16
+
+
+def _pad_head_dim(t):
+    return None if t is None else torch.nn.functional.pad(t, (0, 32 - PADDED_HEAD_DIM))
+
+
+def _cut_head_dim(t):
+    return None if t is None else t[..., :PADDED_HEAD_DIM].contiguous()
+
+
 class HipBackend:
     """Device work of the forward and the backward, through the C ABI.
 
@@ -297,6 +311,11 @@ class HipBackend:
 
     def _fwd(self, q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale, dropout_p=0.0, dropout_seed=0):
         _require_gpu(q, k, v, qt, kt, vt, mask)
+        if q.shape[-1] == PADDED_HEAD_DIM:
+            # zero columns change neither Q K^T nor the columns of P V that are kept
+            o, ot, M, mu = self._fwd(*map(_pad_head_dim, (q, k, v, qt, kt, vt)), mask, mask_kind, causal, sm_scale,
+                                     dropout_p, dropout_seed)
+            return _cut_head_dim(o), _cut_head_dim(ot), M, mu
         lib = load()
         dual = qt is not None
         o = torch.empty_like(q)
@@ -326,6 +345,11 @@ class HipBackend:
     def _bwd(self, q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
              want_tangent_grads=False, dropout_p=0.0, dropout_seed=0):
         _require_gpu(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask)
+        if q.shape[-1] == PADDED_HEAD_DIM:
+            q, k, v, qt, kt, vt, o, ot, go, gt = map(_pad_head_dim, (q, k, v, qt, kt, vt, o, ot, go, gt))
+            grads = self._bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale,
+                              want_tangent_grads, dropout_p, dropout_seed)
+            return tuple(map(_cut_head_dim, grads))
         lib = load()
         Z, H, L, _ = q.shape
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)

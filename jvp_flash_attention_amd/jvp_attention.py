@@ -22,8 +22,9 @@ Differences from the reference, all deliberate:
 * ``fwd_dual`` returns an output whose tangent O' carries an autograd graph, so gradients of
   functions of O' (Hessian-vector products) reach q, k, v and the input tangents.  The
   reference's tangent is a constant (JA:2399, JA:2828) and its backward ignores it (JA:2831).
-* Any sequence length L >= 1 and head dims {32, 64, 128, 256} (the reference: L a multiple of 32,
-  JA:2371-2378, JA:2892).
+* Any sequence length L >= 1 (the reference: an even L >= 32, JA:2375-2378, and a multiple of its tile sizes,
+  JA:2892).  Head dims as there, {16, 32, 64, 128, 256} (JA:2371-2374); 16 runs on the kernels for 32 with zero
+  columns appended.
 * k and v may have fewer heads than q (grouped heads: H a multiple of H_kv) and a length of their own
   (cross-attention); causal then means key index <= query index, as in SDPA.  The reference requires
   q, k, v of one shape (JA:2367-2378).
@@ -49,7 +50,7 @@ from . import _lib
 
 MASK_CONST = -100.0  # JA:48-50: value float masks use for "masked"; far below any real logit
 MIN_SEQUENCE_LENGTH = 32  # JA:51; kept for importers, not a limit of these kernels
-SUPPORTED_HEAD_DIMS = (32, 64, 128, 256)
+SUPPORTED_HEAD_DIMS = (16, 32, 64, 128, 256)
 BLOCK_M = 128  # query rows per workgroup of the forward kernel (only reported through Grid)
 
 

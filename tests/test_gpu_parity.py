@@ -121,6 +121,16 @@ def test_head_dim_256(dt, mode):
     _run_case(1, 2, 200, 256, DTYPES[dt], mode, seed=17)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("mode", ["none", "causal", "keypad", "bias"])
+def test_head_dim_16(dt, mode):
+    """The smallest head dim the reference admits (its jvp_attention.py:2371-2374): the backend appends zero columns
+    and runs the kernels for 32; outputs and all six gradients come back with 16 columns."""
+    _run_case(2, 2, 100, 16, DTYPES[dt], mode, seed=31)
+    if mode == "none":
+        _run_case(1, 2, 70, 16, DTYPES[dt], mode, seed=32, plain=True)
+
+
 @pytest.mark.parametrize("L", [65, 130, 333])
 @pytest.mark.parametrize("mode", ["none", "causal", "keypad", "bool_full"])
 def test_head_dim_256_lengths_across_the_64_row_workgroups(L, mode):

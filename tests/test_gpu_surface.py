@@ -143,6 +143,40 @@ def test_forward_and_backward_replay_from_a_hip_graph(causal):
             assert torch.equal(a, b), f"replay {rep}"
 
 
+def test_surface_head_dim_16_eager_and_compiled():
+    """A head dim of 16, which the reference admits, through the public functions: the tangent from
+    ``torch.func.jvp``, gradients from autograd, and the same call under ``torch.compile``."""
+    from jvp_flash_attention_amd import JVPAttn, attention
+
+    Z, H, L, D = 2, 3, 96, 16
+    q, k, v, qt, kt, vt, go, gt = [_randn((Z, H, L, D), torch.bfloat16, 40 + i) for i in range(8)]
+    f64 = [x.double().cpu().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    ref = dense.forward(*f64[:6], mask=None, causal=True)
+    rb = dense.backward(*f64, mask=None, causal=True)
+    leaves = [x.clone().requires_grad_() for x in (q, k, v, qt, kt, vt)]
+    with fwAD.dual_level():
+        out = JVPAttn.fwd_dual(*(fwAD.make_dual(p, t) for p, t in zip(leaves[:3], leaves[3:])), causal=True)
+        o, ot = fwAD.unpack_dual(out)
+        assert o.shape == (Z, H, L, D) and ot.shape == (Z, H, L, D)
+        grads = torch.autograd.grad((o.float() * go.float()).sum() + (ot.float() * gt.float()).sum(), leaves)
+    assert _rel(o, ref["O"]) <= 2e-2 and _rel(ot, ref["Ot"]) <= 2e-2
+    for n, g in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        assert g.shape == (Z, H, L, D) and _rel(g, rb[n]) <= 2e-2, n
+
+    def f(q, k, v):
+        return (attention(q, k, v, causal=True).float() * go.float()).sum()
+
+    pl = [x.clone().requires_grad_() for x in (q, k, v)]
+    eager = f(*pl)
+    ge = torch.autograd.grad(eager, pl)
+    torch._dynamo.reset()
+    compiled = torch.compile(f, backend="aot_eager", fullgraph=True)(*pl)
+    gc = torch.autograd.grad(compiled, pl)
+    assert torch.equal(eager, compiled)
+    for a, b in zip(ge, gc):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("masked", [False, True])
 def test_plain_attention_inside_torch_compile_without_graph_breaks(masked):
     """``torch.compile(fullgraph=True)`` over a function that calls ``attention``: the kernels enter
