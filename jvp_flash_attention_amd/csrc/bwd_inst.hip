@@ -18,7 +18,7 @@ namespace jvpfa {
 // to itself instead of sharing it with a second workgroup and is still 4 - 9 % ahead; at D = 128 dK, dV, the
 // resident K, V, K' and the tiles already take 452 of the 512 registers and dK', dV' would add 128).
 template <typename T, int D> struct BwdFold {
-  static constexpr bool DQ = sizeof(T) == 2 && D <= 128;
+  static constexpr bool DQ = sizeof(T) == 2;
   static constexpr bool KV = sizeof(T) == 2 && D <= 64;
 };
 
@@ -131,6 +131,7 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
     const long long kblocks = (long long)((p.pr.Lk + CfgP::BLK - 1) / CfgP::BLK) * p.pr.Z * p.pr.Hk;
     if (qblocks > 0x7fffffffLL || kblocks > 0x7fffffffLL) return -2;
     void (*kq)(const BwdParams) = no_go ? bwdp_dq_kernel<T, D, MASK, false> : bwdp_dq_kernel<T, D, MASK, true>;
+    if (six) kq = no_go ? bwdp_dq_kernel<T, D, MASK, false, true> : bwdp_dq_kernel<T, D, MASK, true, true>;
     void (*kkv)(const BwdParams) = no_go ? bwdp_dkdv_kernel<T, D, MASK, false> : bwdp_dkdv_kernel<T, D, MASK, true>;
     int rc = allow_lds(reinterpret_cast<const void *>(kq), CfgP::DQ_LDS);
     if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), CfgP::DKV_LDS);
@@ -148,7 +149,8 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
     if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), CfgK::DKV_LDS);
     if (rc != 0) return rc;
     hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
-    hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(CfgW::NT), CfgW::DQ_LDS, stream, p);
+    // (six: the tangent launch of a six-gradient call, whose dq' the dual launch has written already)
+    if (!(MODE == BWD_TANGENT && six)) hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(CfgW::NT), CfgW::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
   } else {
     auto kq = bwd_dq_kernel<T, D, MODE, MASK>;

@@ -75,7 +75,9 @@ template <int SLOT, int N> __device__ __forceinline__ f32x16 xch_tile(const u32x
 
 #if defined(__HIP_DEVICE_COMPILE__)
 // dq of the dual mode.  Tile slots of a stage: 0 K, 1 V, 2 K', 3 V'.
-template <typename T, int D, int MASK, bool GO>
+// SIX: dq' = scale dS' K as well, from the K fragments and the dS' tiles that dq already has (a call for all six
+// gradients then needs no second launch that forms S and A again).
+template <typename T, int D, int MASK, bool GO, bool SIX = false>
 __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {
   using Cfg = BwdPairCfg<T, D>;
   constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT, DV = Cfg::DV;
@@ -170,9 +172,12 @@ __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {
   const float av = p.a[srow + qld];
   const float dsum = p.d2[srow + qld];
 
-  f32x16 acc[DB];
+  f32x16 acc[DB], accT[SIX ? DB : 1];
 #pragma unroll
-  for (int db = 0; db < DB; ++db) zero_acc(acc[db]);
+  for (int db = 0; db < DB; ++db) {
+    zero_acc(acc[db]);
+    if constexpr (SIX) zero_acc(accT[db]);
+  }
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
@@ -321,6 +326,10 @@ __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {
       mma(acc[2 * dp + 1], as_frag<T>(tk[sl][1]), dsf[c]);
       mma(acc[2 * dp], as_frag<T>(tkt[sl][0]), dspf[c]);
       mma(acc[2 * dp + 1], as_frag<T>(tkt[sl][1]), dspf[c]);
+      if constexpr (SIX) {
+        mma(accT[2 * dp], as_frag<T>(tk[sl][0]), dspf[c]);
+        mma(accT[2 * dp + 1], as_frag<T>(tk[sl][1]), dspf[c]);
+      }
     });
   };
 
@@ -380,6 +389,11 @@ __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) x[e] = acc[db][8 * hf + e] * pr.scale;
         store8<T>(out + 32 * db + 16 * hf + 8 * g, x);
+        if constexpr (SIX) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[e] = accT[db][8 * hf + e] * pr.scale;
+          store8<T>(reinterpret_cast<T *>(p.dqt) + head + (size_t)qrow * D + role * DV + 32 * db + 16 * hf + 8 * g, x);
+        }
       }
     }
   }
@@ -752,7 +766,7 @@ __global__ __launch_bounds__(256, 1) void bwdp_dkdv_kernel(const BwdParams p) {
   }
 }
 #else
-template <typename T, int D, int MASK, bool GO>
+template <typename T, int D, int MASK, bool GO, bool SIX = false>
 __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {}
 template <typename T, int D, int MASK, bool GO>
 __global__ __launch_bounds__(256, 1) void bwdp_dkdv_kernel(const BwdParams p) {}
