@@ -57,10 +57,12 @@ typedef struct jvpfa_problem {
                          added to the scaled logits (SDPA semantics) */
   int64_t mask_stride[4]; /* element strides over (z, h, query, key); 0 broadcasts */
   /* Dropout on the attention probabilities: 0 <= dropout_p < 1, 0 = none.  Entry (z, h, query, key) is kept or
-   * dropped by a counter-based hash of (dropout_seed, entry index) and kept entries are scaled by 1/(1 - p), as
+   * dropped by a counter-based hash of (dropout_seed, z, h, query, key) and kept entries are scaled by 1/(1 - p), as
    * torch's scaled_dot_product_attention does; forward and backward of one call pair must get the same seed.
    * jvpfa_dropout_keep() writes the keep pattern out.  The reference carries dead code for dropout and raises
-   * NotImplementedError (JA:94-122, JA:271-277, JA:2356-2357).  Costs bf16 / fp16 calls 13 - 22 % (D <= 128), fp32 2 - 6 %. */
+   * NotImplementedError (JA:94-122, JA:271-277, JA:2356-2357).  Costs bf16 / fp16 calls 6 - 13 % at D = 128
+   * (a third where the unmasked, non-causal forward leaves its software-pipelined kernel), about 30 % at D = 64,
+   * fp32 1 - 6 %. */
   float dropout_p;
   uint64_t dropout_seed;
 } jvpfa_problem;

@@ -315,7 +315,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(const BwdParams p) {
         if (diag) pv = (key0 + e <= qrow) ? pv : 0.f;
         if (ragged) pv = (key0 + e < Lk) ? pv : 0.f;
         if constexpr (DROP) {  // gO V^T, gT V^T, gT V'^T reach the logits through the kept, rescaled entries only
-          const float ks = drop_scale(pr, ((uint64_t)zh * L + qld) * Lk + (key0 + e));
+          const float ks = drop_scale(pr, zh, qld, key0 + e);
           if constexpr (!TAN) dP[i] *= ks;
           if constexpr (DUAL || TAN) At[i] *= ks;
         }
@@ -585,7 +585,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(const BwdParams p) {
       if (diag) pv = (krow <= qi) ? pv : 0.f;
       float ks = 1.f;  // dropout: 1 / (1 - p) for a kept entry, 0 for a dropped one
       if constexpr (DROP) {
-        ks = drop_scale(pr, (((uint64_t)z * pr.H + h) * L + (qi < L ? qi : L - 1)) * Lk + kld);
+        ks = drop_scale(pr, z * pr.H + h, qi < L ? qi : L - 1, kld);
         if constexpr (!TAN) dP[e] *= ks;
         if constexpr (DUAL || TAN) At[e] *= ks;
       }

@@ -168,6 +168,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
   }
 
   const float Mq = qrow < L ? p.M[srow + qld] : __builtin_inff();
+  const uint32_t drop_row = DROP ? drop_row_word(pr, zh, qld) : 0u;  // dropout: this lane's query row
   const float d1 = (MODE == BWD_PLAIN) ? p.d1[srow + qld] : 0.f;
   const float mu = DUAL ? p.mu[srow + qld] : 0.f;
   const float av = (DUAL || TAN) ? p.a[srow + qld] : 0.f;
@@ -300,11 +301,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
           if constexpr (MASK == MASK_BOOL) keep[e] = mask_keep_of<T, MASK>(mah[hf], e);
         }
       }
-      uint32_t dlo = 0, dhi = 0;
-      if constexpr (DROP) {
-        const uint64_t base = ((uint64_t)zh * L + qld) * Lk + (uint32_t)key0;
-        dlo = (uint32_t)base, dhi = (uint32_t)(base >> 32);
-      }
+      const uint32_t xb = DROP ? drop_row + (uint32_t)key0 * DROP_C_KEY : 0u;  // dropout word of key key0, see params.hpp
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int i = 8 * hf + e;
@@ -314,7 +311,7 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
         if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
         if constexpr (EDGE) pv = (key0 + e <= klim) ? pv : 0.f;
         if constexpr (DROP) {
-          const float ks = drop_scale_at(pr, dlo, dhi, e);
+          const float ks = drop_scale_of(pr, xb + (uint32_t)e * DROP_C_KEY);
           if constexpr (!TAN) dP[i] *= ks;
           if constexpr (DUAL || TAN) At[i] *= ks;
         }
@@ -489,6 +486,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
   const int krow = k0 + wave * 32 + r;
   const int Lk = pr.Lk;  // keys; L counts queries
   const int kld = krow < Lk ? krow : Lk - 1;
+  const uint32_t drop_lane = DROP ? (uint32_t)kld * DROP_C_KEY + (uint32_t)(8 * g) * DROP_C_ROW : 0u;
   if constexpr (MASK != MASK_NONE) {
     // a key block that the caller's hint declares fully masked has zero gradients
     if (pr.klimit && k0 >= pr.klimit[z]) {
@@ -660,6 +658,9 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
   // ih: first query of this half tile; ihn: of the half tile that follows it
   auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn) {
     constexpr int HB = decltype(HBc)::value;
+    // dropout: the 32 queries of a half tile are one block of the pattern (ih is a multiple of 32), so the block's
+    // word is uniform and register e's query adds a constant to it; this lane's key and row group add drop_lane
+    const uint32_t drop_half = DROP ? drop_row_word(pr, z * pr.H + hq, ih) + drop_lane : 0u;
     constexpr bool EDGE = decltype(EDGEc)::value;
     constexpr int RO = HB * 32 * ROWB;
     // ---- recompute ------------------------------------------------------------------------------
@@ -788,7 +789,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
           if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
           float ks = 1.f;  // dropout: 1 / (1 - p) for a kept entry, 0 for a dropped one
           if constexpr (DROP) {
-            ks = drop_scale(pr, (((uint64_t)z * pr.H + hq) * L + min(qi, L - 1)) * Lk + kld);
+            ks = drop_scale_of(pr, drop_half + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_ROW);
             if constexpr (!TAN) dP[e] *= ks;
             if constexpr (DUAL || TAN) At[e] *= ks;
           }

@@ -232,7 +232,7 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
         float ks = 1.f;
         if constexpr (DROP) {
           const int key = j0 + 32 * nb + 16 * (e / 8) + 8 * g + (e % 8);
-          ks = drop_scale(pr, ((uint64_t)zh * L + qld) * Lk + key);
+          ks = drop_scale(pr, zh, qld, key);
         }
         S[nb][e] = pv * ks;
         if constexpr (DUAL) {

@@ -184,6 +184,7 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
+  const uint32_t drop_row = DROP ? drop_row_word(pr, zh, qld) : 0u;  // dropout: this lane's query row, see params.hpp
   bool mask_al = false;  // mask rows can be fetched with aligned vector loads
   if constexpr (MASK != MASK_NONE) mask_al = mask_rows_aligned<T, MASK>(pr);
 
@@ -406,12 +407,11 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     }
     l_i += rs;
     if constexpr (DUAL) mu_i += rmu;
-    if constexpr (DROP) {  // entry index ((z H + h) L + query) Lk + key; register e holds key jh + 16(e/8) + 8g + e%8
-      const uint64_t base = ((uint64_t)zh * L + qld) * Lk + (uint32_t)(jh + 8 * g);
-      const uint32_t blo = (uint32_t)base, bhi = (uint32_t)(base >> 32);
+    if constexpr (DROP) {  // register e holds key jh + 16(e/8) + 8g + e%8 of this lane's query
+      const uint32_t xb = drop_row + (uint32_t)(jh + 8 * g) * DROP_C_KEY;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const float ks = drop_scale_at(pr, blo, bhi, 16 * (e / 8) + (e % 8));
+        const float ks = drop_scale_of(pr, xb + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_KEY);
         S[e] *= ks;
         if constexpr (DUAL) Sp[e] *= ks;
       }

@@ -107,8 +107,10 @@ using namespace jvpfa;
 namespace jvpfa {
 __global__ __launch_bounds__(256) void dropout_keep_kernel(Problem pr, uint64_t n, uint8_t *keep) {
   // a launch holds fewer than 2^32 threads, the pattern may hold more entries: each thread strides over the rest
-  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256)
-    keep[i] = drop_scale(pr, i) != 0.f;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
+    const uint64_t row = i / (uint64_t)pr.Lk;  // (z H + h) L + query
+    keep[i] = drop_scale(pr, (int)(row / (uint64_t)pr.L), (int)(row % (uint64_t)pr.L), (int)(i % (uint64_t)pr.Lk)) != 0.f;
+  }
 }
 }  // namespace jvpfa
 
@@ -118,7 +120,7 @@ extern "C" int jvpfa_dropout_keep(const jvpfa_problem *p, int32_t Lk, uint8_t *k
   jvpfa_problem q = *p;
   q.mask_kind = JVPFA_MASK_NONE;
   const Problem pr = to_problem(q, nullptr, nullptr, nullptr, Lk, 0);
-  const uint64_t n = (uint64_t)p->Z * p->H * p->L * pr.Lk;  // the entry index is ((z H + h) L + i) Lk + j
+  const uint64_t n = (uint64_t)p->Z * p->H * p->L * pr.Lk;  // entry (z, h, i, j) is byte ((z H + h) L + i) Lk + j
   if (n == 0) return JVPFA_OK;
   const uint64_t blocks = std::min<uint64_t>((n + 255) / 256, 1u << 20);
   hipLaunchKernelGGL(dropout_keep_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(hip_stream), pr, n, keep);

@@ -27,16 +27,20 @@ struct Problem {
   int chunks, chunk_tiles;
   float *part;
   // Dropout on the attention probabilities (0 in drop_thr: none).  Entry (z, h, query i, key j) is kept when
-  // drop_hash(((z H + h) L + i) Lk + j) >= drop_thr, and kept entries are scaled by drop_rinv = 1 / (1 - p); the
-  // same function of (seed, index) in the forward, both backward kernels and jvpfa_dropout_keep.
+  // drop_entry_hash(...) >= drop_thr, and kept entries are scaled by drop_rinv = 1 / (1 - p); the same function of
+  // (seed, z, h, i, j) in the forward, both backward kernels and jvpfa_dropout_keep.
   uint32_t drop_thr, drop_s0, drop_s1;
   float drop_rinv;
 };
 
-// Counter-based keep decision: a 32-bit mix of the 64-bit entry index and the seed (two multiply-xorshift rounds).
-__host__ __device__ inline uint32_t drop_hash(uint64_t idx, uint32_t s0, uint32_t s1) {
-  uint32_t x = ((uint32_t)idx * 0x9E3779B1u) ^ s0;
-  x ^= (uint32_t)(idx >> 32) * 0x85EBCA77u + s1;
+// Counter-based keep decision, shaped so that a kernel pays a handful of vector instructions per entry whichever
+// way it walks the matrix.  Query rows are taken in blocks of 32: the block (z H + h) ceil(L / 32) + i / 32 and the
+// seed go through a full 64 -> 32 bit mix (once per lane or per tile in a kernel); inside a block the word moves by a
+// constant per row and a constant per key (two Weyl sequences), and two multiply-xorshift rounds finish the entry.
+constexpr uint32_t DROP_C_KEY = 0x9E3779B1u, DROP_C_ROW = 0x85EBCA77u;
+__host__ __device__ inline uint32_t drop_block_hash(uint64_t block, uint32_t s0, uint32_t s1) {
+  uint32_t x = ((uint32_t)block * 0x9E3779B1u) ^ s0;
+  x ^= (uint32_t)(block >> 32) * 0x85EBCA77u + s1;
   x ^= x >> 16;
   x *= 0x7feb352du;
   x ^= x >> 15;
@@ -44,16 +48,24 @@ __host__ __device__ inline uint32_t drop_hash(uint64_t idx, uint32_t s0, uint32_
   x ^= x >> 16;
   return x;
 }
-// 1 / (1 - p) for a kept entry, 0 for a dropped one
-__host__ __device__ inline float drop_scale(const Problem &pr, uint64_t idx) {
-  return drop_hash(idx, pr.drop_s0, pr.drop_s1) >= pr.drop_thr ? pr.drop_rinv : 0.f;
+__host__ __device__ inline uint32_t drop_finish(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7feb352du;
+  x ^= x >> 15;
+  x *= 0x846ca68bu;
+  return x;
 }
-
-// The same for entry base + off, base a 64-bit index and off a small offset: the carry into the high word is
-// taken from the low-word sum.
-__device__ __forceinline__ float drop_scale_at(const Problem &pr, uint32_t base_lo, uint32_t base_hi, uint32_t off) {
-  const uint32_t lo = base_lo + off, hi = base_hi + (lo < base_lo ? 1u : 0u);
-  return drop_hash(((uint64_t)hi << 32) | lo, pr.drop_s0, pr.drop_s1) >= pr.drop_thr ? pr.drop_rinv : 0.f;
+// the word of row i of head zh = z H + h before the key's share: drop_finish(drop_row_word + j * DROP_C_KEY) is the hash
+__host__ __device__ inline uint32_t drop_row_word(const Problem &pr, int zh, int i) {
+  const uint64_t block = (uint64_t)zh * (uint64_t)((pr.L + 31) / 32) + (uint64_t)(i >> 5);
+  return drop_block_hash(block, pr.drop_s0, pr.drop_s1) + (uint32_t)(i & 31) * DROP_C_ROW;
+}
+// 1 / (1 - p) for a kept entry, 0 for a dropped one, from the entry's word
+__host__ __device__ inline float drop_scale_of(const Problem &pr, uint32_t word) {
+  return drop_finish(word) >= pr.drop_thr ? pr.drop_rinv : 0.f;
+}
+__host__ __device__ inline float drop_scale(const Problem &pr, int zh, int i, int j) {
+  return drop_scale_of(pr, drop_row_word(pr, zh, i) + (uint32_t)j * DROP_C_KEY);
 }
 
 constexpr int TILE_BLOCK = 128, TILE_W = 64;  // geometry of the tile lists

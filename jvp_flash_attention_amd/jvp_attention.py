@@ -31,8 +31,8 @@ Differences from the reference, all deliberate:
 * ``dropout_p`` > 0 works (the reference carries dead code for it and raises ``NotImplementedError``,
   JA:94-122, JA:271-277, JA:2356-2357): dropout on the attention probabilities with SDPA's semantics (kept entries
   scaled by 1/(1-p); the tangent O' sees the same pattern), the pattern a counter-based hash of a seed drawn from
-  torch's CPU generator per call (``torch.manual_seed`` makes it repeatable) and of the entry index, regenerated in
-  the backward.  (bf16 / fp16 calls get 13 - 22 % slower, fp32 2 - 6 %.)
+  torch's CPU generator per call (``torch.manual_seed`` makes it repeatable) and of the entry's coordinates, regenerated in
+  the backward.  (bf16 / fp16 calls get 6 - 13 % slower at head dim 128, about 30 % at 64, fp32 1 - 6 %.)
 * ``attention`` notices dual inputs and then behaves like ``fwd_dual`` (the reference's ``attention``
   is ``JVPAttn.fwd`` and drops the tangent, its README.md:65-67).
 """

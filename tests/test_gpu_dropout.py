@@ -94,9 +94,10 @@ def test_dropout_with_grouped_heads_ragged_and_unequal_lengths(dt):
     _case(1, 4, 77, 128, DTYPES[dt], "causal", p=0.1, seed=1, Hk=1)
 
 
-def test_the_pattern_uses_the_high_index_word_and_both_seed_words():
-    """Past 2^32 entries the index no longer fits one word; a slab across that boundary is read back through a
-    problem whose last rows lie beyond it.  The two seed words both change the pattern."""
+def test_the_pattern_past_two_to_the_32_entries_and_both_seed_words():
+    """The exported pattern is one byte per entry: past 2^32 entries the byte index no longer fits one word; a slab
+    across that boundary is read back through a problem whose last rows lie beyond it.  The two seed words both
+    change the pattern."""
     from jvp_flash_attention_amd import _lib
 
     be = _lib.backend()
@@ -111,8 +112,8 @@ def test_the_pattern_uses_the_high_index_word_and_both_seed_words():
     lo = (1 << 16) - 8
     slab = big[0, 0, lo:lo + 16].cpu().numpy()
     del big
-    idx = (np.arange(lo, lo + 16, dtype=np.uint64)[:, None] * np.uint64(Lk)) + np.arange(Lk, dtype=np.uint64)[None, :]
-    assert np.array_equal(slab, dropout.mix(idx, 99) >= np.uint64(dropout.threshold(0.25)))
+    rows, keys = np.arange(lo, lo + 16, dtype=np.uint64)[:, None], np.arange(Lk, dtype=np.uint64)[None, :]
+    assert np.array_equal(slab, dropout.entry_hash(0, rows, keys, L, 99) >= np.uint64(dropout.threshold(0.25)))
     assert abs(slab.mean() - 0.75) < 0.01
 
 

@@ -264,20 +264,32 @@ def test_dense_with_dropout_matches_the_library_route(mode, with_gt):
 
 
 def test_dropout_pattern_properties():
-    """What the mathematics fixes about the pattern: the mix is a bijection of the low index word for a fixed
-    seed (so no value is favoured), the kept fraction is 1 - p, seeds and rows decorrelate, p = 0 keeps all."""
+    """What the mathematics fixes about the pattern: the block mix is a bijection of the low index word for a fixed
+    seed and the finishing rounds are a bijection of the 32-bit words (so no value is favoured), the kept fraction is
+    1 - p, neighbouring entries along rows, columns and diagonals, and neighbouring seeds, are uncorrelated, p = 0
+    keeps all."""
     from oracle import dropout
 
     idx = np.arange(1 << 16, dtype=np.uint64)
     assert len(np.unique(dropout.mix(idx, 99))) == 1 << 16
+    assert len(np.unique(dropout.finish(idx * np.uint64(0x10001)))) == 1 << 16
     for p in (0.1, 0.5, 0.9):
         kp = dropout.keep(2, 3, 64, 128, p, seed=7)
         assert abs(kp.mean() - (1 - p)) < 0.01
         assert abs(kp[0, 0].mean(axis=-1) - (1 - p)).max() < 0.2  # every row has its own draw
     a, b = dropout.keep(1, 1, 64, 64, 0.5, 1), dropout.keep(1, 1, 64, 64, 0.5, 2)
     assert 0.4 < (a != b).mean() < 0.6
-    assert 0.4 < (a[..., 1:, :] != a[..., :-1, :]).mean() < 0.6
+    # a 512 x 512 head at p = 1/2: the correlation of entries (i, j) and (i + di, j + dj) is noise (sigma 0.002);
+    # rows 31 -> 32 cross a block of the pattern, keys step by the other constant
+    k = dropout.keep(1, 2, 512, 512, 0.5, seed=2**40 + 3)[0, 1].astype(np.float64) - 0.5
+    for di, dj in ((0, 1), (1, 0), (1, 1), (1, -1), (0, 2), (2, 0), (32, 0), (0, 32), (3, 5)):
+        x = k[:512 - di, max(0, -dj):512 - max(0, dj)]
+        y = k[di:, max(0, dj):512 - max(0, -dj)]
+        assert abs((x * y).mean() / 0.25) < 0.01, (di, dj)
     hi = dropout.mix(np.array([5, 5 + (1 << 32)], dtype=np.uint64), 3)
-    assert hi[0] != hi[1]  # the high index word takes part
+    assert hi[0] != hi[1]  # the high word of the block index takes part
+    # heads differ although their rows and keys have the same numbers
+    two = dropout.keep(1, 2, 64, 64, 0.5, 11)
+    assert 0.4 < (two[0, 0] != two[0, 1]).mean() < 0.6
     assert dropout.keep(1, 1, 4, 4, 0.0, 5).all() and dropout.keep_scale(1, 1, 4, 4, 0.0, 5) is None
     assert dropout.threshold(0.5) == 1 << 31 and dropout.threshold(1e-12) == 1
