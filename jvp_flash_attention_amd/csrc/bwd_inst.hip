@@ -35,8 +35,7 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
   const long long kv_blocks = (long long)((p.pr.Lk + BWD_BLK - 1) / BWD_BLK) * p.pr.Z * p.pr.Hk;
   if (kv_blocks > 0x7fffffffLL) return -2;
   if (p.pr.drop_thr != 0) {
-    // dropout: the direct-to-LDS kernels carry it for the 16-bit types up to D = 128, the register-staged ones
-    // for fp32 and for D = 256
+    // dropout: the direct-to-LDS kernels carry it for the 16-bit types, the register-staged ones for fp32
     if constexpr (sizeof(T) == 2 && D <= 128) {
       using Cfg2 = Bwd2Cfg<T, D, MODE>;
       const bool no_go = MODE == BWD_DUAL && p.go == nullptr;
@@ -51,6 +50,31 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
       if (rc != 0) return rc;
       hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
       hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
+      return hipGetLastError() == hipSuccess ? 0 : -6;
+    } else if constexpr (sizeof(T) == 2 && D == 256 && MODE == BWD_DUAL) {
+      using CfgP = BwdPairCfg<T, D>;
+      const bool no_go = p.go == nullptr;
+      const long long qblocks = (long long)((p.pr.L + CfgP::BLK - 1) / CfgP::BLK) * p.pr.Z * p.pr.H;
+      const long long kblocks = (long long)((p.pr.Lk + CfgP::BLK - 1) / CfgP::BLK) * p.pr.Z * p.pr.Hk;
+      if (qblocks > 0x7fffffffLL || kblocks > 0x7fffffffLL) return -2;
+      void (*kq)(const BwdParams) = no_go ? bwdp_dq_kernel<T, D, MASK, false, false, true> : bwdp_dq_kernel<T, D, MASK, true, false, true>;
+      void (*kkv)(const BwdParams) = no_go ? bwdp_dkdv_kernel<T, D, MASK, false, true> : bwdp_dkdv_kernel<T, D, MASK, true, true>;
+      int rc = allow_lds(reinterpret_cast<const void *>(kq), CfgP::DQ_LDS);
+      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), CfgP::DKV_LDS);
+      if (rc != 0) return rc;
+      hipLaunchKernelGGL(kkv, dim3((unsigned)kblocks), dim3(CfgP::NT), CfgP::DKV_LDS, stream, p);
+      hipLaunchKernelGGL(kq, dim3((unsigned)qblocks), dim3(CfgP::NT), CfgP::DQ_LDS, stream, p);
+      return hipGetLastError() == hipSuccess ? 0 : -6;
+    } else if constexpr (sizeof(T) == 2 && D == 256) {
+      using CfgW = BwdWideCfg<T, D, MODE>;
+      using CfgK = BwdWideKvCfg<T, D, MODE>;
+      auto kq = bwdw_dq_kernel<T, D, MODE, MASK, true>;
+      auto kkv = bwdw_dkdv_kernel<T, D, MODE, MASK, true>;
+      int rc = allow_lds(reinterpret_cast<const void *>(kq), CfgW::DQ_LDS);
+      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), CfgK::DKV_LDS);
+      if (rc != 0) return rc;
+      hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(CfgK::NT), CfgK::DKV_LDS, stream, p);
+      hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(CfgW::NT), CfgW::DQ_LDS, stream, p);
       return hipGetLastError() == hipSuccess ? 0 : -6;
     } else {
       auto kq = bwd_dq_kernel<T, D, MODE, MASK, true>;

@@ -77,7 +77,8 @@ template <int SLOT, int N> __device__ __forceinline__ f32x16 xch_tile(const u32x
 // dq of the dual mode.  Tile slots of a stage: 0 K, 1 V, 2 K', 3 V'.
 // SIX: dq' = scale dS' K as well, from the K fragments and the dS' tiles that dq already has (a call for all six
 // gradients then needs no second launch that forms S and A again).
-template <typename T, int D, int MASK, bool GO, bool SIX = false>
+// DROP: dropout (see bwd_kernel.hpp): gO V^T, gT V^T and gT V'^T reach the logits through the kept, rescaled entries.
+template <typename T, int D, int MASK, bool GO, bool SIX = false, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {
   using Cfg = BwdPairCfg<T, D>;
   constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT, DV = Cfg::DV;
@@ -171,6 +172,7 @@ __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {
   const float mu = p.mu[srow + qld];
   const float av = p.a[srow + qld];
   const float dsum = p.d2[srow + qld];
+  const uint32_t drop_row = DROP ? drop_row_word(pr, zh, qld) : 0u;  // dropout: this lane's query row, see params.hpp
 
   f32x16 acc[DB], accT[SIX ? DB : 1];
 #pragma unroll
@@ -290,9 +292,15 @@ __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {
         float pv = fast_exp2(s - Mq);
         if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
         if constexpr (EDGE) pv = (key0 + e <= klim) ? pv : 0.f;
-        const float sp = Sp[i] * pr.scale, am = At[i] - av;
+        float dpv = dP[i], atv = At[i];
+        if constexpr (DROP) {
+          const float ks = drop_scale_of(pr, drop_row + (uint32_t)(key0 + e) * DROP_C_KEY);
+          dpv *= ks;
+          atv *= ks;
+        }
+        const float sp = Sp[i] * pr.scale, am = atv - av;
         Sp[i] = pv * am;
-        S[i] = pv * (dP[i] + am * sp - At[i] * mu - dsum);
+        S[i] = pv * (dpv + am * sp - atv * mu - dsum);
       }
     }
     Frag<T> dsf[2], dspf[2];
@@ -401,7 +409,7 @@ __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {
 
 // dk, dv of the dual mode: workgroup = 64 keys of a key/value head (two pairs), loop over 32-query tiles.
 // Tile slots of a stage: 0 Q, 1 gT, 2 Q', 3 gO; statistics slots M, mu, a, d2 (= d1 + d2).
-template <typename T, int D, int MASK, bool GO>
+template <typename T, int D, int MASK, bool GO, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwdp_dkdv_kernel(const BwdParams p) {
   using Cfg = BwdPairCfg<T, D>;
   constexpr int CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW, BT = Cfg::BT;
@@ -423,6 +431,7 @@ __global__ __launch_bounds__(256, 1) void bwdp_dkdv_kernel(const BwdParams p) {
   const int k0 = kb * Cfg::BLK;
   const int krow = k0 + pairi * 32 + r;
   const int kld = krow < Lk ? krow : Lk - 1;
+  const uint32_t drop_lane = DROP ? (uint32_t)kld * DROP_C_KEY + (uint32_t)(8 * g) * DROP_C_ROW : 0u;
   // role 0 writes dV, role 1 dK
   T *out = reinterpret_cast<T *>(role ? p.dk : p.dv) + head + (size_t)krow * D;
   if constexpr (MASK != MASK_NONE) {
@@ -590,6 +599,9 @@ __global__ __launch_bounds__(256, 1) void bwdp_dkdv_kernel(const BwdParams p) {
   };
   auto tile_body = [&](auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn) {
     constexpr bool EDGE = decltype(EDGEc)::value;
+    // dropout: the 32 queries of a tile are one block of the pattern (ih is a multiple of 32), so the block's word
+    // is uniform and register e's query adds a constant to it; this lane's key and row group add drop_lane
+    const uint32_t drop_tile = DROP ? drop_row_word(pr, z * pr.H + h, ih) + drop_lane : 0u;
     // ---- this role's two tiles: X = f1 A, Y = f2 A + f1 B -----------------------------------------
     FragN f1[2], f2[2];
     auto issue_n = [&](auto kkc) {
@@ -668,7 +680,7 @@ __global__ __launch_bounds__(256, 1) void bwdp_dkdv_kernel(const BwdParams p) {
         constexpr int younger = (c4 + 1 < 4) ? 4 : 0;
         lds_wait4<younger>(stq[sl][0], stq[sl][1], stq[sl][2], stq[sl][3]);
         auto stat = [&](int s_, int e) { return __uint_as_float(stq[sl][s_][e % 4]); };
-        float pv4[4], sp4[4];
+        float pv4[4], sp4[4], ks4[4];
 #pragma unroll
         for (int e = 4 * c4; e < 4 * c4 + 4; ++e) {
           const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
@@ -681,19 +693,22 @@ __global__ __launch_bounds__(256, 1) void bwdp_dkdv_kernel(const BwdParams p) {
           if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
           pv4[e % 4] = pv;
           sp4[e % 4] = Sp[e] * pr.scale;
+          ks4[e % 4] = DROP ? drop_scale_of(pr, drop_tile + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_ROW) : 1.f;
         }
         if (role) {  // X = A, Y = dP
 #pragma unroll
           for (int e = 4 * c4; e < 4 * c4 + 4; ++e) {
-            const float pv = pv4[e % 4], m_ = stat(1, e), am = X[e] - stat(2, e);
-            Fa[e - 8 * c] = pv * (Y[e] + am * sp4[e % 4] - X[e] * m_ - stat(3, e));
+            const float at = DROP ? X[e] * ks4[e % 4] : X[e], dp = DROP ? Y[e] * ks4[e % 4] : Y[e];
+            const float pv = pv4[e % 4], m_ = stat(1, e), am = at - stat(2, e);
+            Fa[e - 8 * c] = pv * (dp + am * sp4[e % 4] - at * m_ - stat(3, e));
             Fb[e - 8 * c] = pv * am;
           }
         } else {
 #pragma unroll
           for (int e = 4 * c4; e < 4 * c4 + 4; ++e) {
-            Fa[e - 8 * c] = pv4[e % 4] * (sp4[e % 4] - stat(1, e));
-            Fb[e - 8 * c] = pv4[e % 4];
+            const float pw = DROP ? pv4[e % 4] * ks4[e % 4] : pv4[e % 4];
+            Fa[e - 8 * c] = pw * (sp4[e % 4] - stat(1, e));
+            Fb[e - 8 * c] = pw;
           }
         }
       });
@@ -766,9 +781,9 @@ __global__ __launch_bounds__(256, 1) void bwdp_dkdv_kernel(const BwdParams p) {
   }
 }
 #else
-template <typename T, int D, int MASK, bool GO, bool SIX = false>
+template <typename T, int D, int MASK, bool GO, bool SIX = false, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwdp_dq_kernel(const BwdParams p) {}
-template <typename T, int D, int MASK, bool GO>
+template <typename T, int D, int MASK, bool GO, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwdp_dkdv_kernel(const BwdParams p) {}
 #endif
 

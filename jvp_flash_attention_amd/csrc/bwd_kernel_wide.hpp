@@ -37,7 +37,8 @@ template <typename T, int D, int MODE> struct BwdWideCfg {
 __device__ __forceinline__ int swz_w(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
 #if defined(__HIP_DEVICE_COMPILE__)
-template <typename T, int D, int MODE, int MASK>
+// DROP: dropout (see bwd_kernel.hpp): gO V^T (gT V^T) reaches the logits through the kept, rescaled entries only.
+template <typename T, int D, int MODE, int MASK, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   using Cfg = BwdWideCfg<T, D, MODE>;
   constexpr bool TAN = MODE == BWD_TANGENT;
@@ -118,6 +119,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
 
   const float Mq = qrow < L ? p.M[srow + qld] : __builtin_inff();
   const float sub = TAN ? p.a[srow + qld] : p.d1[srow + qld];  // what the row takes off dP (PLAIN) or A (TANGENT)
+  const uint32_t drop_row = DROP ? drop_row_word(pr, zh, qld) : 0u;  // dropout: this lane's query row, see params.hpp
 
   f32x16 acc[DB];
 #pragma unroll
@@ -217,7 +219,9 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
         float pv = fast_exp2(s - Mq);
         if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
         if constexpr (EDGE) pv = (key0 + e <= klim) ? pv : 0.f;
-        S[i] = pv * (G[i] - sub);
+        float gv = G[i];
+        if constexpr (DROP) gv *= drop_scale_of(pr, drop_row + (uint32_t)(key0 + e) * DROP_C_KEY);
+        S[i] = pv * (gv - sub);
       }
     }
     Frag<T> dsf[2];
@@ -307,7 +311,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {
   }
 }
 #else
-template <typename T, int D, int MODE, int MASK>
+template <typename T, int D, int MODE, int MASK, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwdw_dq_kernel(const BwdParams p) {}
 #endif
 
@@ -322,7 +326,7 @@ template <typename T, int D, int MODE> struct BwdWideKvCfg : BwdWideCfg<T, D, MO
 };
 
 #if defined(__HIP_DEVICE_COMPILE__)
-template <typename T, int D, int MODE, int MASK>
+template <typename T, int D, int MODE, int MASK, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   using Cfg = BwdWideKvCfg<T, D, MODE>;
   constexpr bool TAN = MODE == BWD_TANGENT;
@@ -344,6 +348,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   const int k0 = kb * Cfg::BLK;
   const int krow = k0 + wave * 32 + r;
   const int kld = krow < Lk ? krow : Lk - 1;
+  const uint32_t drop_lane = DROP ? (uint32_t)kld * DROP_C_KEY + (uint32_t)(8 * g) * DROP_C_ROW : 0u;
   T *outk = reinterpret_cast<T *>(TAN ? p.dkt : p.dk) + head + (size_t)krow * D;
   T *outv = reinterpret_cast<T *>(TAN ? p.dvt : p.dv) + head + (size_t)krow * D;
   if constexpr (MASK != MASK_NONE) {
@@ -518,6 +523,9 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   // ih: first query of this tile; ihn: of the tile that follows it
   auto tile_body = [&](auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn) {
     constexpr bool EDGE = decltype(EDGEc)::value;
+    // dropout: the 32 queries of a tile are one block of the pattern (ih is a multiple of 32), so the block's word
+    // is uniform and register e's query adds a constant to it; this lane's key and row group add drop_lane
+    const uint32_t drop_tile = DROP ? drop_row_word(pr, z * pr.H + h, ih) + drop_lane : 0u;
     // ---- recompute: S and dP = gO V^T (PLAIN) or A = gT V^T (TANGENT) -----------------------------
     FragN fq[2], fg[2];
     auto issue_n = [&](auto kkc) {
@@ -591,8 +599,14 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
           float pv = fast_exp2(s - stat(0, e));
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
           if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
-          S[e] = pv;
-          G[e] = pv * (G[e] - stat(1, e));
+          if constexpr (DROP) {
+            const float ks = drop_scale_of(pr, drop_tile + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_ROW);
+            S[e] = pv * ks;
+            G[e] = pv * (G[e] * ks - stat(1, e));
+          } else {
+            S[e] = pv;
+            G[e] = pv * (G[e] - stat(1, e));
+          }
         }
       });
       const Frag<T> pf = to_frag<T>(S, c), dsf = to_frag<T>(G, c);
@@ -663,7 +677,7 @@ __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {
   }
 }
 #else
-template <typename T, int D, int MODE, int MASK>
+template <typename T, int D, int MODE, int MASK, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void bwdw_dkdv_kernel(const BwdParams p) {}
 #endif
 

@@ -58,13 +58,13 @@ static int launch_fwd3_one(const FwdParams &p, hipStream_t stream) {
 }
 
 // D = 256.
-template <typename T, int D, bool DUAL, int MASK>
+template <typename T, int D, bool DUAL, int MASK, bool DROP = false>
 static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
   // Without tangents one workgroup holds all columns.  The dual forward runs that kernel first (O, M)
   // and then the tangent pass (O', mu) with the final M: seven products, where two workgroups with a
   // column half each would compute nine.
   using Cfg = FwdWideCfg<T, D, false>;
-  auto kern = fwd_wide_kernel<T, D, false, MASK>;
+  auto kern = fwd_wide_kernel<T, D, false, MASK, false, DROP>;
   int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
   if (rc != 0) return rc;
   const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
@@ -73,7 +73,7 @@ static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
   if constexpr (DUAL) {
     using CfgT = FwdWideCfg<T, D, true>;
-    auto kt = fwd_wide_kernel<T, D, true, MASK, true>;
+    auto kt = fwd_wide_kernel<T, D, true, MASK, true, DROP>;
     rc = allow_lds(reinterpret_cast<const void *>(kt), CfgT::LDS_BYTES);
     if (rc != 0) return rc;
     hipLaunchKernelGGL(kt, dim3((unsigned)blocks), dim3(CfgT::NT), CfgT::LDS_BYTES, stream, p);
@@ -84,9 +84,14 @@ static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
 template <typename T, int D, int BN, bool DUAL>
 static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
   if (p.pr.drop_thr != 0) {
-    // dropout: the direct-to-LDS kernel carries it for the 16-bit types up to D = 128, the register-staged one
-    // for fp32 and for D = 256
-    if constexpr (sizeof(T) == 2 && D <= 128) {
+    // dropout: the direct-to-LDS kernels carry it for the 16-bit types, the register-staged one for fp32
+    if constexpr (sizeof(T) == 2 && D == 256) {
+      switch (mask) {
+        case MASK_NONE: return launch_fwd_wide_one<T, D, DUAL, MASK_NONE, true>(p, stream);
+        case MASK_BOOL: return launch_fwd_wide_one<T, D, DUAL, MASK_BOOL, true>(p, stream);
+        case MASK_ADD: return launch_fwd_wide_one<T, D, DUAL, MASK_ADD, true>(p, stream);
+      }
+    } else if constexpr (sizeof(T) == 2 && D <= 128) {
       switch (mask) {
         case MASK_NONE: return launch_fwd2_one<T, D, DUAL, MASK_NONE, true>(p, stream);
         case MASK_BOOL: return launch_fwd2_one<T, D, DUAL, MASK_BOOL, true>(p, stream);

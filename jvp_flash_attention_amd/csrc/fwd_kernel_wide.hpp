@@ -42,7 +42,8 @@ template <typename T, int D, bool DUAL> struct FwdWideCfg {
 };
 
 // TPASS (with DUAL): the second pass of the dual forward, see above.
-template <typename T, int D, bool DUAL, int MASK, bool TPASS = false>
+// DROP: dropout on the probabilities (see fwd_kernel.hpp), in both passes.
+template <typename T, int D, bool DUAL, int MASK, bool TPASS = false, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
   static_assert(!TPASS || DUAL);
   using Cfg = FwdWideCfg<T, D, DUAL>;
@@ -151,6 +152,7 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
+  const uint32_t drop_row = DROP ? drop_row_word(pr, zh, qld) : 0u;  // dropout: this lane's query row, see params.hpp
   bool mask_al = false;
   if constexpr (MASK != MASK_NONE) mask_al = mask_rows_aligned<T, MASK>(pr);
 
@@ -340,6 +342,15 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
     }
     l_i += rs;
     if constexpr (DUAL) mu_i += rmu;
+    if constexpr (DROP) {  // register e holds key j0 + 16(e/8) + 8g + e%8 of this lane's query
+      const uint32_t xb = drop_row + (uint32_t)(j0 + 8 * g) * DROP_C_KEY;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float ks = drop_scale_of(pr, xb + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_KEY);
+        S[e] *= ks;
+        if constexpr (DUAL) Sp[e] *= ks;
+      }
+    }
 
     Frag<T> pf[2], psf[2];
 #pragma unroll

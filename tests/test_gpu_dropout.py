@@ -123,6 +123,14 @@ def test_dropout_at_head_dim_256(dt, mode):
     _case(1, 2, 200, 256, DTYPES[dt], mode, p=0.25, seed=31337)
 
 
+def test_dropout_at_head_dim_256_grouped_heads_unequal_lengths_and_longer_rows():
+    """The D = 256 kernels walk the pattern three ways (a lane per query in the forward and dq, a lane per key in
+    dk/dv with the block of 32 queries mixed once per tile, two waves per row in the dual backward)."""
+    _case(2, 4, 100, 256, torch.bfloat16, "none", p=0.1, seed=77, Hk=2, Lk=333)
+    _case(1, 1, 600, 256, torch.float16, "causal", p=0.3, seed=78)
+    _case(1, 2, 130, 256, torch.bfloat16, "keypad", p=0.3, seed=79, plain=True)
+
+
 def test_zero_probability_is_the_path_without_dropout_and_bad_arguments_are_refused():
     from jvp_flash_attention_amd import _lib
 
