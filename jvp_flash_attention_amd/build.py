@@ -76,7 +76,7 @@ def _compile(unit):
 
 def build(jobs: int | None = None, verbose: bool = True, extra_flags=(), lib: str = LIB, objdir: str = OBJ) -> str:
     """Compile and link.  ``extra_flags`` / ``lib`` / ``objdir`` build a variant next to the default
-    library (used to compare kernel tuning constants, e.g. ``-DJVPFA_RING=4``)."""
+    library (e.g. a build with an extra ``-D`` flag, to compare two versions of a kernel on the same box)."""
     os.makedirs(objdir, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
     us = [(*u, objdir, list(extra_flags)) for u in units()]
