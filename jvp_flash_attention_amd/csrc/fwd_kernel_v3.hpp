@@ -28,9 +28,9 @@ template <bool FIRST> __device__ __forceinline__ void mfma_s(f32x16 &c, const f1
   if constexpr (FIRST) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
   else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
 }
-__device__ __forceinline__ void anchor(float &x) { asm volatile("" : "+v"(x)); }
-__device__ __forceinline__ void anchor(bf16x8 &x) { asm volatile("" : "+v"(x)); }
-__device__ __forceinline__ void anchor(f16x8 &x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void anchor(const float &x) { asm volatile("" : : "v"(x)); }
+__device__ __forceinline__ void anchor(const bf16x8 &x) { asm volatile("" : : "v"(x)); }
+__device__ __forceinline__ void anchor(const f16x8 &x) { asm volatile("" : : "v"(x)); }
 
 template <int N>
 __device__ __forceinline__ void lds_wait6(u32x4 &a, u32x4 &b, u32x2 &c, u32x2 &d, u32x2 &e, u32x2 &f) {
@@ -241,7 +241,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     static_assert(!NEXT || (NSS % RD == 0 && QK && PV), "the fragment ring continues into the next slot");
 
     // ---- softmax state and units ----------------------------------------------------------------
-    float mxa = NEG_INF, mxb = NEG_INF, mx = NEG_INF, alpha = 1.f, m_use = 0.f, rs = 0.f, rmu = 0.f;
+    float mxa = NEG_INF, mxb = NEG_INF, mx = NEG_INF, alpha = 1.f, m_use = 0.f, rs = 0.f, rmu = 0.f, xarg = 0.f;
     float pv[16], sv[16];
     bool any_up = false, outweighs = false, up_l = false;
     auto unit = [&](auto uc) {
@@ -279,11 +279,14 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
         anchor(alpha);
       } else if constexpr (u == 4) {
         m_use = (m_i == NEG_INF) ? 0.f : m_i;
+        xarg = GEN ? Sc[0] - m_use : __builtin_fmaf(Sc[0], sl2, -m_use);
       } else if constexpr (u < 37) {
         constexpr int e = (u - 5) / 2;
         if constexpr ((u - 5) % 2 == 0) {
-          if constexpr (GEN) pv[e] = fast_exp2(Sc[e] - m_use);
-          else pv[e] = fast_exp2(__builtin_fmaf(Sc[e], sl2, -m_use));
+          // the exponent of the next element is formed behind this element's exponential, so that a vector
+          // instruction stands between a transcendental and the first reader of its result (in the next gap)
+          pv[e] = fast_exp2(xarg);
+          if constexpr (e + 1 < 16) xarg = GEN ? Sc[e + 1] - m_use : __builtin_fmaf(Sc[e + 1], sl2, -m_use);
           if constexpr (DUAL) sv[e] = __builtin_fmaf(Spc[e], pr.scale, -c_i);
           anchor(pv[e]);
         } else {
