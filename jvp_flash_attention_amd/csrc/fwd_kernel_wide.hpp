@@ -148,7 +148,14 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
     }
   }
   float m_i = NEG_INF, l_i = 0.f, mu_i = 0.f;
+  // Second pass: S' enters T and mu as S' - c, with c the row's weighted mean of S' over the first tile in which the
+  // row has any weight (so tiles skipped because nothing in them is attended do not change it).  O' = T - mu O
+  // subtracts two sums of about |S'| |V| whose first one went through 16-bit P S' operands; measured from c both
+  // are small wherever one tile holds most of the row's weight (a row with a single key: exactly 0).  p is already
+  // normalised by the final M, so c never has to move once it is set.
+  float c_i = 0.f;
   if constexpr (TPASS) m_i = qrow < L ? p.M[(size_t)zh * L + qld] : __builtin_inff();  // +inf: a row without keys
+  bool c_set = !TPASS || !(m_i < __builtin_inff());  // rows without keys never set c and need none
 
   const float sl2 = pr.scale * LOG2E;
   const int64_t mrow = MASK != MASK_NONE ? z * pr.ms[0] + h * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
@@ -331,11 +338,27 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) S[e] = fast_exp2(__builtin_fmaf(S[e], sl2, -m_use));
     }
+    if constexpr (TPASS) {
+      if (__any(!c_set)) {  // the first tile or two (a branch among vector instructions only)
+        float w0 = 0.f, w1 = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          w0 += S[e];
+          w1 = __builtin_fmaf(S[e], Sp[e] * pr.scale, w1);
+        }
+        w0 += xor32(w0);  // the row's other half of the tile
+        w1 += xor32(w1);
+        if (!c_set && w0 > 0.f) {
+          c_i = w1 / w0;
+          c_set = true;
+        }
+      }
+    }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       rs += S[e];
       if constexpr (DUAL) {
-        const float ps = S[e] * (Sp[e] * pr.scale);
+        const float ps = S[e] * __builtin_fmaf(Sp[e], pr.scale, -c_i);
         Sp[e] = ps;
         rmu += ps;
       }
@@ -428,7 +451,8 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
   l_i += xor32(l_i);
   if constexpr (DUAL) mu_i += xor32(mu_i);
   if constexpr (TPASS) {
-    // p was normalised by the final M, so T and mu are final as they stand; O comes from the first pass
+    // p was normalised by the final M, so T and mu (both measured from c) are final as they stand: T - mu O is the
+    // same with or without c, since sum(p) = 1; O comes from the first pass
     if (qrow < L) {
       const T *Og = reinterpret_cast<const T *>(p.o) + head + (size_t)qrow * D;
       T *Otg = reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D;
@@ -444,7 +468,7 @@ __global__ __launch_bounds__(256, 1) void fwd_wide_kernel(const FwdParams p) {
           store8<T>(Otg + d0, t8);
         }
       }
-      if (g == 0) p.mu[(size_t)zh * L + qrow] = mu_i;
+      if (g == 0) p.mu[(size_t)zh * L + qrow] = __builtin_fmaf(c_i, l_i, mu_i);
     }
   } else {
     const bool dead = !(l_i > 0.f);

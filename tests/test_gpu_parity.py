@@ -145,6 +145,40 @@ def test_head_dim_256_tiles_away_from_every_edge():
     _run_case(1, 1, 520, 256, torch.float16, "none", seed=26, plain=True)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+def test_head_dim_256_rows_whose_weight_sits_on_one_key(dt):
+    """A batch entry padded down to a single key next to an ordinary one, 24 queries over 183 keys: every row of
+    the first has all its weight on key 0, so O' = V'[0] and its gradients through the scores are exactly zero, and
+    what the kernels leave there instead is measured against the other entry's gradients (the tensor's maximum).
+    The second forward pass measures S' from the row's mean over its first tile for this: with S' as it stands,
+    T - mu O is the difference of two sums of size |S'| |V|, one of them through 16-bit operands, and dk of the
+    padded entry came out at 3e-2 of the maximum."""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H, L, Lk, D = 2, 2, 24, 183, 256
+    dtype = DTYPES[dt]
+    g = torch.Generator().manual_seed(7098)
+    q, qt, go, gt = (torch.randn(Z, H, L, D, generator=g).to(dtype) for _ in range(4))
+    k, v, kt, vt = (torch.randn(Z, H, Lk, D, generator=g).to(dtype) for _ in range(4))
+    lens = torch.tensor([1, 126])
+    mask = (torch.arange(Lk)[None, :] < lens[:, None]).view(Z, 1, 1, Lk)
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    be, scale = _lib.backend(), D**-0.5
+    print(f"case one key per row {dt} D{D}", flush=True)
+    o, ot, M, mu = be.fwd(*dev[:6], mask.cuda(), _lib.MASK_BOOL, False, scale)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], mask.cuda(), _lib.MASK_BOOL, False, scale, want_tangent_grads=True)
+    ref = dense.forward(*f64[:6], mask=mask.numpy(), causal=False, scale=scale)
+    rb = dense.backward(*f64, mask=mask.numpy(), causal=False, scale=scale)
+    _tol_check("O", o, ref["O"], dtype)
+    _tol_check("O'", ot, ref["Ot"], dtype)
+    # the padded entry alone: O' is V'[0] to the rounding of the element type (no cancellation left)
+    assert (ot[0].float().cpu() - vt[0, :, :1].float()).abs().max().item() <= 2.0**-7 * vt[0, :, :1].float().abs().max().item()
+    assert np.abs(mu.double().cpu().numpy() - ref["mu"]).max() <= 1e-3 * max(1.0, np.abs(ref["mu"]).max())  # (mu = mu_c + c)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
+        _tol_check(n, t, rb[n], dtype)
+
+
 def test_head_dim_256_in_fp32_plain_and_at_a_benchmark_length():
     """fp32 at D = 256 reads its own rows' fragments from global memory instead of keeping them in registers:
     the plain path, and a length with many interior tiles (causal, so that both loops' edges are crossed)."""
