@@ -120,8 +120,8 @@ def hvp_sweep(be, _lib):
 def shape_rows(be, _lib):
     """Shapes next to the headline one, no mask: the other benchmark configurations' shapes, D = 32 and
     D = 256 (the smallest and the largest head dim the reference admits), 16 query heads over 4 key/value heads, and 4096 queries over 512 keys (the last two are
-    shapes the reference refuses), fp32 at D = 256, and the headline shape with dropout.  Dual forward and dual backward, counted as 12 and 24 flops per
-    (query, key, d) triple."""
+    shapes the reference refuses), fp32 at D = 256, and the headline shape with dropout; then benchmark configurations 3 and 4 with their masks
+    (causal; key padding; additive bias).  Dual forward and dual backward, counted as 12 and 24 flops per (query, key, d) triple."""
     import torch
 
     dev = torch.device("cuda:0")
@@ -149,6 +149,31 @@ def shape_rows(be, _lib):
                                        dropout_p=dp, dropout_seed=7), 5, 2)
         n = float(Zs) * Hs * Lq * Lk * Ds
         rows[name] = {"fwd_ms": ms_f, "fwd_tflops": 12 * n / (ms_f * 1e-3) / 1e12,
+                      "bwd_ms": ms_b, "bwd_tflops": 24 * n / (ms_b * 1e-3) / 1e12}
+    # the benchmark configurations that come with a mask, as they are specified: flops counted over the attended
+    # (query, key) pairs only
+    for name, (Zs, Hs, Ls, Ds, dtype, mode) in {
+        "fp16_B2_H32_L4096_D128_config3_causal": (2, 32, 4096, 128, torch.float16, "causal"),
+        "fp32_B4_H8_L1024_D64_config4a_key_padding": (4, 8, 1024, 64, torch.float32, "keypad"),
+        "fp32_B4_H8_L1024_D64_config4b_additive_bias": (4, 8, 1024, 64, torch.float32, "bias"),
+    }.items():
+        g = torch.Generator(device=dev).manual_seed(13)
+        q, k, v, qt, kt, vt, go, gt = [torch.randn(Zs, Hs, Ls, Ds, generator=g, device=dev).to(dtype) for _ in range(8)]
+        mask, kind, causal, frac = None, _lib.MASK_NONE, False, 1.0
+        if mode == "causal":
+            causal, frac = True, (Ls + 1) / (2.0 * Ls)
+        elif mode == "keypad":  # valid length per batch entry uniform in [L/2, L]
+            lens = torch.randint(Ls // 2, Ls + 1, (Zs,), generator=g, device=dev)
+            mask, kind = (torch.arange(Ls, device=dev)[None, :] < lens[:, None]).view(Zs, 1, 1, Ls), _lib.MASK_BOOL
+            frac = lens.float().mean().item() / Ls
+        else:
+            mask, kind = torch.randn(Zs, Hs, Ls, Ls, generator=g, device=dev).to(dtype), _lib.MASK_ADD
+        scale = Ds**-0.5
+        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, mask, kind, causal, scale), 10, 3)
+        o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, mask, kind, causal, scale)
+        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, kind, causal, scale), 5, 2)
+        n = float(Zs) * Hs * Ls * Ls * Ds * frac
+        rows[name] = {"attended_fraction": frac, "fwd_ms": ms_f, "fwd_tflops": 12 * n / (ms_f * 1e-3) / 1e12,
                       "bwd_ms": ms_b, "bwd_tflops": 24 * n / (ms_b * 1e-3) / 1e12}
     return rows
 
