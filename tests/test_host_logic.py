@@ -347,3 +347,15 @@ def test_dropout_draws_one_seed_per_call_and_replays_it_in_the_backward():
         out, ctx = JVPAttn.apply(q, k, v, None, None, None, None, 0.25, False, None, True, True)
         assert ctx.dropout_p == 0.25 and ctx.ENABLE_DROPOUT and ctx.philox_seed == fake.calls[-1][-1]
         assert torch.equal(attention(q, k, v, dropout_p=0.0), attention(q, k, v))
+
+
+def test_bench_measures_one_gpu_and_says_so():
+    """`bench.py --gpus N` with N above 1 exits with a message instead of measuring anything."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr)
