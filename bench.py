@@ -215,8 +215,9 @@ def mask_rows(be, _lib, q, k, v, qt, kt, vt, go, gt, scale):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=40,
+                    help="untimed launches before the timed ones: the clock of the chip settles over the first 30 or so")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--fwd-only", action="store_true", help="time only the headline forward (for profiling)")
     ap.add_argument("--bwd-only", action="store_true",
