@@ -21,6 +21,10 @@ and to copy each result away at once, in front of the wait: the copy holds whate
 
 The sources provide those slots themselves (``s_nop 1`` in front of the matrix instructions whose
 operands live long enough to be parked, ``tiles_ready()`` = ``s_nop 15; s_nop 3`` after each group).
+A result also counts as written once two further 32x32 matrix instructions have been issued behind its
+producer: the matrix pipe takes them one after another, each for its 8 or 16 passes, so the second cannot
+start before the producer has been through (the one-pass backward reads its dq tile that way, with atomic
+adds placed between the matrix instructions of the next phase).
 ``scan()`` checks the ISA text of a translation unit for both; ``build()`` runs it on every kernel unit it
 compiles and fails on a finding.  ``python -m jvp_flash_attention_amd.asm_lint [unit names]`` compiles
 units to ISA text on its own and scans them.
@@ -51,12 +55,12 @@ def _regs(tok: str) -> set[tuple[str, int]]:
 def scan(isa_text: str, where: str = "") -> list[str]:
     """Findings (one line each) in the ISA text of one translation unit."""
     out = []
-    kern, inasm, hist, pending = "?", False, [], set()
+    kern, inasm, hist, pending = "?", False, [], {}  # pending: register -> matrix instructions issued since
     flying: list[set] = []  # destinations of the inline-asm LDS reads in flight, oldest first
     for ln in isa_text.splitlines():
         t = ln.strip()
         if t.startswith("_Z") and ":" in t and "$" not in t.split(":")[0]:
-            kern, hist, pending, flying = t.split(":")[0], [], set(), []
+            kern, hist, pending, flying = t.split(":")[0], [], {}, []
             continue
         if "ASMSTART" in t:
             inasm = True
@@ -72,7 +76,7 @@ def scan(isa_text: str, where: str = "") -> list[str]:
         op = t.split()[0]
         ops = [x.strip() for x in t.split(None, 1)[1].split(",")] if " " in t else []
         if op == "s_nop" and ops and int(ops[0]) >= 15:
-            pending = set()  # tiles_ready(): results of the group are readable from here on
+            pending = {}  # tiles_ready(): results of the group are readable from here on
         if op.startswith("ds_read") and inasm:
             flying.append(_regs(ops[0]))
             hist.append((op, ops))
@@ -92,20 +96,24 @@ def scan(isa_text: str, where: str = "") -> list[str]:
             dst, srcs = _regs(ops[0]), set()
             for o in ops[1:4]:
                 srcs |= _regs(o)
+            if op.startswith("v_mfma_f32_32x32"):  # two younger ones: the producer has written its result
+                pending = {r: n + 1 for r, n in pending.items() if n + 1 < 2}
             if inasm:
                 guarded = bool(hist) and hist[-1][0] == "s_nop"
                 if not guarded:
                     for pop, pops in hist[-2:]:
                         if pop.startswith("v_") and not pop.startswith("v_mfma") and pops and (_regs(pops[0]) & srcs):
                             out.append(f"{where} {kern}: '{pop} {pops[0]}' feeds '{t[:60]}' without idle slots")
-                pending |= dst  # vector registers, and accumulation registers (read back by v_accvgpr_read)
+                for r in dst:  # vector registers, and accumulation registers (read back by v_accvgpr_read)
+                    pending[r] = 0
             else:
-                pending -= dst
-        elif pending and op.startswith(("v_", "ds_write", "global_store", "buffer_store", "scratch_store")):
+                for r in dst:
+                    pending.pop(r, None)
+        elif pending and op.startswith(("v_", "ds_write", "global_store", "buffer_store", "scratch_store", "global_atomic")):
             srcs = set()
             for o in (ops[1:] if op.startswith("v_") else ops):
                 srcs |= _regs(o)
-            if srcs & pending:
+            if srcs & pending.keys():
                 out.append(f"{where} {kern}: '{t[:60]}' reads a matrix result before the wait that follows its group")
         hist.append((op, ops))
     return out

@@ -9,6 +9,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "common.hpp"
 #include "params.hpp"
 
@@ -33,17 +35,19 @@ inline SplitPlan split_plan(long long blocks, int ntiles_max, int cus) {
   return s;
 }
 
-// Compute units of the current device (0 if it cannot be asked), looked up once per device.
+// Compute units of the current device (0 if it cannot be asked), looked up once per device.  Callable from any
+// thread: the cache is atomic, and two threads that both find it empty store the same value.
 inline int device_cus() {
-  static int cached[64] = {0};
+  static std::atomic<int> cached[64];
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-  if (cached[dev] == 0) {
-    int n = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
-    cached[dev] = n > 0 ? n : -1;
+    n = n > 0 ? n : -1;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached[dev] > 0 ? cached[dev] : 0;
+  return n > 0 ? n : 0;
 }
 
 // Workspace of the forward: per chunk and query row 2 D accumulator values (O, T, not yet divided by l) and
