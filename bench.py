@@ -225,8 +225,6 @@ def main():
     ap.add_argument("--plain-only", action="store_true",
                     help="time the headline shape without tangents (what attention() runs in first-order training): forward, "
                          "then the backward of gO (for profiling); prints its own line")
-    ap.add_argument("--one-pass", action="store_true",
-                    help="with --plain-only: the backward in one pass (dq added up with fp32 atomic adds by the dk/dv workgroups)")
     ap.add_argument("--bwd6-only", action="store_true",
                     help="run one forward, then time the backward that also returns dq', dk', dv' (for profiling)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -270,7 +268,6 @@ def main():
                           "tflops_algorithmic": bwd_flops / (ms_b * 1e-3) / 1e12}), flush=True)
         return
     if args.plain_only:
-        _lib.set_one_pass_backward(args.one_pass)
         ms_pf, _ = timed(lambda: be.fwd(q, k, v, None, None, None, None, _lib.MASK_NONE, False, scale), args.steps, args.warmup)
         o, _, M, _ = be.fwd(q, k, v, None, None, None, None, _lib.MASK_NONE, False, scale)
         ms_pb, _ = timed(lambda: be.bwd(q, k, v, None, None, None, o, None, M, None, go, None, None, _lib.MASK_NONE, False, scale),

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define JVPFA_ABI_VERSION 8
+#define JVPFA_ABI_VERSION 7
 
 enum jvpfa_dtype { JVPFA_BF16 = 0, JVPFA_FP16 = 1, JVPFA_FP32 = 2 };
 
@@ -148,25 +148,11 @@ typedef struct jvpfa_bwd_args {
   const int32_t *tiles_k;   /* the other list of jvpfa_mask_tiles() (dk/dv kernels);
                                tiles_q and tiles_k are both NULL or both set */
   int32_t Lk, Hk;           /* as in jvpfa_fwd_args; dk, dv, dkt, dvt have the shape of k */
-  /* optional opt-in to the one-pass first-order backward, or NULL: jvpfa_bwd_dq_accum_bytes(&p, Lk, Hk) bytes of
-   * device memory, 16-byte aligned, contents don't-care.  With it a call without tangents (gt == NULL; bf16 / fp16,
-   * D 64 or 128, no dropout, k and v with q's head count, a grid that fills the GPU) forms the score gradients
-   * once: the dk/dv workgroups also add their key block's share of dq into this fp32 buffer with atomic adds and
-   * a small kernel converts it, instead of a second kernel that recomputes S and dP for dq as the reference's two
-   * loops do (JA:1415-1563, JA:1567-1707, both run by JA:2008-2233).  The atomic adds land in an order that
-   * differs from run to run, so dq then agrees with the default path to rounding but is not bitwise
-   * reproducible; dk and dv are.  Ignored (the default two kernels run) when the call is not eligible. */
-  void *dq_accum;
-  uint64_t dq_accum_bytes;
 } jvpfa_bwd_args;
 
 int jvpfa_bwd(const jvpfa_bwd_args *args, void *hip_stream);
 
 size_t jvpfa_bwd_workspace_bytes(int32_t Z, int32_t H, int32_t L);
-
-/* Bytes of dq_accum with which a jvpfa_bwd call without tangents would run as one pass on the current device; 0
- * if it would not (element type, head dim, dropout, grouped heads, or a grid smaller than the GPU). */
-size_t jvpfa_bwd_dq_accum_bytes(const jvpfa_problem *p, int32_t Lk, int32_t Hk);
 
 /*
  * jvpfa_bwd for callers that cannot hand over a workspace because they cannot allocate one: code

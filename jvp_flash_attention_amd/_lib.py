@@ -15,10 +15,10 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libjvpfa.so")
 
-ABI_VERSION = 8
+ABI_VERSION = 7
 DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
-EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_bwd_dq_accum_bytes", "jvpfa_fwd_split_workspace_bytes", "jvpfa_dropout_keep", "jvpfa_bwd_workspace_bytes", "jvpfa_bwd_static", "jvpfa_bwd_static_max_rows", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
+EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_fwd_split_workspace_bytes", "jvpfa_dropout_keep", "jvpfa_bwd_workspace_bytes", "jvpfa_bwd_static", "jvpfa_bwd_static_max_rows", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
            "jvpfa_abi_version", "jvpfa_error_string")
 
 
@@ -64,7 +64,6 @@ class BwdArgs(C.Structure):
         ("key_limit", C.c_void_p),
         ("tiles_q", C.c_void_p), ("tiles_k", C.c_void_p),
         ("Lk", C.c_int32), ("Hk", C.c_int32),
-        ("dq_accum", C.c_void_p), ("dq_accum_bytes", C.c_uint64),
     ]
 
 
@@ -87,8 +86,6 @@ def load() -> C.CDLL:
         lib.jvpfa_bwd.restype = C.c_int
         lib.jvpfa_bwd_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         lib.jvpfa_bwd_workspace_bytes.restype = C.c_size_t
-        lib.jvpfa_bwd_dq_accum_bytes.argtypes = [C.POINTER(Problem), C.c_int32, C.c_int32]
-        lib.jvpfa_bwd_dq_accum_bytes.restype = C.c_size_t
         lib.jvpfa_bwd_static.argtypes = [C.POINTER(BwdArgs), C.c_void_p]
         lib.jvpfa_bwd_static.restype = C.c_int
         lib.jvpfa_bwd_static_max_rows.argtypes = []
@@ -200,19 +197,6 @@ def set_split(enabled: bool) -> None:
     partial results, see ``split_workspace`` in ``include/jvpfa.h``."""
     global _split_enabled
     _split_enabled = bool(enabled)
-
-
-_one_pass_backward = False
-
-
-def set_one_pass_backward(enabled: bool) -> None:
-    """Opt in to (or out of) the one-pass first-order backward (default off).  With it a backward without tangents
-    whose problem the library takes (bf16 / fp16, head dim 64 or 128, no dropout, k and v with q's head count, a
-    grid that fills the GPU) forms the score gradients once and adds dq up in an fp32 buffer with atomic adds,
-    see ``dq_accum`` in ``include/jvpfa.h``: faster, and dq is then no longer bitwise reproducible from run to
-    run (dk, dv are)."""
-    global _one_pass_backward
-    _one_pass_backward = bool(enabled)
 
 
 TILE_LISTS_MIN_L = 512  # below this a mask has too few tiles for skipping some to pay for the scan
@@ -389,11 +373,6 @@ class HipBackend:
             a.key_limit = _ptr(lim)
             tq, tk = tile_lists(q, mask, mask_kind, True, k.shape[2])
             a.tiles_q, a.tiles_k = _ptr(tq), _ptr(tk)
-            if _one_pass_backward and gt is None:
-                nacc = lib.jvpfa_bwd_dq_accum_bytes(C.byref(a.p), a.Lk, a.Hk)
-                if nacc:
-                    acc = torch.empty(nacc, device=q.device, dtype=torch.uint8)
-                    a.dq_accum, a.dq_accum_bytes = acc.data_ptr(), nacc
             check(lib.jvpfa_bwd(C.byref(a), _stream(q)))
         return dq, dk, dv, dqt, dkt, dvt
 

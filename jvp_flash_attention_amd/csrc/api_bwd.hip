@@ -7,7 +7,6 @@
 #include <mutex>
 
 #include "api_common.hpp"
-#include "split.hpp"
 
 namespace jvpfa {
 #define JVPFA_DECL(name) int name(const BwdParams &, int, bool, bool, hipStream_t);
@@ -30,23 +29,6 @@ extern "C" size_t jvpfa_bwd_workspace_bytes(int32_t Z, int32_t H, int32_t L) {
   return 3 * stat_floats(Z, H, L) * sizeof(float);
 }
 
-// The one-pass first-order backward: which problems it takes, and the size of its fp32 copy of dq (rows padded
-// to whole 64-row tiles per head).
-static size_t dq_accum_bytes(const jvpfa_problem &p, int32_t Lk, int32_t Hk) {
-  if (p.dtype == JVPFA_FP32 || (p.D != 64 && p.D != 128) || p.dropout_p > 0.f) return 0;
-  if (Hk > 0 && Hk != p.H) return 0;
-  // smaller grids run the dk/dv and dq workgroups side by side in one launch, which the one pass would halve
-  const long long kv_blocks = (long long)(((Lk > 0 ? Lk : p.L) + 127) / 128) * p.Z * p.H;
-  const int cus = device_cus();
-  if (cus <= 0 || kv_blocks < cus) return 0;
-  return (size_t)p.Z * p.H * (size_t)((p.L + 63) / 64 * 64) * p.D * sizeof(float);
-}
-
-extern "C" size_t jvpfa_bwd_dq_accum_bytes(const jvpfa_problem *p, int32_t Lk, int32_t Hk) {
-  if (!p || check_problem(*p) != JVPFA_OK || check_kv_shape(*p, Lk, Hk) != JVPFA_OK) return 0;
-  return dq_accum_bytes(*p, Lk, Hk);
-}
-
 // Everything jvpfa_bwd does, with the row statistics of the pre-pass in `workspace`.
 static int bwd_impl(const jvpfa_bwd_args *a, void *workspace, void *hip_stream) {
   if (!a) return JVPFA_E_NULL;
@@ -66,7 +48,7 @@ static int bwd_impl(const jvpfa_bwd_args *a, void *workspace, void *hip_stream) 
   const int ntg = (a->dqt != nullptr) + (a->dkt != nullptr) + (a->dvt != nullptr);
   if (ntg != 0 && (ntg != 3 || !dual)) return JVPFA_E_NULL;
   const void *ptrs[] = {a->q,  a->k,  a->v,  a->qt, a->kt, a->vt,  a->o,   a->ot,  a->go,
-                        a->gt, a->dq, a->dk, a->dv, a->dqt, a->dkt, a->dvt, workspace, a->dq_accum};
+                        a->gt, a->dq, a->dk, a->dv, a->dqt, a->dkt, a->dvt, workspace};
   for (const void *ptr : ptrs)
     if (ptr && !aligned16(ptr)) return JVPFA_E_ALIGN;
 
@@ -82,11 +64,6 @@ static int bwd_impl(const jvpfa_bwd_args *a, void *workspace, void *hip_stream) 
   p.d1 = static_cast<float *>(workspace);
   p.a = p.d1 + n;
   p.d2 = p.a + n;
-  p.dq_acc = nullptr;
-  if (a->dq_accum && !dual) {
-    const size_t need = dq_accum_bytes(a->p, a->Lk, a->Hk);
-    if (need != 0 && a->dq_accum_bytes >= need) p.dq_acc = static_cast<float *>(a->dq_accum);
-  }
   return kBwd[slot(a->p)](p, a->p.mask_kind, dual, ntg == 3, static_cast<hipStream_t>(hip_stream));
 }
 

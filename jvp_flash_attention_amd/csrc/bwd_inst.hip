@@ -90,21 +90,6 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
   if constexpr (sizeof(T) == 2 && D <= 128) {  // direct-to-LDS, double-buffered kernels
    {
     using Cfg2 = Bwd2Cfg<T, D, MODE>;
-    if constexpr (MODE == BWD_PLAIN && (D == 64 || D == 128)) {
-      // one pass: the dk/dv workgroups also add their share of dq to the caller's fp32 buffer (the API layer sets
-      // dq_acc only for the problems this takes); then scale and convert
-      if (p.dq_acc) {
-        auto k1 = bwd1_kernel<T, D, MASK>;
-        int rc1 = allow_lds(reinterpret_cast<const void *>(k1), Cfg2::DKV1_LDS);
-        if (rc1 != 0) return rc1;
-        hipLaunchKernelGGL(k1, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), Cfg2::DKV1_LDS, stream, p);
-        const long long rows = (long long)p.pr.Z * p.pr.H * p.pr.L;
-        constexpr int RPB = 256 / (D / 8);
-        hipLaunchKernelGGL((bwd_dq_convert_kernel<T, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream,
-                           p.dq_acc, reinterpret_cast<T *>(p.dq), rows, p.pr.L, (p.pr.L + 63) / 64 * 64, p.pr.scale);
-        return hipGetLastError() == hipSuccess ? 0 : -6;
-      }
-    }
     // gO may be absent only in the dual mode (loss depends on O' alone)
     const bool no_go = MODE == BWD_DUAL && p.go == nullptr;
     constexpr bool NG = MODE != BWD_DUAL;  // the GO template argument of the kernels without gO

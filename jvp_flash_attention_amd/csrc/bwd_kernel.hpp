@@ -54,13 +54,6 @@ __global__ __launch_bounds__(256) void bwd_prepass_kernel(const BwdParams p, lon
     sa += __shfl_xor(sa, w, 64);
     s2 += __shfl_xor(s2, w, 64);
   }
-  if (p.dq_acc && row < rows) {  // the one-pass backward adds to an fp32 dq that starts at zero
-    const int L = p.pr.L, Lpad = (L + 63) / 64 * 64;
-    float *z = p.dq_acc + ((size_t)(row / L) * Lpad + (size_t)(row % L)) * D + part * 8;
-    const f32x4 z4 = {0.f, 0.f, 0.f, 0.f};
-    *reinterpret_cast<f32x4 *>(z) = z4;
-    *reinterpret_cast<f32x4 *>(z + 4) = z4;
-  }
   if (row < rows && part == 0) {
     p.d1[row] = s1;
     if (dual) {

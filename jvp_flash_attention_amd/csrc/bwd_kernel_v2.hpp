@@ -31,10 +31,6 @@ template <typename T, int D, int MODE> struct Bwd2Cfg {
   static constexpr int STATB = NSTAT * BT * 4;        // row statistics of a query tile (dk/dv only)
   static constexpr size_t DQ_LDS = 2 * (size_t)STAGEB;
   static constexpr size_t DKV_LDS = 2 * (size_t)STAGEB + 2 * (size_t)STATB;
-  // one-pass backward: the score gradients of a tile (128 keys x 64 queries, 16-bit) change hands through LDS,
-  // two buffers
-  static constexpr int XCHB = BLK * BT * 2;
-  static constexpr size_t DKV1_LDS = DKV_LDS + 2 * (size_t)XCHB;
 };
 
 // One LDS fragment (8 elements per lane) read ahead with lds_b128 / two lds_tr64.
@@ -479,20 +475,11 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(160))) void 
 // one keeps its pointers loop-invariant).
 // SIX (dual mode only): dk' = scale dS'^T Q and dv' = P^T gT as well, from the fragments and tiles that dk, dv
 // already have (two more accumulators: fits for D <= 64).
-// ONEPASS (plain mode, D = 64 or 128): dq as well, so that no second kernel forms S and dP again.  The workgroup
-// holds dS of a 64-query tile for its 128 keys, which is this key block's whole contribution dS K to those 64
-// rows of dq.  Each wave leaves its 32 keys of dS in LDS (16-bit, [key][query]); one tile later (behind the next
-// barrier, so no barrier of its own) every wave reads all 128 keys of it with transposing reads, multiplies by
-// the 32 columns of K it keeps resident as a B operand and adds the 32-column slab of the 64 x D result to an
-// fp32 copy of dq in global memory with atomic adds (p.dq_acc, rows padded to whole tiles per head, zeroed by
-// the pre-pass; bwd_dq_convert_kernel scales and converts it).  The sums arrive in an order that differs from
-// run to run, so dq is not bitwise reproducible; dk and dv are.
-template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED, bool SIX, bool DROP = false, bool ONEPASS = false>
+template <typename T, int D, int MODE, int MASK, bool GO, bool GROUPED, bool SIX, bool DROP = false>
 __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
   static_assert(!SIX || (DUAL && D <= 64), "dk', dv' ride on the dual mode, where the accumulators fit");
-  static_assert(!ONEPASS || (MODE == BWD_PLAIN && !GROUPED && (D == 64 || D == 128)), "one pass: plain mode, one head");
   JVPFA_BWD2_COMMON(Cfg, pr.L, pr.Lk, pr.Hk)  // owns key rows (h: key/value head), streams query tiles
   const int kb = id % nblk;  // causal: the first key blocks have the longest query loops
   const int k0 = kb * Cfg::BLK;
@@ -538,60 +525,6 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     if constexpr (DUAL) {
       pin_acc(Ktf[kk]);  // V' stays in vector registers: the accumulation file also holds dK, dV
     }
-  }
-  // one pass: wave -> (32 columns of dq, 32-query blocks of the tile): D = 128 four column blocks x both query
-  // blocks, D = 64 two column blocks x one query block
-  constexpr int NKS = Cfg::BLK / 16;                  // contraction steps over the workgroup's keys
-  constexpr int QPW = ONEPASS ? DB / 2 : 1;           // query blocks per wave
-  const int dbw = wave % DB, qb0 = (wave / DB) * QPW;
-  Frag<T> Kq[ONEPASS ? NKS : 1];
-  uint32_t xw[2] = {0, 0}, xr[QPW][2];
-  const uint32_t xch0 = stat0 + 2 * Cfg::STATB;  // two buffers of 128 keys x 64 queries, rows of 128 bytes
-  float *dq_head = nullptr;
-  uint32_t dq_lane = 0;
-  if constexpr (ONEPASS) {
-    // B operand of dQ += dS K: lane (r, g) holds K[k0 + 16 ks + 8 g + i][32 dbw + r], i = 0..7.  Keys past the
-    // end count as rows of zeros: the lanes that own them recompute the last key's scores (their dk, dv are
-    // not stored), which must not reach dq.
-    const T *Kh = reinterpret_cast<const T *>(p.k) + head + 32 * dbw + r;
-#pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int key = k0 + 16 * ks + 8 * g + i;
-        const T x = Kh[(size_t)min(key, Lk - 1) * D];
-        Kq[ks][i] = key < Lk ? x : (T)0.f;
-      }
-    }
-#pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) pin_acc(Kq[ks]);
-    // exchange rows are keys; the 16-byte chunk (8 queries) index is XORed with swz_v<8>(row) (0 or 4), which
-    // keeps the transposing reads of four consecutive rows off each other's banks
-    {
-      const int row = wave * 32 + r, sw = swz_v<8>(row);
-      // writer: chunk 4 HB + 2 c + g of this lane's key row; HB picks xw[HB], c is an immediate offset
-#pragma unroll
-      for (int hb = 0; hb < 2; ++hb) xw[hb] = row * 128 + (((4 * hb + g) ^ sw) * 16);
-      // reader (see toff above): rows 8 g + 4 hh + j/4 of a 16-key step, chunk 4 qb + 2 a + j % 2
-      const int a_ = (lane >> 4) & 1, j_ = lane & 15;
-#pragma unroll
-      for (int u = 0; u < QPW; ++u) {
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-          const int rw = 8 * g + 4 * hh + (j_ >> 2);
-          xr[u][hh] = rw * 128 + (((4 * (qb0 + u) + 2 * a_ + (j_ & 1)) ^ swz_v<8>(rw)) * 16) + 8 * ((j_ >> 1) & 1);
-        }
-      }
-    }
-    // fp32 dq: rows padded to whole tiles per head; this lane adds to column 32 dbw + r of rows 8 g + ...
-    const size_t Lpad = (size_t)((L + BT - 1) / BT) * BT;
-    dq_head = p.dq_acc + (size_t)zh * Lpad * D;
-    dq_lane = (uint32_t)((32 * qb0 + 8 * g) * D + 32 * dbw + r);
-    // the first tile's dq step finds a buffer of zeros
-    const u32x4 z4 = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int i = 0; i < Cfg::XCHB / 16 / Cfg::NT; ++i)
-      *(JVPFA_LDS(u32x4))(uintptr_t)(xch0 + Cfg::XCHB + (i * Cfg::NT + tid) * 16) = z4;
   }
 
   f32x16 dK[DB], dV[DB], dKt[SIX ? DB : 1], dVt[SIX ? DB : 1];
@@ -723,19 +656,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     }
   };
   // ih: first query of this half tile; ihn: of the half tile that follows it
-  // one pass: xwbuf is the exchange buffer this tile's dS goes to; dqa holds the dq contribution of the tile
-  // before, whose atomic adds (to the rows at dq_dst) are issued a few at a time between the matrix
-  // instructions of the first half tile
-  constexpr int NATOM = ONEPASS ? 16 * QPW : 0, APS = NATOM / KK;
-  auto dq_add = [&](auto ac, const f32x16 (&dqa)[QPW], const float *const (&dq_dst)[2 * QPW]) {
-    constexpr int a = decltype(ac)::value, u = a / 16, e = a % 16;
-    const uint32_t off = dq_lane * 4u;
-    const float x = dqa[u][e];
-    const float *base = dq_dst[2 * u + e / 8];
-    asm volatile("global_atomic_add_f32 %0, %1, %2 offset:%3" : : "v"(off), "v"(x), "s"(base), "n"((e % 8) * D * 4));
-  };
-  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn, uint32_t xwbuf,
-                       const f32x16 (&dqa)[QPW], const float *const (&dq_dst)[2 * QPW]) {
+  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn) {
     constexpr int HB = decltype(HBc)::value;
     // dropout: the 32 queries of a half tile are one block of the pattern (ih is a multiple of 32), so the block's
     // word is uniform and register e's query adds a constant to it; this lane's key and row group add drop_lane
@@ -786,9 +707,6 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
       const Frag<T> q_ = as_frag<T>(fq[sl]), g_ = as_frag<T>(fg[sl]);
       mma_vra<F>(S, q_, Kf[kk]);
       if constexpr (MODE == BWD_PLAIN) mma_vra<F>(dP, g_, Vf[kk]);
-      // (behind two younger matrix instructions the dq tile, produced before them, has been written)
-      if constexpr (ONEPASS && HB == 0)
-        static_for<APS>([&](auto ic) { dq_add(std::integral_constant<int, kk * APS + decltype(ic)::value>{}, dqa, dq_dst); });
       if constexpr (TAN) mma_vra<F>(At, g_, Vf[kk]);
       if constexpr (DUAL) {
         const Frag<T> gt_ = as_frag<T>(fgt[sl]);
@@ -891,8 +809,6 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
       const Frag<T> pf = to_frag<T>(S, c);
       Frag<T> dsf, dspf, ppf;
       if constexpr (!TAN) dsf = to_frag<T>(dP, c);
-      if constexpr (ONEPASS)  // this lane's key, queries 32 HB + 16 c + 8 g .. + 7
-        asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(xwbuf + xw[HB]), "v"(__builtin_bit_cast(u32x4, dsf)), "n"(c * 32));
       if constexpr (DUAL || TAN) dspf = to_frag<T>(Sp, c);
       if constexpr (DUAL) {
 #pragma unroll
@@ -928,39 +844,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     });
   };
 
-  // one pass: dqa = dS K of the tile whose dS sits in exchange buffer xrbuf (this wave's columns and query blocks,
-  // all 128 keys); fragments are read one step ahead
-  auto dq_products = [&](f32x16 (&dqa)[QPW], uint32_t xrbuf) {
-   if constexpr (ONEPASS) {
-    FragT fa[2][QPW];
-    auto issue_x = [&](auto ksc) {
-      constexpr int ks = decltype(ksc)::value, sl = ks % 2;
-#pragma unroll
-      for (int u = 0; u < QPW; ++u) {
-        fa[sl][u].lo = lds_tr64<ks * 16 * 128>(xrbuf + xr[u][0]);
-        fa[sl][u].hi = lds_tr64<ks * 16 * 128>(xrbuf + xr[u][1]);
-      }
-    };
-    issue_x(std::integral_constant<int, 0>{});
-    static_for<NKS>([&](auto ksc) {
-      constexpr int ks = decltype(ksc)::value, sl = ks % 2;
-      if constexpr (ks + 1 < NKS) issue_x(std::integral_constant<int, ks + 1>{});
-      constexpr int younger = (ks + 1 < NKS) ? 2 * QPW : 0;
-      if constexpr (QPW == 2) lds_wait<younger>(fa[sl][0], fa[sl][1]);
-      else lds_wait<younger>(fa[sl][0].lo, fa[sl][0].hi);
-#pragma unroll
-      for (int u = 0; u < QPW; ++u) mma_vra<ks == 0>(dqa[u], as_frag<T>(fa[sl][u]), Kq[ks]);
-    });
-   }
-  };
-  // rows of the fp32 dq that a tile's atomic adds go to, one pointer per run of 8 rows x 16 that shares an
-  // immediate offset range
-  auto dq_rows = [&](const float *(&dst)[2 * QPW], int i0) {
-#pragma unroll
-    for (int j = 0; j < 2 * QPW; ++j) dst[j] = dq_head + (size_t)(i0 + 16 * j) * D;
-  };
   int tcur = 0, tnext = 0;  // the tile of this step and of the next
-  int iprev = 0;            // one pass: first query of the tile before (its dq is added during this one)
   auto tile = [&](int t, auto EDGEc) {
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -971,20 +855,10 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     prepare_loads(stage ^ 1, i0n, t + 1 < ntiles);
     load_stats();
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB, sstat = stat0 + stage * Cfg::STATB;
-    const uint32_t xwbuf = xch0 + stage * Cfg::XCHB;
-    f32x16 dqa[QPW];
-    const float *dq_dst[2 * QPW];
-    if constexpr (ONEPASS) {
-      // the tile before left its dS in the other buffer (the first tile finds zeros there and adds them to its
-      // own rows)
-      dq_products(dqa, xch0 + (stage ^ 1) * Cfg::XCHB);
-      dq_rows(dq_dst, t > 0 ? iprev : i0);
-      iprev = i0;
-    }
-    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, sstat, i0, i0 + 32, xwbuf, dqa, dq_dst);
+    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, sstat, i0, i0 + 32);
     // always both halves: a half past the last query contributes exact zeros, and a branch here would
     // make the accumulators change register file around it
-    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32, i0n, xwbuf, dqa, dq_dst);
+    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32, i0n);
     if constexpr (MASK != MASK_NONE) {
       const int listed = list_take(tahead);
       tnext2 = tlist ? min(max(listed, 0), tmax) : tnext2;
@@ -1013,18 +887,6 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     for (; t < ntiles && tcur < t_end; ++t) tile(t, std::false_type{});
     for (; t < ntiles; ++t) tile(t, std::true_type{});
     __builtin_amdgcn_s_waitcnt(0x0F70);
-    if constexpr (ONEPASS) {
-      if (t > 0) {  // the last tile's dq
-        __syncthreads();
-        f32x16 dqa[QPW];
-        const float *dq_dst[2 * QPW];
-        dq_products(dqa, xch0 + ((t + 1) & 1) * Cfg::XCHB);
-        dq_rows(dq_dst, iprev);
-        if constexpr (QPW == 2) tiles_ready(dqa[0], dqa[1]);
-        else tiles_ready(dqa[0]);
-        static_for<NATOM>([&](auto ac) { dq_add(ac, dqa, dq_dst); });
-      }
-    }
   }
 
   if (krow < Lk) {
@@ -1062,27 +924,6 @@ __global__ __launch_bounds__(256, 1) void bwd2_dkdv_kernel(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   bwd2_dkdv_body<T, D, MODE, MASK, GO, GROUPED, SIX, DROP>(p, blockIdx.x);
 #endif
-}
-// dk, dv and dq in one pass (plain mode): see ONEPASS above
-template <typename T, int D, int MASK>
-__global__ __launch_bounds__(256, 1) void bwd1_kernel(const BwdParams p) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  bwd2_dkdv_body<T, D, BWD_PLAIN, MASK, true, false, false, false, true>(p, blockIdx.x);
-#endif
-}
-// fp32 dq of the one-pass kernel -> dq: scale, convert; one thread per 8 columns.  acc rows are padded to
-// whole 64-row tiles per head (Lpad rows).
-template <typename T, int D>
-__global__ __launch_bounds__(256) void bwd_dq_convert_kernel(const float *acc, T *dq, long long rows, int L, int Lpad, float scale) {
-  constexpr int LPR = D / 8;
-  const long long row = (long long)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
-  if (row >= rows) return;
-  const int d0 = (threadIdx.x % LPR) * 8;
-  const long long zh = row / L, i = row % L;
-  const float *src = acc + ((size_t)zh * Lpad + i) * D + d0;
-  const f32x4 a = *reinterpret_cast<const f32x4 *>(src), b = *reinterpret_cast<const f32x4 *>(src + 4);
-  float x[8] = {a[0] * scale, a[1] * scale, a[2] * scale, a[3] * scale, b[0] * scale, b[1] * scale, b[2] * scale, b[3] * scale};
-  store8<T>(dq + (size_t)row * D + d0, x);
 }
 // The same code with the vector registers capped, for D = 64: together with the accumulation registers
 // the kernel then needs at most 256 registers and two workgroups share a compute unit.

@@ -98,10 +98,6 @@ struct BwdParams {
   const void *go, *gt;
   void *dq, *dk, *dv, *dqt, *dkt, *dvt;
   float *d1, *a, *d2;  // row statistics produced by the pre-pass, each (Z, H, L)
-  // One-pass first-order backward (null: dq has a kernel of its own): fp32 copy of dq that the dk/dv workgroups
-  // add their share to with atomic adds, (Z, H, L rounded up to whole 64-row tiles, D); the pre-pass clears
-  // rows 0 .. L-1 of every head and the padding rows are never read.
-  float *dq_acc;
 };
 
 // What a backward launch computes.
