@@ -19,6 +19,17 @@ and to copy each result away at once, in front of the wait: the copy holds whate
 
 3. No instruction may read a register while an inline-asm LDS read into it is still in flight.
 
+The forward kernels rescale and re-centre their accumulators in place with an asm statement that names the
+accumulator elements as inputs and writes them all the same (``acc_move_in_place``: as in/out operands the
+compiler gives the tiles a second home behind the rarely taken block and copies them there on every half
+tile).  That is sound only while the registers the statement is handed are the very ones the in-place matrix
+instructions (``mfma_acc``) accumulate into:
+
+4. In a kernel that contains such a statement (an asm block with two ``v_accvgpr_write_b32``), the registers those
+   blocks write must be exactly the destinations of the kernel's in-place inline-asm matrix instructions, and behind
+   the first of those no ``v_accvgpr_mov_b32`` outside asm may read or write one of them (a copy would mean a
+   second home; in front of it the compiler zeroes the tiles that way).
+
 The sources provide those slots themselves (``s_nop 1`` in front of the matrix instructions whose
 operands live long enough to be parked, ``tiles_ready()`` = ``s_nop 15; s_nop 3`` after each group).
 A result also counts as written once two further 32x32 matrix instructions have been issued behind its
@@ -57,16 +68,36 @@ def scan(isa_text: str, where: str = "") -> list[str]:
     out = []
     kern, inasm, hist, pending = "?", False, [], {}  # pending: register -> matrix instructions issued since
     flying: list[set] = []  # destinations of the inline-asm LDS reads in flight, oldest first
+    # rule 4, per kernel: destinations of in-place asm matrix instructions, registers written by in-place-move
+    # blocks, accumulation-file copies made by the compiler
+    acc_dst, moved, copies, block_writes = set(), set(), [], []
+
+    def rule4():
+        if not moved:
+            return
+        if moved != acc_dst:
+            extra, missing = sorted(moved - acc_dst), sorted(acc_dst - moved)
+            out.append(f"{where} {kern}: in-place accumulator moves write a{[r[1] for r in extra]} outside, and miss "
+                       f"a{[r[1] for r in missing]} of, the in-place matrix instructions' destinations")
+        for line, regs in copies:
+            if regs & acc_dst:
+                out.append(f"{where} {kern}: '{line[:60]}' copies an accumulator that is also moved in place")
+
     for ln in isa_text.splitlines():
         t = ln.strip()
         if t.startswith("_Z") and ":" in t and "$" not in t.split(":")[0]:
+            rule4()
             kern, hist, pending, flying = t.split(":")[0], [], {}, []
+            acc_dst, moved, copies, block_writes = set(), set(), [], []
             continue
         if "ASMSTART" in t:
             inasm = True
+            block_writes = []
             continue
         if "ASMEND" in t:
             inasm = False
+            if len(block_writes) == 2:  # acc_move_in_place
+                moved |= set(block_writes)
             continue
         if not t or t[0] in ";.":
             continue
@@ -75,6 +106,10 @@ def scan(isa_text: str, where: str = "") -> list[str]:
             continue
         op = t.split()[0]
         ops = [x.strip() for x in t.split(None, 1)[1].split(",")] if " " in t else []
+        if op == "v_accvgpr_write_b32" and inasm:
+            block_writes += list(_regs(ops[0]))
+        if op == "v_accvgpr_mov_b32" and not inasm and acc_dst:  # (before the first accumulation: the zeroing)
+            copies.append((t, _regs(ops[0]) | _regs(ops[1])))
         if op == "s_nop" and ops and int(ops[0]) >= 15:
             pending = {}  # tiles_ready(): results of the group are readable from here on
         if op.startswith("ds_read") and inasm:
@@ -106,6 +141,8 @@ def scan(isa_text: str, where: str = "") -> list[str]:
                             out.append(f"{where} {kern}: '{pop} {pops[0]}' feeds '{t[:60]}' without idle slots")
                 for r in dst:  # vector registers, and accumulation registers (read back by v_accvgpr_read)
                     pending[r] = 0
+                if len(ops) >= 4 and ops[0] == ops[3] and ops[0].startswith("a"):
+                    acc_dst |= dst  # accumulation in place (mfma_acc)
             else:
                 for r in dst:
                     pending.pop(r, None)
@@ -116,6 +153,7 @@ def scan(isa_text: str, where: str = "") -> list[str]:
             if srcs & pending.keys():
                 out.append(f"{where} {kern}: '{t[:60]}' reads a matrix result before the wait that follows its group")
         hist.append((op, ops))
+    rule4()
     return out
 
 

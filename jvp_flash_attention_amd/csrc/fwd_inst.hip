@@ -37,11 +37,11 @@ static int launch_fwd2_one(const FwdParams &p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }
 
-// ... and, without an explicit mask, its software-pipelined form.
-template <typename T, int D, bool DUAL>
+// ... and its software-pipelined form (D = 128).
+template <typename T, int D, bool DUAL, int MASK = MASK_NONE, bool DROP = false>
 static int launch_fwd3_one(const FwdParams &p, hipStream_t stream) {
   using Cfg = Fwd2Cfg<T, D, DUAL>;
-  auto kern = fwd3_kernel<T, D, DUAL>;
+  auto kern = fwd3_kernel<T, D, DUAL, MASK, DROP>;
   int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
   if (rc != 0) return rc;
   const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
@@ -93,7 +93,10 @@ static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
       }
     } else if constexpr (sizeof(T) == 2 && D <= 128) {
       switch (mask) {
-        case MASK_NONE: return launch_fwd2_one<T, D, DUAL, MASK_NONE, true>(p, stream);
+        case MASK_NONE:
+          // (with a mask and dropout together the pipelined kernel runs out of registers)
+          if constexpr (D == 128) return launch_fwd3_one<T, D, DUAL, MASK_NONE, true>(p, stream);
+          else return launch_fwd2_one<T, D, DUAL, MASK_NONE, true>(p, stream);
         case MASK_BOOL: return launch_fwd2_one<T, D, DUAL, MASK_BOOL, true>(p, stream);
         case MASK_ADD: return launch_fwd2_one<T, D, DUAL, MASK_ADD, true>(p, stream);
       }
@@ -114,12 +117,17 @@ static int launch_fwd_mask(const FwdParams &p, int mask, hipStream_t stream) {
       case MASK_ADD: return launch_fwd_wide_one<T, D, DUAL, MASK_ADD>(p, stream);
     }
     return -3;
-  } else if constexpr (sizeof(T) == 2 && D <= 128) {
+  } else if constexpr (sizeof(T) == 2 && D == 128) {
+    // the pipelined kernel pays off where a slot has enough matrix work to hide the softmax behind
     switch (mask) {
-      case MASK_NONE:
-        // the pipelined kernel pays off where a slot has enough matrix work to hide the softmax behind
-        if constexpr (D >= 128) return launch_fwd3_one<T, D, DUAL>(p, stream);
-        else return launch_fwd2_one<T, D, DUAL, MASK_NONE>(p, stream);
+      case MASK_NONE: return launch_fwd3_one<T, D, DUAL>(p, stream);
+      case MASK_BOOL: return launch_fwd3_one<T, D, DUAL, MASK_BOOL>(p, stream);
+      case MASK_ADD: return launch_fwd3_one<T, D, DUAL, MASK_ADD>(p, stream);
+    }
+    return -3;
+  } else if constexpr (sizeof(T) == 2 && D < 128) {
+    switch (mask) {
+      case MASK_NONE: return launch_fwd2_one<T, D, DUAL, MASK_NONE>(p, stream);
       case MASK_BOOL: return launch_fwd2_one<T, D, DUAL, MASK_BOOL>(p, stream);
       case MASK_ADD: return launch_fwd2_one<T, D, DUAL, MASK_ADD>(p, stream);
     }

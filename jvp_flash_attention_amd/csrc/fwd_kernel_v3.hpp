@@ -1,6 +1,7 @@
-// Software-pipelined fused dual forward for 16-bit element types, D in {64, 128}, no explicit mask
-// (causal and ragged sequence ends are handled).  Same tiles, swizzles, fragment layouts and
-// mathematics as fwd_kernel_v2.hpp; what changes is the order of work inside a wave.
+// Software-pipelined fused dual forward for 16-bit element types, D in {64, 128}: causal, boolean and
+// additive masks (with the key limit and the tile lists), ragged sequence ends, dropout.  Same tiles,
+// swizzles, fragment layouts and mathematics as fwd_kernel_v2.hpp; what changes is the order of work
+// inside a wave.
 //
 // A wave issues instructions in order, but a matrix instruction occupies the issue port for a
 // fraction of the time the matrix pipe needs to execute it, so independent vector instructions
@@ -40,7 +41,12 @@ template <int N> __device__ __forceinline__ void lds_wait3(u32x4 &a, u32x2 &c, u
   asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a), "+v"(c), "+v"(d) : "n"(N));
 }
 
-template <typename T, int D, bool DUAL>
+// MASK: mask values are requested with vector loads a whole iteration before the softmax that applies them
+// (mask.hpp), and tiles that the caller's key limit or tile list leaves out are not visited.
+// DROP: dropout on the probabilities (see fwd_kernel.hpp): what enters the products with V, V' is
+// P * keep / (1 - p), hashed per entry in the gaps between the matrix instructions; l, mu stay those of the
+// full softmax.
+template <typename T, int D, bool DUAL, int MASK = MASK_NONE, bool DROP = false>
 __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (and has no buffer descriptor type)
   using Cfg = Fwd2Cfg<T, D, DUAL>;
@@ -77,9 +83,23 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   const int qld = qrow < L ? qrow : L - 1;
   // This workgroup's keys: all of them, or the tiles of its chunk.  From here on key indices are counted from
   // the chunk's first key k0: Lk is the number of keys left from there, and the causal limits move with it.
-  const int nt_all = ((pr.causal ? min(pr.Lk, q0 + Cfg::BM) : pr.Lk) + BN - 1) / BN;
+  int kend = pr.causal ? min(pr.Lk, q0 + Cfg::BM) : pr.Lk;
+  // padded batches: the caller's hint says the mask hides every key from klimit[z] on, so those tiles
+  // need not be visited (at least one tile is, which keeps rows without any key well defined)
+  if constexpr (MASK != MASK_NONE) {
+    if (pr.klimit) kend = min(kend, max(pr.klimit[zh / pr.H], 1));
+  }
+  const int nt_all = (kend + BN - 1) / BN;
   const int t_first = chunks > 1 ? min(chunk * pr.chunk_tiles, nt_all) : 0;
-  const int ntiles = chunks > 1 ? min(nt_all - t_first, pr.chunk_tiles) : nt_all;  // 0: nothing for this chunk
+  // Tiles visited: t_first .. t_first + ntiles - 1, or (with a mask) the caller's list of the tiles of this query
+  // block that hold an attended entry (ascending; a tile left out would have contributed exact zeros).
+  const int *tlist = nullptr;
+  if constexpr (MASK != MASK_NONE) {
+    if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset_q(pr, zh / pr.H, zh % pr.H, qb);
+  }
+  const int tmax = (pr.Lk + BN - 1) / BN - 1;  // index of the last tile of the sequence: bounds whatever a list holds
+  const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1)
+                           : (chunks > 1 ? min(nt_all - t_first, pr.chunk_tiles) : nt_all);  // 0: nothing for this chunk
   const int k0 = t_first * BN;
   const int Lk = pr.Lk - k0;
   // partial results of a chunk: [chunk][row][O | T][D] floats, then [chunk][row][m, l, mu_acc, c]
@@ -160,6 +180,17 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   const float sl2 = pr.scale * LOG2E;
   const bool neg_scale = !(sl2 > 0.f);
   const int qlim = pr.causal ? qrow - k0 : 0x7fffffff;  // keys above this index are masked
+  const int64_t mrow = MASK != MASK_NONE ? (zh / pr.H) * pr.ms[0] + (zh % pr.H) * pr.ms[1] + (int64_t)qld * pr.ms[2] : 0;
+  bool mask_al = false;  // mask rows can be fetched with aligned vector loads
+  if constexpr (MASK != MASK_NONE) mask_al = mask_rows_aligned<T, MASK>(pr);
+  const uint32_t drop_row = DROP ? drop_row_word(pr, zh, qld) : 0u;  // dropout: this lane's query row, see params.hpp
+  // List elements are requested an iteration ahead, unconditionally (from a harmless address when there is no
+  // list: a branch around the read would split the loop's straight-line body).
+  auto list_slot = [&](int i) { return tlist ? tlist + 1 + i : reinterpret_cast<const int *>(p.q); };
+  auto tile_first_key = [&](int i) {  // first key of the i-th tile visited (i clamped to the last one)
+    const int ic = min(i, max(ntiles - 1, 0));
+    return (tlist ? min(max(tlist[1 + ic], 0), tmax) : ic) * BN;
+  };
 
   // ---- next-tile loads, one instruction per super-step -------------------------------------------
   constexpr int NLOAD = IPW * Cfg::NTILE;
@@ -182,20 +213,21 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     return __builtin_amdgcn_make_buffer_rsrc((void *)(base + (size_t)j * ROWB), 0, rows * ROWB, 0x00020000);
   };
   // iteration t loads K(t+1) into the K half of stage (t+1)&1 and V(t) into the V half of stage t&1
-  auto prepare_loads = [&](int t) {
+  // (jv, jk: first keys of tile t and of tile t + 1)
+  auto prepare_loads = [&](int t, int jv, int jk) {
     ld_dst_k = lds0 + ((t + 1) & 1) * Cfg::STAGEB + (wave * IPW) * 1024;
     ld_dst_v = lds0 + (t & 1) * Cfg::STAGEB + (wave * IPW) * 1024;
-    ld_rs[0] = tile_rsrc(Kg, (t + 1) * BN, t + 1 < ntiles);
-    ld_rs[1] = tile_rsrc(Vg, t * BN, t < ntiles);
+    ld_rs[0] = tile_rsrc(Kg, jk, t + 1 < ntiles);
+    ld_rs[1] = tile_rsrc(Vg, jv, t < ntiles);
     if constexpr (DUAL) {
-      ld_rs[2] = tile_rsrc(Ktg, (t + 1) * BN, t + 1 < ntiles);
-      ld_rs[3] = tile_rsrc(Vtg, t * BN, t < ntiles);
+      ld_rs[2] = tile_rsrc(Ktg, jk, t + 1 < ntiles);
+      ld_rs[3] = tile_rsrc(Vtg, jv, t < ntiles);
     }
   };
-  auto prepare_first = [&]() {
+  auto prepare_first = [&](int jk) {
     ld_dst_k = lds0 + (wave * IPW) * 1024;
-    ld_rs[0] = tile_rsrc(Kg, 0, true);
-    if constexpr (DUAL) ld_rs[2] = tile_rsrc(Ktg, 0, true);
+    ld_rs[0] = tile_rsrc(Kg, jk, true);
+    if constexpr (DUAL) ld_rs[2] = tile_rsrc(Ktg, jk, true);
   };
   auto load_piece = [&](auto pc) {
     constexpr int pi = decltype(pc)::value, i = pi / Cfg::NTILE, ts = pi % Cfg::NTILE;
@@ -220,15 +252,20 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
 
   // One slot.  QK: scores of a half tile (K rows at LDS address kaddr) into Sn, Spn.  PV: accumulate
   // the half tile whose V rows are at vaddr, with fragments pfp, psfp.  SM: softmax of Sc, Spc (first
-  // key jh) into pfn, psfn.  GEN: the softmax applies the causal / sequence-end limits.  LB: index of
-  // the first load step of this slot, or -1.
+  // key jh) into pfn, psfn.  GEN: 0 the softmax takes the scores as they are; 1 it applies the mask values
+  // mah (keys 16 c + 8 g .. + 7 of the half tile in mah[c]); 2 the mask and the causal / sequence-end limits.
+  // LB: index of the first load step of this slot, or -1.
   u32x4 ka[RD], kb[RD];
   u32x2 va[RD][2], vb[RD][2];
   auto slot = [&](auto QKc, auto PVc, auto SMc, auto GENc, auto LBc, auto PREc, auto NEXTc, uint32_t kaddr, uint32_t vaddr, f32x16 &Sc,
                   f32x16 &Spc, f32x16 &Sn, f32x16 &Spn, Frag<T>(&pfp)[2], Frag<T>(&psfp)[2], Frag<T>(&pfn)[2],
-                  Frag<T>(&psfn)[2], int jh) {
+                  Frag<T>(&psfn)[2], int jh, const MaskAhead<T, MASK>(&mah)[2]) {
     constexpr bool QK = decltype(QKc)::value, PV = decltype(PVc)::value, SM = decltype(SMc)::value;
-    constexpr bool GEN = decltype(GENc)::value;
+    constexpr int GENL = decltype(GENc)::value;
+    constexpr bool GEN = GENL != 0, LIM = GENL == 2;
+    static_assert(MASK == MASK_NONE || GEN || !SM, "a masked softmax applies its mask");
+    // dropout: register e holds key jh + 16(e/8) + 8g + e%8 of this lane's query
+    const uint32_t xb = DROP ? drop_row + (uint32_t)(jh + 8 * g) * DROP_C_KEY : 0u;
     constexpr int LB = decltype(LBc)::value;
     // PRE: the reads of the first PD super-steps were issued by the previous slot; NEXT: issue those of
     // the next slot, which works on the other half of the same two tiles
@@ -253,8 +290,12 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
           if constexpr (GEN) {
             const int key = jh + 16 * (e / 8) + 8 * g + (e % 8);
             float s = Sc[e] * sl2;
-            s = (key <= qlim) ? s : NEG_INF;
-            s = (key < Lk) ? s : NEG_INF;
+            if constexpr (MASK == MASK_ADD) s = __builtin_fmaf((float)mah[e / 8].f[e % 8], LOG2E, s);
+            if constexpr (MASK == MASK_BOOL) s = mask_keep_of<T, MASK>(mah[e / 8], e % 8) ? s : NEG_INF;
+            if constexpr (LIM) {
+              s = (key <= qlim) ? s : NEG_INF;
+              s = (key < Lk) ? s : NEG_INF;
+            }
             Sc[e] = s;
             m8 = fmaxf(m8, s);
           } else {
@@ -294,6 +335,11 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
           if constexpr (DUAL) {
             sv[e] *= pv[e];
             rmu += sv[e];
+          }
+          if constexpr (DROP) {  // the row sums above are those of the full softmax
+            const float ks = drop_scale_of(pr, xb + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_KEY);
+            pv[e] *= ks;
+            if constexpr (DUAL) sv[e] *= ks;
           }
           if constexpr (e % 2 == 1) {
             constexpr int c = e / 8, j = e % 8;
@@ -458,6 +504,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
             float pe;
             if constexpr (GEN) pe = fast_exp2(Sc[e] - m_again);
             else pe = fast_exp2(__builtin_fmaf(Sc[e], sl2, -m_again));
+            if constexpr (DROP) pe *= drop_scale_of(pr, xb + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_KEY);
             psfn[e / 8][e % 8] = (T)(pe * __builtin_fmaf(Spc[e], pr.scale, -c_i));
           }
         }
@@ -476,50 +523,112 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   using B0 = std::false_type;
   using B1 = std::true_type;
   using XP = std::integral_constant<bool, NSS % RD == 0>;  // fragment prefetch across the two slots of an iteration
+  using GI = std::integral_constant<int, MASK != MASK_NONE ? 1 : 0>;  // softmax of interior tiles, see slot()
+  using G2 = std::integral_constant<int, 2>;                           // ... of tiles that meet a limit
   f32x16 SX, SpX, SY, SpY;
   Frag<T> pfA[2], psfA[2], pfB[2], psfB[2];
 
+  // Mask values of the two half tiles whose softmax an iteration runs: [0] second half of the tile before,
+  // [1] first half of this iteration's tile; each by 16-key group.  They travel from HBM or the far caches:
+  // those of iteration t + 1 are requested at the top of iteration t.
+  MaskAhead<T, MASK> mcur[2][2], mnext[2][2];
+  auto fetch_half = [&](MaskAhead<T, MASK>(&dst)[2], int jh) {
+    if constexpr (MASK != MASK_NONE) {
+      if (mask_al && jh + 32 <= pr.Lk) {  // aligned rows, all 32 keys exist: one vector load per 8 keys
+#pragma unroll
+        for (int c = 0; c < 2; ++c) dst[c] = mask_fetch8<T, MASK>(pr, mrow, jh + 16 * c + 8 * g);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) dst[c] = mask_fetch8_any<T, MASK>(pr, mrow, jh + 16 * c + 8 * g);
+      }
+    }
+  };
+  // first keys of the tiles of iterations t - 1, t, t + 1
+  int jA = 0, jB = 0, jC = BN;
+  if constexpr (MASK != MASK_NONE) {
+    jB = tile_first_key(0);
+    jC = tile_first_key(1);
+  }
+  // at the end of iteration t: the tile of iteration t + 2 comes from the list element requested at its top
+  auto advance = [&](int t, int tahead) {
+    if constexpr (MASK != MASK_NONE) {
+      const int listed = list_take(tahead);
+      jA = jB;
+      jB = jC;
+      jC = (tlist ? min(max(listed, 0), tmax) : min(t + 2, ntiles - 1)) * BN;
+    }
+  };
+
   // ---- prologue: K(0) in one burst ---------------------------------------------------------------
-  prepare_first();
+  prepare_first(jB);
   static_for<NLOAD>([&](auto pc) {
     if constexpr (decltype(pc)::value % 2 == 0) load_piece(pc);
   });
+  fetch_half(mcur[1], jB);
   auto kad = [&](int t, int hb) { return lds0 + (t & 1) * Cfg::STAGEB + hb * 32 * ROWB; };
 
   // iteration 0: scores of half tiles 0 and 1, softmax of half tile 0
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
-  prepare_loads(0);
-  slot(B1{}, B0{}, B0{}, B1{}, std::integral_constant<int, 0>{}, B0{}, B0{}, kad(0, 0), 0u, SX, SpX, SY, SpY, pfA, psfA, pfB, psfB, 0);
-  slot(B1{}, B0{}, B1{}, B1{}, std::integral_constant<int, NSS>{}, B0{}, B0{}, kad(0, 1), 0u, SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0);
-  // Iterations whose softmax needs the causal / sequence-end limits form the tail of the loop; they
-  // get a loop of their own so that the common iteration is one straight-line block.
-  int t_gen = (Lk >= 32) ? (Lk - 32) / BN + 1 : 0;
-  if (pr.causal) t_gen = min(t_gen, max(q0 - k0 + 32, 0) / BN);
-  t_gen = neg_scale ? 1 : max(1, t_gen);
-  int t = 1;
-  for (; t < min(t_gen, ntiles); ++t) {
+  {
+    int tahead = 0;
+    if constexpr (MASK != MASK_NONE) {
+      tahead = list_request(list_slot(min(2, ntiles - 1)));
+      fetch_half(mnext[0], jB + 32);
+      fetch_half(mnext[1], jC);
+    }
+    prepare_loads(0, jB, jC);
+    slot(B1{}, B0{}, B0{}, G2{}, std::integral_constant<int, 0>{}, B0{}, B0{}, kad(0, 0), 0u, SX, SpX, SY, SpY, pfA, psfA, pfB, psfB, jB, mcur[1]);
+    slot(B1{}, B0{}, B1{}, G2{}, std::integral_constant<int, NSS>{}, B0{}, B0{}, kad(0, 1), 0u, SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, jB, mcur[1]);
+    advance(0, tahead);
+  }
+  auto iteration = [&](int t, auto GENc) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of K(t), V(t-1) has landed
     __syncthreads();                      // ... everyone's has, and K(t-1), V(t-2) are no longer read
-    prepare_loads(t);
-    slot(B1{}, B1{}, B1{}, B0{}, std::integral_constant<int, 0>{}, B0{}, XP{}, kad(t, 0), kad(t - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB, 0);
-    slot(B1{}, B1{}, B1{}, B0{}, std::integral_constant<int, NSS>{}, XP{}, B0{}, kad(t, 1), kad(t - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0);
+    int tahead = 0;
+    if constexpr (MASK != MASK_NONE) {
+      tahead = list_request(list_slot(min(t + 2, ntiles - 1)));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mcur[i / 2][i % 2] = mnext[i / 2][i % 2];
+      fetch_half(mnext[0], jB + 32);
+      fetch_half(mnext[1], jC);
+    } else {
+      jA = (t - 1) * BN;
+      jB = t * BN;
+      jC = (t + 1) * BN;
+    }
+    prepare_loads(t, jB, jC);
+    slot(B1{}, B1{}, B1{}, GENc, std::integral_constant<int, 0>{}, B0{}, XP{}, kad(t, 0), kad(t - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
+         jA + 32, mcur[0]);
+    slot(B1{}, B1{}, B1{}, GENc, std::integral_constant<int, NSS>{}, XP{}, B0{}, kad(t, 1), kad(t - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA,
+         jB, mcur[1]);
+    advance(t, tahead);
+  };
+  // Iterations whose softmax needs the causal / sequence-end limits form the tail of the loop; they
+  // get a loop of their own so that the common iteration is one straight-line block.
+  int t = 1;
+  if constexpr (MASK == MASK_NONE) {
+    int t_gen = (Lk >= 32) ? (Lk - 32) / BN + 1 : 0;
+    if (pr.causal) t_gen = min(t_gen, max(q0 - k0 + 32, 0) / BN);
+    t_gen = neg_scale ? 1 : max(1, t_gen);
+    for (; t < min(t_gen, ntiles); ++t) iteration(t, GI{});
+  } else {
+    // (tiles come in ascending order, so only the last ones can reach past the last key)
+    for (; t < ntiles && jB + 32 <= pr.Lk; ++t) iteration(t, GI{});
   }
-  for (; t < ntiles; ++t) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    prepare_loads(t);
-    slot(B1{}, B1{}, B1{}, B1{}, std::integral_constant<int, 0>{}, B0{}, XP{}, kad(t, 0), kad(t - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
-         (t - 1) * BN + 32);
-    slot(B1{}, B1{}, B1{}, B1{}, std::integral_constant<int, NSS>{}, XP{}, B0{}, kad(t, 1), kad(t - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA,
-         t * BN);
-  }
+  for (; t < ntiles; ++t) iteration(t, G2{});
   // drain: softmax of the last half tile, accumulation of the last two
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
-  slot(B0{}, B1{}, B1{}, B1{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
-       (ntiles - 1) * BN + 32);
-  slot(B0{}, B1{}, B0{}, B1{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0);
+  if constexpr (MASK != MASK_NONE) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c) mcur[0][c] = mnext[0][c];
+  } else {
+    jA = (ntiles - 1) * BN;
+  }
+  slot(B0{}, B1{}, B1{}, G2{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
+       jA + 32, mcur[0]);
+  slot(B0{}, B1{}, B0{}, G2{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0, mcur[0]);
   // the last accumulation has written its registers
   if constexpr (DUAL) accs_ready(Oacc, Tacc);
   else accs_ready(Oacc);

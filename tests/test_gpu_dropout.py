@@ -76,10 +76,57 @@ def test_dual_with_dropout(dt, D, mode):
     _case(2, 2, 256, D, DTYPES[dt], mode, p=0.2, seed=0x1234_5678_9ABC_DEF0)
 
 
-@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+@pytest.mark.parametrize("dt", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("mode", ["keypad", "bias", "bool_full"])
-def test_dual_with_dropout_and_masks(dt, mode):
-    _case(2, 2, 192, 64, DTYPES[dt], mode, p=0.35, seed=77)
+def test_dual_with_dropout_and_masks(dt, D, mode):
+    """Every head dim and element type: the masked forward kernels with dropout all carry the in-place rescale of
+    their accumulators, and every instantiation of it is run here."""
+    _case(2, 2, 192, D, DTYPES[dt], mode, p=0.35, seed=77)
+
+
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("L,Lk", [(33, 65), (64, 129), (130, 200)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_keep_decisions_entry_by_entry_through_the_16_bit_kernels(D, L, Lk, causal):
+    """q = 0 makes the probabilities uniform over the keys a row sees, and one-hot columns in v, v' make every entry of
+    O, O' the sum of at most two entries of P * W: a single wrong keep decision (an off-by-one at a tile or
+    32-row-block edge of a kernel's walk through the pattern) then moves an entry by about half its size, where
+    the ordinary dropout cases would bury it under the 2e-2 bar.  Lengths straddle 32, 64 and 128; one kernel
+    family per head dim (direct-to-LDS, software-pipelined, the D = 256 kernels); gO one-hot exposes the pattern
+    in dv the same way."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    dtype, p, seed = torch.bfloat16, 0.3, 0xABCDEF
+    Z, H = 1, 2
+    g = torch.Generator().manual_seed(9)
+    q = torch.zeros(Z, H, L, D)
+    k = torch.randn(Z, H, Lk, D, generator=g)
+    qt, kt = torch.zeros(Z, H, L, D), torch.zeros(Z, H, Lk, D)
+    eye = lambda n, shift: torch.nn.functional.one_hot((torch.arange(n) + shift) % D, D).float().expand(Z, H, n, D)  # noqa: E731
+    v, vt, go, gt = eye(Lk, 0), eye(Lk, 1), eye(L, 2), eye(L, 3)
+    t = [x.to(dtype).contiguous() for x in (q, k, v, qt, kt, vt, go, gt)]
+    f64 = [x.double().numpy() for x in t]
+    dev = [x.cuda() for x in t]
+    scale = D**-0.5
+    W = dropout.keep_scale(Z, H, L, Lk, p, seed)
+    ref = dense.forward(*f64[:6], mask=None, causal=causal, scale=scale, keep_scale=W)
+    o, ot, M, mu = be.fwd(*dev[:6], None, _lib.MASK_NONE, causal, scale, p, seed)
+    # every entry to a fraction of the smallest nonzero one: 1 / ((1 - p) * keys seen) in bf16
+    smallest = 1.0 / ((1 - p) * Lk)
+    def off(got, want):  # beyond 16-bit rounding of the entry itself
+        return (np.abs(got.double().cpu().numpy() - want) - 0.01 * np.abs(want)).max()
+
+    for name, got, want in (("O", o, ref["O"]), ("O'", ot, ref["Ot"])):
+        err = off(got, want)
+        assert err < 0.05 * smallest, f"{name}: an entry is off by {err:.3e}, entries are multiples of about {smallest:.3e}"
+    rb = dense.backward(*f64, mask=None, causal=causal, scale=scale, keep_scale=W)
+    grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], None, _lib.MASK_NONE, causal, scale, dropout_p=p, dropout_seed=seed)
+    err = off(grads[2], rb["dv"])
+    assert err < 0.05 * smallest, f"dv: an entry is off by {err:.3e}"
+    for n, got in zip(("dq", "dk", "dv"), grads[:3]):
+        _tol_check(n, got, rb[n], dtype)
 
 
 @pytest.mark.parametrize("dt", ["bf16", "fp32"])
