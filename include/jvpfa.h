@@ -62,7 +62,10 @@ typedef struct jvpfa_problem {
    * jvpfa_dropout_keep() writes the keep pattern out.  The reference carries dead code for dropout and raises
    * NotImplementedError (JA:94-122, JA:271-277, JA:2356-2357).  Costs bf16 / fp16 calls 6 - 13 % at D = 128
    * (a third where the unmasked, non-causal forward leaves its software-pipelined kernel), about 30 % at D = 64,
-   * fp32 1 - 6 %. */
+   * fp32 1 - 6 %.
+   * The seed is an argument of the kernels: a launch recorded into a HIP graph replays with the seed it was
+   * recorded with, i.e. the same keep pattern on every replay; a caller that wants a fresh pattern per step
+   * records the graph anew (or runs the dropout calls outside it). */
   float dropout_p;
   uint64_t dropout_seed;
 } jvpfa_problem;
@@ -165,6 +168,9 @@ size_t jvpfa_bwd_workspace_bytes(int32_t Z, int32_t H, int32_t L);
  * nothing is launched.  The GPU the stream belongs to must be the current device.  Every call on a
  * GPU uses that GPU's one array: two calls that overlap in time on one GPU (different streams, or
  * different threads) race; calls on one stream, one after another, are fine.
+ * The first call on a GPU looks the array's address up (hipGetSymbolAddress, which makes the runtime load
+ * the library's code object there and commit the 12 MiB): make that one call, with any valid arguments,
+ * outside graph capture and before memory is measured; every later call on that GPU only launches kernels.
  */
 #define JVPFA_STATIC_ROWS (1 << 20)
 int jvpfa_bwd_static(const jvpfa_bwd_args *args, void *hip_stream);

@@ -75,10 +75,9 @@ __global__ __launch_bounds__(256, 1) void fwd_kernel(const FwdParams p) {
   const int qrow = q0 + wave * 32 + r; // this lane's query row
   const int qld = qrow < L ? qrow : L - 1;
 
-  // D = 256 (fp32; 16-bit types come here with dropout only): Q, Q' resident would be up to 256 registers next to
-  // 256 of accumulators, so
-  // there the lane's fragments are read from global memory where they are used (the same 32 bytes per lane on
-  // every tile: cache hits)
+  // D = 256 (fp32 only: the 16-bit types have kernels of their own at this head dim, fwd_kernel_wide.hpp): Q, Q'
+  // resident would be up to 256 registers next to 256 of accumulators, so there the lane's fragments are read
+  // from global memory where they are used (the same 32 bytes per lane on every tile: cache hits)
   constexpr bool SB = D == 256;
   const T *Qrow = Qg + (size_t)qld * D + 8 * g, *Qtrow = DUAL ? Qtg + (size_t)qld * D + 8 * g : nullptr;
   Frag<T> Qf[SB ? 1 : KK], Qtf[(DUAL && !SB) ? KK : 1];

@@ -87,7 +87,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   // padded batches: the caller's hint says the mask hides every key from klimit[z] on, so those tiles
   // need not be visited (at least one tile is, which keeps rows without any key well defined)
   if constexpr (MASK != MASK_NONE) {
-    if (pr.klimit) kend = min(kend, max(pr.klimit[zh / pr.H], 1));
+    if (pr.klimit) kend = min(kend, max(__builtin_amdgcn_readfirstlane(pr.klimit[zh / pr.H]), 1));
   }
   const int nt_all = (kend + BN - 1) / BN;
   const int t_first = chunks > 1 ? min(chunk * pr.chunk_tiles, nt_all) : 0;
@@ -98,7 +98,8 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     if (pr.tiles_q) tlist = pr.tiles_q + tile_list_offset_q(pr, zh / pr.H, zh % pr.H, qb);
   }
   const int tmax = (pr.Lk + BN - 1) / BN - 1;  // index of the last tile of the sequence: bounds whatever a list holds
-  const int ntiles = tlist ? min(max(tlist[0], 1), tmax + 1)
+  // (what is read from a list is the same in every lane; saying so keeps the tile pointers in scalar registers)
+  const int ntiles = tlist ? __builtin_amdgcn_readfirstlane(min(max(tlist[0], 1), tmax + 1))
                            : (chunks > 1 ? min(nt_all - t_first, pr.chunk_tiles) : nt_all);  // 0: nothing for this chunk
   const int k0 = t_first * BN;
   const int Lk = pr.Lk - k0;
@@ -215,6 +216,10 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   // iteration t loads K(t+1) into the K half of stage (t+1)&1 and V(t) into the V half of stage t&1
   // (jv, jk: first keys of tile t and of tile t + 1)
   auto prepare_loads = [&](int t, int jv, int jk) {
+    if constexpr (MASK != MASK_NONE) {  // (the same in every lane, see above)
+      jv = __builtin_amdgcn_readfirstlane(jv);
+      jk = __builtin_amdgcn_readfirstlane(jk);
+    }
     ld_dst_k = lds0 + ((t + 1) & 1) * Cfg::STAGEB + (wave * IPW) * 1024;
     ld_dst_v = lds0 + (t & 1) * Cfg::STAGEB + (wave * IPW) * 1024;
     ld_rs[0] = tile_rsrc(Kg, jk, t + 1 < ntiles);
@@ -243,7 +248,9 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     }
   };
 
-  constexpr float RESCALE_TAU = 8.f;
+  // fp16: p <= 2^TAU multiplies S' - c in a 16-bit operand that overflows at 65504, so the slack is 2^2 there
+  // (|S' - c| up to 16 000; the reference's p <= 1 gives 65 504); bf16 has the exponent range for 2^8
+  constexpr float RESCALE_TAU = __is_same(T, _Float16) ? 2.f : 8.f;
   constexpr int NQ = DUAL ? 3 : 1, NP = DUAL ? 3 : 1;  // matrix instructions per super-step: scores, accumulation
   constexpr int NRS = DUAL ? 2 : 1, NRV = DUAL ? 4 : 2;  // LDS reads per super-step
   constexpr int NU = 38;                                 // vector units of one softmax
@@ -252,18 +259,26 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
 
   // One slot.  QK: scores of a half tile (K rows at LDS address kaddr) into Sn, Spn.  PV: accumulate
   // the half tile whose V rows are at vaddr, with fragments pfp, psfp.  SM: softmax of Sc, Spc (first
-  // key jh) into pfn, psfn.  GEN: 0 the softmax takes the scores as they are; 1 it applies the mask values
-  // mah (keys 16 c + 8 g .. + 7 of the half tile in mah[c]); 2 the mask and the causal / sequence-end limits.
+  // key jh) into pfn, psfn.  GEN: 0 the softmax takes the scores as they are; 1 it adds the mask terms madd
+  // (0 or -inf for a boolean mask, the bias in log2 units for an additive one) to the scaled scores; 2 it
+  // applies the causal / sequence-end limits (kernels without a mask).  With a mask, a slot that forms scores
+  // also forms the mask terms that go with them, in its gaps: madd is read by the front of the softmax and
+  // refilled behind it from the mask words mah of the half tile whose scores the slot forms (keys
+  // 16 c + 8 g .. + 7 in mah[c]; keys past the end come masked from the fetch).
   // LB: index of the first load step of this slot, or -1.
   u32x4 ka[RD], kb[RD];
   u32x2 va[RD][2], vb[RD][2];
   auto slot = [&](auto QKc, auto PVc, auto SMc, auto GENc, auto LBc, auto PREc, auto NEXTc, uint32_t kaddr, uint32_t vaddr, f32x16 &Sc,
                   f32x16 &Spc, f32x16 &Sn, f32x16 &Spn, Frag<T>(&pfp)[2], Frag<T>(&psfp)[2], Frag<T>(&pfn)[2],
-                  Frag<T>(&psfn)[2], int jh, const MaskAhead<T, MASK>(&mah)[2]) {
+                  Frag<T>(&psfn)[2], int jh, const MaskAhead<T, MASK>(&mah)[2], float (&madd)[16]) {
     constexpr bool QK = decltype(QKc)::value, PV = decltype(PVc)::value, SM = decltype(SMc)::value;
     constexpr int GENL = decltype(GENc)::value;
     constexpr bool GEN = GENL != 0, LIM = GENL == 2;
-    static_assert(MASK == MASK_NONE || GEN || !SM, "a masked softmax applies its mask");
+    static_assert(MASK == MASK_NONE ? GENL != 1 : (GENL == 1 || !SM), "a masked softmax adds its mask terms, no other does");
+    constexpr bool PREC = MASK != MASK_NONE && QK;  // mask terms for the scores this slot forms
+    constexpr int NPRE = PREC ? 8 : 0;              // ... as this many vector units of two entries
+    uint32_t vzero = 0u, vninf = 0xff800000u;
+    if constexpr (PREC && MASK == MASK_BOOL) asm volatile("" : "+v"(vzero), "+v"(vninf));  // vector registers that hold 0 and -inf
     // dropout: register e holds key jh + 16(e/8) + 8g + e%8 of this lane's query
     const uint32_t xb = DROP ? drop_row + (uint32_t)(jh + 8 * g) * DROP_C_KEY : 0u;
     constexpr int LB = decltype(LBc)::value;
@@ -272,7 +287,8 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     constexpr bool PRE = decltype(PREc)::value, NEXT = decltype(NEXTc)::value;
     constexpr int MPS = (QK ? NQ : 0) + (PV ? NP : 0);  // matrix instructions per super-step
     constexpr int NG = NSS * MPS;                       // gaps of the slot
-    constexpr int UPG = SM ? (NU - NU0 + NG - 1) / NG : 0;  // vector units per gap
+    constexpr int NUS = SM ? NU - NU0 : 0;                  // softmax units behind the front
+    constexpr int UPG = (NUS + NPRE + NG - 1) / NG;         // vector units per gap
     constexpr int RPS = (QK ? NRS : 0) + (PV ? NRV : 0);
     static_assert((PD - 1) * RPS <= 15, "lgkmcnt is a 4-bit counter");
     static_assert(!NEXT || (NSS % RD == 0 && QK && PV), "the fragment ring continues into the next slot");
@@ -289,9 +305,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
         for (int e = 8 * u; e < 8 * u + 8; ++e) {
           if constexpr (GEN) {
             const int key = jh + 16 * (e / 8) + 8 * g + (e % 8);
-            float s = Sc[e] * sl2;
-            if constexpr (MASK == MASK_ADD) s = __builtin_fmaf((float)mah[e / 8].f[e % 8], LOG2E, s);
-            if constexpr (MASK == MASK_BOOL) s = mask_keep_of<T, MASK>(mah[e / 8], e % 8) ? s : NEG_INF;
+            float s = MASK != MASK_NONE ? __builtin_fmaf(Sc[e], sl2, madd[e]) : Sc[e] * sl2;
             if constexpr (LIM) {
               s = (key <= qlim) ? s : NEG_INF;
               s = (key < Lk) ? s : NEG_INF;
@@ -336,10 +350,10 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
             sv[e] *= pv[e];
             rmu += sv[e];
           }
-          if constexpr (DROP) {  // the row sums above are those of the full softmax
-            const float ks = drop_scale_of(pr, xb + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_KEY);
-            pv[e] *= ks;
-            if constexpr (DUAL) sv[e] *= ks;
+          if constexpr (DROP) {  // the row sums above are those of the full softmax; 1 / (1 - p) waits for the epilogue
+            const bool kept = drop_finish(xb + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_KEY) >= pr.drop_thr;
+            pv[e] = kept ? pv[e] : 0.f;
+            if constexpr (DUAL) sv[e] = kept ? sv[e] : 0.f;
           }
           if constexpr (e % 2 == 1) {
             constexpr int c = e / 8, j = e % 8;
@@ -371,12 +385,23 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     // the vector work that follows matrix instruction number gi of the slot
     auto gap = [&](auto gc) {
       constexpr int gi = decltype(gc)::value;
-      if constexpr (SM) {
-        static_for<UPG>([&](auto uc) {
-          constexpr int u = NU0 + gi * UPG + decltype(uc)::value;
-          if constexpr (u < NU) unit(std::integral_constant<int, u>{});
-        });
-      }
+      static_for<UPG>([&](auto uc) {
+        constexpr int k = gi * UPG + decltype(uc)::value;
+        if constexpr (k < NUS) {
+          unit(std::integral_constant<int, NU0 + k>{});
+        } else if constexpr (k < NUS + NPRE) {  // mask terms of entries 2 (k - NUS), + 1 for the next softmax
+          static_for<2>([&](auto jc) {
+            constexpr int e = 2 * (k - NUS) + decltype(jc)::value;
+            if constexpr (MASK == MASK_BOOL) {  // byte e % 8 of the eight
+              const uint32_t word = (e % 8) < 4 ? (uint32_t)mah[e / 8].w : (uint32_t)(mah[e / 8].w >> 32);
+              madd[e] = mask_term_of_byte<e % 4>(word, vzero, vninf);
+            }
+            if constexpr (MASK == MASK_ADD) madd[e] = (float)mah[e / 8].f[e % 8] * LOG2E;
+          });
+          anchor(madd[2 * (k - NUS)]);
+          anchor(madd[2 * (k - NUS) + 1]);
+        }
+      });
       __builtin_amdgcn_sched_barrier(0);
     };
 
@@ -504,7 +529,7 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
             float pe;
             if constexpr (GEN) pe = fast_exp2(Sc[e] - m_again);
             else pe = fast_exp2(__builtin_fmaf(Sc[e], sl2, -m_again));
-            if constexpr (DROP) pe *= drop_scale_of(pr, xb + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_KEY);
+            if constexpr (DROP) pe = drop_finish(xb + (uint32_t)(16 * (e / 8) + (e % 8)) * DROP_C_KEY) >= pr.drop_thr ? pe : 0.f;
             psfn[e / 8][e % 8] = (T)(pe * __builtin_fmaf(Spc[e], pr.scale, -c_i));
           }
         }
@@ -523,35 +548,36 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   using B0 = std::false_type;
   using B1 = std::true_type;
   using XP = std::integral_constant<bool, NSS % RD == 0>;  // fragment prefetch across the two slots of an iteration
-  using GI = std::integral_constant<int, MASK != MASK_NONE ? 1 : 0>;  // softmax of interior tiles, see slot()
-  using G2 = std::integral_constant<int, 2>;                           // ... of tiles that meet a limit
+  constexpr bool MASKED = MASK != MASK_NONE;
+  using GI = std::integral_constant<int, MASKED ? 1 : 0>;  // softmax of interior tiles, see slot()
+  using GE = std::integral_constant<int, MASKED ? 1 : 2>;  // ... of tiles that meet a limit (with a mask the fetch applies it)
   f32x16 SX, SpX, SY, SpY;
   Frag<T> pfA[2], psfA[2], pfB[2], psfB[2];
 
-  // Mask values of the two half tiles whose softmax an iteration runs: [0] second half of the tile before,
-  // [1] first half of this iteration's tile; each by 16-key group.  They travel from HBM or the far caches:
-  // those of iteration t + 1 are requested at the top of iteration t.
+  // Mask words of the two half tiles of an iteration's tile, each by 16-key group, and of the tile after it.
+  // They travel from HBM or the far caches: those of iteration t + 1 are requested at the top of iteration t.
   MaskAhead<T, MASK> mcur[2][2], mnext[2][2];
+  float madd[16];  // mask terms of the scores in flight, see slot()
   auto fetch_half = [&](MaskAhead<T, MASK>(&dst)[2], int jh) {
-    if constexpr (MASK != MASK_NONE) {
+    if constexpr (MASKED) {
       if (mask_al && jh + 32 <= pr.Lk) {  // aligned rows, all 32 keys exist: one vector load per 8 keys
 #pragma unroll
         for (int c = 0; c < 2; ++c) dst[c] = mask_fetch8<T, MASK>(pr, mrow, jh + 16 * c + 8 * g);
       } else {
 #pragma unroll
-        for (int c = 0; c < 2; ++c) dst[c] = mask_fetch8_any<T, MASK>(pr, mrow, jh + 16 * c + 8 * g);
+        for (int c = 0; c < 2; ++c) dst[c] = mask_fetch8_lim<T, MASK>(pr, mrow, jh + 16 * c + 8 * g);
       }
     }
   };
   // first keys of the tiles of iterations t - 1, t, t + 1
   int jA = 0, jB = 0, jC = BN;
-  if constexpr (MASK != MASK_NONE) {
-    jB = tile_first_key(0);
-    jC = tile_first_key(1);
+  if constexpr (MASKED) {
+    jB = __builtin_amdgcn_readfirstlane(tile_first_key(0));
+    jC = __builtin_amdgcn_readfirstlane(tile_first_key(1));
   }
   // at the end of iteration t: the tile of iteration t + 2 comes from the list element requested at its top
   auto advance = [&](int t, int tahead) {
-    if constexpr (MASK != MASK_NONE) {
+    if constexpr (MASKED) {
       const int listed = list_take(tahead);
       jA = jB;
       jB = jC;
@@ -564,7 +590,8 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   static_for<NLOAD>([&](auto pc) {
     if constexpr (decltype(pc)::value % 2 == 0) load_piece(pc);
   });
-  fetch_half(mcur[1], jB);
+  fetch_half(mcur[0], jB);
+  fetch_half(mcur[1], jB + 32);
   auto kad = [&](int t, int hb) { return lds0 + (t & 1) * Cfg::STAGEB + hb * 32 * ROWB; };
 
   // iteration 0: scores of half tiles 0 and 1, softmax of half tile 0
@@ -572,26 +599,28 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
   __syncthreads();
   {
     int tahead = 0;
-    if constexpr (MASK != MASK_NONE) {
+    if constexpr (MASKED) {
       tahead = list_request(list_slot(min(2, ntiles - 1)));
-      fetch_half(mnext[0], jB + 32);
-      fetch_half(mnext[1], jC);
+      fetch_half(mnext[0], jC);
+      fetch_half(mnext[1], jC + 32);
     }
     prepare_loads(0, jB, jC);
-    slot(B1{}, B0{}, B0{}, G2{}, std::integral_constant<int, 0>{}, B0{}, B0{}, kad(0, 0), 0u, SX, SpX, SY, SpY, pfA, psfA, pfB, psfB, jB, mcur[1]);
-    slot(B1{}, B0{}, B1{}, G2{}, std::integral_constant<int, NSS>{}, B0{}, B0{}, kad(0, 1), 0u, SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, jB, mcur[1]);
+    slot(B1{}, B0{}, B0{}, GE{}, std::integral_constant<int, 0>{}, B0{}, B0{}, kad(0, 0), 0u, SX, SpX, SY, SpY, pfA, psfA, pfB, psfB, jB,
+         mcur[0], madd);
+    slot(B1{}, B0{}, B1{}, GE{}, std::integral_constant<int, NSS>{}, B0{}, B0{}, kad(0, 1), 0u, SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, jB,
+         mcur[1], madd);
     advance(0, tahead);
   }
   auto iteration = [&](int t, auto GENc) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of K(t), V(t-1) has landed
     __syncthreads();                      // ... everyone's has, and K(t-1), V(t-2) are no longer read
     int tahead = 0;
-    if constexpr (MASK != MASK_NONE) {
+    if constexpr (MASKED) {
       tahead = list_request(list_slot(min(t + 2, ntiles - 1)));
 #pragma unroll
       for (int i = 0; i < 4; ++i) mcur[i / 2][i % 2] = mnext[i / 2][i % 2];
-      fetch_half(mnext[0], jB + 32);
-      fetch_half(mnext[1], jC);
+      fetch_half(mnext[0], jC);
+      fetch_half(mnext[1], jC + 32);
     } else {
       jA = (t - 1) * BN;
       jB = t * BN;
@@ -599,36 +628,29 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     }
     prepare_loads(t, jB, jC);
     slot(B1{}, B1{}, B1{}, GENc, std::integral_constant<int, 0>{}, B0{}, XP{}, kad(t, 0), kad(t - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
-         jA + 32, mcur[0]);
+         jA + 32, mcur[0], madd);
     slot(B1{}, B1{}, B1{}, GENc, std::integral_constant<int, NSS>{}, XP{}, B0{}, kad(t, 1), kad(t - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA,
-         jB, mcur[1]);
+         jB, mcur[1], madd);
     advance(t, tahead);
   };
-  // Iterations whose softmax needs the causal / sequence-end limits form the tail of the loop; they
-  // get a loop of their own so that the common iteration is one straight-line block.
+  // Without a mask, iterations whose softmax needs the causal / sequence-end limits form the tail of the loop;
+  // they get a loop of their own so that the common iteration is one straight-line block.
   int t = 1;
-  if constexpr (MASK == MASK_NONE) {
+  if constexpr (!MASKED) {
     int t_gen = (Lk >= 32) ? (Lk - 32) / BN + 1 : 0;
     if (pr.causal) t_gen = min(t_gen, max(q0 - k0 + 32, 0) / BN);
     t_gen = neg_scale ? 1 : max(1, t_gen);
     for (; t < min(t_gen, ntiles); ++t) iteration(t, GI{});
-  } else {
-    // (tiles come in ascending order, so only the last ones can reach past the last key)
-    for (; t < ntiles && jB + 32 <= pr.Lk; ++t) iteration(t, GI{});
   }
-  for (; t < ntiles; ++t) iteration(t, G2{});
+  for (; t < ntiles; ++t) iteration(t, GE{});
   // drain: softmax of the last half tile, accumulation of the last two
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
-  if constexpr (MASK != MASK_NONE) {
-#pragma unroll
-    for (int c = 0; c < 2; ++c) mcur[0][c] = mnext[0][c];
-  } else {
-    jA = (ntiles - 1) * BN;
-  }
-  slot(B0{}, B1{}, B1{}, G2{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
-       jA + 32, mcur[0]);
-  slot(B0{}, B1{}, B0{}, G2{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0, mcur[0]);
+  if constexpr (!MASKED) jA = (ntiles - 1) * BN;
+  slot(B0{}, B1{}, B1{}, GE{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 0), SX, SpX, SY, SpY, pfA, psfA, pfB, psfB,
+       jA + 32, mcur[0], madd);
+  slot(B0{}, B1{}, B0{}, GE{}, std::integral_constant<int, -1>{}, B0{}, B0{}, 0u, kad(ntiles - 1, 1), SY, SpY, SX, SpX, pfB, psfB, pfA, psfA, 0,
+       mcur[0], madd);
   // the last accumulation has written its registers
   if constexpr (DUAL) accs_ready(Oacc, Tacc);
   else accs_ready(Oacc);
@@ -662,8 +684,9 @@ __global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
     return;
   }
   const bool dead = !(l_i > 0.f);
-  const float inv = dead ? 0.f : 1.f / l_i;
-  const float mu_n = mu_i * inv;
+  const float inv_l = dead ? 0.f : 1.f / l_i;
+  const float mu_n = mu_i * inv_l;
+  const float inv = DROP ? inv_l * pr.drop_rinv : inv_l;  // the kept entries' 1 / (1 - p) is common to O and T
   if (qrow < L) {
     T *Og = reinterpret_cast<T *>(p.o) + head + (size_t)qrow * D;
     T *Otg = DUAL ? reinterpret_cast<T *>(p.ot) + head + (size_t)qrow * D : nullptr;

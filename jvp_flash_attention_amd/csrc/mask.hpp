@@ -78,9 +78,46 @@ __device__ __forceinline__ MaskAhead<T, MASK> mask_fetch8_any(const Problem &pr,
   }
   return m;
 }
+// The same with keys past the end delivered as masked (byte 0 / minus infinity), for callers that apply no limit
+// of their own.
+template <typename T, int MASK>
+__device__ __forceinline__ MaskAhead<T, MASK> mask_fetch8_lim(const Problem &pr, int64_t rowoff, int key0) {
+  MaskAhead<T, MASK> m;
+  if constexpr (MASK == MASK_BOOL) {
+    const uint8_t *base = reinterpret_cast<const uint8_t *>(pr.mask) + rowoff;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t raw = base[(int64_t)min(key0 + e, pr.Lk - 1) * pr.ms[3]];
+      const uint32_t b = (raw != 0 && key0 + e < pr.Lk) ? 0xffu : 0u;
+      if (e < 4) lo |= b << (8 * e);
+      else hi |= b << (8 * (e - 4));
+    }
+    m.w = (uint64_t)lo | ((uint64_t)hi << 32);
+  } else {
+    const T *base = reinterpret_cast<const T *>(pr.mask) + rowoff;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const T raw = base[(int64_t)min(key0 + e, pr.Lk - 1) * pr.ms[3]];
+      m.f[e] = key0 + e < pr.Lk ? raw : (T)(-__builtin_inff());
+    }
+  }
+  return m;
+}
 template <typename T, int MASK> __device__ __forceinline__ bool mask_keep_of(const MaskAhead<T, MASK> &m, int e) {
   const uint32_t half = e < 4 ? (uint32_t)m.w : (uint32_t)(m.w >> 32);  // 32-bit tests: 64-bit shifts are slow
   return (half & (0xffu << (8 * (e & 3)))) != 0;
+}
+// 0 for an attended key, minus infinity for a masked one, from byte K of a word of four mask bytes (two
+// instructions: the comparison selects its byte itself).  zero and ninf are vector registers that hold 0 and the
+// bits of minus infinity (a literal next to vcc would be one constant-bus operand too many).
+template <int K> __device__ __forceinline__ float mask_term_of_byte(uint32_t word, uint32_t zero, uint32_t ninf) {
+  float t;
+  if constexpr (K == 0) asm("v_cmp_eq_u32_sdwa vcc, %1, %2 src0_sel:BYTE_0 src1_sel:DWORD\n\tv_cndmask_b32_e32 %0, 0, %3, vcc" : "=v"(t) : "v"(word), "v"(zero), "v"(ninf) : "vcc");
+  if constexpr (K == 1) asm("v_cmp_eq_u32_sdwa vcc, %1, %2 src0_sel:BYTE_1 src1_sel:DWORD\n\tv_cndmask_b32_e32 %0, 0, %3, vcc" : "=v"(t) : "v"(word), "v"(zero), "v"(ninf) : "vcc");
+  if constexpr (K == 2) asm("v_cmp_eq_u32_sdwa vcc, %1, %2 src0_sel:BYTE_2 src1_sel:DWORD\n\tv_cndmask_b32_e32 %0, 0, %3, vcc" : "=v"(t) : "v"(word), "v"(zero), "v"(ninf) : "vcc");
+  if constexpr (K == 3) asm("v_cmp_eq_u32_sdwa vcc, %1, %2 src0_sel:BYTE_3 src1_sel:DWORD\n\tv_cndmask_b32_e32 %0, 0, %3, vcc" : "=v"(t) : "v"(word), "v"(zero), "v"(ninf) : "vcc");
+  return t;
 }
 template <typename T, int MASK> __device__ __forceinline__ float mask_bias_of(const MaskAhead<T, MASK> &m, int e) {
   return (float)m.f[e] * LOG2E;

@@ -246,3 +246,33 @@ def test_dropout_inside_torch_compile_runs_between_two_compiled_pieces():
     for a, b in zip(g, gref):
         assert torch.equal(a, b)
     assert not torch.equal(f(q, k, v), ref)  # the next draw is another pattern
+
+
+def test_a_recorded_dropout_call_replays_its_pattern():
+    """The seed is a kernel argument drawn on the host: a forward with dropout recorded into a HIP graph replays with
+    the seed it was recorded with, the same keep pattern every time (callers that want a fresh pattern per step
+    record anew).  Pinned here so that the behaviour is a documented one."""
+    from jvp_flash_attention_amd import _lib
+
+    be = _lib.backend()
+    Z, H, L, D = 1, 2, 256, 64
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q, k, v = [torch.randn(Z, H, L, D, generator=g, device="cuda").to(torch.bfloat16) for _ in range(3)]
+    scale = D**-0.5
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        be.fwd(q, k, v, None, None, None, None, _lib.MASK_NONE, False, scale, 0.5, 1234)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o = be.fwd(q, k, v, None, None, None, None, _lib.MASK_NONE, False, scale, 0.5, 1234)[0]
+    graph.replay()
+    torch.cuda.synchronize()
+    first = o.clone()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(first, o)
+    assert torch.equal(first, be.fwd(q, k, v, None, None, None, None, _lib.MASK_NONE, False, scale, 0.5, 1234)[0])
+    assert not torch.equal(first, be.fwd(q, k, v, None, None, None, None, _lib.MASK_NONE, False, scale, 0.5, 1235)[0])

@@ -24,6 +24,10 @@ def _tol_check(name, got, ref, dtype, floor=1e-30):
     err = np.abs(got - ref).max()
     if dtype == torch.float32:
         assert err <= 1e-4, f"{name}: max-abs {err:.3e} > 1e-4"
+    elif np.abs(ref).max() == 0.0:
+        # a quantity that is exactly zero (every row attends a single key, so dS cancels): the 16-bit kernels
+        # return the rounding residue of the stored O, O', held to the absolute bound of test_single_key
+        assert err <= 5e-2, f"{name}: max-abs {err:.3e} > 5e-2 where the exact value is 0"
     else:
         rel = err / max(np.abs(ref).max(), floor)
         assert rel <= 2e-2, f"{name}: relative {rel:.3e} > 2e-2"
@@ -605,12 +609,31 @@ def test_growing_row_maximum_exercises_the_rescale_path(dt, D, causal):
         got = got.double().cpu().numpy()
         rel = np.abs(got - want).max() / np.abs(want).max()
         assert np.isfinite(got).all() and rel <= (2e-5 if dtype == torch.float32 else 2e-2), (name, rel)
-    assert np.abs(M.double().cpu().numpy() - ref["M"]).max() < (1e-3 if dtype == torch.float32 else 0.25)
+    # M is kept in fp32 from identical inputs in every element type: log2 units at values near 90
+    assert np.abs(M.double().cpu().numpy() - ref["M"]).max() < (1e-3 if dtype == torch.float32 else 2e-2)
     grads = be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], None, _lib.MASK_NONE, causal, scale, want_tangent_grads=True)
     for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), grads):
         got = t.double().cpu().numpy()
         rel = np.abs(got - rb[n]).max() / np.abs(rb[n]).max()
         assert np.isfinite(got).all() and rel <= (5e-5 if dtype == torch.float32 else 2e-2), (n, rel)
+
+
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("mode", ["none", "causal", "bias"])
+@pytest.mark.parametrize("std", [64.0, 256.0])
+def test_fp16_tangents_of_large_norm(D, mode, std):
+    """An HVP caller passes a vector of whatever norm it has.  The operand P (S' - c) of the tangent accumulation is
+    a 16-bit number: with fp16 it overflows once p |S' - c| passes 65504, and the lazy rescale lets p exceed 1, so
+    the fp16 kernels keep its slack at 2^2 (|S' - c| reaches about 2000 here; the reference's p <= 1 holds to
+    65504).  Every forward kernel family for fp16 (direct-to-LDS, software-pipelined with and without a mask, the
+    D = 256 pair of passes) and the backward behind it."""
+    _run_case(1, 2, 320, D, torch.float16, mode, seed=71, tangent_std=std)
+
+
+def test_config1_shape_and_seed_on_the_gpu():
+    """Benchmark configuration 1 (fp32, B2 H4 L128 D64, seed 0, every tensor iid N(0,1), no mask) is the
+    reference's CPU plumbing case; the same tensors through the HIP kernels, held to max-abs 1e-4."""
+    _run_case(2, 4, 128, 64, torch.float32, "none", seed=0)
 
 
 @pytest.mark.parametrize("dt,D", [("bf16", 64), ("fp32", 64), ("bf16", 32), ("bf16", 128), ("bf16", 256)])
@@ -692,8 +715,6 @@ def test_grouped_heads_and_a_key_length_of_its_own(dt, D, shape, mode):
 def test_head_dim_256_with_grouped_heads_key_lengths_and_tiny_shapes(dt, shape, mode):
     """The D = 256 kernels (two forward passes over 32-key tiles; a backward whose workgroups are two pairs
     of waves that share 32 rows) on the shapes of the test above, down to a single query."""
-    if mode == "causal" and shape == (1, 1, 1, 3):
-        pytest.skip("one query sees one key under the causal rule: every gradient of q is exactly zero")
     _run_kv_shape_case(dt, 256, shape, mode)
 
 

@@ -51,6 +51,52 @@ def test_static_scratch_backward_matches_the_workspace_backward_twice_in_a_row()
     _both_ways(_lib, 2, 4, 700, 128, torch.bfloat16, True, 3)
 
 
+def test_static_scratch_backward_under_graph_capture_allocates_nothing():
+    """What the entry point is for: after one eager call on the device (which looks the array's address up), a call
+    recorded into a HIP graph; replays with fresh inputs match the workspace backward bit for bit, and the device's
+    free memory does not move across the eager calls that follow the first."""
+    from jvp_flash_attention_amd import _lib
+
+    lib = _lib.load()
+    Z, H, L, D, dtype, causal = 2, 4, 300, 128, torch.bfloat16, True
+    scale = D**-0.5
+    g = torch.Generator(device="cuda").manual_seed(11)
+    t = [torch.randn(Z, H, L, D, generator=g, device="cuda").to(dtype) for _ in range(8)]
+    o, ot, M, mu = _lib.backend().fwd(*t[:6], None, _lib.MASK_NONE, causal, scale)
+    ws = torch.empty(lib.jvpfa_bwd_workspace_bytes(Z, H, L), device="cuda", dtype=torch.uint8)
+    got = [torch.empty_like(t[0]) for _ in range(6)]
+    want = [torch.empty_like(t[0]) for _ in range(6)]
+    args = _args(_lib, t, o, ot, M, mu, got, causal, scale, None)
+    stream = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib.jvpfa_bwd_static(C.byref(args), stream))  # the first call on this device resolves the array
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        _lib.check(lib.jvpfa_bwd_static(C.byref(args), stream))
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "a later call changed the device's free memory"
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    print("case static scratch under capture", flush=True)
+    with torch.cuda.graph(graph, stream=side):
+        _lib.check(lib.jvpfa_bwd_static(C.byref(args), torch.cuda.current_stream().cuda_stream))
+    for rep in range(3):
+        g2 = torch.Generator(device="cuda").manual_seed(100 + rep)
+        for x in t:
+            x.copy_(torch.randn(Z, H, L, D, generator=g2, device="cuda").to(dtype))
+        fo, fot, fM, fmu = _lib.backend().fwd(*t[:6], None, _lib.MASK_NONE, causal, scale)
+        for dst, src in ((o, fo), (ot, fot), (M, fM), (mu, fmu)):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        _lib.check(lib.jvpfa_bwd(C.byref(_args(_lib, t, o, ot, M, mu, want, causal, scale, ws)), stream))
+        torch.cuda.synchronize()
+        for name, a_, b_ in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), got, want):
+            assert torch.equal(a_, b_), f"replay {rep}: {name}"
+
+
 def test_static_scratch_backward_refuses_what_does_not_fit():
     from jvp_flash_attention_amd import _lib
 
