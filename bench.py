@@ -51,7 +51,11 @@ def timed(fn, steps, warmup):
 
 
 def cpu_baseline():
-    """Reference CPU route on a B=1, H=2 slab of the headline shape, scaled to the full shape."""
+    """Reference CPU route (math SDPA under torch.func.jvp, fp32) on this host's cores: one warm-up and three timed
+    runs of a bounded sample of the headline workload, the median reported.  The sample is sized for about 5 s per
+    run (the whole B*H = 64 heads where the host is fast enough, otherwise as many heads as fit)."""
+    import statistics
+
     import torch
 
     from oracle import sdpa_jvp
@@ -66,22 +70,21 @@ def cpu_baseline():
         sdpa_jvp.forward(q, k, v, qt, kt, vt)
         return time.perf_counter() - t0
 
-    run(1, 1)  # warm-up
+    run(1, 1)  # pages in the libraries
     t2 = run(1, 2)
-    # size the sample for roughly 15 s of CPU work, at most the whole B*H = 64 heads
-    zb, hb = 1, 2
-    dt = t2
-    heads = int(min(Z * H, max(2, 15.0 / max(t2 / 2, 1e-3))))
-    if heads > 2:
-        zb, hb = (1, heads) if heads <= H else (heads // H, H)
-        dt = run(zb, hb)
+    heads = int(min(Z * H, max(2, 5.0 / max(t2 / 2, 1e-3))))
+    zb, hb = (1, heads) if heads <= H else (heads // H, H)
+    run(zb, hb)  # warm-up at the sample's size
+    runs = sorted(run(zb, hb) for _ in range(3))
+    dt = statistics.median(runs)
     flops = 12.0 * zb * hb * L * L * D
     return {
         "value": flops / dt / 1e12,
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"math SDPA + torch.func.jvp fp32 dual forward on B={zb},H={hb},L={L},D={D} ({dt:.1f} s)"
+        "sample": f"math SDPA + torch.func.jvp fp32 dual forward on B={zb},H={hb},L={L},D={D}: 1 warm-up + 3 runs, median "
+                  f"{dt:.2f} s (min {runs[0]:.2f}, max {runs[-1]:.2f})"
                   + ("; the whole headline shape" if zb * hb == Z * H
                      else f"; {zb * hb} of {Z * H} heads, the whole shape would take ~{dt * Z * H / (zb * hb):.0f} s"),
     }

@@ -64,13 +64,26 @@ static int launch_fwd_wide_one(const FwdParams &p, hipStream_t stream) {
   // and then the tangent pass (O', mu) with the final M: seven products, where two workgroups with a
   // column half each would compute nine.
   using Cfg = FwdWideCfg<T, D, false>;
-  auto kern = fwd_wide_kernel<T, D, false, MASK, false, DROP>;
-  int rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
-  if (rc != 0) return rc;
   const int nqb = (p.pr.L + Cfg::BM - 1) / Cfg::BM;
   const long long blocks = (long long)nqb * p.pr.Z * p.pr.H;
   if (blocks > 0x7fffffffLL) return -2;
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
+  int rc = 0;
+  if constexpr (MASK == MASK_NONE && !DROP && !DUAL) {
+    // O and M from the software-pipelined kernel: without tangents its resident Q and accumulator fit at
+    // D = 256 too (64-key tiles, two stages of K and V = 128 KB of LDS).  (As the first pass of the dual forward
+    // it is 7 % faster as well, but the tangent pass's O' then misses the 2e-2 bar on dq in one test with very
+    // peaked rows, where its reference c for S', the first tile's mean, is far from the row's mu.)
+    using Cfg3 = Fwd2Cfg<T, D, false>;
+    auto k3 = fwd3_kernel<T, D, false>;
+    rc = allow_lds(reinterpret_cast<const void *>(k3), Cfg3::LDS_BYTES);
+    if (rc != 0) return rc;
+    hipLaunchKernelGGL(k3, dim3((unsigned)blocks), dim3(Cfg3::NT), Cfg3::LDS_BYTES, stream, p);
+  } else {
+    auto kern = fwd_wide_kernel<T, D, false, MASK, false, DROP>;
+    rc = allow_lds(reinterpret_cast<const void *>(kern), Cfg::LDS_BYTES);
+    if (rc != 0) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, p);
+  }
   if constexpr (DUAL) {
     using CfgT = FwdWideCfg<T, D, true>;
     auto kt = fwd_wide_kernel<T, D, true, MASK, true, DROP>;

@@ -133,10 +133,13 @@ __device__ __forceinline__ void pin_acc(f32x16 &c) { asm volatile("" : "+a"(c));
 // 32 idle issue slots behind the last in-place accumulation, tied to the tiles: code the compiler generates to
 // read them (the epilogue) cannot be scheduled in front of the wait, which a bare asm statement would allow.
 template <int N> __device__ __forceinline__ void accs_ready(f32x16 (&o)[N]) {
-  static_assert(N == 1 || N == 2 || N == 4);
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8);
   if constexpr (N == 1) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]));
   if constexpr (N == 2) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]));
   if constexpr (N == 4) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]));
+  if constexpr (N == 8)
+    asm volatile("s_nop 15\n\ts_nop 15"
+                 : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7]));
 }
 template <int N> __device__ __forceinline__ void accs_ready(f32x16 (&o)[N], f32x16 (&t)[N]) {
   static_assert(N == 1 || N == 2 || N == 4);
@@ -194,7 +197,7 @@ __device__ __forceinline__ int list_take(int v) {
 // (CH = 4, rows of 64 bytes: four rows share a line of 256 bytes, which the transposing read of four
 // consecutive rows covers exactly, so only the row-wise read needs its chunks moved)
 template <int CH> __device__ __forceinline__ int swz_k(int row) {
-  return CH == 16 ? (row & 15) : CH == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3);
+  return (CH == 32 || CH == 16) ? (row & 15) : CH == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
 // Tiles read by the transposing read only.  (CH = 32, 16: every row starts a 256-byte line, rows 0..3 move
 // bits 2-3; CH = 8: two rows share a line and differ in the bank already, rows 2-3 move bit 2.)

@@ -1,9 +1,10 @@
 // Small grids: when a launch has fewer workgroups than the GPU has compute units (one sequence of a few
 // thousand tokens, a handful of heads), the kernels for 16-bit element types with D = 128 and no mask split
 // the streamed tiles of every block of owned rows over several workgroups ("chunks").  Each writes fp32
-// partial results to a workspace and a merge kernel combines them: for the backward a plain sum, for the
-// forward the online-softmax merge (every running quantity is linear in p once the reference points m and c
-// are made common).  The reference has nothing like it (one program per 32 query rows, jvp_attention.py:2474).
+// partial results to a workspace and a merge kernel combines them with the online-softmax merge (every running
+// quantity is linear in p once the reference points m and c are made common).  Forward only: the backward of
+// such a launch runs its dk/dv and dq workgroups side by side in one launch instead (bwd2_both_kernel).  The
+// reference has nothing like it (one program per 32 query rows, jvp_attention.py:2474).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stddef.h>
@@ -53,11 +54,6 @@ inline int device_cus() {
 // Workspace of the forward: per chunk and query row 2 D accumulator values (O, T, not yet divided by l) and
 // four statistics (m, l, mu_acc, c).
 inline size_t fwd_part_floats(int chunks, long long rows, int D) { return (size_t)chunks * rows * (2 * (size_t)D + 4); }
-// Workspace of the backward: per chunk dq (rows x D) and dk, dv (kv_rows x D each).
-inline size_t bwd_part_floats(int chunks, long long rows, long long kv_rows, int D) {
-  return (size_t)chunks * ((size_t)rows + 2 * (size_t)kv_rows) * D;
-}
-
 // The kernels that can split: 16-bit element types, D = 128, no mask (the software-pipelined forward and the
 // direct-to-LDS backward kernels).  Tiles are 64 wide, blocks 128 rows.
 template <typename P> inline bool split_capable(const P &p) {
@@ -129,27 +125,6 @@ __global__ __launch_bounds__(256) void fwd_merge_kernel(const float *part, int c
     M[row] = dead ? __builtin_inff() : m + __builtin_amdgcn_logf(l);
     if constexpr (DUAL) mu[row] = dead ? 0.f : mu_n + cref;
   }
-}
-
-// Backward: out = sum over chunks of part[chunk][n], n over rows x D (already scaled by the kernels).
-template <typename T, int D>
-__global__ __launch_bounds__(256) void bwd_merge_kernel(const float *part, size_t chunk_stride, int chunks, long long n8,
-                                                        T *out) {
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n8) return;
-  float x[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) x[e] = 0.f;
-  for (int c = 0; c < chunks; ++c) {
-    const float *src = part + (size_t)c * chunk_stride + (size_t)i * 8;
-    const f32x4 a = *reinterpret_cast<const f32x4 *>(src), b = *reinterpret_cast<const f32x4 *>(src + 4);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      x[e] += a[e];
-      x[4 + e] += b[e];
-    }
-  }
-  store8<T>(out + (size_t)i * 8, x);
 }
 
 }  // namespace jvpfa
