@@ -126,6 +126,7 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
       }
     } else {
       if (plain_q) kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG> : bwd2_dq_kernel<T, D, MODE, MASK, true>;
+      if constexpr (D == 128 && MODE == BWD_PLAIN) kq = bwd2_dq_kernel_2wg_plain<T, D, MODE, MASK>;
       if (!plain_kv) {
       } else if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true>;
       else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;

@@ -137,7 +137,9 @@ __device__ __forceinline__ void zero_acc(f32x16 &x) {
 // SIX (dual mode only): dq' = scale dS' K as well, from the K fragments and the dS' tiles that dq already has.
 // DROP: dropout (see bwd_kernel.hpp): gO V^T, gT V^T and gT V'^T reach the logits through the kept, rescaled
 // entries only.
-template <typename T, int D, int MODE, int MASK, bool GO, bool SIX, bool DROP = false>
+// LEAN: one tile loop (every tile takes the limit tests) instead of an interior loop and an edge loop: less for
+// the compiler to keep in registers, for the variant that must stay within 256 of them.
+template <typename T, int D, int MODE, int MASK, bool GO, bool SIX, bool DROP = false, bool LEAN = false>
 __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) {
   using Cfg = Bwd2Cfg<T, D, MODE>;
   constexpr bool DUAL = MODE == BWD_DUAL, TAN = MODE == BWD_TANGENT;
@@ -427,7 +429,9 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
   if (pr.causal) t_edge = min(t_edge, q0 / BT);
   if (MASK != MASK_NONE && !mask_al) t_edge = 0;  // interior tiles fetch mask rows with aligned vector loads
   int t = 0;
-  for (; t < ntiles && tcur < t_edge; ++t) tile(t, std::false_type{});
+  if constexpr (!LEAN) {
+    for (; t < ntiles && tcur < t_edge; ++t) tile(t, std::false_type{});
+  }
   for (; t < ntiles; ++t) tile(t, std::true_type{});
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the redirected loads of the last iteration must not outlive the kernel
 
@@ -463,6 +467,16 @@ template <typename T, int D, int MODE, int MASK, bool GO, bool SIX = false>
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(160))) void bwd2_dq_kernel_2wg(const BwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   bwd2_dq_body<T, D, MODE, MASK, GO, SIX>(p, blockIdx.x);
+#endif
+}
+
+// D = 128 without tangents: Q, gO and the dq accumulator are 128 accumulation registers, so with the vector
+// registers capped at 128 a wave stays within 256 and two workgroups (64 KB of LDS each) share a compute unit.
+template <typename T, int D, int MODE, int MASK>
+__global__ __launch_bounds__(256, 2) void bwd2_dq_kernel_2wg_plain(const BwdParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  static_assert(MODE == BWD_PLAIN && D == 128);
+  bwd2_dq_body<T, D, MODE, MASK, true, false, false, MASK == MASK_NONE>(p, blockIdx.x);
 #endif
 }
 

@@ -46,8 +46,12 @@ template <int N> __device__ __forceinline__ void lds_wait3(u32x4 &a, u32x2 &c, u
 // DROP: dropout on the probabilities (see fwd_kernel.hpp): what enters the products with V, V' is
 // P * keep / (1 - p), hashed per entry in the gaps between the matrix instructions; l, mu stay those of the
 // full softmax.
-template <typename T, int D, bool DUAL, int MASK = MASK_NONE, bool DROP = false>
-__global__ __launch_bounds__(256, 1) void fwd3_kernel(const FwdParams p) {
+// WGS: workgroups meant to share a compute unit.  Without tangents at D = 128, Q and the accumulator are 96
+// registers and a stage pair 64 KB, so two fit; the unmasked kernel stays within 256 registers by itself, the
+// masked ones are told to.
+template <typename T, int D, bool DUAL, int MASK = MASK_NONE, bool DROP = false,
+          int WGS = (!DUAL && D <= 128 && (MASK != MASK_NONE || DROP)) ? 2 : 1>
+__global__ __launch_bounds__(256, WGS) void fwd3_kernel(const FwdParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (and has no buffer descriptor type)
   using Cfg = Fwd2Cfg<T, D, DUAL>;
   constexpr int BN = Cfg::BN, CH = Cfg::CH, ROWB = Cfg::ROWB, TILEB = Cfg::TILEB, IPW = Cfg::IPW;
