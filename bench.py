@@ -146,10 +146,10 @@ def shape_rows(be, _lib):
         q, qt, go, gt = [mk(Hs, Lq) for _ in range(4)]
         k, v, kt, vt = [mk(Hk, Lk) for _ in range(4)]
         scale = Ds**-0.5
-        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale, dp, 7), 10, 3)
+        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale, dp, 7), 20, 12)
         o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale, dp, 7)
         ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, None, _lib.MASK_NONE, False, scale,
-                                       dropout_p=dp, dropout_seed=7), 5, 2)
+                                       dropout_p=dp, dropout_seed=7), 10, 6)
         n = float(Zs) * Hs * Lq * Lk * Ds
         rows[name] = {"fwd_ms": ms_f, "fwd_tflops": 12 * n / (ms_f * 1e-3) / 1e12,
                       "bwd_ms": ms_b, "bwd_tflops": 24 * n / (ms_b * 1e-3) / 1e12}
@@ -172,9 +172,9 @@ def shape_rows(be, _lib):
         else:
             mask, kind = torch.randn(Zs, Hs, Ls, Ls, generator=g, device=dev).to(dtype), _lib.MASK_ADD
         scale = Ds**-0.5
-        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, mask, kind, causal, scale), 10, 3)
+        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, mask, kind, causal, scale), 20, 12)
         o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, mask, kind, causal, scale)
-        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, kind, causal, scale), 5, 2)
+        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, kind, causal, scale), 10, 6)
         n = float(Zs) * Hs * Ls * Ls * Ds * frac
         rows[name] = {"attended_fraction": frac, "fwd_ms": ms_f, "fwd_tflops": 12 * n / (ms_f * 1e-3) / 1e12,
                       "bwd_ms": ms_b, "bwd_tflops": 24 * n / (ms_b * 1e-3) / 1e12}
@@ -199,16 +199,16 @@ def mask_rows(be, _lib, q, k, v, qt, kt, vt, go, gt, scale):
     }
     rows = {}
     for name, m in masks.items():
-        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, m, _lib.MASK_BOOL, False, scale), 10, 3)
+        ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, m, _lib.MASK_BOOL, False, scale), 20, 12)
         o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, m, _lib.MASK_BOOL, False, scale)
-        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, m, _lib.MASK_BOOL, False, scale), 5, 2)
+        ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, m, _lib.MASK_BOOL, False, scale), 10, 6)
 
         def scan():
             if hasattr(m, "_jvpfa_tiles"):
                 del m._jvpfa_tiles
             _lib.tile_lists(q, m, _lib.MASK_BOOL, True)
 
-        ms_s, _ = timed(scan, 5, 2)
+        ms_s, _ = timed(scan, 10, 6)
         rows[name] = {"attended_fraction": m.float().mean().item(), "fwd_ms": ms_f, "bwd_ms": ms_b, "scan_ms": ms_s,
                       "scan_GBps": 2.0 * m.numel() / (ms_s * 1e-3) / 1e9}
         del m

@@ -254,9 +254,10 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
   // maximum exceeds it by more than RESCALE_TAU (log2 units), so p <= 2^TAU and the accumulators,
   // which live in the matrix-core accumulation registers, are touched by VALU code only on the few
   // tiles where the running maximum really grows.  O = acc / l is unchanged by the choice of m_i.
-  // (fp16: p multiplies S' - c in a 16-bit operand that overflows at 65504, so the slack is 2^2 there: |S' - c| up
-  // to 16 000, where the reference's p <= 1 gives 65 504; bf16 has the exponent range for 2^8)
-  constexpr float RESCALE_TAU = __is_same(T, _Float16) ? 2.f : 8.f;
+  // (fp16: p multiplies S' - c in a 16-bit operand that overflows at 65504, so the slack is 2^4 there: |S' - c| up
+  // to 4 000, where the reference's p <= 1 gives 65 504, see fwd_kernel_v3.hpp; bf16 has the exponent range for 2^8)
+  constexpr float RESCALE_TAU = __is_same(T, _Float16) ? 4.f : 8.f;
+  constexpr float RESCALE_LEAD = __is_same(T, _Float16) ? 2.f : 0.f;  // the reference point moves this far past the new maximum
   MaskAhead<T, MASK> mcur[2][2], mnext[2][2];  // mask values of this tile and the next: [half tile][16-key group]
   const int klim = min(pr.causal ? qrow : 0x7fffffff, Lk - 1);  // keys above this index are masked
   // EDGE: the half tile may cross the causal diagonal or the end of the sequence, the scale may be
@@ -353,8 +354,10 @@ __global__ __launch_bounds__(256, 1) void fwd2_kernel(const FwdParams p) {
     const bool up = mx > m_i + RESCALE_TAU;
     float alpha = 1.f;
     if (__builtin_expect(__any(up), 0)) {
-      alpha = up ? fast_exp2(m_i - mx) : 1.f;
-      m_i = up ? mx : m_i;
+      float m_new = mx;
+      if constexpr (RESCALE_LEAD != 0.f) m_new = mx + RESCALE_LEAD;
+      alpha = up ? fast_exp2(m_i - m_new) : 1.f;
+      m_i = up ? m_new : m_i;
     }
     // V fragments of the first PV steps travel while the softmax runs
     static_for<(PD < NPV ? PD : NPV)>([&](auto ic) { issue_v(ic); });

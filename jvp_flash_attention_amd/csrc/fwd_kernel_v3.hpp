@@ -252,9 +252,16 @@ __global__ __launch_bounds__(256, WGS) void fwd3_kernel(const FwdParams p) {
     }
   };
 
-  // fp16: p <= 2^TAU multiplies S' - c in a 16-bit operand that overflows at 65504, so the slack is 2^2 there
-  // (|S' - c| up to 16 000; the reference's p <= 1 gives 65 504); bf16 has the exponent range for 2^8
-  constexpr float RESCALE_TAU = __is_same(T, _Float16) ? 2.f : 8.f;
+  // fp16: p <= 2^TAU multiplies S' - c in a 16-bit operand that overflows at 65504, so the slack is 2^4 there
+  // (|S' - c| up to 4 000; the reference's p <= 1 gives 65 504).  The running maximum of a row of unit-variance
+  // logits grows by about 2 log2 units between its first tile and its 64th, so 2^4 is still rarely crossed; with
+  // 2^2 every row crosses it about once and the rescale block costs 27 % of the kernel.  bf16 has the exponent
+  // range for 2^8.
+  constexpr float RESCALE_TAU = __is_same(T, _Float16) ? 4.f : 8.f;
+  // ... and when the reference point does move, fp16 puts it 2 log2 units above the new maximum (p <= 1/4 on that
+  // tile, and the next move waits for a maximum 6 above this one), so that the smaller slack does not make the
+  // moves frequent: rows whose maximum climbs by more than 4 over the sequence are common, by more than 6 rare
+  constexpr float RESCALE_LEAD = __is_same(T, _Float16) ? 2.f : 0.f;
   constexpr int NQ = DUAL ? 3 : 1, NP = DUAL ? 3 : 1;  // matrix instructions per super-step: scores, accumulation
   constexpr int NRS = DUAL ? 2 : 1, NRV = DUAL ? 4 : 2;  // LDS reads per super-step
   constexpr int NU = 38;                                 // vector units of one softmax
@@ -333,8 +340,10 @@ __global__ __launch_bounds__(256, WGS) void fwd3_kernel(const FwdParams p) {
         const bool up = mx > m_i + RESCALE_TAU;
         up_l = up;
         if constexpr (!DUAL) any_up = __any(up);
-        alpha = up ? fast_exp2(m_i - mx) : 1.f;
-        m_i = up ? mx : m_i;
+        float m_new = mx;
+        if constexpr (RESCALE_LEAD != 0.f) m_new = mx + RESCALE_LEAD;
+        alpha = up ? fast_exp2(m_i - m_new) : 1.f;
+        m_i = up ? m_new : m_i;
         anchor(alpha);
       } else if constexpr (u == 4) {
         m_use = (m_i == NEG_INF) ? 0.f : m_i;

@@ -624,8 +624,8 @@ def test_growing_row_maximum_exercises_the_rescale_path(dt, D, causal):
 def test_fp16_tangents_of_large_norm(D, mode, std):
     """An HVP caller passes a vector of whatever norm it has.  The operand P (S' - c) of the tangent accumulation is
     a 16-bit number: with fp16 it overflows once p |S' - c| passes 65504, and the lazy rescale lets p exceed 1, so
-    the fp16 kernels keep its slack at 2^2 (|S' - c| reaches about 2000 here; the reference's p <= 1 holds to
-    65504).  Every forward kernel family for fp16 (direct-to-LDS, software-pipelined with and without a mask, the
+    the fp16 kernels keep its slack at 2^4 (|S' - c| reaches about 2000 here, the kernels hold to 4000; the
+    reference's p <= 1 holds to 65504).  Every forward kernel family for fp16 (direct-to-LDS, software-pipelined with and without a mask, the
     D = 256 pair of passes) and the backward behind it."""
     _run_case(1, 2, 320, D, torch.float16, mode, seed=71, tangent_std=std)
 
