@@ -142,17 +142,16 @@ __global__ __launch_bounds__(256, WGS) void fwd3_kernel(const FwdParams p) {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) koff[kk] = pr32 * ROWB + (((2 * kk + g) ^ x) * 16);
   }
-  uint32_t voff[DB][2];
+  // (the second transposing read of a fragment takes rows 4 further down: the same chunk, since the V-type swizzle
+  // only looks at the two low bits of the row, so it is the first one's address plus a constant)
+  uint32_t voff[DB];
   {
     const int a = (lane >> 4) & 1, j = lane & 15;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        const int row = 8 * g + 4 * hh + (j >> 2);
-        const int ch = (4 * db + 2 * a + (j & 1)) ^ swz_v<CH>(row);
-        voff[db][hh] = row * ROWB + ch * 16 + 8 * ((j >> 1) & 1);
-      }
+      const int row = 8 * g + (j >> 2);
+      const int ch = (4 * db + 2 * a + (j & 1)) ^ swz_v<CH>(row);
+      voff[db] = row * ROWB + ch * 16 + 8 * ((j >> 1) & 1);
     }
   }
 
@@ -431,12 +430,13 @@ __global__ __launch_bounds__(256, WGS) void fwd3_kernel(const FwdParams p) {
       if constexpr (PV) {
         constexpr int c = i / DB, db = i % DB;
         constexpr int VO = HO + TILEB + c * 16 * ROWB;
-        const uint32_t a0 = vaddr + voff[db][0], a1 = vaddr + voff[db][1];
+        const uint32_t a0 = vaddr + voff[db];
+        static_assert(VO + (DUAL ? 2 * TILEB : 0) + 4 * ROWB < 65536, "the offset field of an LDS instruction has 16 bits");
         va[sl][0] = lds_tr64<VO>(a0);
-        va[sl][1] = lds_tr64<VO>(a1);
+        va[sl][1] = lds_tr64<VO + 4 * ROWB>(a0);
         if constexpr (DUAL) {
           vb[sl][0] = lds_tr64<VO + 2 * TILEB>(a0);
-          vb[sl][1] = lds_tr64<VO + 2 * TILEB>(a1);
+          vb[sl][1] = lds_tr64<VO + 2 * TILEB + 4 * ROWB>(a0);
         }
       }
     };
