@@ -228,6 +228,9 @@ def main():
     ap.add_argument("--plain-only", action="store_true",
                     help="time the headline shape without tangents (what attention() runs in first-order training): forward, "
                          "then the backward of gO (for profiling); prints its own line")
+    ap.add_argument("--masked-fwd-only", action="store_true",
+                    help="time the headline dual forward with a dense boolean mask, with an additive mask and with dropout "
+                         "0.1 next to the unmasked one (for profiling); prints its own line")
     ap.add_argument("--bwd6-only", action="store_true",
                     help="run one forward, then time the backward that also returns dq', dk', dv' (for profiling)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -278,6 +281,19 @@ def main():
         print(json.dumps({"workload": "bf16 B4 H16 L4096 D128 without tangents: forward (4 N flops), backward of gO (10 N)",
                           "fwd_ms": ms_pf, "fwd_tflops": 4.0 * N / (ms_pf * 1e-3) / 1e12,
                           "bwd_ms": ms_pb, "bwd_tflops": 10.0 * N / (ms_pb * 1e-3) / 1e12}), flush=True)
+        return
+    if args.masked_fwd_only:
+        gm = torch.Generator(device=dev).manual_seed(7)
+        mb = torch.rand(Z, H, L, L, generator=gm, device=dev) > 0.1
+        ma = torch.randn(Z, 1, L, L, generator=gm, device=dev).to(torch.bfloat16)
+        row = {"workload": "bf16 B4 H16 L4096 D128 dual forward: no mask | dense boolean mask (Z,H,L,L), 90 % attended | "
+                           "additive mask (Z,1,L,L) | dropout 0.1"}
+        for name, call in (("none", lambda: fwd()),
+                           ("bool", lambda: be.fwd(q, k, v, qt, kt, vt, mb, _lib.MASK_BOOL, False, scale)),
+                           ("additive", lambda: be.fwd(q, k, v, qt, kt, vt, ma, _lib.MASK_ADD, False, scale)),
+                           ("dropout", lambda: be.fwd(q, k, v, qt, kt, vt, None, _lib.MASK_NONE, False, scale, 0.1, 7))):
+            row[name + "_ms"], _ = timed(call, args.steps, args.warmup)
+        print(json.dumps(row), flush=True)
         return
     if args.bwd6_only:
         o, ot, M, mu = fwd()
