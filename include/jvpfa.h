@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define JVPFA_ABI_VERSION 7
+#define JVPFA_ABI_VERSION 8
 
 enum jvpfa_dtype { JVPFA_BF16 = 0, JVPFA_FP16 = 1, JVPFA_FP32 = 2 };
 
@@ -151,6 +151,7 @@ typedef struct jvpfa_bwd_args {
   const int32_t *tiles_k;   /* the other list of jvpfa_mask_tiles() (dk/dv kernels);
                                tiles_q and tiles_k are both NULL or both set */
   int32_t Lk, Hk;           /* as in jvpfa_fwd_args; dk, dv, dkt, dvt have the shape of k */
+  const uint32_t *mask_bits; /* optional, boolean masks only: the copy written by jvpfa_mask_bits(), or NULL */
 } jvpfa_bwd_args;
 
 int jvpfa_bwd(const jvpfa_bwd_args *args, void *hip_stream);
@@ -194,6 +195,21 @@ size_t jvpfa_bwd_static_max_rows(void);
  */
 size_t jvpfa_mask_tiles_bytes(const jvpfa_problem *p, int32_t Lk, int32_t keys_owned);
 int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t Lk, int32_t *tiles_q, int32_t *tiles_k, void *hip_stream);
+
+/*
+ * A boolean mask packed along the query axis, for the dk/dv kernels: their lanes own a key and walk down the
+ * queries, so from the mask itself they fetch one byte per entry, a mask row apart; from this copy one 32-bit
+ * word per 32 queries.  No counterpart in the reference, whose kernels load the mask block by block
+ * (JA:1451-1463, JA:1607-1619).  Layout: for every mask plane (as for jvpfa_mask_tiles), block of 32 query
+ * rows b < ceil(L/32) and key j < Lk the word [(plane * ceil(L/32) + b) * Lk + j], whose bit i is 1 where the
+ * mask entry of (query 32 b + i, key j) is nonzero; bits of rows past L are 0.  The buffer is
+ * jvpfa_mask_bits_bytes(p, Lk) bytes of device memory (an eighth of the broadcast mask), 4-byte aligned; it
+ * describes the mask's contents: rebuild it when those change.  Only p->Z, H, L, mask_kind (must be
+ * JVPFA_MASK_BOOL), mask and mask_stride are read.  Handing it to jvpfa_bwd is optional and changes no result;
+ * the kernels for 16-bit element types at D <= 128 use it, the others read the mask itself.
+ */
+size_t jvpfa_mask_bits_bytes(const jvpfa_problem *p, int32_t Lk);
+int jvpfa_mask_bits(const jvpfa_problem *p, int32_t Lk, uint32_t *bits, void *hip_stream);
 
 /*
  * The keep pattern of dropout for this problem (only Z, H, L, dropout_p, dropout_seed are read) and Lk keys

@@ -15,10 +15,11 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libjvpfa.so")
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 MASK_NONE, MASK_BOOL, MASK_ADD = 0, 1, 2
 EXPORTS = ("jvpfa_fwd", "jvpfa_bwd", "jvpfa_fwd_split_workspace_bytes", "jvpfa_dropout_keep", "jvpfa_bwd_workspace_bytes", "jvpfa_bwd_static", "jvpfa_bwd_static_max_rows", "jvpfa_mask_tiles", "jvpfa_mask_tiles_bytes",
+           "jvpfa_mask_bits", "jvpfa_mask_bits_bytes",
            "jvpfa_abi_version", "jvpfa_error_string")
 
 
@@ -64,6 +65,7 @@ class BwdArgs(C.Structure):
         ("key_limit", C.c_void_p),
         ("tiles_q", C.c_void_p), ("tiles_k", C.c_void_p),
         ("Lk", C.c_int32), ("Hk", C.c_int32),
+        ("mask_bits", C.c_void_p),
     ]
 
 
@@ -98,6 +100,10 @@ def load() -> C.CDLL:
         lib.jvpfa_mask_tiles_bytes.restype = C.c_size_t
         lib.jvpfa_mask_tiles.argtypes = [C.POINTER(Problem), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.jvpfa_mask_tiles.restype = C.c_int
+        lib.jvpfa_mask_bits_bytes.argtypes = [C.POINTER(Problem), C.c_int32]
+        lib.jvpfa_mask_bits_bytes.restype = C.c_size_t
+        lib.jvpfa_mask_bits.argtypes = [C.POINTER(Problem), C.c_int32, C.c_void_p, C.c_void_p]
+        lib.jvpfa_mask_bits.restype = C.c_int
         lib.jvpfa_abi_version.argtypes = []
         lib.jvpfa_abi_version.restype = C.c_int
         lib.jvpfa_error_string.argtypes = [C.c_int]
@@ -152,7 +158,7 @@ def forget_mask(mask) -> None:
     are keyed by the tensor's version counter, which ordinary in-place operations bump; writes that bypass it
     (``mask.data``, a custom kernel writing through ``data_ptr()``, a dlpack / numpy alias) do not, and after
     such a write this must be called before the mask is used again."""
-    for name in ("_jvpfa_verified", "_jvpfa_key_limit", "_jvpfa_tiles"):
+    for name in ("_jvpfa_verified", "_jvpfa_key_limit", "_jvpfa_tiles", "_jvpfa_bits"):
         try:
             delattr(mask, name)
         except AttributeError:
@@ -253,6 +259,43 @@ def tile_lists(q, mask, mask_kind, want_k, Lk=None):
             except (AttributeError, RuntimeError):
                 pass
     return tq, (tk if want_k else None)
+
+
+MASK_BITS_MIN_L = 512  # below this the backward is too short for the packed copy to pay for its pass over the mask
+_mask_bits_enabled = True
+
+
+def set_mask_bits(enabled: bool) -> None:
+    """Switch the bit-packed copy of boolean masks for the dk/dv kernels on or off (default on)."""
+    global _mask_bits_enabled
+    _mask_bits_enabled = bool(enabled)
+
+
+def mask_bits(q, mask, mask_kind, Lk=None):
+    """For a boolean mask with a row per query (shape [*, *, L, Lk]) and a 16-bit element type at D <= 128: the
+    mask packed along the query axis by ``jvpfa_mask_bits`` (one uint32 per 32 queries and key; an eighth of the
+    broadcast mask's bytes), which the dk/dv kernels read instead of one byte per entry.  None otherwise.  Cached
+    on the mask tensor, keyed by its version counter, like the tile lists."""
+    Z, H, L, D = q.shape
+    Lk = L if Lk is None else Lk
+    if not _mask_bits_enabled or mask is None or mask_kind != MASK_BOOL or max(L, Lk) < MASK_BITS_MIN_L:
+        return None
+    if mask.dim() != 4 or mask.shape[2] != L or mask.shape[3] != Lk or q.element_size() != 2 or D > 128:
+        return None
+    version = mask_version(mask)
+    cached = getattr(mask, "_jvpfa_bits", None)
+    if cached is not None and version is not None and cached[0] == version:
+        return cached[1]
+    lib = load()
+    prob = make_problem(q, mask, mask_kind, False, 1.0)
+    bits = torch.empty(lib.jvpfa_mask_bits_bytes(C.byref(prob), Lk) // 4, device=q.device, dtype=torch.int32)
+    check(lib.jvpfa_mask_bits(C.byref(prob), Lk, _ptr(bits), _stream(q)))
+    if version is not None:
+        try:
+            mask._jvpfa_bits = (version, bits)
+        except (AttributeError, RuntimeError):
+            pass
+    return bits
 
 
 def _require_gpu(*tensors):
@@ -373,6 +416,8 @@ class HipBackend:
             a.key_limit = _ptr(lim)
             tq, tk = tile_lists(q, mask, mask_kind, True, k.shape[2])
             a.tiles_q, a.tiles_k = _ptr(tq), _ptr(tk)
+            bits = mask_bits(q, mask, mask_kind, k.shape[2])
+            a.mask_bits = _ptr(bits)
             check(lib.jvpfa_bwd(C.byref(a), _stream(q)))
         return dq, dk, dv, dqt, dkt, dvt
 

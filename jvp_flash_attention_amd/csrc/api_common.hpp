@@ -32,7 +32,7 @@ inline int check_kv_shape(const jvpfa_problem &p, int32_t Lk, int32_t Hk) {
 }
 
 inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit, const int32_t *tiles_q,
-                          const int32_t *tiles_k, int32_t Lk = 0, int32_t Hk = 0) {
+                          const int32_t *tiles_k, int32_t Lk = 0, int32_t Hk = 0, const uint32_t *mask_bits = nullptr) {
   Problem r;
   r.Lk = Lk > 0 ? Lk : p.L;
   r.Hk = Hk > 0 ? Hk : p.H;
@@ -41,6 +41,7 @@ inline Problem to_problem(const jvpfa_problem &p, const int32_t *key_limit, cons
   const bool lists = masked;
   r.tiles_q = lists ? tiles_q : nullptr;
   r.tiles_k = lists ? tiles_k : nullptr;
+  r.bits_k = p.mask_kind == JVPFA_MASK_BOOL ? mask_bits : nullptr;
   r.klimit = (masked && !r.tiles_q && !r.tiles_k) ? key_limit : nullptr;
   r.chunks = 1;
   r.chunk_tiles = 0;

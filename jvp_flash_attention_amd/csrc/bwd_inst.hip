@@ -22,6 +22,38 @@ template <typename T, int D> struct BwdFold {
   static constexpr bool KV = sizeof(T) == 2 && D <= 64;
 };
 
+// The dk/dv kernel of the direct-to-LDS family for one launch.  MK is MASK, or MASK_BITS for a boolean mask
+// whose bit-packed copy the caller handed over.  fold_kv: the dual variant that also writes dk', dv'.
+template <typename T, int D, int MODE, int MK>
+static auto pick_dkdv(bool no_go, bool grouped, bool fold_kv, bool drop) -> void (*)(const BwdParams) {
+  constexpr bool NG = MODE != BWD_DUAL;  // the GO template argument of the kernels without gO
+  if (drop) {
+    if (grouped) return no_go ? bwd2_dkdv_kernel<T, D, MODE, MK, NG, true, false, true> : bwd2_dkdv_kernel<T, D, MODE, MK, true, true, false, true>;
+    return no_go ? bwd2_dkdv_kernel<T, D, MODE, MK, NG, false, false, true> : bwd2_dkdv_kernel<T, D, MODE, MK, true, false, false, true>;
+  }
+  if constexpr (MODE == BWD_DUAL && BwdFold<T, D>::KV) {
+    if (fold_kv) {
+      if (grouped) return no_go ? bwd2_dkdv_kernel<T, D, MODE, MK, false, true, true> : bwd2_dkdv_kernel<T, D, MODE, MK, true, true, true>;
+      return no_go ? bwd2_dkdv_kernel<T, D, MODE, MK, false, false, true> : bwd2_dkdv_kernel<T, D, MODE, MK, true, false, true>;
+    }
+  }
+  // D = 64: the register-capped twins, two workgroups per compute unit (D = 32 needs no cap for that); the masked
+  // dual kernel needs a few registers more than the cap leaves
+  if constexpr (D == 64 && (MK == MASK_NONE || MODE != BWD_DUAL)) {
+    if (grouped) return no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MK, NG, true> : bwd2_dkdv_kernel_2wg<T, D, MODE, MK, true, true>;
+    return no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MK, NG> : bwd2_dkdv_kernel_2wg<T, D, MODE, MK, true>;
+  }
+  if (grouped) return no_go ? bwd2_dkdv_kernel<T, D, MODE, MK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MK, true, true>;
+  return no_go ? bwd2_dkdv_kernel<T, D, MODE, MK, NG> : bwd2_dkdv_kernel<T, D, MODE, MK, true>;
+}
+template <typename T, int D, int MODE, int MASK>
+static auto pick_dkdv_for(const BwdParams &p, bool no_go, bool grouped, bool fold_kv, bool drop) -> void (*)(const BwdParams) {
+  if constexpr (MASK == MASK_BOOL) {
+    if (p.pr.bits_k) return pick_dkdv<T, D, MODE, MASK_BITS>(no_go, grouped, fold_kv, drop);
+  }
+  return pick_dkdv<T, D, MODE, MASK>(no_go, grouped, fold_kv, drop);
+}
+
 // six: all six gradients were asked for.  The dual launch then also writes what BwdFold says, and the tangent
 // launch skips the kernels whose outputs exist already.
 template <typename T, int D, int MODE, int MASK>
@@ -42,9 +74,7 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
       constexpr bool NG = MODE != BWD_DUAL;
       const bool grouped = p.pr.Hk != p.pr.H;
       void (*kq)(const BwdParams) = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG, false, true> : bwd2_dq_kernel<T, D, MODE, MASK, true, false, true>;
-      void (*kkv)(const BwdParams);
-      if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true, false, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true, false, true>;
-      else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, false, false, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, false, false, true>;
+      void (*kkv)(const BwdParams) = pick_dkdv_for<T, D, MODE, MASK>(p, no_go, grouped, false, true);
       int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
       if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);
       if (rc != 0) return rc;
@@ -107,30 +137,16 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
         // their registers before they have arrived, which the build's lint refuses: that variant runs uncapped)
         if constexpr (D == 64) kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, false, true> : bwd2_dq_kernel_2wg<T, D, MODE, MASK, true, true>;
         else kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, false, true> : bwd2_dq_kernel<T, D, MODE, MASK, true, true>;
-        if constexpr (Fold::KV) {
-          if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, false, true, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true, true>;
-          else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, false, false, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, false, true>;
-        }
       }
     }
-    const bool plain_q = !(MODE == BWD_DUAL && six), plain_kv = !(MODE == BWD_DUAL && six && Fold::KV);
+    const bool plain_q = !(MODE == BWD_DUAL && six);
     if constexpr (D == 64) {  // the register-capped twins: two workgroups per compute unit (D = 32 needs no cap for that)
       if (plain_q) kq = no_go ? bwd2_dq_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dq_kernel_2wg<T, D, MODE, MASK, true>;
-      if (!plain_kv) {
-      } else if constexpr (MASK == MASK_NONE || MODE != BWD_DUAL) {
-        if (grouped) kkv = no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, true, true>;
-        else kkv = no_go ? bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel_2wg<T, D, MODE, MASK, true>;
-      } else {  // the masked dual dk/dv kernel needs a few registers more than the cap leaves
-        if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true>;
-        else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
-      }
     } else {
       if (plain_q) kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG> : bwd2_dq_kernel<T, D, MODE, MASK, true>;
       if constexpr (D == 128 && MODE == BWD_PLAIN) kq = bwd2_dq_kernel_2wg_plain<T, D, MODE, MASK>;
-      if (!plain_kv) {
-      } else if (grouped) kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MASK, true, true>;
-      else kkv = no_go ? bwd2_dkdv_kernel<T, D, MODE, MASK, NG> : bwd2_dkdv_kernel<T, D, MODE, MASK, true>;
     }
+    kkv = pick_dkdv_for<T, D, MODE, MASK>(p, no_go, grouped, MODE == BWD_DUAL && six, false);
     // a grid smaller than the GPU: both roles in one launch, side by side
     const int cus = device_cus();
     if (!grouped && !six && blocks < cus && kv_blocks < cus) {

@@ -569,6 +569,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
   int hq = h * group;
   const char *Qb = nullptr, *gTb = nullptr, *Gb = nullptr, *Qtb = nullptr;
   const float *st_p[4] = {nullptr, nullptr, nullptr, nullptr};
+  const uint32_t *bits_head = nullptr;  // MASK_BITS: the packed mask words of the current query head's plane
   auto set_query_head = [&](int hq_) {
     hq = hq_;
     const size_t qhead = ((size_t)z * pr.H + hq) * L * D * sizeof(T), qrow0 = ((size_t)z * pr.H + hq) * L;
@@ -580,6 +581,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     st_p[1] = MODE == BWD_PLAIN ? p.d1 + qrow0 : (DUAL ? p.mu + qrow0 : p.a + qrow0);
     st_p[2] = DUAL ? p.a + qrow0 : nullptr;
     st_p[3] = DUAL ? p.d2 + qrow0 : nullptr;
+    if constexpr (MASK == MASK_BITS) bits_head = pr.bits_k + mask_bits_offset(pr, z, hq, 0);
   };
   set_query_head(h * group);
 
@@ -643,11 +645,19 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
   // the far caches, so they are requested a whole half tile before their use.  (Where two workgroups
   // share a compute unit, D = 64 outside the dual mode, each value is instead fetched where it is used:
   // the other workgroup covers the wait and the registers stay within the cap.)
-  constexpr bool MAHEAD = D > 64 || MODE == BWD_DUAL;
+  // MASK_BITS: one word per half tile and lane, bit i = (query ihn + i, this lane's key), moved so that bit
+  // 16(e/8) + e%8 belongs to register e; always requested a half tile ahead (it costs one register).
+  constexpr bool MAHEAD = D > 64 || MODE == BWD_DUAL || MASK == MASK_BITS;
   T mnext_a[MASK == MASK_ADD ? 16 : 1];
   uint8_t mnext_b[MASK == MASK_BOOL ? 16 : 1];
+  uint32_t mnext_w = 0;
+  const int nqb = (L + 31) >> 5;
   auto fetch_mask_half = [&](int ihn) {
-    if constexpr (MASK != MASK_NONE) {
+    if constexpr (MASK == MASK_BITS) {
+      // (the second half of the last tile may start past the last row: its entries are masked by index)
+      const uint32_t *wp = bits_head + (size_t)min(ihn >> 5, nqb - 1) * (size_t)Lk;
+      mnext_w = wp[kld] >> (8 * g);
+    } else if constexpr (MASK != MASK_NONE) {
       if (mask_small && ihn + 32 <= L) {
         // uniform 64-bit row pointer + 32-bit lane offset: no per-lane address arithmetic per element
         const int64_t mrow0 = z * pr.ms[0] + hq * pr.ms[1];
@@ -698,6 +708,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     T mraw_a[MASK == MASK_ADD ? 16 : 1];
     uint8_t mraw_b[MASK == MASK_BOOL ? 16 : 1];
     const int64_t mcol_use = MASK != MASK_NONE ? z * pr.ms[0] + hq * pr.ms[1] + (int64_t)kld * pr.ms[3] : 0;
+    const uint32_t mraw_w = mnext_w;
     if constexpr (MASK != MASK_NONE && MAHEAD) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
@@ -800,6 +811,8 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
           if constexpr (MASK == MASK_BOOL) keep = mraw_b[MAHEAD ? e : 0] != 0;
           float pv = fast_exp2(s - stat(0, e));
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
+          if constexpr (MASK == MASK_BITS)  // the entry's bit spread over a word (0 or all ones), and-ed onto P
+            pv = __uint_as_float(__float_as_uint(pv) & (uint32_t)__builtin_amdgcn_sbfe((int)mraw_w, 16 * (e / 8) + (e % 8), 1));
           if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
           float ks = 1.f;  // dropout: 1 / (1 - p) for a kept entry, 0 for a dropped one
           if constexpr (DROP) {

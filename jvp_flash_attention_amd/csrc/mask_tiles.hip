@@ -100,6 +100,47 @@ static int launch_both(const jvpfa_problem &p, int Lk, int *tq, int *tk, hipStre
                        s[1], s[2], s[3], hm, p.L, Lk, tk);
   return hipGetLastError() == hipSuccess ? JVPFA_OK : JVPFA_E_LAUNCH;
 }
+
+// Boolean mask -> one word per (block of 32 query rows, key): bit i = entry (query 32 b + i, key) != 0.
+// A thread owns four consecutive keys of one block of rows; a workgroup 1024 keys.  HBM-bound: reads the mask
+// once (four bytes per thread and row, the rows of a block all in flight), writes an eighth of it.
+__global__ __launch_bounds__(256) void mask_bits_kernel(const uint8_t *mask, int64_t s0, int64_t s1, int64_t s2,
+                                                        int64_t s3, int hm, int Lq, int Lk, int kchunks,
+                                                        uint32_t *out) {
+  const int nqb = (Lq + 31) / 32;
+  const int kc = blockIdx.x % kchunks;
+  const int qb = (blockIdx.x / kchunks) % nqb;
+  const int plane = blockIdx.x / kchunks / nqb;
+  const int key0 = kc * 1024 + 4 * threadIdx.x;
+  if (key0 >= Lk) return;
+  const uint8_t *base = mask + (int64_t)(plane / hm) * s0 + (int64_t)(plane % hm) * s1 + (int64_t)key0 * s3;
+  const int rows = min(32, Lq - 32 * qb);
+  const bool vec = s3 == 1 && key0 + 4 <= Lk && ((reinterpret_cast<uintptr_t>(base) | (uintptr_t)s2) & 3u) == 0;
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  if (vec) {
+    uint32_t x[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+      x[i] = i < rows ? *reinterpret_cast<const uint32_t *>(base + (int64_t)(32 * qb + i) * s2) : 0u;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] |= ((x[i] >> (8 * j)) & 0xffu) ? (1u << i) : 0u;
+    }
+  } else {
+    const int nk = min(4, Lk - key0);
+    for (int i = 0; i < rows; ++i) {
+      const uint8_t *rp = base + (int64_t)(32 * qb + i) * s2;
+      for (int j = 0; j < nk; ++j) w[j] |= rp[(int64_t)j * s3] ? (1u << i) : 0u;
+    }
+  }
+  uint32_t *dst = out + ((size_t)plane * nqb + qb) * (size_t)Lk + key0;
+  if (key0 + 4 <= Lk && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+    *reinterpret_cast<uint4 *>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+  } else {
+    for (int j = 0; j < min(4, Lk - key0); ++j) dst[j] = w[j];
+  }
+}
 }  // namespace jvpfa
 
 using namespace jvpfa;
@@ -151,4 +192,32 @@ extern "C" int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t Lk, int32_t *til
     case JVPFA_FP16: return launch_both<_Float16, false>(*p, lk, tiles_q, tiles_k, stream);
     default: return launch_both<float, false>(*p, lk, tiles_q, tiles_k, stream);
   }
+}
+
+static inline size_t mask_planes(const jvpfa_problem *p) {
+  return (size_t)(p->mask_stride[0] ? p->Z : 1) * (p->mask_stride[1] ? p->H : 1);
+}
+
+extern "C" size_t jvpfa_mask_bits_bytes(const jvpfa_problem *p, int32_t Lk) {
+  if (!p || p->Z < 1 || p->H < 1 || p->L < 1 || Lk < 0) return 0;
+  const size_t lk = Lk > 0 ? Lk : p->L;
+  return mask_planes(p) * (((size_t)p->L + 31) / 32) * lk * sizeof(uint32_t);
+}
+
+extern "C" int jvpfa_mask_bits(const jvpfa_problem *p, int32_t Lk, uint32_t *bits, void *hip_stream) {
+  if (!p || !bits) return JVPFA_E_NULL;
+  if (p->Z < 1 || p->H < 1 || p->L < 1 || Lk < 0) return JVPFA_E_SHAPE;
+  if (p->mask_kind != JVPFA_MASK_BOOL) return JVPFA_E_DTYPE;
+  if (!p->mask) return JVPFA_E_NULL;
+  for (int i = 0; i < 4; ++i)
+    if (p->mask_stride[i] < 0) return JVPFA_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(bits) & 3u) return JVPFA_E_ALIGN;
+  const int lk = Lk > 0 ? Lk : p->L;
+  const int hm = p->mask_stride[1] ? p->H : 1, kchunks = (lk + 1023) / 1024;
+  const long long blocks = (long long)mask_planes(p) * ((p->L + 31) / 32) * kchunks;
+  if (blocks > 0x7fffffffLL) return JVPFA_E_SHAPE;
+  const int64_t *s = p->mask_stride;
+  hipLaunchKernelGGL(mask_bits_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(hip_stream),
+                     static_cast<const uint8_t *>(p->mask), s[0], s[1], s[2], s[3], hm, p->L, lk, kchunks, bits);
+  return hipGetLastError() == hipSuccess ? JVPFA_OK : JVPFA_E_LAUNCH;
 }

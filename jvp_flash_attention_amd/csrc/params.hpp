@@ -4,7 +4,9 @@
 
 namespace jvpfa {
 
-enum MaskKind { MASK_NONE = 0, MASK_BOOL = 1, MASK_ADD = 2 };
+// MASK_BITS is a boolean mask read by the dk/dv kernels from its bit-packed transposed copy (Problem::bits_k);
+// it exists as a template argument of those kernels only.
+enum MaskKind { MASK_NONE = 0, MASK_BOOL = 1, MASK_ADD = 2, MASK_BITS = 3 };
 
 struct Problem {
   int Z, H, L;  // batch, query heads, query length
@@ -20,6 +22,10 @@ struct Problem {
   // 1 + ceil(L/64) ints (count >= 1, then ascending indices of 64-wide tiles).  tiles_q: key tiles
   // per query block; tiles_k: query tiles per key block.
   const int *tiles_q, *tiles_k;
+  // A boolean mask packed along the query axis, or null: per mask plane, block of 32 query rows and key one
+  // word whose bit i is the mask entry of (query 32 * block + i, key); rows past L are zero bits.  The dk/dv
+  // kernels, whose lanes own a key, read one word per 32 queries instead of 32 bytes a mask row apart.
+  const uint32_t *bits_k;
   // Split of the streamed tiles of one block of owned rows over `chunks` workgroups (1 = no split), used when
   // a launch would otherwise leave most compute units idle: workgroup c of a block takes the tiles
   // c * chunk_tiles .. (c + 1) * chunk_tiles - 1 and writes fp32 partial results to `part`, which a merge
@@ -82,6 +88,11 @@ __host__ __device__ inline size_t tile_list_offset_q(const Problem &pr, int z, i
 __host__ __device__ inline size_t tile_list_offset_k(const Problem &pr, int z, int h, int block) {
   const int nblk = (pr.Lk + TILE_BLOCK - 1) / TILE_BLOCK, nt = (pr.L + TILE_W - 1) / TILE_W;
   return (tile_list_plane(pr, z, h) * nblk + block) * (size_t)(nt + 1);
+}
+
+// first word of (plane of (z, h), block of 32 query rows) in the bit-packed mask
+__host__ __device__ inline size_t mask_bits_offset(const Problem &pr, int z, int h, int qblock) {
+  return (tile_list_plane(pr, z, h) * (size_t)((pr.L + 31) / 32) + (size_t)qblock) * (size_t)pr.Lk;
 }
 
 struct FwdParams {

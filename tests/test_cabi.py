@@ -136,6 +136,47 @@ def test_tile_lists_are_only_made_for_masks_with_a_row_per_query():
         _lib.set_tile_lists(True)
 
 
+def test_the_packed_mask_is_only_made_where_a_kernel_reads_it():
+    import torch
+
+    q = torch.empty(2, 2, 1024, 64, dtype=torch.bfloat16)
+    full = torch.ones(2, 1, 1024, 1024, dtype=torch.bool)
+    cases = [
+        (q, torch.ones(2, 1, 1, 1024, dtype=torch.bool), _lib.MASK_BOOL),  # key padding: no row per query
+        (q[:, :, :256], full[:, :, :256, :256], _lib.MASK_BOOL),            # too short to pay for the pass
+        (q.float(), full, _lib.MASK_BOOL),                                   # fp32 kernels read the mask itself
+        (torch.empty(2, 2, 1024, 256, dtype=torch.bfloat16), full, _lib.MASK_BOOL),  # and so do those for D = 256
+        (q, full.to(torch.bfloat16), _lib.MASK_ADD),                        # additive masks have no bits
+        (q, None, _lib.MASK_NONE),
+    ]
+    for qq, m, kind in cases:
+        assert _lib.mask_bits(qq, m, kind) is None
+    _lib.set_mask_bits(False)
+    try:
+        assert _lib.mask_bits(q, full, _lib.MASK_BOOL) is None
+    finally:
+        _lib.set_mask_bits(True)
+
+
+def test_packed_mask_size_and_argument_checks():
+    """Host-side part of jvpfa_mask_bits: buffer size and refusals (nothing is launched)."""
+    lib = _lib.load()
+    p = _lib.Problem()
+    p.Z, p.H, p.L, p.D, p.dtype, p.mask_kind = 2, 3, 100, 64, 0, _lib.MASK_BOOL
+    p.mask_stride = (C.c_int64 * 4)(0, 100 * 70, 70, 1)  # shared by the batch: 3 planes
+    assert lib.jvpfa_mask_bits_bytes(C.byref(p), 70) == 3 * 4 * 70 * 4  # planes * ceil(100/32) * keys * 4 bytes
+    assert lib.jvpfa_mask_bits_bytes(C.byref(p), 0) == 3 * 4 * 100 * 4
+    assert lib.jvpfa_mask_bits(C.byref(p), 70, None, None) == -1            # no buffer
+    assert lib.jvpfa_mask_bits(C.byref(p), 70, C.c_void_p(64), None) == -1  # no mask
+    p.mask = 4096
+    assert lib.jvpfa_mask_bits(C.byref(p), 70, C.c_void_p(66), None) == -4  # misaligned buffer
+    p.mask_kind = _lib.MASK_ADD
+    assert lib.jvpfa_mask_bits(C.byref(p), 70, C.c_void_p(64), None) == -3  # additive masks are not packed
+    p.mask_kind = _lib.MASK_BOOL
+    p.mask_stride = (C.c_int64 * 4)(0, 100 * 70, -70, 1)
+    assert lib.jvpfa_mask_bits(C.byref(p), 70, C.c_void_p(64), None) == -2
+
+
 def test_mask_tile_list_sizes_and_argument_checks():
     """Host-side part of jvpfa_mask_tiles: buffer sizes and refusals (nothing is launched)."""
     lib = _lib.load()

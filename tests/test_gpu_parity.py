@@ -321,6 +321,95 @@ def test_mask_tile_lists_match_a_numpy_scan(kind, as_bias, L):
             assert row[0] == len(want) and row[1:1 + row[0]] == want
 
 
+def _numpy_mask_bits(keep):
+    """(P, ceil(L/32), Lk) uint32 from a (P, L, Lk) boolean array: bit i of word [p, b, j] = keep[p, 32 b + i, j]."""
+    P, L, Lk = keep.shape
+    nqb = (L + 31) // 32
+    padded = np.zeros((P, nqb * 32, Lk), dtype=np.uint32)
+    padded[:, :L] = keep
+    weights = (np.uint32(1) << np.arange(32, dtype=np.uint32))[None, None, :, None]
+    return (padded.reshape(P, nqb, 32, Lk) * weights).sum(axis=2, dtype=np.uint64).astype(np.uint32)
+
+
+@pytest.mark.parametrize("shape", [(2, 2, 700, 700), (2, 1, 333, 515), (1, 3, 640, 1030), (1, 1, 33, 2050)])
+@pytest.mark.parametrize("layout", ["dense", "offset", "strided"])
+def test_the_packed_mask_matches_a_numpy_packing(shape, layout):
+    """jvpfa_mask_bits against numpy: ragged row and key counts, masks shared by heads or batch, and masks whose
+    rows do not start on a 4-byte boundary or whose keys are not contiguous (the loop that reads byte by byte)."""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H, L, Lk = shape
+    g = torch.Generator().manual_seed(L + Lk)
+    keep = torch.rand(Z, H, L, Lk, generator=g) > 0.3
+    keep[0, 0, 5] = False
+    keep[0, 0, :, 7] = False
+    if layout == "dense":
+        dmask = keep.cuda()
+    elif layout == "offset":  # every row starts one byte past a multiple of four
+        big = torch.zeros(Z, H, L, Lk + 8 - Lk % 4, dtype=torch.bool, device="cuda")
+        dmask = big[..., 1:1 + Lk]
+        dmask.copy_(keep)
+    else:  # keys two bytes apart
+        big = torch.zeros(Z, H, L, 2 * Lk, dtype=torch.bool, device="cuda")
+        dmask = big[..., ::2]
+        dmask.copy_(keep)
+    # a mask axis of size one is shared by the problem's batch entries / heads
+    q = torch.empty(Z if Z > 1 else 2, H if H > 1 else 3, L, 64, dtype=torch.bfloat16, device="cuda")
+    lib = _lib.load()
+    prob = _lib.make_problem(q, dmask, _lib.MASK_BOOL, False, 1.0)
+    n = lib.jvpfa_mask_bits_bytes(C.byref(prob), Lk) // 4
+    assert n == Z * H * ((L + 31) // 32) * Lk
+    bits = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    _lib.check(lib.jvpfa_mask_bits(C.byref(prob), Lk, bits.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    got = bits.cpu().numpy().view(np.uint32).reshape(Z * H, -1, Lk)
+    assert np.array_equal(got, _numpy_mask_bits(keep.reshape(Z * H, L, Lk).numpy()))
+
+
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("Lq,Lk,Hk", [(700, 700, 4), (545, 830, 2)])
+def test_the_packed_mask_changes_no_bit_of_the_backward(dt, D, Lq, Lk, Hk):
+    """The dk/dv kernels read a boolean mask from its bit-packed copy when they are handed one: every gradient
+    of every kind of call (first order, both output gradients, all six gradients, no gO, dropout) must equal,
+    bit for bit, what the same kernels give when they read the mask itself."""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H = 2, 4
+    dtype = DTYPES[dt]
+    g = torch.Generator().manual_seed(Lq + D)
+    q, qt, go, gt = (torch.randn(Z, H, Lq, D, generator=g).to(dtype).cuda() for _ in range(4))
+    k, v, kt, vt = (torch.randn(Z, Hk, Lk, D, generator=g).to(dtype).cuda() for _ in range(4))
+    keep = torch.rand(Z, H, Lq, Lk, generator=g) > 0.2
+    keep[1, 2, 40:75] = False  # rows that attend nothing
+    keep[0, 1, :, 100:300] = False  # keys that nothing attends
+    be, scale = _lib.backend(), D**-0.5
+    print(f"case packed mask {dt} D{D} Lq{Lq} Lk{Lk} Hk{Hk}", flush=True)
+
+    def run(dmask):
+        o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, dmask, _lib.MASK_BOOL, False, scale)
+        out = list(be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, dmask, _lib.MASK_BOOL, False, scale, want_tangent_grads=True))
+        out += be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, dmask, _lib.MASK_BOOL, False, scale)[:3]
+        out += be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, None, gt, dmask, _lib.MASK_BOOL, False, scale)[:3]
+        out += be.bwd(q, k, v, None, None, None, o, None, M, None, go, None, dmask, _lib.MASK_BOOL, False, scale)[:3]
+        od, otd, Md, mud = be.fwd(q, k, v, qt, kt, vt, dmask, _lib.MASK_BOOL, False, scale, 0.2, 11)
+        out += be.bwd(q, k, v, qt, kt, vt, od, otd, Md, mud, go, gt, dmask, _lib.MASK_BOOL, False, scale,
+                      dropout_p=0.2, dropout_seed=11)[:3]
+        return out
+
+    dmask = keep.cuda()
+    packed = run(dmask)
+    assert getattr(dmask, "_jvpfa_bits")[1] is not None
+    _lib.set_mask_bits(False)
+    try:
+        other = keep.cuda()
+        from_bytes = run(other)
+        assert not hasattr(other, "_jvpfa_bits")
+    finally:
+        _lib.set_mask_bits(True)
+    for a, b in zip(packed, from_bytes):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("dt,D", [("bf16", 32), ("bf16", 64), ("bf16", 128), ("bf16", 256),
                                   ("fp32", 32), ("fp32", 64), ("fp32", 128), ("fp32", 256)])
 @pytest.mark.parametrize("kind", ["blockdiag", "band", "pad2d", "lower"])
