@@ -198,12 +198,12 @@ int jvpfa_mask_tiles(const jvpfa_problem *p, int32_t Lk, int32_t *tiles_q, int32
 
 /*
  * A boolean mask packed along the query axis, for the dk/dv kernels: their lanes own a key and walk down the
- * queries, so from the mask itself they fetch one byte per entry, a mask row apart; from this copy one 32-bit
- * word per 32 queries.  No counterpart in the reference, whose kernels load the mask block by block
- * (JA:1451-1463, JA:1607-1619).  Layout: for every mask plane (as for jvpfa_mask_tiles), block of 32 query
- * rows b < ceil(L/32) and key j < Lk the word [(plane * ceil(L/32) + b) * Lk + j], whose bit i is 1 where the
- * mask entry of (query 32 b + i, key j) is nonzero; bits of rows past L are 0.  The buffer is
- * jvpfa_mask_bits_bytes(p, Lk) bytes of device memory (an eighth of the broadcast mask), 4-byte aligned; it
+ * queries, so from the mask itself they fetch one byte per entry, a mask row apart; from this copy one pair of
+ * 32-bit words per 64 queries.  No counterpart in the reference, whose kernels load the mask block by block
+ * (JA:1451-1463, JA:1607-1619).  Layout: for every mask plane (as for jvpfa_mask_tiles), tile of 64 query
+ * rows t < ceil(L/64), key j < Lk and half hf < 2 the word [((plane * ceil(L/64) + t) * Lk + j) * 2 + hf], whose
+ * bit i is 1 where the mask entry of (query 64 t + 32 hf + i, key j) is nonzero; bits of rows past L are 0.  The
+ * buffer is jvpfa_mask_bits_bytes(p, Lk) bytes of device memory (an eighth of the broadcast mask), 8-byte aligned; it
  * describes the mask's contents: rebuild it when those change.  Only p->Z, H, L, mask_kind (must be
  * JVPFA_MASK_BOOL), mask and mask_stride are read.  Handing it to jvpfa_bwd is optional and changes no result;
  * the kernels for 16-bit element types at D <= 128 use it, the others read the mask itself.

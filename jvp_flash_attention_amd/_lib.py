@@ -273,8 +273,8 @@ def set_mask_bits(enabled: bool) -> None:
 
 def mask_bits(q, mask, mask_kind, Lk=None):
     """For a boolean mask with a row per query (shape [*, *, L, Lk]) and a 16-bit element type at D <= 128: the
-    mask packed along the query axis by ``jvpfa_mask_bits`` (one uint32 per 32 queries and key; an eighth of the
-    broadcast mask's bytes), which the dk/dv kernels read instead of one byte per entry.  None otherwise.  Cached
+    mask packed along the query axis by ``jvpfa_mask_bits`` (a pair of uint32 per 64 queries and key; an eighth of
+    the broadcast mask's bytes), which the dk/dv kernels read instead of one byte per entry.  None otherwise.  Cached
     on the mask tensor, keyed by its version counter, like the tile lists."""
     Z, H, L, D = q.shape
     Lk = L if Lk is None else Lk

@@ -53,7 +53,7 @@ static int bwd_impl(const jvpfa_bwd_args *a, void *workspace, void *hip_stream) 
     if (ptr && !aligned16(ptr)) return JVPFA_E_ALIGN;
 
   BwdParams p;
-  if (a->mask_bits && (reinterpret_cast<uintptr_t>(a->mask_bits) & 3u)) return JVPFA_E_ALIGN;
+  if (a->mask_bits && (reinterpret_cast<uintptr_t>(a->mask_bits) & 7u)) return JVPFA_E_ALIGN;
   p.pr = to_problem(a->p, a->key_limit, a->tiles_q, a->tiles_k, a->Lk, a->Hk, a->mask_bits);
   p.q = a->q; p.k = a->k; p.v = a->v;
   p.qt = a->qt; p.kt = a->kt; p.vt = a->vt;

@@ -581,7 +581,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     st_p[1] = MODE == BWD_PLAIN ? p.d1 + qrow0 : (DUAL ? p.mu + qrow0 : p.a + qrow0);
     st_p[2] = DUAL ? p.a + qrow0 : nullptr;
     st_p[3] = DUAL ? p.d2 + qrow0 : nullptr;
-    if constexpr (MASK == MASK_BITS) bits_head = pr.bits_k + mask_bits_offset(pr, z, hq, 0);
+    if constexpr (MASK == MASK_BITS) bits_head = pr.bits_k + mask_bits_offset(pr, z, hq);
   };
   set_query_head(h * group);
 
@@ -645,19 +645,21 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
   // the far caches, so they are requested a whole half tile before their use.  (Where two workgroups
   // share a compute unit, D = 64 outside the dual mode, each value is instead fetched where it is used:
   // the other workgroup covers the wait and the registers stay within the cap.)
-  // MASK_BITS: one word per half tile and lane, bit i = (query ihn + i, this lane's key), moved so that bit
-  // 16(e/8) + e%8 belongs to register e; always requested a half tile ahead (it costs one register).
-  constexpr bool MAHEAD = D > 64 || MODE == BWD_DUAL || MASK == MASK_BITS;
+  constexpr bool MAHEAD = (D > 64 || MODE == BWD_DUAL) && MASK != MASK_BITS;
   T mnext_a[MASK == MASK_ADD ? 16 : 1];
   uint8_t mnext_b[MASK == MASK_BOOL ? 16 : 1];
-  uint32_t mnext_w = 0;
-  const int nqb = (L + 31) >> 5;
+  // MASK_BITS: this lane's key against the 64 queries of a tile is one pair of words (bit i of word hf = query
+  // 32 hf + i of the tile).  The pair of the next tile is requested at the top of a tile, before any of the
+  // tile's direct loads, and taken over behind the wait for everything at the top of the next one: the loop
+  // body then holds no wait of its own for it (a wait in mid-tile would also wait for the direct loads issued
+  // before it, which are meant to be in flight until the tile ends).
+  u32x2 bits_next = {0u, 0u};
+  auto fetch_bits = [&](int tile_index) {
+    if constexpr (MASK == MASK_BITS)
+      bits_next = *reinterpret_cast<const u32x2 *>(bits_head + ((size_t)tile_index * (size_t)Lk + (size_t)kld) * 2);
+  };
   auto fetch_mask_half = [&](int ihn) {
-    if constexpr (MASK == MASK_BITS) {
-      // (the second half of the last tile may start past the last row: its entries are masked by index)
-      const uint32_t *wp = bits_head + (size_t)min(ihn >> 5, nqb - 1) * (size_t)Lk;
-      mnext_w = wp[kld] >> (8 * g);
-    } else if constexpr (MASK != MASK_NONE) {
+    if constexpr (MASK != MASK_NONE && MASK != MASK_BITS) {
       if (mask_small && ihn + 32 <= L) {
         // uniform 64-bit row pointer + 32-bit lane offset: no per-lane address arithmetic per element
         const int64_t mrow0 = z * pr.ms[0] + hq * pr.ms[1];
@@ -680,7 +682,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     }
   };
   // ih: first query of this half tile; ihn: of the half tile that follows it
-  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn) {
+  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn, uint32_t bits_word) {
     constexpr int HB = decltype(HBc)::value;
     // dropout: the 32 queries of a half tile are one block of the pattern (ih is a multiple of 32), so the block's
     // word is uniform and register e's query adds a constant to it; this lane's key and row group add drop_lane
@@ -708,7 +710,8 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     T mraw_a[MASK == MASK_ADD ? 16 : 1];
     uint8_t mraw_b[MASK == MASK_BOOL ? 16 : 1];
     const int64_t mcol_use = MASK != MASK_NONE ? z * pr.ms[0] + hq * pr.ms[1] + (int64_t)kld * pr.ms[3] : 0;
-    const uint32_t mraw_w = mnext_w;
+    // MASK_BITS: moved so that bit 16(e/8) + e%8 belongs to register e
+    const uint32_t mraw_w = bits_word >> (8 * g);
     if constexpr (MASK != MASK_NONE && MAHEAD) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
@@ -796,7 +799,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
           const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
           float s = S[e] * sl2;
           bool keep = true;
-          if constexpr (MASK != MASK_NONE && !MAHEAD) {
+          if constexpr (MASK != MASK_NONE && MASK != MASK_BITS && !MAHEAD) {
             if constexpr (!EDGE) {  // uniform row pointer + 32-bit lane offset, as above
               const int64_t urow = z * pr.ms[0] + hq * pr.ms[1] + (int64_t)(ih + 16 * (e / 8) + (e % 8)) * pr.ms[2];
               if constexpr (MASK == MASK_ADD) mraw_a[0] = (reinterpret_cast<const T *>(pr.mask) + urow)[mlane];
@@ -811,8 +814,13 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
           if constexpr (MASK == MASK_BOOL) keep = mraw_b[MAHEAD ? e : 0] != 0;
           float pv = fast_exp2(s - stat(0, e));
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
-          if constexpr (MASK == MASK_BITS)  // the entry's bit spread over a word (0 or all ones), and-ed onto P
-            pv = __uint_as_float(__float_as_uint(pv) & (uint32_t)__builtin_amdgcn_sbfe((int)mraw_w, 16 * (e / 8) + (e % 8), 1));
+          if constexpr (MASK == MASK_BITS) {
+            // the entry's bit spread over a word (0 or all ones), and-ed onto P: two instructions (written as
+            // asm: from the builtin the compiler makes a bit test, a compare and a select)
+            uint32_t spread;
+            asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(spread) : "v"(mraw_w), "n"(16 * (e / 8) + (e % 8)));
+            pv = __uint_as_float(__float_as_uint(pv) & spread);
+          }
           if constexpr (EDGE) pv = (qi >= qmin && qi < L) ? pv : 0.f;
           float ks = 1.f;  // dropout: 1 / (1 - p) for a kept entry, 0 for a dropped one
           if constexpr (DROP) {
@@ -876,16 +884,21 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
+    u32x2 bits_cur = bits_next;
+    if constexpr (MASK == MASK_BITS) {
+      asm volatile("" : "+v"(bits_cur));  // taken over here, behind the wait above
+      fetch_bits(tnext);
+    }
     int tnext2 = min(t + 2, ntiles - 1), tahead = 0;
     if constexpr (MASK != MASK_NONE) tahead = list_request(list_slot(tnext2));
     const int i0 = istart + tcur * BT, i0n = istart + tnext * BT;
     prepare_loads(stage ^ 1, i0n, t + 1 < ntiles);
     load_stats();
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB, sstat = stat0 + stage * Cfg::STATB;
-    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, sstat, i0, i0 + 32);
+    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, sstat, i0, i0 + 32, bits_cur[0]);
     // always both halves: a half past the last query contributes exact zeros, and a branch here would
     // make the accumulators change register file around it
-    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32, i0n);
+    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32, i0n, bits_cur[1]);
     if constexpr (MASK != MASK_NONE) {
       const int listed = list_take(tahead);
       tnext2 = tlist ? min(max(listed, 0), tmax) : tnext2;
@@ -906,6 +919,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     tcur = tlist ? min(max(tlist[1], 0), tmax) : 0;
     tnext = tlist ? min(max(tlist[1 + min(1, ntiles - 1)], 0), tmax) : min(1, ntiles - 1);
     if constexpr (MASK != MASK_NONE && MAHEAD) fetch_mask_half(istart + tcur * BT);
+    if constexpr (MASK == MASK_BITS) fetch_bits(tcur);
     prepare_loads(0, istart + tcur * BT, true);
     static_for<NLOAD>([&](auto pc) { load_piece(pc); });
     load_stats();

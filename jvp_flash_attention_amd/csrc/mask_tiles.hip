@@ -101,20 +101,21 @@ static int launch_both(const jvpfa_problem &p, int Lk, int *tq, int *tk, hipStre
   return hipGetLastError() == hipSuccess ? JVPFA_OK : JVPFA_E_LAUNCH;
 }
 
-// Boolean mask -> one word per (block of 32 query rows, key): bit i = entry (query 32 b + i, key) != 0.
-// A thread owns four consecutive keys of one block of rows; a workgroup 1024 keys.  HBM-bound: reads the mask
+// Boolean mask -> a pair of words per (tile of 64 query rows, key): bit i of word hf = entry (query
+// 64 t + 32 hf + i, key) != 0.  A thread owns four consecutive keys of one half tile (32 rows); a workgroup
+// 1024 keys.  HBM-bound: reads the mask
 // once (four bytes per thread and row, the rows of a block all in flight), writes an eighth of it.
 __global__ __launch_bounds__(256) void mask_bits_kernel(const uint8_t *mask, int64_t s0, int64_t s1, int64_t s2,
                                                         int64_t s3, int hm, int Lq, int Lk, int kchunks,
                                                         uint32_t *out) {
-  const int nqb = (Lq + 31) / 32;
+  const int nqb = 2 * ((Lq + 63) / 64);  // half tiles, an even number: the last may lie wholly past the last row
   const int kc = blockIdx.x % kchunks;
   const int qb = (blockIdx.x / kchunks) % nqb;
   const int plane = blockIdx.x / kchunks / nqb;
   const int key0 = kc * 1024 + 4 * threadIdx.x;
   if (key0 >= Lk) return;
   const uint8_t *base = mask + (int64_t)(plane / hm) * s0 + (int64_t)(plane % hm) * s1 + (int64_t)key0 * s3;
-  const int rows = min(32, Lq - 32 * qb);
+  const int rows = max(0, min(32, Lq - 32 * qb));
   const bool vec = s3 == 1 && key0 + 4 <= Lk && ((reinterpret_cast<uintptr_t>(base) | (uintptr_t)s2) & 3u) == 0;
   uint32_t w[4] = {0u, 0u, 0u, 0u};
   if (vec) {
@@ -134,12 +135,10 @@ __global__ __launch_bounds__(256) void mask_bits_kernel(const uint8_t *mask, int
       for (int j = 0; j < nk; ++j) w[j] |= rp[(int64_t)j * s3] ? (1u << i) : 0u;
     }
   }
-  uint32_t *dst = out + ((size_t)plane * nqb + qb) * (size_t)Lk + key0;
-  if (key0 + 4 <= Lk && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
-    *reinterpret_cast<uint4 *>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
-  } else {
-    for (int j = 0; j < min(4, Lk - key0); ++j) dst[j] = w[j];
-  }
+  // (a plane has ceil(Lq / 64) tiles; the second half of a last tile that ends early is written as zeros by
+  // the workgroups of the block of rows that does not exist: see the launch)
+  uint32_t *dst = out + (((size_t)plane * (nqb / 2) + qb / 2) * (size_t)Lk + key0) * 2 + (qb & 1);
+  for (int j = 0; j < min(4, Lk - key0); ++j) dst[2 * j] = w[j];
 }
 }  // namespace jvpfa
 
@@ -201,7 +200,7 @@ static inline size_t mask_planes(const jvpfa_problem *p) {
 extern "C" size_t jvpfa_mask_bits_bytes(const jvpfa_problem *p, int32_t Lk) {
   if (!p || p->Z < 1 || p->H < 1 || p->L < 1 || Lk < 0) return 0;
   const size_t lk = Lk > 0 ? Lk : p->L;
-  return mask_planes(p) * (((size_t)p->L + 31) / 32) * lk * sizeof(uint32_t);
+  return mask_planes(p) * (((size_t)p->L + 63) / 64) * lk * 2 * sizeof(uint32_t);
 }
 
 extern "C" int jvpfa_mask_bits(const jvpfa_problem *p, int32_t Lk, uint32_t *bits, void *hip_stream) {
@@ -211,10 +210,10 @@ extern "C" int jvpfa_mask_bits(const jvpfa_problem *p, int32_t Lk, uint32_t *bit
   if (!p->mask) return JVPFA_E_NULL;
   for (int i = 0; i < 4; ++i)
     if (p->mask_stride[i] < 0) return JVPFA_E_SHAPE;
-  if (reinterpret_cast<uintptr_t>(bits) & 3u) return JVPFA_E_ALIGN;
+  if (reinterpret_cast<uintptr_t>(bits) & 7u) return JVPFA_E_ALIGN;
   const int lk = Lk > 0 ? Lk : p->L;
   const int hm = p->mask_stride[1] ? p->H : 1, kchunks = (lk + 1023) / 1024;
-  const long long blocks = (long long)mask_planes(p) * ((p->L + 31) / 32) * kchunks;
+  const long long blocks = (long long)mask_planes(p) * (2 * ((p->L + 63) / 64)) * kchunks;
   if (blocks > 0x7fffffffLL) return JVPFA_E_SHAPE;
   const int64_t *s = p->mask_stride;
   hipLaunchKernelGGL(mask_bits_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(hip_stream),

@@ -22,9 +22,10 @@ struct Problem {
   // 1 + ceil(L/64) ints (count >= 1, then ascending indices of 64-wide tiles).  tiles_q: key tiles
   // per query block; tiles_k: query tiles per key block.
   const int *tiles_q, *tiles_k;
-  // A boolean mask packed along the query axis, or null: per mask plane, block of 32 query rows and key one
-  // word whose bit i is the mask entry of (query 32 * block + i, key); rows past L are zero bits.  The dk/dv
-  // kernels, whose lanes own a key, read one word per 32 queries instead of 32 bytes a mask row apart.
+  // A boolean mask packed along the query axis, or null: per mask plane, tile of 64 query rows and key a pair
+  // of words, bit i of word hf being the mask entry of (query 64 * tile + 32 * hf + i, key); rows past L are
+  // zero bits.  The dk/dv kernels, whose lanes own a key, read one pair per 64 queries instead of 64 bytes a
+  // mask row apart.
   const uint32_t *bits_k;
   // Split of the streamed tiles of one block of owned rows over `chunks` workgroups (1 = no split), used when
   // a launch would otherwise leave most compute units idle: workgroup c of a block takes the tiles
@@ -90,9 +91,9 @@ __host__ __device__ inline size_t tile_list_offset_k(const Problem &pr, int z, i
   return (tile_list_plane(pr, z, h) * nblk + block) * (size_t)(nt + 1);
 }
 
-// first word of (plane of (z, h), block of 32 query rows) in the bit-packed mask
-__host__ __device__ inline size_t mask_bits_offset(const Problem &pr, int z, int h, int qblock) {
-  return (tile_list_plane(pr, z, h) * (size_t)((pr.L + 31) / 32) + (size_t)qblock) * (size_t)pr.Lk;
+// first word of the plane of (z, h) in the bit-packed mask
+__host__ __device__ inline size_t mask_bits_offset(const Problem &pr, int z, int h) {
+  return tile_list_plane(pr, z, h) * (size_t)((pr.L + 63) / 64) * (size_t)pr.Lk * 2;
 }
 
 struct FwdParams {

@@ -164,12 +164,12 @@ def test_packed_mask_size_and_argument_checks():
     p = _lib.Problem()
     p.Z, p.H, p.L, p.D, p.dtype, p.mask_kind = 2, 3, 100, 64, 0, _lib.MASK_BOOL
     p.mask_stride = (C.c_int64 * 4)(0, 100 * 70, 70, 1)  # shared by the batch: 3 planes
-    assert lib.jvpfa_mask_bits_bytes(C.byref(p), 70) == 3 * 4 * 70 * 4  # planes * ceil(100/32) * keys * 4 bytes
-    assert lib.jvpfa_mask_bits_bytes(C.byref(p), 0) == 3 * 4 * 100 * 4
+    assert lib.jvpfa_mask_bits_bytes(C.byref(p), 70) == 3 * 2 * 70 * 8  # planes * ceil(100/64) * keys * 8 bytes
+    assert lib.jvpfa_mask_bits_bytes(C.byref(p), 0) == 3 * 2 * 100 * 8
     assert lib.jvpfa_mask_bits(C.byref(p), 70, None, None) == -1            # no buffer
     assert lib.jvpfa_mask_bits(C.byref(p), 70, C.c_void_p(64), None) == -1  # no mask
     p.mask = 4096
-    assert lib.jvpfa_mask_bits(C.byref(p), 70, C.c_void_p(66), None) == -4  # misaligned buffer
+    assert lib.jvpfa_mask_bits(C.byref(p), 70, C.c_void_p(68), None) == -4  # misaligned buffer
     p.mask_kind = _lib.MASK_ADD
     assert lib.jvpfa_mask_bits(C.byref(p), 70, C.c_void_p(64), None) == -3  # additive masks are not packed
     p.mask_kind = _lib.MASK_BOOL

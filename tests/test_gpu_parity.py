@@ -322,13 +322,15 @@ def test_mask_tile_lists_match_a_numpy_scan(kind, as_bias, L):
 
 
 def _numpy_mask_bits(keep):
-    """(P, ceil(L/32), Lk) uint32 from a (P, L, Lk) boolean array: bit i of word [p, b, j] = keep[p, 32 b + i, j]."""
+    """(P, ceil(L/64), Lk, 2) uint32 from a (P, L, Lk) boolean array: bit i of word [p, t, j, hf] =
+    keep[p, 64 t + 32 hf + i, j], rows past L counting as masked."""
     P, L, Lk = keep.shape
-    nqb = (L + 31) // 32
-    padded = np.zeros((P, nqb * 32, Lk), dtype=np.uint32)
+    nqt = (L + 63) // 64
+    padded = np.zeros((P, nqt * 64, Lk), dtype=np.uint32)
     padded[:, :L] = keep
-    weights = (np.uint32(1) << np.arange(32, dtype=np.uint32))[None, None, :, None]
-    return (padded.reshape(P, nqb, 32, Lk) * weights).sum(axis=2, dtype=np.uint64).astype(np.uint32)
+    weights = (np.uint32(1) << np.arange(32, dtype=np.uint32))[None, None, None, :, None]
+    words = (padded.reshape(P, nqt, 2, 32, Lk) * weights).sum(axis=3, dtype=np.uint64).astype(np.uint32)
+    return words.transpose(0, 1, 3, 2)
 
 
 @pytest.mark.parametrize("shape", [(2, 2, 700, 700), (2, 1, 333, 515), (1, 3, 640, 1030), (1, 1, 33, 2050)])
@@ -358,10 +360,10 @@ def test_the_packed_mask_matches_a_numpy_packing(shape, layout):
     lib = _lib.load()
     prob = _lib.make_problem(q, dmask, _lib.MASK_BOOL, False, 1.0)
     n = lib.jvpfa_mask_bits_bytes(C.byref(prob), Lk) // 4
-    assert n == Z * H * ((L + 31) // 32) * Lk
+    assert n == Z * H * ((L + 63) // 64) * Lk * 2
     bits = torch.full((n,), -1, dtype=torch.int32, device="cuda")
     _lib.check(lib.jvpfa_mask_bits(C.byref(prob), Lk, bits.data_ptr(), torch.cuda.current_stream().cuda_stream))
-    got = bits.cpu().numpy().view(np.uint32).reshape(Z * H, -1, Lk)
+    got = bits.cpu().numpy().view(np.uint32).reshape(Z * H, -1, Lk, 2)
     assert np.array_equal(got, _numpy_mask_bits(keep.reshape(Z * H, L, Lk).numpy()))
 
 
