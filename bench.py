@@ -29,7 +29,7 @@ Z, H, L, D = 4, 16, 4096, 128
 # HBM bytes per forward launch.  A recorded constant, not measured in this run: rocprofv3 --pmc
 # FETCH_SIZE (x2.0, the factor a plain copy of known size gives) and WRITE_SIZE (x1.0) read 403.0 MB +
 # 136.3 MB; the counter runs and their commands are in profiles/fwd3_kernel_bf16_B4_H16_L4096_D128.md.
-MEASURED_FWD_TRAFFIC_BYTES = 539.6e6
+MEASURED_FWD_TRAFFIC_BYTES = 540.9e6
 TRAFFIC_SOURCE = "recorded from the rocprofv3 --pmc runs in profiles/fwd3_kernel_bf16_B4_H16_L4096_D128.md, not measured in this run"
 
 
