@@ -46,10 +46,28 @@ static auto pick_dkdv(bool no_go, bool grouped, bool fold_kv, bool drop) -> void
   if (grouped) return no_go ? bwd2_dkdv_kernel<T, D, MODE, MK, NG, true> : bwd2_dkdv_kernel<T, D, MODE, MK, true, true>;
   return no_go ? bwd2_dkdv_kernel<T, D, MODE, MK, NG> : bwd2_dkdv_kernel<T, D, MODE, MK, true>;
 }
+// An additive mask can be streamed through LDS as tiles (MASK_TILE) when its rows are runs of contiguous keys
+// that start on 16-byte boundaries wherever a tile starts, and 64 rows stay within a 32-bit offset.
+template <typename T> static bool mask_rows_tileable(const Problem &pr) {
+  const int64_t es = sizeof(T);
+  if (pr.ms[3] != 1 || (reinterpret_cast<uintptr_t>(pr.mask) & 15u)) return false;
+  for (int i = 0; i < 3; ++i)
+    if (pr.ms[i] < 0 || (pr.ms[i] * es) % 16 != 0) return false;
+  return 64 * pr.ms[2] * es < ((int64_t)1 << 31);
+}
+// *lds: the dynamic LDS bytes of the kernel returned
 template <typename T, int D, int MODE, int MASK>
-static auto pick_dkdv_for(const BwdParams &p, bool no_go, bool grouped, bool fold_kv, bool drop) -> void (*)(const BwdParams) {
+static auto pick_dkdv_for(const BwdParams &p, bool no_go, bool grouped, bool fold_kv, bool drop, size_t *lds) -> void (*)(const BwdParams) {
+  using Cfg2 = Bwd2Cfg<T, D, MODE>;
+  *lds = Cfg2::DKV_LDS;
   if constexpr (MASK == MASK_BOOL) {
     if (p.pr.bits_k) return pick_dkdv<T, D, MODE, MASK_BITS>(no_go, grouped, fold_kv, drop);
+  }
+  if constexpr (MASK == MASK_ADD && Cfg2::MTILE_FITS) {
+    if (mask_rows_tileable<T>(p.pr)) {
+      *lds = Cfg2::DKV_LDS_MTILE;
+      return pick_dkdv<T, D, MODE, MASK_TILE>(no_go, grouped, fold_kv, drop);
+    }
   }
   return pick_dkdv<T, D, MODE, MASK>(no_go, grouped, fold_kv, drop);
 }
@@ -74,11 +92,12 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
       constexpr bool NG = MODE != BWD_DUAL;
       const bool grouped = p.pr.Hk != p.pr.H;
       void (*kq)(const BwdParams) = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG, false, true> : bwd2_dq_kernel<T, D, MODE, MASK, true, false, true>;
-      void (*kkv)(const BwdParams) = pick_dkdv_for<T, D, MODE, MASK>(p, no_go, grouped, false, true);
+      size_t kv_lds = 0;
+      void (*kkv)(const BwdParams) = pick_dkdv_for<T, D, MODE, MASK>(p, no_go, grouped, false, true, &kv_lds);
       int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
-      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);
+      if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), kv_lds);
       if (rc != 0) return rc;
-      hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
+      hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), kv_lds, stream, p);
       hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
       return hipGetLastError() == hipSuccess ? 0 : -6;
     } else if constexpr (sizeof(T) == 2 && D == 256 && MODE == BWD_DUAL) {
@@ -146,7 +165,8 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
       if (plain_q) kq = no_go ? bwd2_dq_kernel<T, D, MODE, MASK, NG> : bwd2_dq_kernel<T, D, MODE, MASK, true>;
       if constexpr (D == 128 && MODE == BWD_PLAIN) kq = bwd2_dq_kernel_2wg_plain<T, D, MODE, MASK>;
     }
-    kkv = pick_dkdv_for<T, D, MODE, MASK>(p, no_go, grouped, MODE == BWD_DUAL && six, false);
+    size_t kv_lds = 0;
+    kkv = pick_dkdv_for<T, D, MODE, MASK>(p, no_go, grouped, MODE == BWD_DUAL && six, false, &kv_lds);
     // a grid smaller than the GPU: both roles in one launch, side by side
     const int cus = device_cus();
     if (!grouped && !six && blocks < cus && kv_blocks < cus) {
@@ -158,9 +178,9 @@ static int launch_bwd_mode(const BwdParams &p, bool six, hipStream_t stream) {
       return hipGetLastError() == hipSuccess ? 0 : -6;
     }
     int rc = allow_lds(reinterpret_cast<const void *>(kq), Cfg2::DQ_LDS);
-    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), Cfg2::DKV_LDS);
+    if (rc == 0) rc = allow_lds(reinterpret_cast<const void *>(kkv), kv_lds);
     if (rc != 0) return rc;
-    if (run_kv) hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), Cfg2::DKV_LDS, stream, p);
+    if (run_kv) hipLaunchKernelGGL(kkv, dim3((unsigned)kv_blocks), dim3(Cfg2::NT), kv_lds, stream, p);
     if (run_q) hipLaunchKernelGGL(kq, dim3((unsigned)blocks), dim3(Cfg2::NT), Cfg2::DQ_LDS, stream, p);
     return hipGetLastError() == hipSuccess ? 0 : -6;
    }

@@ -31,6 +31,10 @@ template <typename T, int D, int MODE> struct Bwd2Cfg {
   static constexpr int STATB = NSTAT * BT * 4;        // row statistics of a query tile (dk/dv only)
   static constexpr size_t DQ_LDS = 2 * (size_t)STAGEB;
   static constexpr size_t DKV_LDS = 2 * (size_t)STAGEB + 2 * (size_t)STATB;
+  // MASK_TILE: two stages of a 64-query x 128-key tile of a 16-bit additive mask behind the statistics
+  static constexpr int MTILEB = BT * 256;
+  static constexpr size_t DKV_LDS_MTILE = DKV_LDS + 2 * (size_t)MTILEB;
+  static constexpr bool MTILE_FITS = DKV_LDS_MTILE <= 160 * 1024;
 };
 
 // One LDS fragment (8 elements per lane) read ahead with lds_b128 / two lds_tr64.
@@ -561,6 +565,32 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     mask_small = pr.ms[2] >= 0 && pr.ms[3] >= 0 && 8 * pr.ms[2] + (int64_t)Lk * pr.ms[3] < lim;
     mlane = (uint32_t)(8 * g * pr.ms[2] + (int64_t)kld * pr.ms[3]);
   }
+  // MASK_TILE: the mask tile of (64 queries, this workgroup's 128 keys) is an operand tile of 256-byte rows in
+  // all but name: direct loads with the chunks swizzled on the global side (wave w brings rows 16w .. 16w+15,
+  // four instructions of four rows), and this lane's 16 values of a half tile (queries 16c + 8g + 0..7, its key)
+  // come from the transposing fragment read of d-block `wave`.
+  uint32_t mt_o[4] = {0u, 0u, 0u, 0u}, mt_f[2] = {0u, 0u};
+  const uint32_t mt0 = lds0 + 2 * Cfg::STAGEB + 2 * Cfg::STATB;
+  const char *mt_head = nullptr;       // first byte of (plane of the current query head, query 0, key k0)
+  int64_t mt_row = 0;                  // bytes from a mask row to the next
+  __amdgpu_buffer_rsrc_t mt_rs;
+  uint32_t mt_dst = 0;
+  if constexpr (MASK == MASK_TILE) {
+    mt_row = pr.ms[2] * (int64_t)sizeof(T);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 16 * wave + 4 * i + lane / 16;
+      mt_o[i] = (uint32_t)(row * mt_row) + (uint32_t)(((lane % 16) ^ swz_u<16>(row)) * 16);
+    }
+    const int a_ = (lane >> 4) & 1, j_ = lane & 15;
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const int row = 8 * g + 4 * hh + (j_ >> 2);
+      // (the operand fragments take chunk j%2, half (j/2)%2, which hands lane r the column perm32(r); the mask
+      // value must be that of the lane's own key, column r: chunk and half change places)
+      mt_f[hh] = row * 256 + ((4 * wave + 2 * a_ + ((j_ >> 1) & 1)) ^ swz_u<16>(row)) * 16 + 8 * (j_ & 1);
+    }
+  }
   // The query heads that read this key/value head are visited one after another (one, h itself, for
   // the shapes the reference admits); hq is the current one, and what depends on it is set per head:
   // tile slots 0 Q, 1 G (gO; gT in TANGENT; gT again in DUAL without gO), 2 Q', 3 gT, and the
@@ -582,6 +612,8 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     st_p[2] = DUAL ? p.a + qrow0 : nullptr;
     st_p[3] = DUAL ? p.d2 + qrow0 : nullptr;
     if constexpr (MASK == MASK_BITS) bits_head = pr.bits_k + mask_bits_offset(pr, z, hq);
+    if constexpr (MASK == MASK_TILE)
+      mt_head = reinterpret_cast<const char *>(pr.mask) + (z * pr.ms[0] + hq * pr.ms[1] + (int64_t)k0) * (int64_t)sizeof(T);
   };
   set_query_head(h * group);
 
@@ -619,6 +651,15 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
       ld_rs[2] = tile_rsrc(Qtb, i0, on);
       ld_rs[3] = tile_rsrc(gTb, i0, on);
     }
+    if constexpr (MASK == MASK_TILE) {
+      // from (query i0, key k0) to the end of the last row's keys: rows past L and keys past Lk of the last
+      // row read as zeros; keys past Lk of the other rows read the row that follows (lanes whose key does not
+      // exist keep nothing)
+      const int rows = on ? max(L - i0, 0) : 0;
+      const int64_t bytes = rows > 0 ? (int64_t)(rows - 1) * mt_row + (int64_t)(Lk - k0) * (int64_t)sizeof(T) : 0;
+      mt_rs = __builtin_amdgcn_make_buffer_rsrc((void *)(mt_head + (int64_t)i0 * mt_row), 0, (int)min(bytes, (int64_t)0x7fffffff), 0x00020000);
+      mt_dst = mt0 + stage * Cfg::MTILEB + (wave * 4) * 1024;
+    }
     i0 = on ? i0 : istart;
     st_row = min(i0 + lane, L - 1);
     st_dst = stat0 + stage * Cfg::STATB;
@@ -630,13 +671,24 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
                                        (JVPFA_LDS(void))(uintptr_t)(st_dst + wave * BT * 4), 4, 0, 0);
     }
   };
+  // MASK_TILE: four more pieces per wave, rows 4i .. 4i+3 of the wave's 16
+  constexpr int NLOAD_ALL = NLOAD + (MASK == MASK_TILE ? 4 : 0);
+  auto load_any = [&](auto pc) {
+    constexpr int pi = decltype(pc)::value;
+    if constexpr (pi < NLOAD) {
+      load_piece(pc);
+    } else {
+      constexpr int i = pi - NLOAD;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(mt_rs, (JVPFA_LDS(void))(uintptr_t)(mt_dst + i * 1024), 16, mt_o[i], 0, 0, 0);
+    }
+  };
   auto load_step = [&](auto gc) {
     constexpr int gi = decltype(gc)::value;
     // spread over the first NSPREAD steps only: the last load then has time to land before the barrier
     constexpr int NSPREAD = bwd_spread(NSTEP);
     if constexpr (gi < NSPREAD) {
-      constexpr int lo = (gi * NLOAD + NSPREAD - 1) / NSPREAD, hi = ((gi + 1) * NLOAD + NSPREAD - 1) / NSPREAD;
-      static_for<hi - lo>([&](auto dc) { load_piece(std::integral_constant<int, lo + decltype(dc)::value>{}); });
+      constexpr int lo = (gi * NLOAD_ALL + NSPREAD - 1) / NSPREAD, hi = ((gi + 1) * NLOAD_ALL + NSPREAD - 1) / NSPREAD;
+      static_for<hi - lo>([&](auto dc) { load_any(std::integral_constant<int, lo + decltype(dc)::value>{}); });
     }
   };
 
@@ -645,7 +697,8 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
   // the far caches, so they are requested a whole half tile before their use.  (Where two workgroups
   // share a compute unit, D = 64 outside the dual mode, each value is instead fetched where it is used:
   // the other workgroup covers the wait and the registers stay within the cap.)
-  constexpr bool MAHEAD = (D > 64 || MODE == BWD_DUAL) && MASK != MASK_BITS;
+  constexpr bool MBYTES = MASK == MASK_BOOL || MASK == MASK_ADD;  // the mask itself, element by element
+  constexpr bool MAHEAD = (D > 64 || MODE == BWD_DUAL) && MBYTES;
   T mnext_a[MASK == MASK_ADD ? 16 : 1];
   uint8_t mnext_b[MASK == MASK_BOOL ? 16 : 1];
   // MASK_BITS: this lane's key against the 64 queries of a tile is one pair of words (bit i of word hf = query
@@ -659,7 +712,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
       bits_next = *reinterpret_cast<const u32x2 *>(bits_head + ((size_t)tile_index * (size_t)Lk + (size_t)kld) * 2);
   };
   auto fetch_mask_half = [&](int ihn) {
-    if constexpr (MASK != MASK_NONE && MASK != MASK_BITS) {
+    if constexpr (MBYTES) {
       if (mask_small && ihn + 32 <= L) {
         // uniform 64-bit row pointer + 32-bit lane offset: no per-lane address arithmetic per element
         const int64_t mrow0 = z * pr.ms[0] + hq * pr.ms[1];
@@ -682,7 +735,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     }
   };
   // ih: first query of this half tile; ihn: of the half tile that follows it
-  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn, uint32_t bits_word) {
+  auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn, uint32_t bits_word, uint32_t mbase) {
     constexpr int HB = decltype(HBc)::value;
     // dropout: the 32 queries of a half tile are one block of the pattern (ih is a multiple of 32), so the block's
     // word is uniform and register e's query adds a constant to it; this lane's key and row group add drop_lane
@@ -719,6 +772,16 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
         if constexpr (MASK == MASK_BOOL) mraw_b[e] = mnext_b[e];
       }
       fetch_mask_half(ihn);
+    }
+    // MASK_TILE: the 16 values of this half tile, four transposing reads issued ahead of every fragment read
+    // of the half tile (LDS reads complete in order, so the first fragment wait covers them)
+    u32x2 mtv[2][2];
+    if constexpr (MASK == MASK_TILE) {
+      static_for<2>([&](auto cc) {
+        constexpr int c = decltype(cc)::value, MO = (HB * 32 + c * 16) * 256;
+        mtv[c][0] = lds_tr64<MO>(mbase + mt_f[0]);
+        mtv[c][1] = lds_tr64<MO>(mbase + mt_f[1]);
+      });
     }
     // tiles in ordinary vector registers; in DUAL, dP also collects gT V'^T (the B term)
     f32x16 S, dP, Sp, At;
@@ -782,6 +845,12 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     };
     constexpr int NRT = DUAL ? 8 : 4;
     if constexpr (SAHEAD) issue_s(std::integral_constant<int, 0>{});
+    Frag<T> mfr[2];
+    if constexpr (MASK == MASK_TILE) {
+      lds_wait<SAHEAD ? Cfg::NSTAT : 0>(mtv[0][0], mtv[0][1], mtv[1][0], mtv[1][1]);  // long since there
+      mfr[0] = as_frag<T>(FragT{mtv[0][0], mtv[0][1]});
+      mfr[1] = as_frag<T>(FragT{mtv[1][0], mtv[1][1]});
+    }
     static_for<2>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
       f32x8 Pp;  // P * (S' - mu) of this chunk
@@ -799,7 +868,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
           const int qi = ih + 16 * (e / 8) + 8 * g + (e % 8);
           float s = S[e] * sl2;
           bool keep = true;
-          if constexpr (MASK != MASK_NONE && MASK != MASK_BITS && !MAHEAD) {
+          if constexpr (MBYTES && !MAHEAD) {
             if constexpr (!EDGE) {  // uniform row pointer + 32-bit lane offset, as above
               const int64_t urow = z * pr.ms[0] + hq * pr.ms[1] + (int64_t)(ih + 16 * (e / 8) + (e % 8)) * pr.ms[2];
               if constexpr (MASK == MASK_ADD) mraw_a[0] = (reinterpret_cast<const T *>(pr.mask) + urow)[mlane];
@@ -811,6 +880,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
             }
           }
           if constexpr (MASK == MASK_ADD) s += (float)mraw_a[MAHEAD ? e : 0] * LOG2E;
+          if constexpr (MASK == MASK_TILE) s += (float)mfr[e / 8][e % 8] * LOG2E;
           if constexpr (MASK == MASK_BOOL) keep = mraw_b[MAHEAD ? e : 0] != 0;
           float pv = fast_exp2(s - stat(0, e));
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
@@ -895,10 +965,11 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     prepare_loads(stage ^ 1, i0n, t + 1 < ntiles);
     load_stats();
     const uint32_t sbase = lds0 + stage * Cfg::STAGEB, sstat = stat0 + stage * Cfg::STATB;
-    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, sstat, i0, i0 + 32, bits_cur[0]);
+    const uint32_t mbase = mt0 + stage * Cfg::MTILEB;
+    half_tile(std::integral_constant<int, 0>{}, EDGEc, sbase, sstat, i0, i0 + 32, bits_cur[0], mbase);
     // always both halves: a half past the last query contributes exact zeros, and a branch here would
     // make the accumulators change register file around it
-    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32, i0n, bits_cur[1]);
+    half_tile(std::integral_constant<int, 1>{}, EDGEc, sbase, sstat, i0 + 32, i0n, bits_cur[1], mbase);
     if constexpr (MASK != MASK_NONE) {
       const int listed = list_take(tahead);
       tnext2 = tlist ? min(max(listed, 0), tmax) : tnext2;
@@ -921,7 +992,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     if constexpr (MASK != MASK_NONE && MAHEAD) fetch_mask_half(istart + tcur * BT);
     if constexpr (MASK == MASK_BITS) fetch_bits(tcur);
     prepare_loads(0, istart + tcur * BT, true);
-    static_for<NLOAD>([&](auto pc) { load_piece(pc); });
+    static_for<NLOAD_ALL>([&](auto pc) { load_any(pc); });
     load_stats();
     int t = 0;
     for (; t < t_diag; ++t) tile(t, std::true_type{});

@@ -4,9 +4,10 @@
 
 namespace jvpfa {
 
-// MASK_BITS is a boolean mask read by the dk/dv kernels from its bit-packed transposed copy (Problem::bits_k);
-// it exists as a template argument of those kernels only.
-enum MaskKind { MASK_NONE = 0, MASK_BOOL = 1, MASK_ADD = 2, MASK_BITS = 3 };
+// MASK_BITS is a boolean mask read by the dk/dv kernels from its bit-packed transposed copy (Problem::bits_k),
+// MASK_TILE an additive mask whose 64-query x 128-key tiles those kernels stream through LDS like the operand
+// tiles (rows of 16-byte aligned, contiguous keys); both exist as template arguments of those kernels only.
+enum MaskKind { MASK_NONE = 0, MASK_BOOL = 1, MASK_ADD = 2, MASK_BITS = 3, MASK_TILE = 4 };
 
 struct Problem {
   int Z, H, L;  // batch, query heads, query length

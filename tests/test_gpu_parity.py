@@ -412,6 +412,56 @@ def test_the_packed_mask_changes_no_bit_of_the_backward(dt, D, Lq, Lk, Hk):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "fp16"])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("Lq,Lk,Hk,planes", [(704, 704, 16, "zh"), (545, 832, 4, "z1"), (300, 1160, 16, "11")])
+def test_additive_masks_whose_tiles_go_through_lds(dt, D, Lq, Lk, Hk, planes):
+    """An additive mask whose rows are contiguous keys starting on 16-byte boundaries reaches the dk/dv kernels as
+    tiles in LDS (where they have the room); any other layout is fetched element by element.  Both against the
+    oracle, and against each other: the same values one element further on in memory (rows no longer aligned)
+    must give the same gradients to rounding of the last bit.  (64 heads: with fewer workgroups than compute
+    units the backward runs as one launch of both roles, which reads every mask element by element.)"""
+    from jvp_flash_attention_amd import _lib
+
+    Z, H = 4, 16
+    dtype = DTYPES[dt]
+    g = torch.Generator().manual_seed(Lq + Lk + D)
+    q, qt, go, gt = (torch.randn(Z, H, Lq, D, generator=g).to(dtype) for _ in range(4))
+    k, v, kt, vt = (torch.randn(Z, Hk, Lk, D, generator=g).to(dtype) for _ in range(4))
+    shape = {"zh": (Z, H, Lq, Lk), "z1": (Z, 1, Lq, Lk), "11": (1, 1, Lq, Lk)}[planes]
+    bias = torch.randn(*shape, generator=g).to(dtype)
+    bias[..., 17:90] = float("-inf")       # keys nobody attends
+    bias[0, 0, 33:70, :] = float("-inf")   # rows that attend nothing
+    bias[0, 0, 200:, 500:] = float("-inf")
+    f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
+    dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
+    be, scale = _lib.backend(), D**-0.5
+    print(f"case mask tiles {dt} D{D} Lq{Lq} Lk{Lk} Hk{Hk} {planes}", flush=True)
+
+    def run(dmask):
+        o, ot, M, mu = be.fwd(*dev[:6], dmask, _lib.MASK_ADD, False, scale)
+        out = list(be.bwd(*dev[:6], o, ot, M, mu, dev[6], dev[7], dmask, _lib.MASK_ADD, False, scale, want_tangent_grads=True))
+        out += be.bwd(*dev[:6], o, ot, M, mu, None, dev[7], dmask, _lib.MASK_ADD, False, scale)[:3]
+        out += be.bwd(dev[0], dev[1], dev[2], None, None, None, o, None, M, None, dev[6], None, dmask, _lib.MASK_ADD, False, scale)[:3]
+        return o, ot, out
+
+    aligned = bias.cuda()
+    assert aligned.data_ptr() % 16 == 0 and (Lk * aligned.element_size()) % 16 == 0
+    o, ot, tiled = run(aligned)
+    shifted = torch.empty(bias.numel() + 1, dtype=dtype, device="cuda")[1:].view(shape)  # one element off: no tiles
+    shifted.copy_(bias)
+    _, _, by_element = run(shifted)
+    for a, b in zip(tiled, by_element):
+        assert torch.allclose(a.float(), b.float(), rtol=0, atol=2e-2 * float(b.float().abs().max()) + 1e-30)
+    npm = np.broadcast_to(bias.float().numpy(), (Z, H, Lq, Lk))
+    ref = dense.forward(*f64[:6], mask=npm, causal=False, scale=scale)
+    rb = dense.backward(*f64, mask=npm, causal=False, scale=scale)
+    _tol_check("O", o, ref["O"], dtype)
+    _tol_check("O'", ot, ref["Ot"], dtype)
+    for n, t in zip(("dq", "dk", "dv", "dqt", "dkt", "dvt"), tiled[:6]):
+        _tol_check(n, t, rb[n], dtype)
+
+
 @pytest.mark.parametrize("dt,D", [("bf16", 32), ("bf16", 64), ("bf16", 128), ("bf16", 256),
                                   ("fp32", 32), ("fp32", 64), ("fp32", 128), ("fp32", 256)])
 @pytest.mark.parametrize("kind", ["blockdiag", "band", "pad2d", "lower"])
