@@ -184,8 +184,8 @@ def shape_rows(be, _lib):
 def mask_rows(be, _lib, q, k, v, qt, kt, vt, go, gt, scale):
     """The headline shape with explicit masks: dual forward / backward times for a dense random boolean
     mask (nothing to skip), a block-diagonal mask of four segments and a band of +-256 keys (tiles
-    without an attended entry are skipped through the tile lists), and the time of the scan that makes
-    the lists (an HBM-bound pass: it reads the mask once per list)."""
+    without an attended entry are skipped through the tile lists), the time of the scan that makes
+    the lists (an HBM-bound pass: it reads the mask once per list), and an additive mask shared by the heads."""
     import torch
 
     dev = q.device
@@ -212,6 +212,13 @@ def mask_rows(be, _lib, q, k, v, qt, kt, vt, go, gt, scale):
         rows[name] = {"attended_fraction": m.float().mean().item(), "fwd_ms": ms_f, "bwd_ms": ms_b, "scan_ms": ms_s,
                       "scan_GBps": 2.0 * m.numel() / (ms_s * 1e-3) / 1e9}
         del m
+    # an additive mask (a bias shared by the heads): dual forward / backward and the backward without tangents
+    bias = torch.randn(Z, 1, L, L, generator=g, device=dev).to(q.dtype)
+    ms_f, _ = timed(lambda: be.fwd(q, k, v, qt, kt, vt, bias, _lib.MASK_ADD, False, scale), 20, 12)
+    o, ot, M, mu = be.fwd(q, k, v, qt, kt, vt, bias, _lib.MASK_ADD, False, scale)
+    ms_b, _ = timed(lambda: be.bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, bias, _lib.MASK_ADD, False, scale), 10, 6)
+    ms_p, _ = timed(lambda: be.bwd(q, k, v, None, None, None, o, None, M, None, go, None, bias, _lib.MASK_ADD, False, scale), 10, 6)
+    rows["additive_bias_Z1LL"] = {"attended_fraction": 1.0, "fwd_ms": ms_f, "bwd_ms": ms_b, "bwd_without_tangents_ms": ms_p}
     return rows
 
 

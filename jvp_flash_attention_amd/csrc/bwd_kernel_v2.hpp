@@ -303,7 +303,8 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
       if constexpr (MASK != MASK_NONE) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          if constexpr (MASK == MASK_ADD) bias[e] = mask_bias_of<T, MASK>(mah[hf], e);
+          // the mask value and the row's reference point in one term: the exponent is then one fused multiply-add
+          if constexpr (MASK == MASK_ADD) bias[e] = fmaf((float)mah[hf].f[e], LOG2E, -Mq);
           if constexpr (MASK == MASK_BOOL) keep[e] = mask_keep_of<T, MASK>(mah[hf], e);
         }
       }
@@ -311,9 +312,9 @@ __device__ __forceinline__ void bwd2_dq_body(const BwdParams &p, const int bid) 
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int i = 8 * hf + e;
-        float s = S[i] * sl2;
-        if constexpr (MASK == MASK_ADD) s += bias[e];
-        float pv = fast_exp2(s - Mq);
+        float pv;
+        if constexpr (MASK == MASK_ADD) pv = fast_exp2(fmaf(S[i], sl2, bias[e]));
+        else pv = fast_exp2(S[i] * sl2 - Mq);
         if constexpr (MASK == MASK_BOOL) pv = keep[e] ? pv : 0.f;
         if constexpr (EDGE) pv = (key0 + e <= klim) ? pv : 0.f;
         if constexpr (DROP) {
@@ -879,10 +880,12 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
               if constexpr (MASK == MASK_BOOL) mraw_b[0] = reinterpret_cast<const uint8_t *>(pr.mask)[off];
             }
           }
-          if constexpr (MASK == MASK_ADD) s += (float)mraw_a[MAHEAD ? e : 0] * LOG2E;
-          if constexpr (MASK == MASK_TILE) s += (float)mfr[e / 8][e % 8] * LOG2E;
           if constexpr (MASK == MASK_BOOL) keep = mraw_b[MAHEAD ? e : 0] != 0;
-          float pv = fast_exp2(s - stat(0, e));
+          // (additive: the mask value and the row's reference point in one term, the exponent one fused multiply-add)
+          float pv;
+          if constexpr (MASK == MASK_ADD) pv = fast_exp2(fmaf(S[e], sl2, fmaf((float)mraw_a[MAHEAD ? e : 0], LOG2E, -stat(0, e))));
+          else if constexpr (MASK == MASK_TILE) pv = fast_exp2(fmaf(S[e], sl2, fmaf((float)mfr[e / 8][e % 8], LOG2E, -stat(0, e))));
+          else pv = fast_exp2(s - stat(0, e));
           if constexpr (MASK == MASK_BOOL) pv = keep ? pv : 0.f;
           if constexpr (MASK == MASK_BITS) {
             // the entry's bit spread over a word (0 or all ones), and-ed onto P: two instructions (written as
