@@ -63,7 +63,7 @@ static auto pick_dkdv_for(const BwdParams &p, bool no_go, bool grouped, bool fol
   if constexpr (MASK == MASK_BOOL) {
     if (p.pr.bits_k) return pick_dkdv<T, D, MODE, MASK_BITS>(no_go, grouped, fold_kv, drop);
   }
-  if constexpr (MASK == MASK_ADD && Cfg2::MTILE_FITS) {
+  if constexpr (MASK == MASK_ADD) {
     if (mask_rows_tileable<T>(p.pr)) {
       *lds = Cfg2::DKV_LDS_MTILE;
       return pick_dkdv<T, D, MODE, MASK_TILE>(no_go, grouped, fold_kv, drop);

@@ -31,10 +31,12 @@ template <typename T, int D, int MODE> struct Bwd2Cfg {
   static constexpr int STATB = NSTAT * BT * 4;        // row statistics of a query tile (dk/dv only)
   static constexpr size_t DQ_LDS = 2 * (size_t)STAGEB;
   static constexpr size_t DKV_LDS = 2 * (size_t)STAGEB + 2 * (size_t)STATB;
-  // MASK_TILE: two stages of a 64-query x 128-key tile of a 16-bit additive mask behind the statistics
+  // MASK_TILE: two stages of a 64-query x 128-key tile of a 16-bit additive mask behind the statistics; where
+  // two do not fit (the dual mode at D = 128) one, which every wave empties into registers at the top of a tile,
+  // in front of a second barrier, before the direct loads of the tile refill it
   static constexpr int MTILEB = BT * 256;
-  static constexpr size_t DKV_LDS_MTILE = DKV_LDS + 2 * (size_t)MTILEB;
-  static constexpr bool MTILE_FITS = DKV_LDS_MTILE <= 160 * 1024;
+  static constexpr bool MTILE_SINGLE = DKV_LDS + 2 * (size_t)MTILEB > 160 * 1024;
+  static constexpr size_t DKV_LDS_MTILE = DKV_LDS + (MTILE_SINGLE ? 1 : 2) * (size_t)MTILEB;
 };
 
 // One LDS fragment (8 elements per lane) read ahead with lds_b128 / two lds_tr64.
@@ -659,7 +661,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
       const int rows = on ? max(L - i0, 0) : 0;
       const int64_t bytes = rows > 0 ? (int64_t)(rows - 1) * mt_row + (int64_t)(Lk - k0) * (int64_t)sizeof(T) : 0;
       mt_rs = __builtin_amdgcn_make_buffer_rsrc((void *)(mt_head + (int64_t)i0 * mt_row), 0, (int)min(bytes, (int64_t)0x7fffffff), 0x00020000);
-      mt_dst = mt0 + stage * Cfg::MTILEB + (wave * 4) * 1024;
+      mt_dst = mt0 + (Cfg::MTILE_SINGLE ? 0 : stage * Cfg::MTILEB) + (wave * 4) * 1024;
     }
     i0 = on ? i0 : istart;
     st_row = min(i0 + lane, L - 1);
@@ -735,6 +737,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
       }
     }
   };
+  u32x2 mt_all[2][2][2];  // MASK_TILE with one stage: [half tile][chunk of 16 queries][4-row half]
   // ih: first query of this half tile; ihn: of the half tile that follows it
   auto half_tile = [&](auto HBc, auto EDGEc, uint32_t sbase, uint32_t sstat, int ih, int ihn, uint32_t bits_word, uint32_t mbase) {
     constexpr int HB = decltype(HBc)::value;
@@ -777,7 +780,7 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     // MASK_TILE: the 16 values of this half tile, four transposing reads issued ahead of every fragment read
     // of the half tile (LDS reads complete in order, so the first fragment wait covers them)
     u32x2 mtv[2][2];
-    if constexpr (MASK == MASK_TILE) {
+    if constexpr (MASK == MASK_TILE && !Cfg::MTILE_SINGLE) {
       static_for<2>([&](auto cc) {
         constexpr int c = decltype(cc)::value, MO = (HB * 32 + c * 16) * 256;
         mtv[c][0] = lds_tr64<MO>(mbase + mt_f[0]);
@@ -847,7 +850,10 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     constexpr int NRT = DUAL ? 8 : 4;
     if constexpr (SAHEAD) issue_s(std::integral_constant<int, 0>{});
     Frag<T> mfr[2];
-    if constexpr (MASK == MASK_TILE) {
+    if constexpr (MASK == MASK_TILE && Cfg::MTILE_SINGLE) {
+      mfr[0] = as_frag<T>(FragT{mt_all[HB][0][0], mt_all[HB][0][1]});
+      mfr[1] = as_frag<T>(FragT{mt_all[HB][1][0], mt_all[HB][1][1]});
+    } else if constexpr (MASK == MASK_TILE) {
       lds_wait<SAHEAD ? Cfg::NSTAT : 0>(mtv[0][0], mtv[0][1], mtv[1][0], mtv[1][1]);  // long since there
       mfr[0] = as_frag<T>(FragT{mtv[0][0], mtv[0][1]});
       mfr[1] = as_frag<T>(FragT{mtv[1][0], mtv[1][1]});
@@ -957,6 +963,20 @@ __device__ __forceinline__ void bwd2_dkdv_body(const BwdParams &p, const int bid
     const int stage = t & 1;
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
+    if constexpr (MASK == MASK_TILE && Cfg::MTILE_SINGLE) {
+      // the one stage of the mask tile: every wave takes its 32 values of this tile now; behind the second
+      // barrier the stage belongs to the direct loads of the next tile
+      static_for<4>([&](auto ic) {
+        constexpr int hb = decltype(ic)::value / 2, c = decltype(ic)::value % 2, MO = (hb * 32 + c * 16) * 256;
+        mt_all[hb][c][0] = lds_tr64<MO>(mt0 + mt_f[0]);
+        mt_all[hb][c][1] = lds_tr64<MO>(mt0 + mt_f[1]);
+      });
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier"
+                   : "+v"(mt_all[0][0][0]), "+v"(mt_all[0][0][1]), "+v"(mt_all[0][1][0]), "+v"(mt_all[0][1][1]),
+                     "+v"(mt_all[1][0][0]), "+v"(mt_all[1][0][1]), "+v"(mt_all[1][1][0]), "+v"(mt_all[1][1][1])
+                   :
+                   : "memory");
+    }
     u32x2 bits_cur = bits_next;
     if constexpr (MASK == MASK_BITS) {
       asm volatile("" : "+v"(bits_cur));  // taken over here, behind the wait above
