@@ -414,7 +414,8 @@ def test_the_packed_mask_changes_no_bit_of_the_backward(dt, D, Lq, Lk, Hk):
 
 @pytest.mark.parametrize("dt", ["bf16", "fp16"])
 @pytest.mark.parametrize("D", [32, 64, 128])
-@pytest.mark.parametrize("Lq,Lk,Hk,planes", [(704, 704, 16, "zh"), (545, 832, 4, "z1"), (300, 1160, 16, "11")])
+@pytest.mark.parametrize("Lq,Lk,Hk,planes", [(704, 704, 16, "zh"), (545, 832, 4, "z1"), (300, 1160, 16, "11"),
+                                             (600, 712, 16, "keys")])
 def test_additive_masks_whose_tiles_go_through_lds(dt, D, Lq, Lk, Hk, planes):
     """An additive mask whose rows are contiguous keys starting on 16-byte boundaries reaches the dk/dv kernels as
     tiles in LDS (where they have the room); any other layout is fetched element by element.  Both against the
@@ -428,11 +429,13 @@ def test_additive_masks_whose_tiles_go_through_lds(dt, D, Lq, Lk, Hk, planes):
     g = torch.Generator().manual_seed(Lq + Lk + D)
     q, qt, go, gt = (torch.randn(Z, H, Lq, D, generator=g).to(dtype) for _ in range(4))
     k, v, kt, vt = (torch.randn(Z, Hk, Lk, D, generator=g).to(dtype) for _ in range(4))
-    shape = {"zh": (Z, H, Lq, Lk), "z1": (Z, 1, Lq, Lk), "11": (1, 1, Lq, Lk)}[planes]
+    # "keys": one row of keys per batch entry, shared by heads and queries (a mask row of stride 0)
+    shape = {"zh": (Z, H, Lq, Lk), "z1": (Z, 1, Lq, Lk), "11": (1, 1, Lq, Lk), "keys": (Z, 1, 1, Lk)}[planes]
     bias = torch.randn(*shape, generator=g).to(dtype)
     bias[..., 17:90] = float("-inf")       # keys nobody attends
-    bias[0, 0, 33:70, :] = float("-inf")   # rows that attend nothing
-    bias[0, 0, 200:, 500:] = float("-inf")
+    if planes != "keys":
+        bias[0, 0, 33:70, :] = float("-inf")   # rows that attend nothing
+        bias[0, 0, 200:, 500:] = float("-inf")
     f64 = [x.double().numpy() for x in (q, k, v, qt, kt, vt, go, gt)]
     dev = [x.cuda() for x in (q, k, v, qt, kt, vt, go, gt)]
     be, scale = _lib.backend(), D**-0.5
