@@ -473,5 +473,40 @@ def _(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_sca
     return (*full, *rest)
 
 
+# Dropout inside a compiled graph.  The seed of a call is a host integer, and drawing it in traced code would
+# end the graph, so these two operators draw it themselves: ``jvpfa::fwd_drop`` takes a fresh seed from torch's
+# CPU generator (as the eager path does, so ``torch.manual_seed`` makes either repeatable) and hands it out as a
+# one-element int64 CPU tensor, which the Function saves for ``jvpfa::bwd_drop``.  Tagged as seeded random
+# operators, so the compiler neither merges two such calls nor drops one.
+_RANDOM = (torch.Tag.nondeterministic_seeded,)
+
+
+@torch.library.custom_op("jvpfa::fwd_drop", mutates_args=(), device_types="cuda", tags=_RANDOM)
+def _op_fwd_drop(q: _T, k: _T, v: _T, mask: _OT, mask_kind: int, causal: bool, sm_scale: float,
+                 dropout_p: float) -> Tuple[_T, _T, _T]:
+    seed = torch.randint(0, 2**62, (1,), dtype=torch.int64)
+    o, _ot, M, _mu = _hip._fwd(q, k, v, None, None, None, mask, mask_kind, causal, sm_scale, dropout_p, int(seed.item()))
+    return o, M, seed
+
+
+@_op_fwd_drop.register_fake
+def _(q, k, v, mask, mask_kind, causal, sm_scale, dropout_p):
+    Z, H, L, _ = q.shape
+    return torch.empty_like(q), q.new_empty((Z, H, L), dtype=torch.float32), torch.empty(1, dtype=torch.int64, device="cpu")
+
+
+@torch.library.custom_op("jvpfa::bwd_drop", mutates_args=(), device_types="cuda")
+def _op_bwd_drop(q: _T, k: _T, v: _T, o: _T, M: _T, go: _T, mask: _OT, mask_kind: int, causal: bool, sm_scale: float,
+                 dropout_p: float, seed: _T) -> Tuple[_T, _T, _T]:
+    dq, dk, dv, _, _, _ = _hip._bwd(q, k, v, None, None, None, o, None, M, None, go, None, mask, mask_kind, causal,
+                                    sm_scale, False, dropout_p, int(seed.item()))
+    return dq, dk, dv
+
+
+@_op_bwd_drop.register_fake
+def _(q, k, v, o, M, go, mask, mask_kind, causal, sm_scale, dropout_p, seed):
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
 def backend():
     return _backend

@@ -232,6 +232,33 @@ class _PlainCore(Function):
         return dq, dk, dv, None, None, None, None, None, None
 
 
+class _PlainCoreDrop(Function):
+    """``_PlainCore`` with dropout for code under ``torch.compile``: the operators draw and carry the seed
+    themselves (see ``_lib.py``), so the call stays inside the graph."""
+
+    @staticmethod
+    def forward(q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p):
+        o, M, seed = torch.ops.jvpfa.fwd_drop(q, k, v, mask_tensor, int(MASK_TYPE), bool(causal), float(sm_scale),
+                                              float(dropout_p))
+        return o, M, seed
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p = inputs
+        o, M, seed = outputs
+        ctx.mark_non_differentiable(M, seed)
+        ctx.save_for_backward(q, k, v, o, M, seed)
+        ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale, ctx.dropout_p = mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, go, _gM, _gseed):
+        q, k, v, o, M, seed = ctx.saved_tensors
+        dq, dk, dv = torch.ops.jvpfa.bwd_drop(q, k, v, o, M, _dense(go), ctx.mask_tensor, int(ctx.MASK_TYPE),
+                                              bool(ctx.causal), float(ctx.sm_scale), float(ctx.dropout_p), seed)
+        return dq, dk, dv, None, None, None, None, None
+
+
 class _AttachTangent(Function):
     """Identity on O whose forward-mode tangent is the precomputed O' (the reference's trick of
     JA:2688 and JA:2828, with O' an input so that it keeps its autograd graph)."""
@@ -449,13 +476,15 @@ class JVPAttn(Function):
         if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
             q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         if torch.compiler.is_compiling():
-            if dropout_p > 0.0:  # the seed is drawn on the host: such a call runs between two compiled pieces
-                return _fwd_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
             # the same computation through a Function the tracer can follow (no custom jvp, no
-            # data-dependent mask checks); the kernels appear in the graph as jvpfa::fwd / jvpfa::bwd
+            # data-dependent mask checks); the kernels appear in the graph as jvpfa::fwd / jvpfa::bwd, with
+            # dropout as jvpfa::fwd_drop / jvpfa::bwd_drop, which draw and carry the seed themselves
             _validate(q, k, v, attn_mask, dropout_p, causal)
             scale = q.shape[-1] ** -0.5 if sm_scale is None else sm_scale
             mask_tensor, MASK_TYPE = _classify_mask(attn_mask, q, False)
+            if dropout_p > 0.0:
+                o, _M, _seed = _PlainCoreDrop.apply(q, k, v, mask_tensor, MASK_TYPE, causal, scale, dropout_p)
+                return o
             o, _M = _PlainCore.apply(q, k, v, mask_tensor, MASK_TYPE, causal, scale, 0.0, 0)
             return o
         if fwAD._current_level < 0 and not _transforms_active():
@@ -493,7 +522,7 @@ class JVPAttn(Function):
             # The tracer cannot follow the custom jvp that hands O' to forward-mode AD.  With a
             # forward-mode level active the call is therefore left out of the graph and runs as
             # ordinary Python between two compiled pieces; without one no tangent can exist.
-            if fwAD._current_level >= 0 or dropout_p > 0.0:
+            if fwAD._current_level >= 0:
                 return _fwd_dual_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
             return JVPAttn.fwd(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
         if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
@@ -543,11 +572,6 @@ class JVPAttn(Function):
             dropout_p=ctx.dropout_p, dropout_seed=ctx.philox_seed,
         )
         return JVPAttn.BwdOut(dq, dk, dv, None, None, None, None, None, None, None, None, None, None)
-
-
-@torch.compiler.disable
-def _fwd_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA):
-    return JVPAttn.fwd(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
 
 
 @torch.compiler.disable

@@ -205,6 +205,40 @@ def test_plain_attention_inside_torch_compile_without_graph_breaks(masked):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("masked", [False, True])
+def test_dropout_inside_torch_compile_without_graph_breaks(masked):
+    """``attention`` with dropout under ``torch.compile(fullgraph=True)``: the operators ``jvpfa::fwd_drop`` /
+    ``jvpfa::bwd_drop`` draw the seed from torch's CPU generator themselves, as the eager call does, so after the
+    same ``torch.manual_seed`` output and gradients equal the eager ones bit for bit; a second compiled call
+    draws another pattern."""
+    from jvp_flash_attention_amd import attention
+
+    Z, H, L, D = 2, 4, 256, 64
+    q, k, v = [_randn((Z, H, L, D), torch.bfloat16, 75 + i).requires_grad_() for i in range(3)]
+    kw = dict(causal=True, dropout_p=0.25)
+    if masked:
+        keep = torch.rand(Z, 1, L, L, device="cuda", generator=torch.Generator(device="cuda").manual_seed(6)) > 0.3
+        keep[..., 0] = True
+        kw = dict(attn_mask=keep, dropout_p=0.25)
+
+    def f(q, k, v):
+        return (attention(q * 1.0, k, v, **kw) * 2.0).float().sum()
+
+    torch.manual_seed(11)
+    ref = f(q, k, v)
+    gref = torch.autograd.grad(ref, (q, k, v))
+    torch._dynamo.reset()
+    compiled = torch.compile(f, backend="aot_eager", fullgraph=True)
+    torch.manual_seed(11)
+    out = compiled(q, k, v)
+    g = torch.autograd.grad(out, (q, k, v))
+    assert torch.equal(out, ref)
+    for a, b in zip(g, gref):
+        assert torch.equal(a, b)
+    again = compiled(q, k, v)  # the generator has moved on: another pattern
+    assert not torch.equal(again, ref)
+
+
 def test_dual_tensors_inside_torch_compile_keep_their_tangent():
     """Forward-mode AD inside a compiled function: the attention call is left out of the graph and
     runs between two compiled pieces, so O' is what the eager call gives, not silently dropped."""
