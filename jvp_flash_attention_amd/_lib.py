@@ -482,30 +482,37 @@ _RANDOM = (torch.Tag.nondeterministic_seeded,)
 
 
 @torch.library.custom_op("jvpfa::fwd_drop", mutates_args=(), device_types="cuda", tags=_RANDOM)
-def _op_fwd_drop(q: _T, k: _T, v: _T, mask: _OT, mask_kind: int, causal: bool, sm_scale: float,
-                 dropout_p: float) -> Tuple[_T, _T, _T]:
+def _op_fwd_drop(q: _T, k: _T, v: _T, qt: _OT, kt: _OT, vt: _OT, mask: _OT, mask_kind: int, causal: bool,
+                 sm_scale: float, dropout_p: float) -> Tuple[_T, _T, _T, _T, _T]:
     seed = torch.randint(0, 2**62, (1,), dtype=torch.int64)
-    o, _ot, M, _mu = _hip._fwd(q, k, v, None, None, None, mask, mask_kind, causal, sm_scale, dropout_p, int(seed.item()))
-    return o, M, seed
+    o, ot, M, mu = _hip._fwd(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale, dropout_p, int(seed.item()))
+    return o, (ot if ot is not None else q.new_empty(0)), M, (mu if mu is not None else M.new_empty(0)), seed
 
 
 @_op_fwd_drop.register_fake
-def _(q, k, v, mask, mask_kind, causal, sm_scale, dropout_p):
+def _(q, k, v, qt, kt, vt, mask, mask_kind, causal, sm_scale, dropout_p):
     Z, H, L, _ = q.shape
-    return torch.empty_like(q), q.new_empty((Z, H, L), dtype=torch.float32), torch.empty(1, dtype=torch.int64, device="cpu")
+    stat = q.new_empty((Z, H, L), dtype=torch.float32)
+    seed = torch.empty(1, dtype=torch.int64, device="cpu")
+    if qt is None:
+        return torch.empty_like(q), q.new_empty(0), stat, stat.new_empty(0), seed
+    return torch.empty_like(q), torch.empty_like(q), stat, torch.empty_like(stat), seed
 
 
 @torch.library.custom_op("jvpfa::bwd_drop", mutates_args=(), device_types="cuda")
-def _op_bwd_drop(q: _T, k: _T, v: _T, o: _T, M: _T, go: _T, mask: _OT, mask_kind: int, causal: bool, sm_scale: float,
-                 dropout_p: float, seed: _T) -> Tuple[_T, _T, _T]:
-    dq, dk, dv, _, _, _ = _hip._bwd(q, k, v, None, None, None, o, None, M, None, go, None, mask, mask_kind, causal,
-                                    sm_scale, False, dropout_p, int(seed.item()))
-    return dq, dk, dv
+def _op_bwd_drop(q: _T, k: _T, v: _T, qt: _OT, kt: _OT, vt: _OT, o: _T, ot: _OT, M: _T, mu: _OT, go: _OT, gt: _OT,
+                 mask: _OT, mask_kind: int, causal: bool, sm_scale: float, want_tangent_grads: bool,
+                 dropout_p: float, seed: _T) -> Tuple[_T, _T, _T, _T, _T, _T]:
+    g = _hip._bwd(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale, want_tangent_grads,
+                  dropout_p, int(seed.item()))
+    return tuple(t if t is not None else q.new_empty(0) for t in g)
 
 
 @_op_bwd_drop.register_fake
-def _(q, k, v, o, M, go, mask, mask_kind, causal, sm_scale, dropout_p, seed):
-    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+def _(q, k, v, qt, kt, vt, o, ot, M, mu, go, gt, mask, mask_kind, causal, sm_scale, want_tangent_grads, dropout_p, seed):
+    full = [torch.empty_like(t) for t in (q, k, v)]
+    rest = [torch.empty_like(t) if want_tangent_grads else q.new_empty(0) for t in (q, k, v)]
+    return (*full, *rest)
 
 
 def backend():

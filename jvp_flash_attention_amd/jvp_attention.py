@@ -232,14 +232,34 @@ class _PlainCore(Function):
         return dq, dk, dv, None, None, None, None, None, None
 
 
+class _DualCoreTraced(Function):
+    """``_DualCore`` for code under ``torch.compile``: the same forward and backward without the look through
+    ``torch.func`` wrappers, which the tracer cannot follow (and which do not occur while it traces)."""
+
+    forward = _DualCore.forward
+    setup_context = _DualCore.setup_context
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, go, gt, _gM, _gmu):
+        q, k, v, q_t, k_t, v_t, o, o_t, M, mu = ctx.saved_tensors
+        want_t = any(ctx.needs_input_grad[3:6])
+        dq, dk, dv, dqt, dkt, dvt = _lib.backend().bwd(
+            q, k, v, q_t, k_t, v_t, o, o_t, M, mu, _dense(go), _dense(gt),
+            ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale, want_tangent_grads=want_t,
+            dropout_p=ctx.dropout_p, dropout_seed=ctx.philox_seed,
+        )
+        return dq, dk, dv, dqt, dkt, dvt, None, None, None, None, None, None
+
+
 class _PlainCoreDrop(Function):
     """``_PlainCore`` with dropout for code under ``torch.compile``: the operators draw and carry the seed
     themselves (see ``_lib.py``), so the call stays inside the graph."""
 
     @staticmethod
     def forward(q, k, v, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p):
-        o, M, seed = torch.ops.jvpfa.fwd_drop(q, k, v, mask_tensor, int(MASK_TYPE), bool(causal), float(sm_scale),
-                                              float(dropout_p))
+        o, _ot, M, _mu, seed = torch.ops.jvpfa.fwd_drop(q, k, v, None, None, None, mask_tensor, int(MASK_TYPE),
+                                                        bool(causal), float(sm_scale), float(dropout_p))
         return o, M, seed
 
     @staticmethod
@@ -254,9 +274,39 @@ class _PlainCoreDrop(Function):
     @once_differentiable
     def backward(ctx, go, _gM, _gseed):
         q, k, v, o, M, seed = ctx.saved_tensors
-        dq, dk, dv = torch.ops.jvpfa.bwd_drop(q, k, v, o, M, _dense(go), ctx.mask_tensor, int(ctx.MASK_TYPE),
-                                              bool(ctx.causal), float(ctx.sm_scale), float(ctx.dropout_p), seed)
+        dq, dk, dv, _, _, _ = torch.ops.jvpfa.bwd_drop(
+            q, k, v, None, None, None, o, None, M, None, _dense(go), None, ctx.mask_tensor, int(ctx.MASK_TYPE),
+            bool(ctx.causal), float(ctx.sm_scale), False, float(ctx.dropout_p), seed)
         return dq, dk, dv, None, None, None, None, None
+
+
+class _DualCoreDrop(Function):
+    """``_DualCoreTraced`` with dropout, on the operators that draw and carry the seed themselves."""
+
+    @staticmethod
+    def forward(q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p):
+        return torch.ops.jvpfa.fwd_drop(q, k, v, q_t, k_t, v_t, mask_tensor, int(MASK_TYPE), bool(causal),
+                                        float(sm_scale), float(dropout_p))
+
+    @staticmethod
+    def setup_context(ctx, inputs, outputs):
+        q, k, v, q_t, k_t, v_t, mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p = inputs
+        o, o_t, M, mu, seed = outputs
+        ctx.mark_non_differentiable(M, mu, seed)
+        ctx.save_for_backward(q, k, v, q_t, k_t, v_t, o, o_t, M, mu, seed)
+        ctx.mask_tensor, ctx.MASK_TYPE, ctx.causal, ctx.sm_scale, ctx.dropout_p = mask_tensor, MASK_TYPE, causal, sm_scale, dropout_p
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, go, gt, _gM, _gmu, _gseed):
+        q, k, v, q_t, k_t, v_t, o, o_t, M, mu, seed = ctx.saved_tensors
+        want_t = any(ctx.needs_input_grad[3:6])
+        out = torch.ops.jvpfa.bwd_drop(
+            q, k, v, q_t, k_t, v_t, o, o_t, M, mu, _dense(go), _dense(gt), ctx.mask_tensor, int(ctx.MASK_TYPE),
+            bool(ctx.causal), float(ctx.sm_scale), bool(want_t), float(ctx.dropout_p), seed)
+        dq, dk, dv = out[:3]
+        dqt, dkt, dvt = out[3:] if want_t else (None, None, None)
+        return dq, dk, dv, dqt, dkt, dvt, None, None, None, None, None
 
 
 class _AttachTangent(Function):
@@ -519,11 +569,29 @@ class JVPAttn(Function):
         kernel pass as O.  Both O and O' are differentiable (reverse mode) in q, k, v and in the
         input tangents."""
         if torch.compiler.is_compiling():
-            # The tracer cannot follow the custom jvp that hands O' to forward-mode AD.  With a
-            # forward-mode level active the call is therefore left out of the graph and runs as
-            # ordinary Python between two compiled pieces; without one no tangent can exist.
+            # (without a forward-mode level no tangent can exist: the plain path below)
             if fwAD._current_level >= 0:
-                return _fwd_dual_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
+                # The tracer follows forward-mode levels and dual tensors, but not a Function with a custom jvp:
+                # the tangents are taken off the inputs, O and O' come from the Function that is differentiable
+                # in all six (the kernels enter the graph as jvpfa::fwd / jvpfa::bwd), and O' is put back on O.
+                q_p, q_t = fwAD.unpack_dual(q)
+                k_p, k_t = fwAD.unpack_dual(k)
+                v_p, v_t = fwAD.unpack_dual(v)
+                if q_t is not None or k_t is not None or v_t is not None:
+                    q_p, k_p, v_p = _dense(q_p), _dense(k_p), _dense(v_p)
+                    _validate(q_p, k_p, v_p, attn_mask, dropout_p, causal)
+                    scale = q_p.shape[-1] ** -0.5 if sm_scale is None else sm_scale
+                    mask_tensor, MASK_TYPE = _classify_mask(attn_mask, q_p, False)
+                    q_t = torch.zeros_like(q_p) if q_t is None else _dense(q_t)
+                    k_t = torch.zeros_like(k_p) if k_t is None else _dense(k_t)
+                    v_t = torch.zeros_like(v_p) if v_t is None else _dense(v_t)
+                    if dropout_p > 0.0:
+                        o, o_t, _M, _mu, _seed = _DualCoreDrop.apply(q_p, k_p, v_p, q_t, k_t, v_t, mask_tensor,
+                                                                     MASK_TYPE, causal, scale, dropout_p)
+                    else:
+                        o, o_t, _M, _mu = _DualCoreTraced.apply(q_p, k_p, v_p, q_t, k_t, v_t, mask_tensor, MASK_TYPE,
+                                                                causal, scale, 0.0, 0)
+                    return fwAD.make_dual(o, o_t)
             return JVPAttn.fwd(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
         if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
             q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
@@ -572,11 +640,6 @@ class JVPAttn(Function):
             dropout_p=ctx.dropout_p, dropout_seed=ctx.philox_seed,
         )
         return JVPAttn.BwdOut(dq, dk, dv, None, None, None, None, None, None, None, None, None, None)
-
-
-@torch.compiler.disable
-def _fwd_dual_outside_graph(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA):
-    return JVPAttn.fwd_dual(q, k, v, attn_mask, dropout_p, causal, sm_scale, warp_specialize, USE_TMA)
 
 
 def attention(

@@ -239,9 +239,39 @@ def test_dropout_inside_torch_compile_without_graph_breaks(masked):
     assert not torch.equal(again, ref)
 
 
+@pytest.mark.parametrize("dropout_p", [0.0, 0.3])
+def test_forward_mode_inside_torch_compile_without_graph_breaks(dropout_p):
+    """A forward-mode level opened inside a function compiled with ``fullgraph=True``: ``fwd_dual`` takes the
+    tangents off its inputs, runs the dual kernels as ``jvpfa::fwd`` and puts O' back on O; O, O' and the
+    gradients of a loss on both (through ``jvpfa::bwd``) equal the eager ones bit for bit."""
+    from jvp_flash_attention_amd import JVPAttn
+
+    Z, H, L, D = 2, 2, 192, 64
+    q, k, v = [_randn((Z, H, L, D), torch.bfloat16, 85 + i).requires_grad_() for i in range(3)]
+    qt, kt, vt = [_randn((Z, H, L, D), torch.bfloat16, 88 + i) for i in range(3)]
+
+    def g(q, k, v, qt, kt, vt):
+        with fwAD.dual_level():
+            out = JVPAttn.fwd_dual(fwAD.make_dual(q * 1.0, qt), fwAD.make_dual(k, kt), fwAD.make_dual(v, vt), causal=True,
+                                   dropout_p=dropout_p)
+            o, ot = fwAD.unpack_dual(out * 2.0)
+            return o.float().sum() + (ot.float() ** 2).sum(), o.detach().clone(), ot.detach().clone()
+
+    torch.manual_seed(3)
+    loss1, o1, ot1 = g(q, k, v, qt, kt, vt)
+    g1 = torch.autograd.grad(loss1, (q, k, v))
+    torch._dynamo.reset()
+    torch.manual_seed(3)
+    loss2, o2, ot2 = torch.compile(g, backend="aot_eager", fullgraph=True)(q, k, v, qt, kt, vt)
+    g2 = torch.autograd.grad(loss2, (q, k, v))
+    assert torch.equal(o1, o2) and torch.equal(ot1, ot2) and torch.equal(loss1, loss2)
+    for a, b in zip(g1, g2):
+        assert torch.equal(a, b)
+
+
 def test_dual_tensors_inside_torch_compile_keep_their_tangent():
-    """Forward-mode AD inside a compiled function: the attention call is left out of the graph and
-    runs between two compiled pieces, so O' is what the eager call gives, not silently dropped."""
+    """Forward-mode AD inside a compiled function (here with the ``eager`` backend, which runs the traced graph
+    as it stands): O' is what the eager call gives, not silently dropped."""
     from jvp_flash_attention_amd import JVPAttn
 
     Z, H, L, D = 1, 2, 128, 64
