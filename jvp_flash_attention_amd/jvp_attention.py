@@ -35,6 +35,9 @@ Differences from the reference, all deliberate:
   the backward.  (bf16 / fp16 calls get 6 - 13 % slower at head dim 128, about 30 % at 64, fp32 1 - 6 %.)
 * ``attention`` notices dual inputs and then behaves like ``fwd_dual`` (the reference's ``attention``
   is ``JVPAttn.fwd`` and drops the tangent, its README.md:65-67).
+* Under ``torch.compile`` every call stays inside the graph (``fullgraph=True``), also with a forward-mode level
+  opened inside the compiled function and with dropout; the reference's Function defines ``jvp``, which the tracer
+  refuses, so there every call is a graph break.
 """
 from __future__ import annotations
 
