@@ -456,6 +456,16 @@ def test_additive_masks_whose_tiles_go_through_lds(dt, D, Lq, Lk, Hk, planes):
     _, _, by_element = run(shifted)
     for a, b in zip(tiled, by_element):
         assert torch.allclose(a.float(), b.float(), rtol=0, atol=2e-2 * float(b.float().abs().max()) + 1e-30)
+    if planes == "zh":  # with tile lists (tiles that are -inf throughout are not visited): not a bit changes
+        _lib.set_tile_lists(True, additive=True)
+        try:
+            listed_mask = bias.cuda()
+            _, _, listed = run(listed_mask)
+            assert getattr(listed_mask, "_jvpfa_tiles")[2] is not None
+        finally:
+            _lib.set_tile_lists(True, additive=False)
+        for a, b in zip(listed, tiled):
+            assert torch.equal(a, b)
     npm = np.broadcast_to(bias.float().numpy(), (Z, H, Lq, Lk))
     ref = dense.forward(*f64[:6], mask=npm, causal=False, scale=scale)
     rb = dense.backward(*f64, mask=npm, causal=False, scale=scale)
