@@ -1,7 +1,7 @@
 """Accuracy and speed report for JVP attention on the current GPU.
 
     python -m jvp_flash_attention_amd.validate --dtype bfloat16 [--seq-lengths 32 64 ... 2048]
-                                               [--no-masks] [--no-timing] [--json out.json]
+                                               [--no-masks] [--no-timing] [--json out.json] [--plots DIR]
 
 Counterpart of the reference's script ``tests/test_jvp_attention.py`` (run as a program there,
 README.md:111-113): for every sequence length, mask type (none / boolean / additive) and causal
@@ -12,7 +12,8 @@ forward the way the reference does (10 warm-up + 100 calls, input clones and ``m
 included, lines 129-143 and 770-780) next to math SDPA; (3) records the peak memory of one call.
 After the per-case lines it prints the reference's two tables (summary per case and method, lines 883-937;
 time by mask type, lines 940-976) and its speed-up statistics, and writes them with the rows into the JSON
-file (lines 1172-1227); the reference's PNG plots (lines 977-1091) are not drawn.
+file (lines 1172-1227); with ``--plots DIR`` it also draws the reference's two figures (lines 977-1091): speed-up over
+math SDPA and peak memory per sequence length, one panel per (causal, mask) configuration.
 Shapes default to the reference's (batch 2, 12 heads, head dim 64, lines 225-230); masks are its
 random masks with keep-probability 0.1 (lines 334-394).  TFLOP/s uses the reference's FLOP
 convention ``2 * (4 B H L^2 D + 5 B H L^2)``, halved when causal (lines 49-83).
@@ -195,6 +196,54 @@ def summary_statistics(rows) -> dict:
             "max_grad_error": max((max(r["dq"], r["dk"], r["dv"]) for r in rows), default=0.0)}
 
 
+def plot_report(rows, dtype: str, out_dir: str, masks: bool = True):
+    """The reference's two figures (its test file, lines 977-1091) from the rows of ``run``: for every
+    (causal, mask) configuration one panel with the speed-up over math SDPA per sequence length, and one with the
+    peak memory of one call of either method.  Returns the two file names (named as the reference names them)."""
+    import os
+
+    import matplotlib
+
+    matplotlib.use("Agg")  # files only: no display on a GPU box
+    import matplotlib.pyplot as plt
+
+    panels = {}
+    for r in rows:
+        panels.setdefault((r["causal"], r["mask"]), []).append(r)
+    os.makedirs(out_dir, exist_ok=True)
+    suffix = "_with_masks" if masks else ""
+    paths = [os.path.join(out_dir, f"{dtype}_jvp_attention_{what}{suffix}.png") for what in ("perf", "mem")]
+    n = max(len(panels), 1)
+    fig_p, ax_p = plt.subplots(1, n, figsize=(6 * n, 5), squeeze=False)
+    fig_m, ax_m = plt.subplots(1, n, figsize=(6 * n, 5), squeeze=False)
+    fig_p.suptitle("Speed-up of the fused dual forward over math SDPA under forward-mode AD")
+    fig_m.suptitle("Peak memory of one call")
+    for col, ((causal, mask), rs) in enumerate(sorted(panels.items(), key=lambda kv: (kv[0][0], kv[0][1]))):
+        rs = sorted(rs, key=lambda r: r["L"])
+        xs = list(range(len(rs)))
+        labels = [str(r["L"]) for r in rs]
+        title = f"causal={causal}, mask={mask}"
+        a = ax_p[0, col]
+        bars = a.bar(xs, [r["speedup"] for r in rs], width=0.5, color="tab:green")
+        a.bar_label(bars, labels=[f"{r['speedup']:.1f}x" for r in rs])
+        a.axhline(1.0, color="grey", linestyle="--")
+        a.set(title=title, xlabel="sequence length", ylabel="math SDPA time / JVP attention time", xticks=xs, xticklabels=labels)
+        b = ax_m[0, col]
+        w = 0.38
+        b1 = b.bar([x - w / 2 for x in xs], [r["mem_mb_sdpa"] for r in rs], w, label="math SDPA")
+        b2 = b.bar([x + w / 2 for x in xs], [r["mem_mb"] for r in rs], w, label="JVP attention")
+        b.bar_label(b1, fmt="%.0f", padding=2)
+        b.bar_label(b2, fmt="%.0f", padding=2)
+        b.set(title=title, xlabel="sequence length", ylabel="peak allocated memory (MB)", xticks=xs, xticklabels=labels)
+        b.set_yscale("log")
+        b.legend()
+    for fig, path in ((fig_p, paths[0]), (fig_m, paths[1])):
+        fig.tight_layout(rect=[0, 0.02, 1, 0.95])
+        fig.savefig(path, dpi=120)
+        plt.close(fig)
+    return paths
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--dtype", default="bfloat16", choices=list(DTYPES))
@@ -205,7 +254,12 @@ def main():
     ap.add_argument("--no-masks", action="store_true")
     ap.add_argument("--no-timing", action="store_true", help="one call per case instead of 10 + 100: accuracy only")
     ap.add_argument("--json", default=None)
-    run(ap.parse_args())
+    ap.add_argument("--plots", default=None, metavar="DIR", help="draw the speed-up and memory figures into DIR (needs matplotlib)")
+    args = ap.parse_args()
+    rows = run(args)
+    if args.plots:
+        for path in plot_report(rows, args.dtype, args.plots, not args.no_masks):
+            print("wrote", path)
 
 
 if __name__ == "__main__":

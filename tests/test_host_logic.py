@@ -359,3 +359,21 @@ def test_bench_measures_one_gpu_and_says_so():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "one GPU" in (r.stdout + r.stderr)
+
+
+def test_validation_report_figures_from_synthetic_rows(tmp_path):
+    """``validate.plot_report`` (the reference's two PNG figures): one panel per (causal, mask) configuration,
+    files named as the reference names them; drawn here from made-up rows, no GPU involved."""
+    pytest.importorskip("matplotlib")
+    from jvp_flash_attention_amd import validate
+
+    rows = [{"L": L, "mask": mask, "causal": causal, "speedup": 3.0 + L / 512, "mem_mb": 1.0 + L / 64,
+             "mem_mb_sdpa": 2.0 + (L / 64) ** 2}
+            for L in (128, 512, 2048) for mask, causal in (("none", False), ("none", True), ("boolean", False), ("additive", False))]
+    paths = validate.plot_report(rows, "bfloat16", str(tmp_path), masks=True)
+    assert [p.split("/")[-1] for p in paths] == ["bfloat16_jvp_attention_perf_with_masks.png", "bfloat16_jvp_attention_mem_with_masks.png"]
+    for p in paths:
+        with open(p, "rb") as f:
+            head = f.read(8)
+        assert head == b"\x89PNG\r\n\x1a\n"
+    assert validate.plot_report(rows[:3], "float32", str(tmp_path), masks=False)[0].endswith("float32_jvp_attention_perf.png")
