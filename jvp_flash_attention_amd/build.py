@@ -80,8 +80,16 @@ def build(jobs: int | None = None, verbose: bool = True, extra_flags=(), lib: st
     os.makedirs(objdir, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
     us = [(*u, objdir, list(extra_flags)) for u in units()]
+
+    # the units that take longest (the 16-bit backward kernels, most template variants) start first, so that the
+    # build ends with short ones filling the remaining cores; the link order stays that of units()
+    def cost(u):
+        name = u[0]
+        return -(4 * name.startswith("bwd_") + 2 * ("fp32" not in name) + ("256" not in name))
+
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(_compile, us))
+        done = dict(zip((u[0] for u in sorted(us, key=cost)), ex.map(_compile, sorted(us, key=cost))))
+    objs = [done[u[0]] for u in us]
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", lib]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
