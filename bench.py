@@ -27,9 +27,9 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
 Z, H, L, D = 4, 16, 4096, 128
 
 # HBM bytes per forward launch.  A recorded constant, not measured in this run: rocprofv3 --pmc
-# FETCH_SIZE (x2.0, the factor a plain copy of known size gives) and WRITE_SIZE (x1.0) read 404.6 MB +
+# FETCH_SIZE (x2.0, the factor a plain copy of known size gives) and WRITE_SIZE (x1.0) read 405.4 MB +
 # 136.3 MB; the counter runs and their commands are in profiles/fwd3_kernel_bf16_B4_H16_L4096_D128.md.
-MEASURED_FWD_TRAFFIC_BYTES = 540.9e6
+MEASURED_FWD_TRAFFIC_BYTES = 541.7e6
 TRAFFIC_SOURCE = "recorded from the rocprofv3 --pmc runs in profiles/fwd3_kernel_bf16_B4_H16_L4096_D128.md, not measured in this run"
 
 
