@@ -1,4 +1,4 @@
-// Backward kernels for 16-bit element types (bf16 / fp16), D in {64, 128}, on the forward's memory
+// Backward kernels for 16-bit element types (bf16 / fp16), D in {32, 64, 128}, on the forward's memory
 // pipeline: 64-row tiles of the streamed tensors go global -> LDS with direct-to-LDS loads, double
 // buffered and issued one instruction at a time between the matrix products of the current tile;
 // tiles stay row-major (XOR-swizzled 16-byte chunks) and are read both ways from that one copy:

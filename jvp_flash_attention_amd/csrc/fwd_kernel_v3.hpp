@@ -1,5 +1,5 @@
-// Software-pipelined fused dual forward for 16-bit element types, D in {64, 128}: causal, boolean and
-// additive masks (with the key limit and the tile lists), ragged sequence ends, dropout.  Same tiles,
+// Software-pipelined fused dual forward for 16-bit element types at D = 128 (and the forward without tangents
+// at D = 256): causal, boolean and additive masks (with the key limit and the tile lists), ragged sequence ends, dropout.  Same tiles,
 // swizzles, fragment layouts and mathematics as fwd_kernel_v2.hpp; what changes is the order of work
 // inside a wave.
 //
